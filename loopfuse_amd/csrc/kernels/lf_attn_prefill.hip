@@ -1,0 +1,311 @@
+// lf_attn_prefill.hip — fused attention forward for gfx950 (prefill shapes).
+//
+// One workgroup = LF_NW waves x 32 query rows; it walks the KV sequence in
+// tiles of LF_BN rows that are staged (double-buffered, XOR-swizzled) in LDS.
+// Per KV tile each wave computes, entirely in registers,
+//     S^T = K Q^T          (v_mfma_f32_32x32x16, K fragment from LDS, Q in VGPRs)
+//     score mods + mask    (scale / softcap / causal / window / bounds)
+//     online softmax       (lane-local over the 16*LF_BN/32 scores a lane owns,
+//                           one exchange with lane^32)
+//     O^T += V^T P^T       (V fragment read transposed from LDS)
+// Working on the transposed problem makes the accumulator layout of S^T equal to
+// the B-operand layout of the second product, so P never leaves registers, and
+// makes every per-query quantity (running max, sum, rescale factor) a per-lane
+// scalar.  This is the loop nest the reference's optimiser derives for attention
+// (loopfuse/compiler/passes/factor_acc.py:23-109 for the rescaled accumulation,
+// loopfuse/compiler/passes/skip_loop_iterations.py:343-376 for the tile bounds)
+// and hands to its Triton emitter (loopfuse/codegen.py:699-712).
+//
+// Extra compile-time switches:
+//   LF_V_TR   1: read V fragments with ds_read_b64_tr_b16; 0: scalar LDS reads
+
+#ifndef LF_V_TR
+#define LF_V_TR 1
+#endif
+
+#define LF_BM 128
+#define LF_BN 64
+#define LF_NW 4
+#define LF_NT (LF_NW * 64)
+#define LF_D LF_HEAD_DIM
+#define LF_CPR (LF_D / 8)                    /* 16-byte chunks per K/V row    */
+#define LF_RPS (256 / (LF_D * 2))            /* rows per 256-byte bank span   */
+#define LF_NPASS (LF_BN * LF_CPR / LF_NT)    /* staging passes per tile       */
+#define LF_NKB (LF_BN / 32)                  /* 32-row blocks of S^T per tile */
+#define LF_NKS (LF_D / 16)                   /* k-steps of the QK^T product   */
+#define LF_NDB (LF_D / 32)                   /* 32-row blocks of O^T          */
+#define LF_NKK (LF_BN / 16)                  /* k-steps of the PV product     */
+
+// Physical 16-byte chunk of logical chunk `ch` in row `row` of the K tile: rows
+// that a ds_read_b128 touches together (16 consecutive rows, same logical chunk)
+// land in 16 different chunks, i.e. on all 64 banks.
+__device__ __forceinline__ int lf_k_phys(int row, int ch) {
+  return ch ^ ((row / LF_RPS) & (LF_CPR - 1));
+}
+// Same for the V tile, where a transposed read touches 4 consecutive rows x 64
+// contiguous bytes per 32 lanes: permute the 64-byte groups by the row.
+__device__ __forceinline__ int lf_v_phys(int row, int ch) {
+  return ch ^ (4 * ((row / LF_RPS) & (LF_CPR / 4 - 1)));
+}
+
+extern "C" __global__ void __launch_bounds__(LF_NT, 2) lf_attn_prefill(const LfAttnParams p) {
+  __shared__ __attribute__((aligned(16))) lf_elem lds_k[2][LF_BN * LF_D];
+  __shared__ __attribute__((aligned(16))) lf_elem lds_v[2][LF_BN * LF_D];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int l32 = lane & 31;
+  const int g = lane >> 5;
+
+  // ---- workgroup -> (batch*head, q tile).  Workgroup ids are dealt round-robin
+  // to the 8 XCDs, so ids with equal id%8 share an L2: keep all q tiles of one
+  // (batch, head) on one XCD, heaviest (latest) q tile first.
+  const int nqt = (p.Sq + LF_BM - 1) / LF_BM;
+  const int nbh = p.B * p.Hq;
+  const int xcd = blockIdx.x & 7;
+  const int slot = blockIdx.x >> 3;
+  const int bh = (slot / nqt) * 8 + xcd;
+  if (bh >= nbh) return;
+  const int qt = nqt - 1 - (slot % nqt);
+  const int b = bh / p.Hq;
+  const int h = bh % p.Hq;
+  const int hkv = h / (p.Hq / p.Hkv);
+  const int q0 = qt * LF_BM;
+  const int qlast = min(q0 + LF_BM, p.Sq) - 1;
+  const int nkt = (p.Sk + LF_BN - 1) / LF_BN;
+
+  // ---- block skip: KV tiles [kt_begin, kt_end) are those with at least one
+  // unmasked (i, j) for rows q0..qlast.
+  int kt_begin = 0, kt_end = nkt;
+#if LF_MASK >= 1
+  kt_end = min(nkt, qlast / LF_BN + 1);
+#endif
+#if LF_MASK == 2
+  {
+    int lo = q0 - p.window + 1;
+    if (lo > 0) kt_begin = lo / LF_BN;
+  }
+#endif
+  if (p.visits != nullptr && tid == 0) {
+    for (int kt = kt_begin; kt < kt_end; ++kt)
+      p.visits[((long long)bh * nqt + qt) * nkt + kt] = 1;
+  }
+
+  // ---- this wave's rows
+  const int wq0 = q0 + 32 * wave;
+  const int wqlast = min(wq0 + 31, p.Sq - 1);
+  const bool wave_has_rows = wq0 < p.Sq;
+  const int my_q = wq0 + l32;
+
+  // Q^T fragments (B operand): lane holds row my_q, d = 16*ks + 8*g .. +7.
+  lf_elem8 qf[LF_NKS];
+  {
+    const lf_elem* qrow = p.q + (long long)b * p.q_sb + (long long)h * p.q_sh + (long long)my_q * p.q_ss;
+#pragma unroll
+    for (int ks = 0; ks < LF_NKS; ++ks) {
+      lf_u32x4 raw = {0u, 0u, 0u, 0u};
+      if (my_q < p.Sq) raw = *reinterpret_cast<const lf_u32x4*>(qrow + 16 * ks + 8 * g);
+      qf[ks] = __builtin_bit_cast(lf_elem8, raw);
+    }
+  }
+
+#if LF_SOFTCAP
+  const float sc_in = p.scale / p.softcap;   // tanh argument multiplier
+  const float cexp = LF_LOG2E;               // scores are final before exp
+#else
+  const float cexp = p.scale * LF_LOG2E;     // scale folded into the exponent
+#endif
+
+  lf_f32x16 o[LF_NDB];
+#pragma unroll
+  for (int db = 0; db < LF_NDB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[db][i] = 0.0f;
+  float m_run = LF_NEG_INF;   // running max of the (modified) scores, per query
+  float l_run = 0.0f;         // this lane's share of the running sum
+
+  // ---- staging: thread handles chunk (srow, sch) of every pass
+  lf_u32x4 kst[LF_NPASS], vst[LF_NPASS];
+  auto load_tile = [&](int kt) {
+#pragma unroll
+    for (int ps = 0; ps < LF_NPASS; ++ps) {
+      int idx = tid + LF_NT * ps;
+      int row = idx / LF_CPR;
+      int ch = idx % LF_CPR;
+      int tok = kt * LF_BN + row;
+      lf_u32x4 kz = {0u, 0u, 0u, 0u}, vz = {0u, 0u, 0u, 0u};
+      if (tok < p.Sk) {
+        kz = *reinterpret_cast<const lf_u32x4*>(lf_kv_row(p, 0, b, hkv, tok) + 8 * ch);
+        vz = *reinterpret_cast<const lf_u32x4*>(lf_kv_row(p, 1, b, hkv, tok) + 8 * ch);
+      }
+      kst[ps] = kz;
+      vst[ps] = vz;
+    }
+  };
+  auto store_tile = [&](int buf) {
+#pragma unroll
+    for (int ps = 0; ps < LF_NPASS; ++ps) {
+      int idx = tid + LF_NT * ps;
+      int row = idx / LF_CPR;
+      int ch = idx % LF_CPR;
+      *reinterpret_cast<lf_u32x4*>(&lds_k[buf][row * LF_D + 8 * lf_k_phys(row, ch)]) = kst[ps];
+      *reinterpret_cast<lf_u32x4*>(&lds_v[buf][row * LF_D + 8 * lf_v_phys(row, ch)]) = vst[ps];
+    }
+  };
+
+  if (kt_begin < kt_end) {
+    load_tile(kt_begin);
+    store_tile(0);
+  }
+  __syncthreads();
+
+  for (int kt = kt_begin; kt < kt_end; ++kt) {
+    const int cur = (kt - kt_begin) & 1;
+    const bool have_next = kt + 1 < kt_end;
+    if (have_next) load_tile(kt + 1);
+
+    const int k0 = kt * LF_BN;
+    bool need = wave_has_rows;
+    bool full = (k0 + LF_BN <= p.Sk);
+#if LF_MASK >= 1
+    need = need && (k0 <= wqlast);
+    full = full && (k0 + LF_BN - 1 <= wq0);
+#endif
+#if LF_MASK == 2
+    need = need && (min(k0 + LF_BN, p.Sk) - 1 >= wq0 - p.window + 1);
+    full = full && (wq0 + 31 - k0 < p.window);
+#endif
+
+    if (need) {
+      const lf_elem* kbuf = lds_k[cur];
+      const lf_elem* vbuf = lds_v[cur];
+
+      // ---- S^T = K Q^T
+      lf_f32x16 s[LF_NKB];
+#pragma unroll
+      for (int kb = 0; kb < LF_NKB; ++kb) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[kb][i] = 0.0f;
+        const int row = 32 * kb + l32;
+#pragma unroll
+        for (int ks = 0; ks < LF_NKS; ++ks) {
+          lf_u32x4 raw = *reinterpret_cast<const lf_u32x4*>(&kbuf[row * LF_D + 8 * lf_k_phys(row, 2 * ks + g)]);
+          s[kb] = lf_mfma32(__builtin_bit_cast(lf_elem8, raw), qf[ks], s[kb]);
+        }
+      }
+
+      // ---- score modifications and mask; element i of block kb is kv index
+      // j = k0 + 32*kb + 8*(i/4) + 4*g + i%4, query my_q.
+#if LF_SOFTCAP
+#pragma unroll
+      for (int kb = 0; kb < LF_NKB; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[kb][i] = p.softcap * lf_tanh(s[kb][i] * sc_in);
+#endif
+      if (!full) {
+#pragma unroll
+        for (int kb = 0; kb < LF_NKB; ++kb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            int j = k0 + 32 * kb + 8 * (i / 4) + 4 * g + (i % 4);
+            bool ok = j < p.Sk;
+#if LF_MASK >= 1
+            ok = ok && (j <= my_q);
+#endif
+#if LF_MASK == 2
+            ok = ok && (my_q - j < p.window);
+#endif
+            s[kb][i] = ok ? s[kb][i] : LF_NEG_INF;
+          }
+      }
+
+      // ---- online softmax (per query = per lane pair l, l^32)
+      float mx = LF_NEG_INF;
+#pragma unroll
+      for (int kb = 0; kb < LF_NKB; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kb][i]);
+      mx = fmaxf(mx, lf_swap32(mx));
+      const float m_new = fmaxf(m_run, mx);
+      const float m_sub = (m_new == LF_NEG_INF) ? 0.0f : m_new;
+      const float mc = m_sub * cexp;
+      const float r = lf_exp2(m_run * cexp - mc);
+      m_run = m_new;
+
+      float rs = 0.0f;
+      lf_elem8 pf[LF_NKK];
+#pragma unroll
+      for (int kb = 0; kb < LF_NKB; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          float e = lf_exp2(s[kb][i] * cexp - mc);
+          rs += e;
+          pf[2 * kb + i / 8][i % 8] = lf_from_float(e);
+        }
+      l_run = l_run * r + rs;
+#pragma unroll
+      for (int db = 0; db < LF_NDB; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[db][i] *= r;
+
+      // ---- O^T += V^T P^T.  k-slot s of step kk is kv row
+      // 16*kk + 8*(s/4) + 4*g + s%4 (the order P is held in); A row = d.
+#pragma unroll
+      for (int kk = 0; kk < LF_NKK; ++kk) {
+#pragma unroll
+        for (int db = 0; db < LF_NDB; ++db) {
+          lf_elem8 a;
+#if LF_V_TR
+          // 16-lane group (2g + dh) asks for rows r0..r0+3, columns 32db+16dh..+15:
+          // lane j of the group supplies the 8-byte piece (row r0 + j/4, cols +4*(j%4))
+          // and receives column j of the 4 rows.
+          const int j16 = lane & 15;
+          const int dh = (lane >> 4) & 1;
+          const int col = 32 * db + 16 * dh + 4 * (j16 & 3);
+#pragma unroll
+          for (int half = 0; half < 2; ++half) {
+            const int row = 16 * kk + 8 * half + 4 * g + (j16 >> 2);
+            const lf_elem* src = &vbuf[row * LF_D + 8 * lf_v_phys(row, col / 8) + (col % 8)];
+            lf_s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (__attribute__((address_space(3))) lf_s16x4*)(src));
+            lf_elem4 te = __builtin_bit_cast(lf_elem4, t);
+            a[4 * half + 0] = te[0];
+            a[4 * half + 1] = te[1];
+            a[4 * half + 2] = te[2];
+            a[4 * half + 3] = te[3];
+          }
+#else
+          const int col = 32 * db + l32;
+#pragma unroll
+          for (int sl = 0; sl < 8; ++sl) {
+            const int row = 16 * kk + 8 * (sl / 4) + 4 * g + (sl % 4);
+            a[sl] = vbuf[row * LF_D + 8 * lf_v_phys(row, col / 8) + (col % 8)];
+          }
+#endif
+          o[db] = lf_mfma32(a, pf[kk], o[db]);
+        }
+      }
+    }
+
+    if (have_next) store_tile(cur ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: O[q][d] = O^T[d][q] / l.  Element i of block db is
+  // d = 32*db + 8*(i/4) + 4*g + i%4.
+  if (my_q < p.Sq) {
+    const float l_tot = l_run + lf_swap32(l_run);
+    const float inv = 1.0f / l_tot;
+    lf_elem* orow = p.o + (long long)b * p.o_sb + (long long)h * p.o_sh + (long long)my_q * p.o_ss;
+#pragma unroll
+    for (int db = 0; db < LF_NDB; ++db)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        lf_elem4 w;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[e] = lf_from_float(o[db][4 * i4 + e] * inv);
+        *reinterpret_cast<lf_elem4*>(orow + 32 * db + 8 * i4 + 4 * g) = w;
+      }
+  }
+}

@@ -1,0 +1,148 @@
+// lf_common.hip.h — shared device-side building blocks for the gfx950 attention
+// kernels: element/vector types, the kernel parameter block, MFMA wrappers,
+// cross-half-wave exchange, fast exp2/tanh and K/V row addressing (contiguous or
+// gathered through a page table).
+//
+// Compile-time specialisation (passed as -D options by the host lowering):
+//   LF_DTYPE      0 = bf16, 1 = fp16 storage (accumulation is always fp32)
+//   LF_HEAD_DIM   64 or 128
+//   LF_MASK       0 = none, 1 = causal (j <= i), 2 = causal sliding window
+//                 (j <= i and i - j < window); top-left aligned as in the
+//                 reference (loopfuse/torch_backend/ops.py:675-751)
+//   LF_SOFTCAP    1: s <- cap * tanh(s * scale / cap) before the mask
+//   LF_PAGED      bit 0: K rows, bit 1: V rows are gathered through a page table
+//   LF_TABLE_I64  1: page tables hold int64 ids (else int32)
+//   LF_PAGE_SIZE  tokens per page (power of two) when LF_PAGED
+#ifndef LF_COMMON_HIP_H
+#define LF_COMMON_HIP_H
+
+#ifndef __HIPCC_RTC__
+#include <hip/hip_runtime.h>
+#endif
+
+#ifndef LF_DTYPE
+#define LF_DTYPE 0
+#endif
+#ifndef LF_HEAD_DIM
+#define LF_HEAD_DIM 128
+#endif
+#ifndef LF_MASK
+#define LF_MASK 0
+#endif
+#ifndef LF_SOFTCAP
+#define LF_SOFTCAP 0
+#endif
+#ifndef LF_PAGED
+#define LF_PAGED 0
+#endif
+#ifndef LF_PAGE_SIZE
+#define LF_PAGE_SIZE 16
+#endif
+#ifndef LF_TABLE_I64
+#define LF_TABLE_I64 0
+#endif
+
+#if LF_DTYPE == 0
+typedef __bf16 lf_elem;
+#else
+typedef _Float16 lf_elem;
+#endif
+
+typedef lf_elem lf_elem8 __attribute__((ext_vector_type(8)));
+typedef lf_elem lf_elem4 __attribute__((ext_vector_type(4)));
+typedef lf_elem lf_elem2 __attribute__((ext_vector_type(2)));
+typedef short lf_s16x4 __attribute__((ext_vector_type(4)));
+typedef float lf_f32x2 __attribute__((ext_vector_type(2)));
+typedef float lf_f32x4 __attribute__((ext_vector_type(4)));
+typedef float lf_f32x16 __attribute__((ext_vector_type(16)));
+typedef unsigned int lf_u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int lf_u32x2 __attribute__((ext_vector_type(2)));
+
+#if LF_TABLE_I64
+typedef long long lf_table_t;
+#else
+typedef int lf_table_t;
+#endif
+
+#define LF_NEG_INF (-__builtin_inff())
+#define LF_LOG2E 1.4426950408889634f
+
+// Kernel parameter block.  Mirrors loopfuse_amd/lowering.py::AttnParams field
+// for field (pointers, then 64-bit element strides, then 32-bit scalars).
+struct LfAttnParams {
+  const lf_elem* q;
+  const lf_elem* k;          // contiguous K, or the K page pool when LF_PAGED
+  const lf_elem* v;
+  lf_elem* o;
+  const void* k_table;       // [B, pages_per_seq] page ids (lf_table_t) when paged
+  const void* v_table;
+  float* part_acc;           // split-K scratch: [units, nsplit, rows, D]
+  float* part_ml;            // split-K scratch: [units, nsplit, rows, 2] (max, sum)
+  unsigned char* visits;     // optional [B*Hq*nqt, nkt] visited-tile record
+  long long q_sb, q_sh, q_ss;  // element strides of Q [B, Hq, Sq, D] (d stride 1)
+  long long k_sb, k_sh, k_ss;  // K [B, Hkv, Sk, D]; paged: k_sb = page stride,
+                               // k_ss = stride between tokens inside a page
+  long long v_sb, v_sh, v_ss;
+  long long o_sb, o_sh, o_ss;
+  int B, Hq, Hkv, Sq, Sk;
+  int window;                // sliding-window width (LF_MASK == 2)
+  int kt_stride, vt_stride;  // row strides (elements) of k_table / v_table
+  int nsplit;                // decode: number of KV splits across workgroups
+  int rows;                  // decode: query rows per (batch, kv head) unit
+  int split_len;             // decode: tokens per split (multiple of 16)
+  float scale;               // multiplies QK^T (D^-0.5 in the reference graphs)
+  float softcap;             // cap of cap*tanh(s/cap) (LF_SOFTCAP)
+};
+
+__device__ __forceinline__ lf_f32x16 lf_mfma32(lf_elem8 a, lf_elem8 b, lf_f32x16 c) {
+#if LF_DTYPE == 0
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+#else
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+#endif
+}
+
+__device__ __forceinline__ lf_f32x4 lf_mfma16(lf_elem8 a, lf_elem8 b, lf_f32x4 c) {
+#if LF_DTYPE == 0
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+#else
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+#endif
+}
+
+// Value held by the lane 32 positions away (lane l <-> lane l ^ 32).
+__device__ __forceinline__ float lf_swap32(float x) {
+  return __shfl_xor(x, 32, 64);
+}
+
+__device__ __forceinline__ float lf_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// tanh(x) = 1 - 2 / (2^(2 x log2 e) + 1); exact limits at +-inf.
+__device__ __forceinline__ float lf_tanh(float x) {
+  float e = lf_exp2(x * (2.0f * LF_LOG2E));
+  return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+}
+
+__device__ __forceinline__ lf_elem lf_from_float(float x) { return (lf_elem)x; }
+__device__ __forceinline__ float lf_to_float(lf_elem x) { return (float)x; }
+
+// Pointer to element 0 of row `tok` of K (which = 0) or V (which = 1) for batch
+// b and kv head h.  With LF_PAGED the row lives in page table[b][tok / P] of the
+// pool, at token slot tok % P (reference semantics: out[*s,*t] =
+// buffer[block_table[*s],*t], loopfuse/torch_backend/__init__.py:46-56).
+__device__ __forceinline__ const lf_elem* lf_kv_row(const LfAttnParams& p, int which, int b, int h,
+                                                   int tok) {
+  const lf_elem* base = which ? p.v : p.k;
+  const long long sb = which ? p.v_sb : p.k_sb;
+  const long long sh = which ? p.v_sh : p.k_sh;
+  const long long ss = which ? p.v_ss : p.k_ss;
+  const bool paged = which ? ((LF_PAGED & 2) != 0) : ((LF_PAGED & 1) != 0);
+  if (paged) {
+    const lf_table_t* table = reinterpret_cast<const lf_table_t*>(which ? p.v_table : p.k_table);
+    const long long page = table[(long long)b * (which ? p.vt_stride : p.kt_stride) + (tok / LF_PAGE_SIZE)];
+    return base + page * sb + (long long)(tok % LF_PAGE_SIZE) * ss + (long long)h * sh;
+  }
+  return base + (long long)b * sb + (long long)h * sh + (long long)tok * ss;
+}
+
+#endif  // LF_COMMON_HIP_H

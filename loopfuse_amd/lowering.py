@@ -1,0 +1,351 @@
+"""Lowering: attention plan -> specialised gfx950 HIP kernel -> launcher.
+
+This module is the counterpart of the reference's Triton emitter
+(``loopfuse/codegen.py:100-126`` ``codegen_program`` and the generated
+``launch_kernel_0``, ``codegen.py:215-298``).  Instead of printing a kernel per
+graph it selects hand-written building blocks from ``csrc/kernels`` and
+specialises them with ``-D`` options (dtype, head dim, mask kind, softcap,
+paging, rows per unit); hipRTC compiles the result once per specialisation and
+the code object is cached on disk.
+
+Everything dynamic (batch, heads, sequence lengths, strides, scale, window,
+softcap value) is a run-time kernel parameter, so a new sequence length does not
+recompile (the reference makes every dimension a ``tl.constexpr``,
+``codegen.py:394-396``).
+"""
+from __future__ import annotations
+
+import ctypes
+import dataclasses
+import math
+import os
+import threading
+from typing import Optional
+
+import torch
+
+from . import runtime
+from .skip import PREFILL_BM, PREFILL_BN
+
+MASK_NONE, MASK_CAUSAL, MASK_SLIDING = 0, 1, 2
+_MASK_NAMES = {"none": MASK_NONE, None: MASK_NONE, "causal": MASK_CAUSAL, "sliding": MASK_SLIDING}
+_DTYPE_CODE = {torch.bfloat16: 0, torch.float16: 1}
+
+# hipcc/hipRTC flags common to every kernel.  Packed-FP32 instruction selection
+# (v_pk_*_f32) is switched off on purpose: scalar fp32 VALU code only.
+COMMON_OPTS = ("-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops")
+
+
+class AttnParams(ctypes.Structure):
+    """Mirror of ``struct LfAttnParams`` in csrc/kernels/lf_common.hip.h."""
+
+    _fields_ = (
+        [(n, ctypes.c_void_p) for n in ("q", "k", "v", "o", "k_table", "v_table", "part_acc", "part_ml", "visits")]
+        + [(n, ctypes.c_longlong) for n in (
+            "q_sb", "q_sh", "q_ss", "k_sb", "k_sh", "k_ss", "v_sb", "v_sh", "v_ss", "o_sb", "o_sh", "o_ss")]
+        + [(n, ctypes.c_int) for n in (
+            "B", "Hq", "Hkv", "Sq", "Sk", "window", "kt_stride", "vt_stride", "nsplit", "rows", "split_len")]
+        + [("scale", ctypes.c_float), ("softcap", ctypes.c_float)]
+    )
+
+
+@dataclasses.dataclass(frozen=True)
+class KernelSpec:
+    """Compile-time specialisation of one kernel family (= one code object)."""
+
+    family: str            # "prefill" | "decode"
+    dtype: int             # 0 bf16, 1 fp16
+    head_dim: int          # 64 | 128
+    mask: int = MASK_NONE
+    softcap: bool = False
+    paged: int = 0         # bit 0: K paged, bit 1: V paged
+    page_size: int = 1
+    table_i64: bool = False
+    rows: int = 1          # decode: query rows sharing K/V (1, 2, 4)
+    waves: int = 4         # decode: waves per workgroup
+    v_tr: bool = True      # prefill: transposed LDS reads for V
+
+    def options(self) -> list[str]:
+        o = list(COMMON_OPTS) + [
+            f"-DLF_DTYPE={self.dtype}",
+            f"-DLF_HEAD_DIM={self.head_dim}",
+            f"-DLF_MASK={self.mask}",
+            f"-DLF_SOFTCAP={int(self.softcap)}",
+            f"-DLF_PAGED={self.paged}",
+            f"-DLF_PAGE_SIZE={self.page_size}",
+            f"-DLF_TABLE_I64={int(self.table_i64)}",
+        ]
+        if self.family == "decode":
+            o += [f"-DLF_ROWS={self.rows}", f"-DLF_DW={self.waves}"]
+        else:
+            o += [f"-DLF_V_TR={int(self.v_tr)}"]
+        return o
+
+    def files(self) -> tuple[str, ...]:
+        return ("lf_common.hip.h", "lf_attn_prefill.hip" if self.family == "prefill" else "lf_attn_decode.hip")
+
+    def name(self) -> str:
+        return (f"lf_{self.family}_t{self.dtype}_d{self.head_dim}_m{self.mask}_c{int(self.softcap)}"
+                f"_p{self.paged}x{self.page_size}i{int(self.table_i64)}_r{self.rows}w{self.waves}v{int(self.v_tr)}")
+
+    def source(self) -> str:
+        return runtime.read_kernel_source(*self.files())
+
+
+@dataclasses.dataclass
+class CompiledKernel:
+    """What ``CODEGEN_ONLY`` returns in place of a runnable function (the
+    reference returns ``KernelData(kernel_name, launch_name, code)``,
+    ``loopfuse/codegen.py:66-71``)."""
+
+    spec: KernelSpec
+    code_object: bytes
+    cache_hit: bool
+    log: str
+
+    @property
+    def code(self) -> str:
+        return "// options: " + " ".join(self.spec.options()) + "\n" + self.spec.source()
+
+
+_compiled: dict[KernelSpec, CompiledKernel] = {}
+_loaded: dict[tuple[KernelSpec, int], runtime.Module] = {}
+_lock = threading.Lock()
+
+
+def compile_spec(spec: KernelSpec, arch: str = runtime.DEFAULT_ARCH) -> CompiledKernel:
+    """hipRTC-compile (or fetch from the on-disk cache) one specialisation.  Needs no GPU."""
+    with _lock:
+        ck = _compiled.get(spec)
+        if ck is None:
+            code, hit, log = runtime.compile_source(spec.source(), spec.name(), spec.options(), arch)
+            ck = CompiledKernel(spec, code, hit, log)
+            _compiled[spec] = ck
+        return ck
+
+
+def load_spec(spec: KernelSpec) -> runtime.Module:
+    dev = torch.cuda.current_device()
+    key = (spec, dev)
+    mod = _loaded.get(key)
+    if mod is None:
+        ck = compile_spec(spec)
+        with _lock:
+            mod = _loaded.get(key)
+            if mod is None:
+                mod = runtime.Module(ck.code_object)
+                _loaded[key] = mod
+    return mod
+
+
+_kernels: dict[tuple[KernelSpec, int, str], runtime.Kernel] = {}
+
+
+def get_kernel(spec: KernelSpec, symbol: str) -> runtime.Kernel:
+    key = (spec, torch.cuda.current_device(), symbol)
+    k = _kernels.get(key)
+    if k is None:
+        k = load_spec(spec).kernel(symbol)
+        _kernels[key] = k
+    return k
+
+
+# ----------------------------------------------------------------------------
+# plan
+# ----------------------------------------------------------------------------
+
+@dataclasses.dataclass
+class AttnPlan:
+    """What the front end extracts from a captured graph: the parameters of
+    ``softmax(mask(mods(Q K^T))) V``.  ``scale`` multiplies the raw scores,
+    ``softcap`` (if set) is applied as cap*tanh(s/cap) after scaling and before
+    the mask, exactly the order of the reference graphs
+    (``tests/benchmark.py:142-147``)."""
+
+    mask: str | None = None            # None | "causal" | "sliding"
+    window: int = 0
+    scale: float = 1.0
+    softcap: float | None = None
+    k_paged: bool = False
+    v_paged: bool = False
+
+
+class UnsupportedPlan(ValueError):
+    """The shapes/dtypes cannot be served by the HIP kernels (caller falls back to eager)."""
+
+
+def _check_tensor(name: str, t: torch.Tensor, dtype: torch.dtype) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"loopfuse_amd: {name} is not on the GPU; the HIP path has no CPU fallback")
+    if t.dtype != dtype:
+        raise UnsupportedPlan(f"{name} has dtype {t.dtype}, expected {dtype}")
+    if t.stride(-1) != 1:
+        raise UnsupportedPlan(f"{name} must have unit stride in its last dimension")
+    if t.data_ptr() % 16:
+        raise UnsupportedPlan(f"{name} is not 16-byte aligned")
+    for n, s in zip(t.shape[:-1], t.stride()[:-1]):
+        if n > 1 and s % 8:
+            raise UnsupportedPlan(f"{name} strides must be multiples of 8 elements (16-byte loads)")
+
+
+_scratch: dict[tuple[int, int], torch.Tensor] = {}
+
+
+def _get_scratch(device: torch.device, nfloats: int) -> torch.Tensor:
+    key = (device.index or 0, 0)
+    t = _scratch.get(key)
+    if t is None or t.numel() < nfloats:
+        t = torch.empty(max(nfloats, 1 << 20), dtype=torch.float32, device=device)
+        _scratch[key] = t
+    return t
+
+
+def decode_split(units: int, Sk: int, cus: int = 256) -> int:
+    """Number of KV splits across workgroups: enough workgroups for ~4 per CU,
+    but at least 256 tokens per split."""
+    env = os.environ.get("LOOPFUSE_DECODE_SPLITS")
+    if env:
+        return max(1, int(env))
+    want = max(1, (4 * cus + units - 1) // units)
+    most = max(1, Sk // 256)
+    return max(1, min(want, most))
+
+
+def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
+              k_table: Optional[torch.Tensor] = None, v_table: Optional[torch.Tensor] = None,
+              *, out: Optional[torch.Tensor] = None, record_visits: bool = False,
+              force_family: str | None = None, num_splits: int | None = None, v_tr: bool = True):
+    """Run fused attention on the GPU.
+
+    q : [B, Hq, Sq, D];  k, v : [B, Hkv, Sk, D], or page pools [N, P, Hkv, D]
+    ([N, Hkv, D] for one-token pages) with ``k_table``/``v_table`` [B, Sk/P].
+    Returns O [B, Hq, Sq, D] (and the visited-tile record if asked).
+    """
+    dtype = q.dtype
+    if dtype not in _DTYPE_CODE:
+        raise UnsupportedPlan(f"dtype {dtype} not supported by the MFMA kernels (bf16/fp16 only)")
+    if q.dim() != 4:
+        raise UnsupportedPlan("Q must be [B, Hq, Sq, D]")
+    B, Hq, Sq, D = q.shape
+    if D not in (64, 128):
+        raise UnsupportedPlan(f"head dim {D} not supported (64, 128)")
+    if not (plan.scale > 0.0) or not math.isfinite(plan.scale):
+        raise UnsupportedPlan("score scale must be positive and finite")
+    _check_tensor("Q", q, dtype)
+    _check_tensor("K", k, dtype)
+    _check_tensor("V", v, dtype)
+
+    P = AttnParams()
+    paged = 0
+    page_size = 1
+    table_i64 = False
+
+    def kv_layout(t: torch.Tensor, table: Optional[torch.Tensor], is_paged: bool, which: str):
+        nonlocal paged, page_size, table_i64
+        if not is_paged:
+            if t.dim() != 4 or t.shape[0] != B or t.shape[3] != D:
+                raise UnsupportedPlan(f"{which} must be [B, Hkv, Sk, D]")
+            return t.shape[1], t.shape[2], t.stride(0), t.stride(1), t.stride(2), None, 0
+        if table is None or table.dim() != 2 or table.shape[0] != B:
+            raise UnsupportedPlan(f"{which} page table must be [B, pages]")
+        if table.dtype not in (torch.int32, torch.int64):
+            raise UnsupportedPlan("page table must be int32 or int64")
+        if not table.is_cuda:
+            raise RuntimeError(f"loopfuse_amd: {which} page table is not on the GPU")
+        if table.stride(1) != 1:
+            table = table.contiguous()
+        if t.dim() == 3:       # [N, Hkv, D], one token per page (the reference's format)
+            ps, hk, sp, st, sh = 1, t.shape[1], t.stride(0), 0, t.stride(1)
+        elif t.dim() == 4:     # [N, P, Hkv, D]
+            ps, hk, sp, st, sh = t.shape[1], t.shape[2], t.stride(0), t.stride(1), t.stride(2)
+        else:
+            raise UnsupportedPlan(f"{which} pool must be [N, Hkv, D] or [N, P, Hkv, D]")
+        if ps & (ps - 1):
+            raise UnsupportedPlan("page size must be a power of two")
+        i64 = table.dtype == torch.int64
+        if paged and (page_size != ps or table_i64 != i64):
+            raise UnsupportedPlan("K and V pools must share page size and table dtype")
+        page_size, table_i64 = ps, i64
+        paged |= 1 if which == "K" else 2
+        return hk, table.shape[1] * ps, sp, sh, st, table, table.stride(0)
+
+    Hkv, Sk, P.k_sb, P.k_sh, P.k_ss, kt, P.kt_stride = kv_layout(k, k_table, plan.k_paged, "K")
+    Hkv2, Sk2, P.v_sb, P.v_sh, P.v_ss, vt, P.vt_stride = kv_layout(v, v_table, plan.v_paged, "V")
+    if Hkv != Hkv2 or Sk != Sk2:
+        raise UnsupportedPlan("K and V disagree on heads or length")
+    if Hq % Hkv:
+        raise UnsupportedPlan("Hq must be a multiple of Hkv")
+    group = Hq // Hkv
+    mask = _MASK_NAMES[plan.mask]
+    if mask == MASK_SLIDING and plan.window < 1:
+        raise UnsupportedPlan("sliding mask needs window >= 1")
+
+    if out is None:
+        out = torch.empty((B, Hq, Sq, D), dtype=dtype, device=q.device)
+    else:
+        _check_tensor("O", out, dtype)
+
+    P.q, P.k, P.v, P.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+    P.k_table = kt.data_ptr() if kt is not None else None
+    P.v_table = vt.data_ptr() if vt is not None else None
+    P.B, P.Hq, P.Hkv, P.Sq, P.Sk = B, Hq, Hkv, Sq, Sk
+    P.window = int(plan.window)
+    P.scale = float(plan.scale)
+    P.softcap = float(plan.softcap) if plan.softcap else 0.0
+    P.nsplit, P.rows, P.split_len = 1, 1, 0
+
+    # ---- family: decode when there is no mask and few query rows share a KV head
+    family = force_family
+    if family is None:
+        few = (Sq == 1 and group <= 16) or (group == 1 and Sq <= 16)
+        family = "decode" if (mask == MASK_NONE and few and Sk >= 16) else "prefill"
+    keep = (q, k, v, out, kt, vt)  # noqa: F841  (tensors stay alive until the launch is queued)
+
+    if family == "prefill":
+        P.q_sb, P.q_sh, P.q_ss = q.stride(0), q.stride(1), q.stride(2)
+        P.o_sb, P.o_sh, P.o_ss = out.stride(0), out.stride(1), out.stride(2)
+        spec = KernelSpec("prefill", _DTYPE_CODE[dtype], D, mask, plan.softcap is not None, paged,
+                          page_size, table_i64, v_tr=v_tr)
+        nqt = (Sq + PREFILL_BM - 1) // PREFILL_BM
+        nkt = (Sk + PREFILL_BN - 1) // PREFILL_BN
+        visits = None
+        if record_visits:
+            visits = torch.zeros((B * Hq * nqt, nkt), dtype=torch.uint8, device=q.device)
+            P.visits = visits.data_ptr()
+        grid = 8 * ((B * Hq + 7) // 8) * nqt
+        get_kernel(spec, "lf_attn_prefill").launch((grid, 1, 1), (256, 1, 1), P)
+        return (out, visits) if record_visits else out
+
+    if family != "decode":
+        raise ValueError(f"unknown kernel family {family!r}")
+    if mask != MASK_NONE:
+        raise UnsupportedPlan("the decode kernel takes no mask")
+    # query rows of one unit: the group's heads (Sq == 1) or the Sq rows (group == 1)
+    if Sq == 1:
+        rows = group
+        P.q_sb, P.q_sh, P.q_ss = q.stride(0), group * q.stride(1), q.stride(1)
+        P.o_sb, P.o_sh, P.o_ss = out.stride(0), group * out.stride(1), out.stride(1)
+    elif group == 1:
+        rows = Sq
+        P.q_sb, P.q_sh, P.q_ss = q.stride(0), q.stride(1), q.stride(2)
+        P.o_sb, P.o_sh, P.o_ss = out.stride(0), out.stride(1), out.stride(2)
+    else:
+        raise UnsupportedPlan("decode needs Sq == 1 or group == 1")
+    krows = 4 if rows >= 3 else rows
+    chunks = (rows + krows - 1) // krows
+    units = B * Hkv * chunks
+    nsplit = num_splits if num_splits else decode_split(units, Sk)
+    split_len = ((Sk + nsplit - 1) // nsplit + 15) // 16 * 16
+    nsplit = (Sk + split_len - 1) // split_len
+    P.rows, P.nsplit, P.split_len = rows, nsplit, split_len
+    spec = KernelSpec("decode", _DTYPE_CODE[dtype], D, MASK_NONE, plan.softcap is not None, paged,
+                      page_size, table_i64, rows=krows, waves=4)
+    if nsplit > 1:
+        nrow = B * Hkv * rows * nsplit
+        scratch = _get_scratch(q.device, nrow * (D + 2))
+        P.part_acc = scratch.data_ptr()
+        P.part_ml = scratch.data_ptr() + 4 * nrow * D
+    get_kernel(spec, "lf_attn_decode").launch((units, nsplit, 1), (64 * spec.waves, 1, 1), P)
+    if nsplit > 1:
+        get_kernel(spec, "lf_attn_decode_combine").launch((B * Hkv * rows, 1, 1), (D, 1, 1), P)
+    return out

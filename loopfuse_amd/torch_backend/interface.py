@@ -1,0 +1,125 @@
+"""``loopfuse_backend`` — the ``torch.compile`` backend — and its graph capture.
+
+Same public surface as the reference (``loopfuse/torch_backend/interface.py:
+77-86, 164-170, 640-644``):
+
+    loopfuse_backend(gm, sample_inputs, mode="max-autotune", **kwargs)
+        -> aot_module_simplified(gm, sample_inputs, fw_compiler=loopfuse_compiler)
+    loopfuse_compiler(gm, sample_inputs, input_names=None, symint_names=None, mode=None)
+        -> callable taking the flat placeholder list (tensors and SymInts as ints)
+
+and the same environment switches ``DEBUG``, ``CODEGEN_ONLY`` and
+``USE_HARDCODE_KERNEL`` (``interface.py:23-29``).
+
+Where the reference parses the ATen graph into per-op loop nests, fuses them and
+prints Triton (``interface.py:387-400``, ``optimize.py:34-60``,
+``codegen.py:100-126``), this front end recognises the fused result directly: it
+abstract-interprets the graph (``capture.py``) and, when the graph is
+``softmax(mask(mods(Q K^T))) V``, produces an ``AttnPlan`` that
+``lowering.attention`` runs on the hand-written HIP kernels.
+
+Graphs that are not of that form, and calls on CPU tensors, run the captured
+graph unchanged (the reference raises ``ValueError``/``NotImplementedError``
+there, ``interface.py:157-161``).  Set ``LOOPFUSE_STRICT=1`` to raise instead;
+``stats`` counts which route each call took so tests can insist on the fused one.
+"""
+from __future__ import annotations
+
+import logging
+import os
+from functools import partial
+from typing import Any, Callable
+
+import torch
+from torch._functorch.aot_autograd import aot_module_simplified
+
+from .. import lowering
+from . import capture
+
+log = logging.getLogger("loopfuse_amd")
+
+DEBUG = os.environ.get("DEBUG", "0") == "1"
+CODEGEN_ONLY = os.environ.get("CODEGEN_ONLY", "0") == "1"
+USE_HARDCODE_KERNEL = os.environ.get("USE_HARDCODE_KERNEL", "0") == "1"
+
+# route taken by compiled callables since import: "fused" = HIP kernel launched,
+# "eager_graph" = graph not recognised, "eager_runtime" = recognised but the call's
+# tensors could not be served (CPU tensors, dtype, alignment ...)
+stats = {"fused": 0, "eager_graph": 0, "eager_runtime": 0, "compiled_graphs": 0, "matched_graphs": 0}
+
+
+def _strict() -> bool:
+    return os.environ.get("LOOPFUSE_STRICT", "0") == "1"
+
+
+def get_input_names(gm: torch.fx.GraphModule) -> list[str]:
+    """Placeholder names in order (reference ``interface.py:49-56``)."""
+    return [n.name for n in gm.graph.nodes if n.op == "placeholder"]
+
+
+def loopfuse_backend(gm: torch.fx.GraphModule, sample_inputs, mode="max-autotune", **kwargs):
+    """``torch.compile`` backend entry point (reference ``interface.py:77-86``).
+
+    ``mode`` is accepted for compatibility: the reference uses it to pick the
+    Triton autotune space; the HIP kernels have fixed tile shapes.
+    """
+    if mode:
+        kwargs["mode"] = mode
+    compiler = partial(loopfuse_compiler, input_names=get_input_names(gm), **kwargs)
+    return aot_module_simplified(gm, sample_inputs, fw_compiler=compiler)
+
+
+def loopfuse_compiler(gm: torch.fx.GraphModule, sample_inputs, input_names: list[str] | None = None,
+                      symint_names: dict[str, str] | None = None, mode: str | None = None) -> Callable:
+    """fw_compiler: ATen graph -> callable over the flat placeholder list."""
+    stats["compiled_graphs"] += 1
+    if DEBUG:
+        print("---- loopfuse_amd: ATen graph ----")
+        print(gm.code)
+    try:
+        match = capture.match_attention(gm)
+    except capture.NoMatch as e:
+        match = None
+        reason = str(e)
+    else:
+        reason = ""
+    if match is None:
+        if _strict():
+            raise NotImplementedError(f"loopfuse_amd: graph is not a fused-attention pattern: {reason}")
+        log.info("graph not recognised (%s); running it unfused", reason)
+        if DEBUG:
+            print(f"---- loopfuse_amd: no match ({reason}); eager graph ----")
+
+        def eager_fn(*args):
+            stats["eager_graph"] += 1
+            return gm(*args)
+
+        return eager_fn
+
+    stats["matched_graphs"] += 1
+    if DEBUG:
+        print("---- loopfuse_amd: matched ----")
+        print(match.describe())
+
+    if CODEGEN_ONLY:
+        # no launch: hand back what would be compiled, as the reference hands back
+        # KernelData under CODEGEN_ONLY (interface.py:615-622)
+        def codegen_fn(*args):
+            specs = match.kernel_specs_for(args)
+            return [lowering.compile_spec(s) for s in specs]
+
+        return codegen_fn
+
+    def optimized_fn(*args):
+        try:
+            out = match.run(args)
+        except lowering.UnsupportedPlan as e:
+            if _strict():
+                raise
+            log.info("fused path not applicable to this call (%s); running the graph unfused", e)
+            stats["eager_runtime"] += 1
+            return gm(*args)
+        stats["fused"] += 1
+        return (out,)
+
+    return optimized_fn

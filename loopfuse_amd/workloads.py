@@ -1,0 +1,108 @@
+"""Seeded synthetic inputs for the five benchmark configurations.
+
+Generated on the CPU generator in fp32 and cast, so a CPU checker and the GPU
+kernel see identical bits whatever the device.  Shapes follow the reference's
+benchmark harness (``tests/benchmark.py:68-76, 207-217, 380-398, 510-520``) with
+the sizes of this repository's BASELINE configs.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Optional
+
+import torch
+
+
+@dataclasses.dataclass
+class Workload:
+    name: str
+    q: torch.Tensor
+    k: torch.Tensor                    # dense [B,Hkv,Sk,D] or page pool [N,P,Hkv,D]
+    v: torch.Tensor
+    mask: Optional[str] = None
+    window: int = 0
+    softcap: Optional[float] = None
+    k_table: Optional[torch.Tensor] = None
+    v_table: Optional[torch.Tensor] = None
+
+    @property
+    def scale(self) -> float:
+        return self.q.shape[-1] ** -0.5
+
+    def to(self, device) -> "Workload":
+        mv = lambda t: None if t is None else t.to(device)
+        return dataclasses.replace(self, q=mv(self.q), k=mv(self.k), v=mv(self.v),
+                                   k_table=mv(self.k_table), v_table=mv(self.v_table))
+
+    # work counts, conventions of the reference's benchmark (tests/benchmark.py:110,
+    # 280-284, 369, 452): Q, O and table traffic are not counted
+    def flops(self) -> int:
+        B, Hq, Sq, D = self.q.shape
+        if self.mask == "sliding":
+            w = self.window
+            return 2 * B * Hq * (2 * Sq * w - w * w) * D
+        if self.mask == "causal":
+            return 2 * B * Hq * Sq * Sq * D
+        Sk = self.kv_len()
+        return 4 * B * Hq * Sq * Sk * D
+
+    def kv_len(self) -> int:
+        if self.k_table is not None:
+            return self.k_table.shape[1] * (self.k.shape[1] if self.k.dim() == 4 else 1)
+        return self.k.shape[2]
+
+    def kv_heads(self) -> int:
+        return self.k.shape[-2] if self.k_table is not None else self.k.shape[1]
+
+    def kv_bytes(self) -> int:
+        B, D = self.q.shape[0], self.q.shape[-1]
+        return 2 * self.k.element_size() * B * self.kv_heads() * self.kv_len() * D
+
+
+def _randn(gen, shape, dtype):
+    return torch.randn(shape, generator=gen, dtype=torch.float32).to(dtype)
+
+
+def make(name: str, seed: int = 0, dtype: torch.dtype = torch.bfloat16, *, B=None, S=None) -> Workload:
+    """name in {"c1","c2","c2_softcap","c3","c4","c5"}; B / S override the size (tests)."""
+    g = torch.Generator().manual_seed(seed)
+    if name == "c1":      # fp32 CPU-runnable case
+        B, S = B or 2, S or 512
+        q, k, v = (_randn(g, (B, 8, S, 64), torch.float32) for _ in range(3))
+        return Workload(name, q, k, v, mask="causal")
+    if name in ("c2", "c2_softcap"):
+        B, S = B or 8, S or 2048
+        q, k, v = (_randn(g, (B, 32, S, 128), dtype) for _ in range(3))
+        return Workload(name, q, k, v, mask="causal", softcap=30.0 if name == "c2_softcap" else None)
+    if name == "c3":
+        B, S = B or 8, S or 2048
+        q = _randn(g, (B, 32, S, 128), dtype)
+        k = _randn(g, (B, 8, S, 128), dtype)
+        v = _randn(g, (B, 8, S, 128), dtype)
+        return Workload(name, q, k, v, mask="sliding", window=256, softcap=30.0)
+    if name == "c4":
+        B, S = B or 64, S or 2048
+        q = _randn(g, (B, 32, 1, 128), dtype)
+        k = _randn(g, (B, 32, S, 128), dtype)
+        v = _randn(g, (B, 32, S, 128), dtype)
+        return Workload(name, q, k, v)
+    if name == "c5":
+        B, S = B or 64, S or 2048
+        P = 16
+        pages = S // P
+        n = B * pages
+        q = _randn(g, (B, 32, 1, 128), dtype)
+        kp = _randn(g, (n, P, 8, 128), dtype)
+        vp = _randn(g, (n, P, 8, 128), dtype)
+        table = torch.randperm(n, generator=g).view(B, pages).to(torch.int32)
+        return Workload(name, q, kp, vp, k_table=table, v_table=table.clone())
+    raise ValueError(name)
+
+
+def run(w: Workload, **kw) -> torch.Tensor:
+    """One pass of the hot path over a workload (tensors must be on the GPU)."""
+    from . import lowering
+
+    plan = lowering.AttnPlan(mask=w.mask, window=w.window, scale=w.scale, softcap=w.softcap,
+                             k_paged=w.k_table is not None, v_paged=w.v_table is not None)
+    return lowering.attention(w.q, w.k, w.v, plan, w.k_table, w.v_table, **kw)

@@ -1,0 +1,190 @@
+"""Front end on the CPU: custom-op semantics, graph capture -> plan, CODEGEN_ONLY-style
+compilation of the matched kernels, and eager fallback for everything else."""
+import pytest
+import torch
+
+import loopfuse_amd  # noqa: F401  (registers torch.ops.loopfuse.*)
+from loopfuse_amd import lowering
+from loopfuse_amd.torch_backend import capture, interface
+from oracle import attention_oracle as O
+from torch._functorch.aot_autograd import aot_module_simplified
+
+
+def test_custom_op_semantics():
+    g = torch.Generator().manual_seed(0)
+    a = torch.randn(2, 3, 6, 6, generator=g)
+    assert torch.equal(torch.ops.loopfuse.causal_mask(a), a.masked_fill(~O.dense_mask("causal", 6, 6), float("-inf")))
+    assert torch.equal(torch.ops.loopfuse.sliding_mask(a, 3),
+                       a.masked_fill(~O.dense_mask("sliding", 6, 6, 3), float("-inf")))
+    run, fin = torch.ops.loopfuse.scan_max(a)
+    assert torch.equal(run, torch.cummax(a, -1).values) and torch.equal(fin, a.max(-1, keepdim=True).values)
+    buf = torch.randn(10, 4, 5, generator=g)
+    tab = torch.randint(0, 10, (2, 3), generator=g, dtype=torch.int32)
+    assert torch.equal(torch.ops.loopfuse.paged_load(buf, tab), buf[tab.long()])
+
+
+def capture_graph(fn, inputs, marks=()):
+    """Trace fn with dynamic shapes and return the AttentionMatch (or the NoMatch)."""
+    box = {}
+
+    def backend(gm, sample):
+        def fw(g, _):
+            try:
+                box["match"] = capture.match_attention(g)
+            except capture.NoMatch as e:
+                box["nomatch"] = e
+            box["gm"] = g
+            return g.forward
+
+        return aot_module_simplified(gm, sample, fw_compiler=fw)
+
+    torch._dynamo.reset()
+    for t, dim, kind in marks:
+        (torch._dynamo.mark_static if kind == "static" else torch._dynamo.mark_dynamic)(t, dim)
+    with torch.inference_mode():
+        torch.compile(fn, backend=backend, dynamic=True)(*inputs)
+    return box
+
+
+def bf(*shape, seed=0):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed)).to(torch.bfloat16)
+
+
+def test_capture_causal_static_head_dim():
+    def fn(q, k, v):
+        s = q @ k.transpose(-2, -1) * (q.shape[-1] ** -0.5)
+        return torch.softmax(torch.ops.loopfuse.causal_mask(s), dim=-1) @ v
+
+    q, k, v = bf(2, 4, 96, 64), bf(2, 4, 96, 64, seed=1), bf(2, 4, 96, 64, seed=2)
+    m = capture_graph(fn, (q, k, v), [(q, 3, "static"), (q, 2, "dynamic")])["match"]
+    assert m.mask == "causal" and not m.has_tanh and not m.k.paged
+    assert (m.q.perm, m.k.perm, m.v.perm) == ((0, 1, 2, 3),) * 3
+
+
+def test_capture_gqa_softcap_sliding_and_plan_values():
+    def fn(Q, K, V):
+        g = Q.shape[1] // K.shape[1]
+        K = K.repeat_interleave(g, dim=1)
+        V = V.repeat_interleave(g, dim=1)
+        s = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        s = torch.tanh(s / 30) * 30
+        return torch.softmax(torch.ops.loopfuse.sliding_mask(s, 256), dim=-1) @ V
+
+    q, k, v = bf(2, 8, 80, 64), bf(2, 2, 80, 64, seed=1), bf(2, 2, 80, 64, seed=2)
+    box = capture_graph(fn, (q, k, v))
+    m = box["match"]
+    assert m.mask == "sliding" and m.has_tanh
+    args = [None] * len(m.placeholders)
+    # rebuild the flat argument list: ints for SymInt placeholders, tensors otherwise
+    tensors = iter((q, k, v))
+    for i, p in enumerate(m.placeholders):
+        val = p.meta["val"]
+        args[i] = next(tensors) if isinstance(val, torch.Tensor) else int(val.node.hint)
+    plan = m.plan_for(args)
+    assert plan.mask == "sliding" and plan.window == 256
+    assert plan.softcap == pytest.approx(30.0) and plan.scale == pytest.approx(64 ** -0.5, rel=1e-6)
+
+
+def test_capture_paged_decode():
+    def fn(Q, Kc, kt, Vc, vt):
+        K = torch.ops.loopfuse.paged_load(Kc, kt).transpose(-3, -2)
+        V = torch.ops.loopfuse.paged_load(Vc, vt).transpose(-3, -2)
+        s = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        return torch.softmax(s, dim=-1) @ V
+
+    B, Hkv, grp, D, S = 3, 2, 4, 64, 32
+    Kc, Vc = bf(B * S * 2, Hkv, D), bf(B * S * 2, Hkv, D, seed=1)
+    g = torch.Generator().manual_seed(3)
+    kt = torch.randint(0, B * S * 2, (B, S), generator=g, dtype=torch.int32)
+    vt = torch.randint(0, B * S * 2, (B, S), generator=g, dtype=torch.int32)
+    Q = bf(B, Hkv, grp, D, seed=2)
+    m = capture_graph(fn, (Q, Kc, kt, Vc, vt))["match"]
+    assert m.k.paged and m.v.paged and m.mask is None
+    assert m.k.table_index != m.v.table_index
+
+
+def test_capture_paged_page16_reshape():
+    def fn(Q, Kc, kt, Vc, vt):
+        B, pages = kt.shape
+        P, H, D = Kc.shape[1:]
+        K = torch.ops.loopfuse.paged_load(Kc, kt).reshape(B, pages * P, H, D).transpose(1, 2)
+        V = torch.ops.loopfuse.paged_load(Vc, vt).reshape(B, pages * P, H, D).transpose(1, 2)
+        g = Q.shape[1] // H
+        K = K.repeat_interleave(g, dim=1)
+        V = V.repeat_interleave(g, dim=1)
+        s = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        return torch.softmax(s, dim=-1) @ V
+
+    B, Hkv, grp, D, S, P = 3, 2, 4, 64, 64, 16
+    n = B * S // P
+    Kc, Vc = bf(n, P, Hkv, D), bf(n, P, Hkv, D, seed=1)
+    tab = torch.randperm(n, generator=torch.Generator().manual_seed(3)).view(B, S // P).to(torch.int32)
+    Q = bf(B, Hkv * grp, 1, D, seed=2)
+    box = capture_graph(fn, (Q, Kc, tab, Vc, tab.clone()))
+    assert "match" in box, box.get("nomatch")
+    assert box["match"].k.paged and box["match"].v.paged
+
+
+@pytest.mark.parametrize("which", ["bias", "add", "softmax_matmul", "two_outputs"])
+def test_unrecognised_graphs_do_not_match(which):
+    if which == "bias":
+        def fn(q, k, v, b):
+            s = q @ k.transpose(-2, -1) * 0.125 + b
+            return torch.softmax(torch.ops.loopfuse.causal_mask(s), dim=-1) @ v
+        ins = (bf(1, 2, 32, 64), bf(1, 2, 32, 64, seed=1), bf(1, 2, 32, 64, seed=2), bf(1, 2, 32, 32, seed=3))
+    elif which == "add":
+        def fn(a, b):
+            return a + b
+        ins = (bf(4, 8), bf(4, 8, seed=1))
+    elif which == "softmax_matmul":
+        def fn(x, y):
+            return torch.softmax(x, dim=-1) @ y
+        ins = (bf(2, 2, 16, 8), bf(2, 2, 8, 16, seed=1))
+    else:
+        def fn(q, k, v):
+            s = q @ k.transpose(-2, -1)
+            p = torch.softmax(s, dim=-1)
+            return p @ v, p
+        ins = (bf(1, 2, 32, 64), bf(1, 2, 32, 64, seed=1), bf(1, 2, 32, 64, seed=2))
+    box = capture_graph(fn, ins)
+    assert "match" not in box and "nomatch" in box
+
+
+def test_backend_on_cpu_tensors_runs_graph_unfused():
+    """CPU tensors have no HIP path: the compiled function must still be correct (it
+    runs the captured graph) and must say so in the stats."""
+    def fn(q, k, v):
+        s = q @ k.transpose(-2, -1) * (q.shape[-1] ** -0.5)
+        return torch.softmax(torch.ops.loopfuse.causal_mask(s), dim=-1) @ v
+
+    q, k, v = (torch.randn(1, 2, 48, 64, generator=torch.Generator().manual_seed(s)) for s in (0, 1, 2))
+    torch._dynamo.reset()
+    before = dict(interface.stats)
+    out = torch.compile(fn, backend=loopfuse_amd.loopfuse_backend, dynamic=True)(q, k, v)
+    assert torch.allclose(out, O.attention_reference(q, k, v, mask="causal"), atol=1e-5)
+    assert interface.stats["matched_graphs"] == before["matched_graphs"] + 1
+    assert interface.stats["eager_runtime"] == before["eager_runtime"] + 1
+    assert interface.stats["fused"] == before["fused"]
+
+
+def test_unfused_graph_still_correct():
+    def fn(a, b):
+        return torch.relu(a) + b
+
+    a, b = torch.randn(4, 8), torch.randn(4, 8)
+    torch._dynamo.reset()
+    out = torch.compile(fn, backend=loopfuse_amd.loopfuse_backend, dynamic=True)(a, b)
+    assert torch.equal(out, torch.relu(a) + b)
+
+
+def test_kernel_specs_compile_without_gpu(shim_built):
+    spec = lowering.KernelSpec("prefill", 0, 128, lowering.MASK_CAUSAL)
+    ck = lowering.compile_spec(spec)
+    assert ck.code_object[:4] == b"\x7fELF"
+    assert "lf_attn_prefill" in ck.code and "-DLF_MASK=1" in ck.code
+
+
+def test_cpu_tensors_fail_loudly_on_direct_call():
+    q = torch.randn(1, 1, 16, 64).to(torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        lowering.attention(q, q, q, lowering.AttnPlan(scale=0.125))

@@ -1,0 +1,74 @@
+"""The C-ABI library: loads, exports every symbol include/lf_shim.h declares, and its
+host-side entry points (compile, cache, error reporting) behave.  No GPU, no launches."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from loopfuse_amd import runtime
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_symbols():
+    text = open(os.path.join(ROOT, "include", "lf_shim.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(lf_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_exports_every_declared_symbol(shim_built):
+    syms = header_symbols()
+    assert len(syms) >= 11
+    for s in syms:
+        assert hasattr(shim_built, s), f"{s} declared in lf_shim.h but not exported"
+    assert sorted(runtime.ABI_SYMBOLS) == syms
+    assert shim_built.lf_abi_version() == 1
+
+
+def test_compile_without_gpu_and_cache(shim_built, tmp_path):
+    src = 'extern "C" __global__ void k(float* x) { x[threadIdx.x] *= 2.0f; }'
+    code, hit, log = runtime.compile_source(src, "unit_k", ["-O3"], "gfx950", str(tmp_path))
+    assert code[:4] == b"\x7fELF" and not hit
+    code2, hit2, _ = runtime.compile_source(src, "unit_k", ["-O3"], "gfx950", str(tmp_path))
+    assert hit2 and code2 == code
+    # a different option is a different cache entry
+    _, hit3, _ = runtime.compile_source(src, "unit_k", ["-O2"], "gfx950", str(tmp_path))
+    assert not hit3
+    assert len(os.listdir(tmp_path)) == 2
+
+
+def test_compile_error_is_reported(shim_built):
+    with pytest.raises(runtime.ShimError) as e:
+        runtime.compile_source("this is not HIP", "bad", [], "gfx950", None)
+    assert e.value.code != 0
+    assert "error" in str(e.value).lower()
+
+
+def test_bad_arguments_are_rejected(shim_built):
+    L = shim_built
+    assert L.lf_launch(None, 1, 1, 1, 64, 1, 1, 0, None, None) == -1
+    assert b"null function" in L.lf_last_error()
+    fn = ctypes.c_void_p()
+    assert L.lf_get_function(ctypes.c_void_p(1234), b"k", ctypes.byref(fn)) == -1
+    assert L.lf_module_unload(ctypes.c_void_p(1234)) == -1
+    mod = ctypes.c_void_p()
+    assert L.lf_module_load(None, 0, ctypes.byref(mod)) == -1
+
+
+def test_launch_geometry_checks(shim_built):
+    L = shim_built
+    dummy = ctypes.c_void_p(1)
+    assert L.lf_launch(dummy, 0, 1, 1, 64, 1, 1, 0, None, None) == -1
+    assert L.lf_launch(dummy, 1, 1, 1, 2048, 1, 1, 0, None, None) == -1
+    assert L.lf_launch(dummy, 1, 1, 1, 64, 1, 1, 200 * 1024, None, None) == -1
+
+
+def test_params_struct_layout():
+    from loopfuse_amd.lowering import AttnParams
+
+    # 9 pointers, 12 int64 strides, 11 ints, 2 floats; no implicit padding before the tail
+    assert AttnParams.q.offset == 0 and AttnParams.q_sb.offset == 72
+    assert AttnParams.B.offset == 72 + 96
+    assert AttnParams.scale.offset == 72 + 96 + 44
+    assert ctypes.sizeof(AttnParams) == 224
