@@ -1,0 +1,182 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused-attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one pass of the hot path over one batch of synthetic input.  The
+headline workload is BASELINE config 2 (bf16 causal prefill, B8 H32 S2048 D128):
+``value`` is its algorithmic TFLOP/s with the reference's flop convention
+(2*B*H*S^2*D, reference tests/benchmark.py:110).  The same run also times the
+memory-bound half of the metric, config 5 (paged GQA decode, B64 K_len 2048, page
+16), reported under "decode" in GB/s with the reference's byte convention
+(K and V only, tests/benchmark.py:452).  Inputs are resident in HBM before the
+timed region.  One JSON line on stdout.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16/fp16, published
+HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, published
+
+
+def time_gpu(fn, steps: int, warmup: int):
+    """Average seconds per call over `steps` calls, HIP events on the launch stream."""
+    import torch
+
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(steps):
+        fn(i)
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return start.elapsed_time(stop) * 1e-3 / steps, wall / steps
+
+
+def cpu_baseline(seconds: float = 12.0) -> dict:
+    """The reference's eager CPU path (oracle port) on a bounded slice of the workload."""
+    import torch
+
+    from loopfuse_amd import workloads
+    from oracle import attention_oracle as O
+
+    cores = os.cpu_count() or 1
+    if os.environ.get("OMP_NUM_THREADS"):
+        cores = min(cores, int(os.environ["OMP_NUM_THREADS"]))
+    torch.set_num_threads(cores)
+
+    def run(q, k, v, budget):
+        with torch.inference_mode():
+            for _ in range(2):
+                O.eager_reference_graph(q, k, v)
+            ts = []
+            t_end = time.perf_counter() + budget
+            while time.perf_counter() < t_end and len(ts) < 200:
+                t0 = time.perf_counter()
+                O.eager_reference_graph(q, k, v)
+                ts.append(time.perf_counter() - t0)
+        return statistics.median(ts), len(ts)
+
+    # slice of config 2: one batch, four heads, full S and D; fp32 as the eager path computes
+    w = workloads.make("c2", seed=0, B=1)
+    q, k, v = (t[:, :4].float().contiguous() for t in (w.q, w.k, w.v))
+    t2, n2 = run(q, k, v, seconds * 0.75)
+    flops2 = 2 * 1 * 4 * 2048 * 2048 * 128
+    # config 1 (the reference's own CPU-runnable case): fp32 B2 H8 S512 D64
+    w1 = workloads.make("c1", seed=0)
+    t1, n1 = run(w1.q, w1.k, w1.v, seconds * 0.25)
+    flops1 = 2 * 2 * 8 * 512 * 512 * 64
+    return {
+        "value": flops2 / t2 / 1e12,
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"eager fp32 causal attention on config-2 slice B1 H4 S2048 D128, median of {n2} runs "
+                  f"({t2 * 1e3:.1f} ms); config 1 (B2 H8 S512 D64 fp32): {flops1 / t1 / 1e12:.4f} TFLOP/s, "
+                  f"{t1 * 1e3:.2f} ms median of {n1}",
+        "c1_tflops": flops1 / t1 / 1e12,
+        "c1_ms": t1 * 1e3,
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", choices=["prefill", "decode"], default=None,
+                    help="time only one of the two kernels (profiling aid)")
+    ap.add_argument("--workload", default="c2", help="prefill workload: c2 | c2_softcap | c3")
+    ap.add_argument("--decode-workload", default="c5", help="decode workload: c5 | c4")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (--gpus 1); "
+              "the hot path shards over batch and heads with no exchange", file=sys.stderr)
+        return 2
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        return 3
+    from loopfuse_amd import workloads
+
+    dev = torch.device("cuda:0")
+    out: dict = {}
+
+    pre = None
+    if args.only in (None, "prefill"):
+        w = workloads.make(args.workload, seed=0).to(dev)
+        o = workloads.run(w)     # first call compiles / loads the code object
+        torch.cuda.synchronize()
+        t, wall = time_gpu(lambda i: workloads.run(w, out=o), args.steps, args.warmup)
+        pre = {"workload": args.workload, "sec": t, "wall_sec": wall, "flops": w.flops()}
+
+    dec = None
+    if args.only in (None, "decode"):
+        # rotate over copies of the KV pool so that no launch finds its input in the
+        # 256 MB Infinity Cache
+        base = workloads.make(args.decode_workload, seed=0)
+        nrot = max(2, int(1.5e9 // base.kv_bytes()) + 1)
+        ws = [base.to(dev)]
+        for _ in range(nrot - 1):
+            ws.append(workloads.Workload(base.name, ws[0].q, ws[0].k.clone(), ws[0].v.clone(), base.mask,
+                                         base.window, base.softcap, ws[0].k_table, ws[0].v_table))
+        o = workloads.run(ws[0])
+        torch.cuda.synchronize()
+        t, wall = time_gpu(lambda i: workloads.run(ws[i % nrot], out=o), args.steps, args.warmup)
+        dec = {"workload": args.decode_workload, "sec": t, "wall_sec": wall, "bytes": base.kv_bytes(), "rotation": nrot}
+
+    primary = pre if pre is not None else dec
+    if pre is not None:
+        tflops = pre["flops"] / pre["sec"] / 1e12
+        out.update({
+            "metric": "prefill TFLOP/s + decode HBM GB/s on 1 MI355X (% of roofline)",
+            "value": tflops, "unit": "TFLOP/s",
+        })
+        out["roofline"] = {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                           "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                           "kernel": "lf_attn_prefill", "us_per_launch": pre["sec"] * 1e6}
+    if dec is not None:
+        gbs = dec["bytes"] / dec["sec"] / 1e9
+        d = {"workload": dec["workload"], "value": gbs, "unit": "GB/s", "us_per_launch": dec["sec"] * 1e6,
+             "host_us_per_launch": dec["wall_sec"] * 1e6, "kv_pool_rotation": dec["rotation"],
+             "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": gbs / HBM_PEAK_GBS, "traffic": None, "kernel": "lf_attn_decode(+combine)"}}
+        if pre is None:
+            out.update({"metric": "prefill TFLOP/s + decode HBM GB/s on 1 MI355X (% of roofline)",
+                        "value": gbs, "unit": "GB/s", "roofline": d["roofline"]})
+        out["decode"] = d
+    out.update({
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": primary["sec"] * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": ("config 2: causal prefill bf16 B8 H32 S2048 D128" if pre is not None and args.workload == "c2"
+                                else primary["workload"]),
+                   "decode_workload": "config 5: paged GQA decode bf16 B64 Hq32/Hkv8 K_len2048 D128 page16"
+                   if args.decode_workload == "c5" else args.decode_workload},
+    })
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -22,6 +22,12 @@
 #ifndef LF_V_TR
 #define LF_V_TR 1
 #endif
+#ifndef LF_SETPRIO
+#define LF_SETPRIO 1     /* raise wave priority while it issues MFMAs */
+#endif
+#ifndef LF_LAZY_LOG2
+#define LF_LAZY_LOG2 8   /* slack of the softmax exponent offset, log2 units */
+#endif
 
 #define LF_BM 128
 #define LF_BN 64
@@ -122,42 +128,54 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 2) lf_attn_prefill(const LfA
   for (int db = 0; db < LF_NDB; ++db)
 #pragma unroll
     for (int i = 0; i < 16; ++i) o[db][i] = 0.0f;
-  float m_run = LF_NEG_INF;   // running max of the (modified) scores, per query
+  float mc_ref = LF_NEG_INF;  // exponent offset of this query in log2 units (a lagging running max)
   float l_run = 0.0f;         // this lane's share of the running sum
 
-  // ---- staging: thread handles chunk (srow, sch) of every pass
+  // ---- staging: thread handles chunk (row0 + 16*ps*LF_RPS.., ch) of every pass.
+  // Dense K/V: address = wave-uniform base (batch, head, tile, pass) + a fixed
+  // 32-bit per-thread offset, so the loop carries no 64-bit address arithmetic.
   lf_u32x4 kst[LF_NPASS], vst[LF_NPASS];
+  constexpr int kRowsPerPass = LF_NT / LF_CPR;
+  const int srow = tid / LF_CPR;
+  const int sch = tid % LF_CPR;
+  const lf_elem* k_uni = p.k + (long long)b * p.k_sb + (long long)hkv * p.k_sh;
+  const lf_elem* v_uni = p.v + (long long)b * p.v_sb + (long long)hkv * p.v_sh;
+  const unsigned k_toff = (unsigned)(srow * p.k_ss) + 8u * sch;
+  const unsigned v_toff = (unsigned)(srow * p.v_ss) + 8u * sch;
   auto load_tile = [&](int kt) {
+    const bool tail = (kt + 1) * LF_BN > p.Sk;          // uniform
 #pragma unroll
     for (int ps = 0; ps < LF_NPASS; ++ps) {
-      int idx = tid + LF_NT * ps;
-      int row = idx / LF_CPR;
-      int ch = idx % LF_CPR;
-      int tok = kt * LF_BN + row;
-      lf_u32x4 kz = {0u, 0u, 0u, 0u}, vz = {0u, 0u, 0u, 0u};
-      if (tok < p.Sk) {
-        kz = *reinterpret_cast<const lf_u32x4*>(lf_kv_row(p, 0, b, hkv, tok) + 8 * ch);
-        vz = *reinterpret_cast<const lf_u32x4*>(lf_kv_row(p, 1, b, hkv, tok) + 8 * ch);
+      const int r0 = kt * LF_BN + kRowsPerPass * ps;    // uniform
+      if ((LF_PAGED & 1) || tail) {
+        // rows past the end re-read the last row: their scores are masked (j >= Sk)
+        // and their probabilities are exactly 0, so any finite data will do
+        const int tok = min(r0 + srow, p.Sk - 1);
+        kst[ps] = *reinterpret_cast<const lf_u32x4*>(lf_kv_row(p, 0, b, hkv, tok) + 8 * sch);
+      } else {
+        kst[ps] = *reinterpret_cast<const lf_u32x4*>(k_uni + (long long)r0 * p.k_ss + k_toff);
       }
-      kst[ps] = kz;
-      vst[ps] = vz;
+      if ((LF_PAGED & 2) || tail) {
+        const int tok = min(r0 + srow, p.Sk - 1);
+        vst[ps] = *reinterpret_cast<const lf_u32x4*>(lf_kv_row(p, 1, b, hkv, tok) + 8 * sch);
+      } else {
+        vst[ps] = *reinterpret_cast<const lf_u32x4*>(v_uni + (long long)r0 * p.v_ss + v_toff);
+      }
     }
   };
   auto store_tile = [&](int buf) {
 #pragma unroll
     for (int ps = 0; ps < LF_NPASS; ++ps) {
-      int idx = tid + LF_NT * ps;
-      int row = idx / LF_CPR;
-      int ch = idx % LF_CPR;
-      *reinterpret_cast<lf_u32x4*>(&lds_k[buf][row * LF_D + 8 * lf_k_phys(row, ch)]) = kst[ps];
-      *reinterpret_cast<lf_u32x4*>(&lds_v[buf][row * LF_D + 8 * lf_v_phys(row, ch)]) = vst[ps];
+      const int row = srow + kRowsPerPass * ps;
+      *reinterpret_cast<lf_u32x4*>(&lds_k[buf][row * LF_D + 8 * lf_k_phys(row, sch)]) = kst[ps];
+      *reinterpret_cast<lf_u32x4*>(&lds_v[buf][row * LF_D + 8 * lf_v_phys(row, sch)]) = vst[ps];
     }
   };
 
-  if (kt_begin < kt_end) {
-    load_tile(kt_begin);
-    store_tile(0);
-  }
+  // every valid q tile has at least one KV tile (kt_end >= 1 > kt_begin is not
+  // guaranteed only for Sk == 0, which the host rejects)
+  load_tile(kt_begin);
+  store_tile(0);
   __syncthreads();
 
   for (int kt = kt_begin; kt < kt_end; ++kt) {
@@ -181,19 +199,28 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 2) lf_attn_prefill(const LfA
       const lf_elem* kbuf = lds_k[cur];
       const lf_elem* vbuf = lds_v[cur];
 
-      // ---- S^T = K Q^T
+      // ---- S^T = K Q^T (the LF_NKB accumulator chains are interleaved so that
+      // consecutive MFMAs are independent)
       lf_f32x16 s[LF_NKB];
 #pragma unroll
-      for (int kb = 0; kb < LF_NKB; ++kb) {
+      for (int kb = 0; kb < LF_NKB; ++kb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) s[kb][i] = 0.0f;
-        const int row = 32 * kb + l32;
+#if LF_SETPRIO
+      __builtin_amdgcn_s_setprio(2);
+#endif
 #pragma unroll
-        for (int ks = 0; ks < LF_NKS; ++ks) {
+      for (int ks = 0; ks < LF_NKS; ++ks) {
+#pragma unroll
+        for (int kb = 0; kb < LF_NKB; ++kb) {
+          const int row = 32 * kb + l32;
           lf_u32x4 raw = *reinterpret_cast<const lf_u32x4*>(&kbuf[row * LF_D + 8 * lf_k_phys(row, 2 * ks + g)]);
           s[kb] = lf_mfma32(__builtin_bit_cast(lf_elem8, raw), qf[ks], s[kb]);
         }
       }
+#if LF_SETPRIO
+      __builtin_amdgcn_s_setprio(0);
+#endif
 
       // ---- score modifications and mask; element i of block kb is kv index
       // j = k0 + 32*kb + 8*(i/4) + 4*g + i%4, query my_q.
@@ -220,18 +247,34 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 2) lf_attn_prefill(const LfA
           }
       }
 
-      // ---- online softmax (per query = per lane pair l, l^32)
+      // ---- online softmax (per query = per lane pair l, l^32).  The exponent
+      // offset m_ref is allowed to lag behind the true running max by up to
+      // LF_LAZY_LOG2 (in log2 units): probabilities then reach at most
+      // 2^LF_LAZY_LOG2, which fp32 sums and bf16/fp16 operands hold without loss,
+      // and O and l are rescaled only when some query of the wave exceeds the
+      // slack -- a wave-uniform branch that is rarely taken after the first tiles.
+      // O / l is independent of the offset, so the result is unchanged.
       float mx = LF_NEG_INF;
 #pragma unroll
       for (int kb = 0; kb < LF_NKB; ++kb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kb][i]);
       mx = fmaxf(mx, lf_swap32(mx));
-      const float m_new = fmaxf(m_run, mx);
-      const float m_sub = (m_new == LF_NEG_INF) ? 0.0f : m_new;
-      const float mc = m_sub * cexp;
-      const float r = lf_exp2(m_run * cexp - mc);
-      m_run = m_new;
+      const float mxc = mx * cexp;
+      if (__builtin_amdgcn_ballot_w64(mxc > mc_ref + (float)LF_LAZY_LOG2) != 0ull) {
+        const float mc_new = fmaxf(mc_ref, mxc);          // finite wherever mxc is
+        // 0 on a query's first update (its O and l are still 0); 1 for a query
+        // that still has seen nothing (both offsets -inf)
+        const float r = (mc_new == LF_NEG_INF) ? 1.0f : lf_exp2(mc_ref - mc_new);
+        mc_ref = mc_new;
+        l_run *= r;
+#pragma unroll
+        for (int db = 0; db < LF_NDB; ++db)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o[db][i] *= r;
+      }
+      // a query that has seen no unmasked key yet (offset still -inf) subtracts 0
+      const float mc_sub = (mc_ref == LF_NEG_INF) ? 0.0f : mc_ref;
 
       float rs = 0.0f;
       lf_elem8 pf[LF_NKK];
@@ -239,16 +282,15 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 2) lf_attn_prefill(const LfA
       for (int kb = 0; kb < LF_NKB; ++kb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          float e = lf_exp2(s[kb][i] * cexp - mc);
+          float e = lf_exp2(s[kb][i] * cexp - mc_sub);
           rs += e;
           pf[2 * kb + i / 8][i % 8] = lf_from_float(e);
         }
-      l_run = l_run * r + rs;
-#pragma unroll
-      for (int db = 0; db < LF_NDB; ++db)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) o[db][i] *= r;
+      l_run += rs;
 
+#if LF_SETPRIO
+      __builtin_amdgcn_s_setprio(2);
+#endif
       // ---- O^T += V^T P^T.  k-slot s of step kk is kv row
       // 16*kk + 8*(s/4) + 4*g + s%4 (the order P is held in); A row = d.
 #pragma unroll
@@ -286,6 +328,9 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 2) lf_attn_prefill(const LfA
           o[db] = lf_mfma32(a, pf[kk], o[db]);
         }
       }
+#if LF_SETPRIO
+      __builtin_amdgcn_s_setprio(0);
+#endif
     }
 
     if (have_next) store_tile(cur ^ 1);
