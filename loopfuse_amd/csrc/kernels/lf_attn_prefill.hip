@@ -25,12 +25,29 @@
 #ifndef LF_SETPRIO
 #define LF_SETPRIO 1     /* raise wave priority while it issues MFMAs */
 #endif
+#ifndef LF_KPF
+#define LF_KPF 6         /* K fragments in flight ahead of the MFMA consuming them */
+#endif
+#ifndef LF_VPF
+#define LF_VPF 4         /* V fragments (two transposed reads each) in flight */
+#endif
+#ifndef LF_SCHED
+#define LF_SCHED 1       /* pin read/MFMA interleaving with sched_group_barrier */
+#endif
+#ifndef LF_ABLATE
+#define LF_ABLATE 0      /* profiling aid: 1 = no softmax math, 2 = no staging/barrier, 4 = no PV, 8 = no QK^T (results are wrong) */
+#endif
 #ifndef LF_LAZY_LOG2
 #define LF_LAZY_LOG2 8   /* slack of the softmax exponent offset, log2 units */
 #endif
 
 #define LF_BM 128
+#ifndef LF_BN
 #define LF_BN 64
+#endif
+#ifndef LF_OCC
+#define LF_OCC 2    /* waves per SIMD the register budget is set for */
+#endif
 #define LF_NW 4
 #define LF_NT (LF_NW * 64)
 #define LF_D LF_HEAD_DIM
@@ -54,7 +71,7 @@ __device__ __forceinline__ int lf_v_phys(int row, int ch) {
   return ch ^ (4 * ((row / LF_RPS) & (LF_CPR / 4 - 1)));
 }
 
-extern "C" __global__ void __launch_bounds__(LF_NT, 2) lf_attn_prefill(const LfAttnParams p) {
+extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(const LfAttnParams p) {
   __shared__ __attribute__((aligned(16))) lf_elem lds_k[2][LF_BN * LF_D];
   __shared__ __attribute__((aligned(16))) lf_elem lds_v[2][LF_BN * LF_D];
 
@@ -71,9 +88,13 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 2) lf_attn_prefill(const LfA
   const int nbh = p.B * p.Hq;
   const int xcd = blockIdx.x & 7;
   const int slot = blockIdx.x >> 3;
-  const int bh = (slot / nqt) * 8 + xcd;
+  // within an XCD: groups of 4 (batch, head) pairs (their K/V fit the 4 MB L2
+  // together), each group dealt heaviest q tile first across its 4 members
+  const int grp = slot / (4 * nqt);
+  const int in_grp = slot % (4 * nqt);
+  const int bh = (grp * 4 + (in_grp & 3)) * 8 + xcd;
   if (bh >= nbh) return;
-  const int qt = nqt - 1 - (slot % nqt);
+  const int qt = nqt - 1 - (in_grp >> 2);
   const int b = bh / p.Hq;
   const int h = bh % p.Hq;
   const int hkv = h / (p.Hq / p.Hkv);
@@ -181,7 +202,9 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 2) lf_attn_prefill(const LfA
   for (int kt = kt_begin; kt < kt_end; ++kt) {
     const int cur = (kt - kt_begin) & 1;
     const bool have_next = kt + 1 < kt_end;
+#if !(LF_ABLATE & 2)
     if (have_next) load_tile(kt + 1);
+#endif
 
     const int k0 = kt * LF_BN;
     bool need = wave_has_rows;
@@ -209,14 +232,33 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 2) lf_attn_prefill(const LfA
 #if LF_SETPRIO
       __builtin_amdgcn_s_setprio(2);
 #endif
-#pragma unroll
-      for (int ks = 0; ks < LF_NKS; ++ks) {
-#pragma unroll
-        for (int kb = 0; kb < LF_NKB; ++kb) {
+      {
+        // K fragments are fetched LF_KPF MFMAs ahead of their use: the LDS round
+        // trip (well over 100 cycles) spans several 32-cycle MFMAs
+        constexpr int kNF = ((LF_ABLATE & 8) ? 0 : LF_NKS * LF_NKB);
+        lf_u32x4 kf[kNF > 0 ? kNF : 1];
+        auto k_frag = [&](int f) {
+          const int ks = f / LF_NKB, kb = f % LF_NKB;
           const int row = 32 * kb + l32;
-          lf_u32x4 raw = *reinterpret_cast<const lf_u32x4*>(&kbuf[row * LF_D + 8 * lf_k_phys(row, 2 * ks + g)]);
-          s[kb] = lf_mfma32(__builtin_bit_cast(lf_elem8, raw), qf[ks], s[kb]);
+          return *reinterpret_cast<const lf_u32x4*>(&kbuf[row * LF_D + 8 * lf_k_phys(row, 2 * ks + g)]);
+        };
+#pragma unroll
+        for (int f = 0; f < LF_KPF && f < kNF; ++f) kf[f] = k_frag(f);
+#pragma unroll
+        for (int f = 0; f < kNF; ++f) {
+          if (f + LF_KPF < kNF) kf[f + LF_KPF] = k_frag(f + LF_KPF);
+          s[f % LF_NKB] = lf_mfma32(__builtin_bit_cast(lf_elem8, kf[f]), qf[f / LF_NKB], s[f % LF_NKB]);
         }
+#if LF_SCHED
+        // pin the order: LF_KPF reads, then (MFMA, read) pairs, then the last MFMAs
+        __builtin_amdgcn_sched_group_barrier(0x100, LF_KPF, 0);
+#pragma unroll
+        for (int f = 0; f < kNF - LF_KPF; ++f) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, LF_KPF, 0);
+#endif
       }
 #if LF_SETPRIO
       __builtin_amdgcn_s_setprio(0);
@@ -255,11 +297,13 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 2) lf_attn_prefill(const LfA
       // slack -- a wave-uniform branch that is rarely taken after the first tiles.
       // O / l is independent of the offset, so the result is unchanged.
       float mx = LF_NEG_INF;
+#if !(LF_ABLATE & 1)
 #pragma unroll
       for (int kb = 0; kb < LF_NKB; ++kb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kb][i]);
       mx = fmaxf(mx, lf_swap32(mx));
+#endif
       const float mxc = mx * cexp;
       if (__builtin_amdgcn_ballot_w64(mxc > mc_ref + (float)LF_LAZY_LOG2) != 0ull) {
         const float mc_new = fmaxf(mc_ref, mxc);          // finite wherever mxc is
@@ -282,7 +326,11 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 2) lf_attn_prefill(const LfA
       for (int kb = 0; kb < LF_NKB; ++kb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
+#if LF_ABLATE & 1
+          float e = s[kb][i];
+#else
           float e = lf_exp2(s[kb][i] * cexp - mc_sub);
+#endif
           rs += e;
           pf[2 * kb + i / 8][i % 8] = lf_from_float(e);
         }
@@ -293,10 +341,11 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 2) lf_attn_prefill(const LfA
 #endif
       // ---- O^T += V^T P^T.  k-slot s of step kk is kv row
       // 16*kk + 8*(s/4) + 4*g + s%4 (the order P is held in); A row = d.
-#pragma unroll
-      for (int kk = 0; kk < LF_NKK; ++kk) {
-#pragma unroll
-        for (int db = 0; db < LF_NDB; ++db) {
+      {
+        constexpr int kNF = ((LF_ABLATE & 4) ? 0 : LF_NKK * LF_NDB);
+        lf_elem8 vf[kNF > 0 ? kNF : 1];
+        auto v_frag = [&](int f) {
+          const int kk = f / LF_NDB, db = f % LF_NDB;
           lf_elem8 a;
 #if LF_V_TR
           // 16-lane group (2g + dh) asks for rows r0..r0+3, columns 32db+16dh..+15:
@@ -325,16 +374,34 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 2) lf_attn_prefill(const LfA
             a[sl] = vbuf[row * LF_D + 8 * lf_v_phys(row, col / 8) + (col % 8)];
           }
 #endif
-          o[db] = lf_mfma32(a, pf[kk], o[db]);
+          return a;
+        };
+#pragma unroll
+        for (int f = 0; f < LF_VPF && f < kNF; ++f) vf[f] = v_frag(f);
+#pragma unroll
+        for (int f = 0; f < kNF; ++f) {
+          if (f + LF_VPF < kNF) vf[f + LF_VPF] = v_frag(f + LF_VPF);
+          o[f % LF_NDB] = lf_mfma32(vf[f], pf[f / LF_NDB], o[f % LF_NDB]);
         }
+#if LF_SCHED && LF_V_TR
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * LF_VPF, 0);
+#pragma unroll
+        for (int f = 0; f < kNF - LF_VPF; ++f) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, LF_VPF, 0);
+#endif
       }
 #if LF_SETPRIO
       __builtin_amdgcn_s_setprio(0);
 #endif
     }
 
+#if !(LF_ABLATE & 2)
     if (have_next) store_tile(cur ^ 1);
     __syncthreads();
+#endif
   }
 
   // ---- epilogue: O[q][d] = O^T[d][q] / l.  Element i of block db is

@@ -25,7 +25,7 @@ from typing import Optional
 import torch
 
 from . import runtime
-from .skip import PREFILL_BM, PREFILL_BN
+from .skip import TILE_SHAPES
 
 MASK_NONE, MASK_CAUSAL, MASK_SLIDING = 0, 1, 2
 _MASK_NAMES = {"none": MASK_NONE, None: MASK_NONE, "causal": MASK_CAUSAL, "sliding": MASK_SLIDING}
@@ -64,6 +64,7 @@ class KernelSpec:
     rows: int = 1          # decode: query rows sharing K/V (1, 2, 4)
     waves: int = 4         # decode: waves per workgroup
     v_tr: bool = True      # prefill: transposed LDS reads for V
+    extra: tuple = ()      # further -D options (tuning experiments)
 
     def options(self) -> list[str]:
         o = list(COMMON_OPTS) + [
@@ -77,16 +78,22 @@ class KernelSpec:
         ]
         if self.family == "decode":
             o += [f"-DLF_ROWS={self.rows}", f"-DLF_DW={self.waves}"]
-        else:
+        elif self.family == "prefill":
             o += [f"-DLF_V_TR={int(self.v_tr)}"]
-        return o
+        return o + list(self.extra)
 
     def files(self) -> tuple[str, ...]:
-        return ("lf_common.hip.h", "lf_attn_prefill.hip" if self.family == "prefill" else "lf_attn_decode.hip")
+        return ("lf_common.hip.h", {"prefill": "lf_attn_prefill.hip", "prefill_pipe": "lf_attn_prefill_pipe.hip",
+                                    "decode": "lf_attn_decode.hip"}[self.family])
+
+    def entry(self) -> str:
+        return {"prefill": "lf_attn_prefill", "prefill_pipe": "lf_attn_prefill_pipe",
+                "decode": "lf_attn_decode"}[self.family]
 
     def name(self) -> str:
         return (f"lf_{self.family}_t{self.dtype}_d{self.head_dim}_m{self.mask}_c{int(self.softcap)}"
-                f"_p{self.paged}x{self.page_size}i{int(self.table_i64)}_r{self.rows}w{self.waves}v{int(self.v_tr)}")
+                f"_p{self.paged}x{self.page_size}i{int(self.table_i64)}_r{self.rows}w{self.waves}v{int(self.v_tr)}"
+                + "".join("_" + e.replace("-D", "").replace("=", "") for e in self.extra))
 
     def source(self) -> str:
         return runtime.read_kernel_source(*self.files())
@@ -211,6 +218,16 @@ def decode_split(units: int, Sk: int, cus: int = 256) -> int:
     return max(1, min(want, most))
 
 
+def prefill_variant(Sq: int, v_tr: bool = True) -> str:
+    """Which prefill kernel serves a call.  The two-waves-per-SIMD kernel
+    (``prefill``) is the measured-faster default; LOOPFUSE_PREFILL=pipe selects the
+    one-wave-per-SIMD software-pipelined kernel for comparison."""
+    env = os.environ.get("LOOPFUSE_PREFILL")
+    if env == "pipe" and v_tr:
+        return "prefill_pipe"
+    return "prefill"
+
+
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
               k_table: Optional[torch.Tensor] = None, v_table: Optional[torch.Tensor] = None,
               *, out: Optional[torch.Tensor] = None, record_visits: bool = False,
@@ -302,18 +319,24 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     keep = (q, k, v, out, kt, vt)  # noqa: F841  (tensors stay alive until the launch is queued)
 
     if family == "prefill":
+        family = prefill_variant(Sq, v_tr)
+    if family in ("prefill", "prefill_pipe"):
         P.q_sb, P.q_sh, P.q_ss = q.stride(0), q.stride(1), q.stride(2)
         P.o_sb, P.o_sh, P.o_ss = out.stride(0), out.stride(1), out.stride(2)
-        spec = KernelSpec("prefill", _DTYPE_CODE[dtype], D, mask, plan.softcap is not None, paged,
-                          page_size, table_i64, v_tr=v_tr)
-        nqt = (Sq + PREFILL_BM - 1) // PREFILL_BM
-        nkt = (Sk + PREFILL_BN - 1) // PREFILL_BN
+        spec = KernelSpec(family, _DTYPE_CODE[dtype], D, mask, plan.softcap is not None, paged,
+                          page_size, table_i64, v_tr=v_tr if family == "prefill" else True,
+                          extra=tuple(os.environ.get("LOOPFUSE_KOPTS", "").split()))
+        bm, bn = TILE_SHAPES[family]
+        nqt = (Sq + bm - 1) // bm
+        nkt = (Sk + bn - 1) // bn
         visits = None
         if record_visits:
             visits = torch.zeros((B * Hq * nqt, nkt), dtype=torch.uint8, device=q.device)
             P.visits = visits.data_ptr()
-        grid = 8 * ((B * Hq + 7) // 8) * nqt
-        get_kernel(spec, "lf_attn_prefill").launch((grid, 1, 1), (256, 1, 1), P)
+        # 8 XCD classes x (batch*head pairs per class, padded to the kernel's groups of 4) x q tiles
+        per_xcd = (B * Hq + 7) // 8
+        grid = 8 * ((per_xcd + 3) // 4 * 4) * nqt
+        get_kernel(spec, spec.entry()).launch((grid, 1, 1), (256, 1, 1), P)
         return (out, visits) if record_visits else out
 
     if family != "decode":

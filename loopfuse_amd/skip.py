@@ -14,8 +14,12 @@ Contract (checked bit-exact against the dense mask in the tests):
 """
 from __future__ import annotations
 
-PREFILL_BM = 128   # query rows per workgroup of lf_attn_prefill
-PREFILL_BN = 64    # KV rows per LDS tile
+# (query rows per workgroup, KV rows per LDS tile) of each prefill kernel
+TILE_SHAPES = {
+    "prefill": (128, 64),        # lf_attn_prefill: 4 waves x 32 rows, two waves per SIMD
+    "prefill_pipe": (256, 32),   # lf_attn_prefill_pipe: 4 waves x 64 rows, software-pipelined
+}
+PREFILL_BM, PREFILL_BN = TILE_SHAPES["prefill"]
 
 
 def cdiv(a: int, b: int) -> int:

@@ -127,18 +127,52 @@ def test_paged_kv_prefill_page16_int64():
 
 
 # ---------------------------------------------------------------- block skip
+@pytest.mark.parametrize("variant", ["w32", "pipe"])
 @pytest.mark.parametrize("mask,window,S", [("causal", 0, 593), ("sliding", 256, 2048), ("sliding", 100, 700),
                                            (None, 0, 300)])
-def test_visited_tiles_bit_exact(mask, window, S):
+def test_visited_tiles_bit_exact(mask, window, S, variant, monkeypatch):
+    """The KV tiles each workgroup actually walks == tiles with any unmasked score."""
+    monkeypatch.setenv("LOOPFUSE_PREFILL", variant)
+    bm, bn = skip.TILE_SHAPES[lowering.prefill_variant(S)]
     q, k, v = (rand((1, 2, S, 128), torch.bfloat16, s).to(dev()) for s in (1, 2, 3))
     plan = lowering.AttnPlan(mask=mask, window=window, scale=128 ** -0.5)
     _, visits = lowering.attention(q, k, v, plan, record_visits=True, force_family="prefill")
     torch.cuda.synchronize()
-    nqt = skip.cdiv(S, skip.PREFILL_BM)
+    nqt = skip.cdiv(S, bm)
     visits = visits.cpu().view(2, nqt, -1).bool()
-    dense = O.visited_tiles_dense(mask, S, S, window, skip.PREFILL_BM, skip.PREFILL_BN)
+    dense = O.visited_tiles_dense(mask, S, S, window, bm, bn)
     for h in range(2):
         assert torch.equal(visits[h], dense)
+    # and the host-side closed form agrees with both
+    host = torch.zeros_like(dense)
+    for qt, (b, e) in enumerate(skip.visited_tiles(mask, S, S, window, bm, bn)):
+        host[qt, b:e] = True
+    assert torch.equal(host, dense)
+
+
+@pytest.mark.parametrize("variant", ["w32", "pipe"])
+@pytest.mark.parametrize("case", ["causal593", "sliding", "softcap_gqa", "rect", "tiny"])
+def test_prefill_variants(variant, case, monkeypatch):
+    """Both prefill kernels serve every shape class (the default picks by size)."""
+    monkeypatch.setenv("LOOPFUSE_PREFILL", variant)
+    dt = torch.bfloat16
+    if case == "causal593":
+        q, k, v = (rand((2, 4, 593, 128), dt, s) for s in (1, 2, 3))
+        check(q, k, v, mask="causal")
+    elif case == "sliding":
+        q, k, v = (rand((1, 4, 1100, 64), torch.float16, s) for s in (1, 2, 3))
+        check(q, k, v, mask="sliding", window=77)
+    elif case == "softcap_gqa":
+        q = rand((2, 8, 700, 128), dt, 1)
+        k, v = (rand((2, 2, 700, 128), dt, s) for s in (2, 3))
+        check(q, k, v, mask="causal", softcap=20.0)
+    elif case == "rect":
+        q = rand((1, 2, 300, 128), dt, 1)
+        k, v = (rand((1, 2, 1000, 128), dt, s) for s in (2, 3))
+        check(q, k, v, force_family="prefill")
+    else:
+        q, k, v = (rand((1, 1, 5, 64), dt, s) for s in (1, 2, 3))
+        check(q, k, v, mask="causal")
 
 
 # ---------------------------------------------------------------- decode
