@@ -1,80 +1,96 @@
 // lf_attn_decode.hip — split-K decode attention for gfx950 (few query rows per
-// (batch, kv head), long KV): a pure HBM-streaming kernel.
+// (batch, kv head), long KV): an HBM-streaming kernel with both products on MFMA.
 //
-// A "unit" is one (batch, kv head, row chunk): LF_ROWS (1, 2 or 4) query rows
-// that share every K/V fetch (GQA group rows, reference benchmark.py:439-443).
+// A "unit" is one (batch, kv head, row chunk): up to 16 query rows that share
+// every K/V fetch (GQA group rows, reference tests/benchmark.py:439-443).
 // grid = (units, nsplit); a workgroup of LF_DW waves owns tokens
-// [z*split_len, (z+1)*split_len) of its unit and deals them to its waves in
-// 16-token steps.  Per step a lane (t = lane%16, g = lane/16) loads, straight
-// from global memory into registers and 16 bytes at a time, the pieces
-// d = 32*j + 8*g .. +7 (j < D/32) of K[token t] and V[token t].  Those registers
-// ARE the B operand of v_mfma_f32_16x16x32 (column = token, k = d), so
-//     S[row, t] = sum_d Q[row, d] K[t, d]
-// costs D/32 MFMAs with Q (rows replicated to fill 16) as the A operand, and
-// every lane ends up holding the scores of all LF_ROWS rows for ITS token.  Each
-// lane keeps a private online-softmax state (m, l, acc[row][its 32 d's]) for
-// the tokens it has seen; PV is plain FMAs on the V registers.  No LDS, no
-// barrier and no cross-lane traffic inside the loop.  At the end the 16 token
-// lanes of each wave and the waves of the workgroup are merged through LDS
-// with the usual (max, sum, acc) log-sum-exp combine; with nsplit > 1 the
-// workgroup writes its partial to scratch and lf_attn_decode_combine merges.
+// [z*split_len, (z+1)*split_len) of its unit and deals them to its waves in pairs
+// of 16-token steps.  Nothing is shared between waves until the final merge, so
+// the streaming loop has no barrier.
 //
-// The page-table gather (LF_PAGED) is fused into the row address: page ids for
-// step s+2 are fetched while K/V of step s+1 are in flight and step s is
-// being consumed (reference: loopfuse/codegen.py:738-872).
+// Per step a lane (c = lane%16, g = lane/16) loads, 16 bytes at a time and
+// straight from global memory into registers, the pieces d = 32*j + 8*g .. +7 of
+// K[token c] and V[token c] (paged: through the page table, ids fetched two pairs
+// ahead -- reference loopfuse/codegen.py:738-872).  Four register stages keep two
+// pairs (32 KB per wave) in flight.
+//   S^T = K Q^T :  the K registers ARE the A operand of v_mfma_f32_16x16x32
+//                  (row = token, k = d); Q^T (rows padded to 16) is the B operand.
+//                  Lane (q = c, g) receives S^T[tokens 4g..4g+3][q].
+//   softmax     :  per query column, with one exponent offset per column shared by
+//                  the four lane groups; it may lag the running max by
+//                  2^LF_LAZY_LOG2, so the cross-lane max and the rescale of O sit
+//                  in a rarely taken wave-uniform branch.
+//   O^T += V^T P^T: P^T of a PAIR of steps is, as held, a B operand (k = 32
+//                  tokens); V goes through a wave-private LDS tile and comes back
+//                  transposed (ds_read_b64_tr_b16) as the A operand (row = d).
+// O^T lives in 4*D/16 accumulator registers per lane whatever the number of rows.
+// At the end the LF_DW waves are merged through LDS with the (offset, sum, acc)
+// log-sum-exp combine; with nsplit > 1 the workgroup writes its partial to
+// scratch and lf_attn_decode_combine merges the splits.
 
-#ifndef LF_ROWS
-#define LF_ROWS 1
-#endif
 #ifndef LF_DW
 #define LF_DW 4              /* waves per workgroup */
 #endif
+#ifndef LF_LAZY_LOG2
+#define LF_LAZY_LOG2 8       /* slack of the softmax exponent offset, log2 units */
+#endif
 #define LF_DT (LF_DW * 64)
 #define LF_D LF_HEAD_DIM
-#define LF_NJ (LF_D / 32)    /* 16-byte pieces of a row held by one lane */
+#define LF_NJ (LF_D / 32)    /* 16-byte pieces of a row held by one lane = k-steps of QK^T */
+#define LF_NDB (LF_D / 16)   /* 16-row blocks of O^T */
+#define LF_QROWS 16          /* query rows one unit can hold (MFMA N) */
+#define LF_OSTRIDE (LF_D + 4) /* floats per row of the merge buffer */
 
-struct LfDecStep {
+struct LfDecStage {
   lf_u32x4 k[LF_NJ];
   lf_u32x4 v[LF_NJ];
 };
+struct LfDecIds {            // page ids of one step
+  long long k, v;
+};
 
 extern "C" __global__ void __launch_bounds__(LF_DT, 2) lf_attn_decode(const LfAttnParams p) {
-  // merge buffer: [LF_DW*16 (wave, token lane)][LF_D] floats for one row at a time
-  __shared__ float red[LF_DW * 16 * LF_D];
-  __shared__ float red_m[LF_DW][LF_ROWS];
-  __shared__ float red_l[LF_DW][LF_ROWS];
-  __shared__ float part_sum[LF_DT / LF_D][LF_D];
+  // One buffer, two lives: wave-private V tiles of the pair being consumed
+  // ([LF_DW][2][16*D] elements) during the loop, merge buffer
+  // ([LF_DW][16][LF_OSTRIDE] floats) after it.
+  constexpr int kVBytes = LF_DW * 2 * 16 * LF_D * 2;
+  constexpr int kOBytes = LF_DW * LF_QROWS * LF_OSTRIDE * 4;
+  __shared__ __attribute__((aligned(16))) unsigned char smem[kVBytes > kOBytes ? kVBytes : kOBytes];
+  __shared__ float red_m[LF_DW][LF_QROWS];
+  __shared__ float red_l[LF_DW][LF_QROWS];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int t = lane & 15;
+  const int c = lane & 15;      // token of a step (loads) / query column (MFMA results)
   const int g = lane >> 4;
 
   const int unit = blockIdx.x;
   const int z = blockIdx.y;
-  const int chunks = (p.rows + LF_ROWS - 1) / LF_ROWS;   // row chunks per (b, kv head)
+  const int chunks = (p.rows + LF_QROWS - 1) / LF_QROWS;   // row chunks per (b, kv head)
   const int rc = unit % chunks;
   const int bh = unit / chunks;
   const int hkv = bh % p.Hkv;
   const int b = bh / p.Hkv;
-  const int row0 = rc * LF_ROWS;                           // first query row of this unit
+  const int row0 = rc * LF_QROWS;
+  const int nrows = min(p.rows - row0, LF_QROWS);          // query rows of this unit
 
   const int tok_begin = z * p.split_len;
   const int tok_end = min(tok_begin + p.split_len, p.Sk);
-  const int nsteps = (max(tok_end - tok_begin, 0) + 15) / 16;
+  const int npairs = (max(tok_end - tok_begin, 0) + 31) / 32;
 
-  // ---- A operand: Q rows replicated, lane (m = lane%16, g) holds
-  // Q[row0 + m % LF_ROWS][32*j + 8*g .. +7].  Query row r of the unit is the
-  // tensor row (head = hkv*rows + r) when Sq == 1, i.e. Q viewed [B, Hkv, rows, D].
-  lf_elem8 qa[LF_NJ];
+  // ---- B operand of S^T = K Q^T: lane (q = c, g) holds Q[row0 + q][32*j + 8*g .. +7];
+  // columns past nrows are zero
+  lf_elem8 qb[LF_NJ];
   {
-    int r = row0 + (t % LF_ROWS);
-    if (r >= p.rows) r = p.rows - 1;
-    const lf_elem* qrow = p.q + (long long)b * p.q_sb + (long long)hkv * p.q_sh + (long long)r * p.q_ss;
+    const lf_elem* qrow = p.q + (long long)b * p.q_sb + (long long)hkv * p.q_sh +
+                          (long long)(row0 + min(c, nrows - 1)) * p.q_ss;
 #pragma unroll
-    for (int j = 0; j < LF_NJ; ++j)
-      qa[j] = __builtin_bit_cast(lf_elem8, *reinterpret_cast<const lf_u32x4*>(qrow + 32 * j + 8 * g));
+    for (int j = 0; j < LF_NJ; ++j) {
+      lf_u32x4 raw = *reinterpret_cast<const lf_u32x4*>(qrow + 32 * j + 8 * g);
+      if (c >= nrows) raw = lf_u32x4{0u, 0u, 0u, 0u};
+      qb[j] = __builtin_bit_cast(lf_elem8, raw);
+    }
   }
 
 #if LF_SOFTCAP
@@ -84,162 +100,225 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 2) lf_attn_decode(const LfAt
   const float cexp = p.scale * LF_LOG2E;
 #endif
 
-  float m_run[LF_ROWS], l_run[LF_ROWS];
-  float acc[LF_ROWS][LF_NJ][8];
+  lf_f32x4 o[LF_NDB];          // O^T: lane (q = c, g) holds d = 16*db + 4*g + i
 #pragma unroll
-  for (int r = 0; r < LF_ROWS; ++r) {
-    m_run[r] = LF_NEG_INF;
-    l_run[r] = 0.0f;
-#pragma unroll
-    for (int j = 0; j < LF_NJ; ++j)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc[r][j][e] = 0.0f;
-  }
+  for (int db = 0; db < LF_NDB; ++db) o[db] = lf_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  float mc = LF_NEG_INF;       // exponent offset of column q (same in all 4 lane groups)
+  float l_part = 0.0f;         // this lane's share of the sum
 
-  // ---- token stream of this wave: steps wave, wave + LF_DW, ...
-  auto step_tok = [&](int s) { return tok_begin + 16 * s + t; };
-  auto row_ptrs = [&](int s, const lf_elem*& kp, const lf_elem*& vp) {
-    int tok = min(step_tok(s), p.Sk - 1);      // clamp: masked later, never out of bounds
-    kp = lf_kv_row(p, 0, b, hkv, tok) + 8 * g;
-    vp = lf_kv_row(p, 1, b, hkv, tok) + 8 * g;
-  };
-  auto issue = [&](LfDecStep& st, const lf_elem* kp, const lf_elem* vp) {
-#pragma unroll
-    for (int j = 0; j < LF_NJ; ++j) st.k[j] = *reinterpret_cast<const lf_u32x4*>(kp + 32 * j);
-#pragma unroll
-    for (int j = 0; j < LF_NJ; ++j) st.v[j] = *reinterpret_cast<const lf_u32x4*>(vp + 32 * j);
-  };
-  auto consume = [&](const LfDecStep& st, int s) {
-    lf_f32x4 sc = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-    for (int j = 0; j < LF_NJ; ++j) sc = lf_mfma16(qa[j], __builtin_bit_cast(lf_elem8, st.k[j]), sc);
-    const bool valid = step_tok(s) < tok_end;
-    float vf[LF_NJ][8];
-#pragma unroll
-    for (int j = 0; j < LF_NJ; ++j) {
-      lf_elem8 ve = __builtin_bit_cast(lf_elem8, st.v[j]);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) vf[j][e] = lf_to_float(ve[e]);
+  // ---- addressing
+  constexpr bool kPagedK = (LF_PAGED & 1) != 0;
+  constexpr bool kPagedV = (LF_PAGED & 2) != 0;
+  // pages of >= 16 tokens: a 16-token step lies inside one page, the id is wave-uniform
+  constexpr bool kUniformPage = (LF_PAGE_SIZE % 16) == 0;
+  auto step_tok0 = [&](int st) { return tok_begin + 16 * st; };
+  auto fetch_ids = [&](int st) {
+    LfDecIds id = {0, 0};
+    if (kPagedK || kPagedV) {
+      // clamp: steps past the end re-read the last page (their scores are masked)
+      const int tok = min(step_tok0(st) + (kUniformPage ? 0 : c), p.Sk - 1);
+      const int pi = tok / LF_PAGE_SIZE;
+      if (kPagedK) id.k = reinterpret_cast<const lf_table_t*>(p.k_table)[(long long)b * p.kt_stride + pi];
+      if (kPagedV) id.v = reinterpret_cast<const lf_table_t*>(p.v_table)[(long long)b * p.vt_stride + pi];
     }
-#pragma unroll
-    for (int r = 0; r < LF_ROWS; ++r) {
-      float x = sc[r];                         // C row 4*g + r holds query row r (replicated)
-#if LF_SOFTCAP
-      x = p.softcap * lf_tanh(x * sc_in);
-#endif
-      x = valid ? x : LF_NEG_INF;
-      const float m_new = fmaxf(m_run[r], x);
-      const float m_sub = (m_new == LF_NEG_INF) ? 0.0f : m_new;
-      const float mc = m_sub * cexp;
-      const float resc = lf_exp2(m_run[r] * cexp - mc);
-      const float pe = lf_exp2(x * cexp - mc);
-      m_run[r] = m_new;
-      l_run[r] = l_run[r] * resc + pe;
-#pragma unroll
-      for (int j = 0; j < LF_NJ; ++j)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[r][j][e] = acc[r][j][e] * resc + pe * vf[j][e];
-    }
+    return id;
   };
-
-  {
-    LfDecStep st0, st1;
+  auto issue = [&](LfDecStage& sg, int st, const LfDecIds& id) {
+    const int tok = min(step_tok0(st) + c, p.Sk - 1);      // clamp: masked later, never out of bounds
     const lf_elem *kp, *vp;
-    int s = wave;
-    if (s < nsteps) {
-      row_ptrs(s, kp, vp);
-      issue(st0, kp, vp);
-    }
-    // two steps per trip so both register stages have static names
-    for (; s < nsteps; s += 2 * LF_DW) {
-      const int s1 = s + LF_DW;
-      const int s2 = s + 2 * LF_DW;
-      if (s1 < nsteps) {
-        row_ptrs(s1, kp, vp);
-        issue(st1, kp, vp);
-      }
-      consume(st0, s);
-      if (s2 < nsteps) {
-        row_ptrs(s2, kp, vp);
-        issue(st0, kp, vp);
-      }
-      if (s1 < nsteps) consume(st1, s1);
-    }
-  }
+    if (kPagedK)
+      kp = p.k + id.k * p.k_sb + (long long)(tok % LF_PAGE_SIZE) * p.k_ss + (long long)hkv * p.k_sh + 8 * g;
+    else
+      kp = p.k + (long long)b * p.k_sb + (long long)hkv * p.k_sh + (long long)tok * p.k_ss + 8 * g;
+    if (kPagedV)
+      vp = p.v + id.v * p.v_sb + (long long)(tok % LF_PAGE_SIZE) * p.v_ss + (long long)hkv * p.v_sh + 8 * g;
+    else
+      vp = p.v + (long long)b * p.v_sb + (long long)hkv * p.v_sh + (long long)tok * p.v_ss + 8 * g;
+#pragma unroll
+    for (int j = 0; j < LF_NJ; ++j) sg.k[j] = *reinterpret_cast<const lf_u32x4*>(kp + 32 * j);
+#pragma unroll
+    for (int j = 0; j < LF_NJ; ++j) sg.v[j] = *reinterpret_cast<const lf_u32x4*>(vp + 32 * j);
+  };
 
-  // ---- merge the 16 token lanes x LF_DW waves.  (m, l) do not depend on g.
-  float m_wg[LF_ROWS], l_wg[LF_ROWS];
-#pragma unroll
-  for (int r = 0; r < LF_ROWS; ++r) {
-    float mw = m_run[r];
-#pragma unroll
-    for (int off = 1; off < 16; off <<= 1) mw = fmaxf(mw, __shfl_xor(mw, off, 64));
-    if (lane == 0) red_m[wave][r] = mw;
-  }
-  __syncthreads();
-#pragma unroll
-  for (int r = 0; r < LF_ROWS; ++r) {
-    float mw = red_m[0][r];
-#pragma unroll
-    for (int w = 1; w < LF_DW; ++w) mw = fmaxf(mw, red_m[w][r]);
-    m_wg[r] = mw;
-    const float m_sub = (mw == LF_NEG_INF) ? 0.0f : mw;
-    const float f = lf_exp2(m_run[r] * cexp - m_sub * cexp);   // 0 for lanes that saw nothing
-    float lw = l_run[r] * f;
-#pragma unroll
-    for (int off = 1; off < 16; off <<= 1) lw += __shfl_xor(lw, off, 64);
-    if (lane == 0) red_l[wave][r] = lw;
-#pragma unroll
-    for (int j = 0; j < LF_NJ; ++j)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc[r][j][e] *= f;
-  }
-  __syncthreads();
-#pragma unroll
-  for (int r = 0; r < LF_ROWS; ++r) {
-    float lw = red_l[0][r];
-#pragma unroll
-    for (int w = 1; w < LF_DW; ++w) lw += red_l[w][r];
-    l_wg[r] = lw;
-  }
-
-  const int dcol = tid % LF_D;          // column this thread sums in the merge
-  const int part = tid / LF_D;          // which slice of the (wave, lane) rows
-  constexpr int kParts = LF_DT / LF_D;  // 2 for D = 128 with 256 threads
-  constexpr int kRowsPerPart = LF_DW * 16 / kParts;
-#pragma unroll
-  for (int r = 0; r < LF_ROWS; ++r) {
-    __syncthreads();
+  lf_elem* my_v = reinterpret_cast<lf_elem*>(smem) + wave * 2 * 16 * LF_D;
+  // V rows of a step -> wave-private LDS tile hsel (row = token c, 16-byte chunk
+  // 4j+g, chunk index XORed with 2*(row&3) so that the 4 rows a transposed read
+  // touches sit on different banks)
+  auto stash_v = [&](const LfDecStage& sg, int hsel) {
 #pragma unroll
     for (int j = 0; j < LF_NJ; ++j) {
-      float* dst = &red[(wave * 16 + t) * LF_D + 32 * j + 8 * g];
-      *reinterpret_cast<lf_f32x4*>(dst) = lf_f32x4{acc[r][j][0], acc[r][j][1], acc[r][j][2], acc[r][j][3]};
-      *reinterpret_cast<lf_f32x4*>(dst + 4) = lf_f32x4{acc[r][j][4], acc[r][j][5], acc[r][j][6], acc[r][j][7]};
+      const int ch = (4 * j + g) ^ (2 * (c & 3));
+      *reinterpret_cast<lf_u32x4*>(&my_v[hsel * 16 * LF_D + c * LF_D + 8 * ch]) = sg.v[j];
     }
-    __syncthreads();
-    float sum = 0.0f;
-#pragma unroll 8
-    for (int i = 0; i < kRowsPerPart; ++i) sum += red[(part * kRowsPerPart + i) * LF_D + dcol];
-    if (kParts > 1) {
-      part_sum[part][dcol] = sum;
-      __syncthreads();
-      if (part == 0) {
+  };
+
+  // ---- one pair of steps (32 tokens)
+  auto consume = [&](const LfDecStage& sa, const LfDecStage& sb, int pr) {
+    lf_f32x4 xa = {0.0f, 0.0f, 0.0f, 0.0f}, xb = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int q = 1; q < kParts; ++q) sum += part_sum[q][dcol];
+    for (int j = 0; j < LF_NJ; ++j) {
+      xa = lf_mfma16(__builtin_bit_cast(lf_elem8, sa.k[j]), qb[j], xa);
+      xb = lf_mfma16(__builtin_bit_cast(lf_elem8, sb.k[j]), qb[j], xb);
+    }
+    stash_v(sa, 0);
+    stash_v(sb, 1);
+
+    // lane (q = c, g): xa[i] is token t0 + i, xb[i] token t0 + 16 + i
+    const int t0 = step_tok0(2 * pr) + 4 * g;
+    float x[8];
+    float mx = LF_NEG_INF;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float s = (i < 4) ? xa[i] : xb[i - 4];
+#if LF_SOFTCAP
+      s = p.softcap * lf_tanh(s * sc_in);
+#endif
+      const int tok = t0 + (i < 4 ? i : 12 + i);
+      x[i] = (tok < tok_end) ? s * cexp : LF_NEG_INF;
+      mx = fmaxf(mx, x[i]);
+    }
+    if (__builtin_amdgcn_ballot_w64(mx > mc + (float)LF_LAZY_LOG2) != 0ull) {
+      // bring the column's offset up to its max over all four lane groups
+      float mq = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mq = fmaxf(mq, __shfl_xor(mq, 32, 64));
+      const float m_new = fmaxf(mc, mq);
+      const float r = (m_new == LF_NEG_INF) ? 1.0f : lf_exp2(mc - m_new);
+      mc = m_new;
+      l_part *= r;
+#pragma unroll
+      for (int db = 0; db < LF_NDB; ++db) o[db] *= r;
+    }
+    const float m_sub = (mc == LF_NEG_INF) ? 0.0f : mc;
+    lf_elem8 pb;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float e = lf_exp2(x[i] - m_sub);
+      l_part += e;
+      pb[i] = lf_from_float(e);
+    }
+
+    // O^T += V^T P^T: k-slot s of lane group g is token 4g + s (s < 4) of the first
+    // step and 4g + s - 4 of the second -- the order pb is held in
+    const int trow = 4 * g + (c >> 2);          // row this lane addresses for its 16-lane group
+#pragma unroll
+    for (int db = 0; db < LF_NDB; ++db) {
+      const int col = 16 * db + 4 * (c & 3);
+      const int ch = (col / 8) ^ (2 * (trow & 3));
+      lf_elem8 a;
+#pragma unroll
+      for (int hsel = 0; hsel < 2; ++hsel) {
+        const lf_elem* src = &my_v[hsel * 16 * LF_D + trow * LF_D + 8 * ch + (col % 8)];
+        lf_s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_s16x4*)(src));
+        lf_elem4 te = __builtin_bit_cast(lf_elem4, t);
+        a[4 * hsel + 0] = te[0];
+        a[4 * hsel + 1] = te[1];
+        a[4 * hsel + 2] = te[2];
+        a[4 * hsel + 3] = te[3];
+      }
+      o[db] = lf_mfma16(a, pb, o[db]);
+    }
+  };
+
+  // ---- streaming loop: this wave's pairs are wave, wave + LF_DW, ...; four register
+  // stages (two pairs) rotate, two trips of the pipeline per loop iteration so every
+  // stage has a static name
+  {
+    LfDecStage s0, s1, s2, s3;
+    LfDecIds i0, i1, i2, i3;
+    int pr = wave;
+    i0 = fetch_ids(2 * pr);
+    i1 = fetch_ids(2 * pr + 1);
+    i2 = fetch_ids(2 * (pr + LF_DW));
+    i3 = fetch_ids(2 * (pr + LF_DW) + 1);
+    if (pr < npairs) {
+      issue(s0, 2 * pr, i0);
+      issue(s1, 2 * pr + 1, i1);
+      i0 = fetch_ids(2 * (pr + 2 * LF_DW));
+      i1 = fetch_ids(2 * (pr + 2 * LF_DW) + 1);
+    }
+    if (pr + LF_DW < npairs) {
+      issue(s2, 2 * (pr + LF_DW), i2);
+      issue(s3, 2 * (pr + LF_DW) + 1, i3);
+      i2 = fetch_ids(2 * (pr + 3 * LF_DW));
+      i3 = fetch_ids(2 * (pr + 3 * LF_DW) + 1);
+    }
+    for (; pr < npairs; pr += 2 * LF_DW) {
+      consume(s0, s1, pr);
+      const int pa = pr + 2 * LF_DW;
+      if (pa < npairs) {
+        issue(s0, 2 * pa, i0);
+        issue(s1, 2 * pa + 1, i1);
+        i0 = fetch_ids(2 * (pa + 2 * LF_DW));
+        i1 = fetch_ids(2 * (pa + 2 * LF_DW) + 1);
+      }
+      const int pb2 = pr + LF_DW;
+      if (pb2 < npairs) {
+        consume(s2, s3, pb2);
+        const int pc = pb2 + 2 * LF_DW;
+        if (pc < npairs) {
+          issue(s2, 2 * pc, i2);
+          issue(s3, 2 * pc + 1, i3);
+          i2 = fetch_ids(2 * (pc + 2 * LF_DW));
+          i3 = fetch_ids(2 * (pc + 2 * LF_DW) + 1);
+        }
       }
     }
-    const int qr = row0 + r;
-    if (part == 0 && qr < p.rows) {
-      if (p.nsplit == 1) {
-        lf_elem* orow = p.o + (long long)b * p.o_sb + (long long)hkv * p.o_sh + (long long)qr * p.o_ss;
-        orow[dcol] = lf_from_float(sum / l_wg[r]);
-      } else {
-        const long long slot = ((long long)bh * p.rows + qr) * p.nsplit + z;
-        p.part_acc[slot * LF_D + dcol] = sum;
-        if (dcol == 0) {
-          p.part_ml[slot * 2 + 0] = m_wg[r] * cexp;   // in exponent units (log2 domain)
-          p.part_ml[slot * 2 + 1] = l_wg[r];
-        }
+  }
+
+  // ---- merge: lane groups (sum), then the LF_DW waves
+  float l_wave = l_part + __shfl_xor(l_part, 16, 64);
+  l_wave += __shfl_xor(l_wave, 32, 64);
+  if (g == 0) {
+    red_m[wave][c] = mc;
+    red_l[wave][c] = l_wave;
+  }
+  __syncthreads();   // also: every wave is done with its V tiles, smem changes role
+  float* red_o = reinterpret_cast<float*>(smem);
+  {
+    float m_wg = red_m[0][c];
+#pragma unroll
+    for (int w = 1; w < LF_DW; ++w) m_wg = fmaxf(m_wg, red_m[w][c]);
+    const float m_sub = (m_wg == LF_NEG_INF) ? 0.0f : m_wg;
+    const float f = lf_exp2(mc - m_sub);        // 0 for a wave that saw nothing
+#pragma unroll
+    for (int db = 0; db < LF_NDB; ++db)
+      *reinterpret_cast<lf_f32x4*>(&red_o[(wave * LF_QROWS + c) * LF_OSTRIDE + 16 * db + 4 * g]) = o[db] * f;
+  }
+  __syncthreads();
+  // thread -> (query row qi, 8 consecutive d's)
+  for (int item = tid; item < LF_QROWS * LF_D / 8; item += LF_DT) {
+    const int qi = item / (LF_D / 8);
+    const int d0 = (item % (LF_D / 8)) * 8;
+    if (qi >= nrows) continue;
+    float m_all = red_m[0][qi];
+#pragma unroll
+    for (int w = 1; w < LF_DW; ++w) m_all = fmaxf(m_all, red_m[w][qi]);
+    const float ms = (m_all == LF_NEG_INF) ? 0.0f : m_all;
+    float l_tot = 0.0f;
+#pragma unroll
+    for (int w = 0; w < LF_DW; ++w) l_tot += red_l[w][qi] * lf_exp2(red_m[w][qi] - ms);
+    float sum[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sum[e] = 0.0f;
+#pragma unroll
+    for (int w = 0; w < LF_DW; ++w)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sum[e] += red_o[(w * LF_QROWS + qi) * LF_OSTRIDE + d0 + e];
+    const int qr = row0 + qi;
+    if (p.nsplit == 1) {
+      lf_elem* orow = p.o + (long long)b * p.o_sb + (long long)hkv * p.o_sh + (long long)qr * p.o_ss;
+      const float inv = 1.0f / l_tot;
+      lf_elem8 w8;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) w8[e] = lf_from_float(sum[e] * inv);
+      *reinterpret_cast<lf_elem8*>(orow + d0) = w8;
+    } else {
+      const long long slot = ((long long)bh * p.rows + qr) * p.nsplit + z;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) p.part_acc[slot * LF_D + d0 + e] = sum[e];
+      if (d0 == 0) {
+        p.part_ml[slot * 2 + 0] = m_all;       // exponent offset, log2 units
+        p.part_ml[slot * 2 + 1] = l_tot;
       }
     }
   }

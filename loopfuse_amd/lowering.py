@@ -28,6 +28,7 @@ from . import runtime
 from .skip import TILE_SHAPES
 
 MASK_NONE, MASK_CAUSAL, MASK_SLIDING = 0, 1, 2
+DECODE_QROWS = 16    # query rows one decode unit holds (the MFMA N dimension)
 _MASK_NAMES = {"none": MASK_NONE, None: MASK_NONE, "causal": MASK_CAUSAL, "sliding": MASK_SLIDING}
 _DTYPE_CODE = {torch.bfloat16: 0, torch.float16: 1}
 
@@ -61,7 +62,7 @@ class KernelSpec:
     paged: int = 0         # bit 0: K paged, bit 1: V paged
     page_size: int = 1
     table_i64: bool = False
-    rows: int = 1          # decode: query rows sharing K/V (1, 2, 4)
+    rows: int = 1          # decode: query rows a unit can hold (fixed, the MFMA N dimension)
     waves: int = 4         # decode: waves per workgroup
     v_tr: bool = True      # prefill: transposed LDS reads for V
     extra: tuple = ()      # further -D options (tuning experiments)
@@ -77,7 +78,7 @@ class KernelSpec:
             f"-DLF_TABLE_I64={int(self.table_i64)}",
         ]
         if self.family == "decode":
-            o += [f"-DLF_ROWS={self.rows}", f"-DLF_DW={self.waves}"]
+            o += [f"-DLF_DW={self.waves}"]
         elif self.family == "prefill":
             o += [f"-DLF_V_TR={int(self.v_tr)}"]
         return o + list(self.extra)
@@ -314,7 +315,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     # ---- family: decode when there is no mask and few query rows share a KV head
     family = force_family
     if family is None:
-        few = (Sq == 1 and group <= 16) or (group == 1 and Sq <= 16)
+        few = (Sq == 1 and group <= 64) or (group == 1 and Sq <= 16)
         family = "decode" if (mask == MASK_NONE and few and Sk >= 16) else "prefill"
     keep = (q, k, v, out, kt, vt)  # noqa: F841  (tensors stay alive until the launch is queued)
 
@@ -354,15 +355,16 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         P.o_sb, P.o_sh, P.o_ss = out.stride(0), out.stride(1), out.stride(2)
     else:
         raise UnsupportedPlan("decode needs Sq == 1 or group == 1")
-    krows = 4 if rows >= 3 else rows
-    chunks = (rows + krows - 1) // krows
+    chunks = (rows + DECODE_QROWS - 1) // DECODE_QROWS
     units = B * Hkv * chunks
     nsplit = num_splits if num_splits else decode_split(units, Sk)
-    split_len = ((Sk + nsplit - 1) // nsplit + 15) // 16 * 16
+    split_len = ((Sk + nsplit - 1) // nsplit + 31) // 32 * 32     # whole pairs of 16-token steps
     nsplit = (Sk + split_len - 1) // split_len
     P.rows, P.nsplit, P.split_len = rows, nsplit, split_len
     spec = KernelSpec("decode", _DTYPE_CODE[dtype], D, MASK_NONE, plan.softcap is not None, paged,
-                      page_size, table_i64, rows=krows, waves=4)
+                      page_size, table_i64, rows=DECODE_QROWS,
+                      waves=int(os.environ.get("LOOPFUSE_DECODE_WAVES", "4")),
+                      extra=tuple(os.environ.get("LOOPFUSE_KOPTS", "").split()))
     if nsplit > 1:
         nrow = B * Hkv * rows * nsplit
         scratch = _get_scratch(q.device, nrow * (D + 2))
