@@ -102,6 +102,8 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="time only one of the two kernels (profiling aid)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 512 MiB device copy (reference point for FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--workload", default="c2", help="prefill workload: c2 | c2_softcap | c3")
     ap.add_argument("--decode-workload", default="c5", help="decode workload: c5 | c4")
     args = ap.parse_args()
@@ -119,6 +121,15 @@ def main() -> int:
 
     dev = torch.device("cuda:0")
     out: dict = {}
+
+    if args.copy_calibration:
+        # a kernel whose HBM traffic is known exactly: 512 MiB read + 512 MiB written
+        src = torch.empty(512 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     pre = None
     if args.only in (None, "prefill"):

@@ -34,6 +34,9 @@
 #ifndef LF_SCHED
 #define LF_SCHED 1       /* pin read/MFMA interleaving with sched_group_barrier */
 #endif
+#ifndef LF_TIMING
+#define LF_TIMING 0      /* profiling aid: per-phase s_memtime totals of one wave into part_acc */
+#endif
 #ifndef LF_ABLATE
 #define LF_ABLATE 0      /* profiling aid: 1 = no softmax math, 2 = no staging/barrier, 4 = no PV, 8 = no QK^T (results are wrong) */
 #endif
@@ -58,22 +61,45 @@
 #define LF_NKS (LF_D / 16)                   /* k-steps of the QK^T product   */
 #define LF_NDB (LF_D / 32)                   /* 32-row blocks of O^T          */
 #define LF_NKK (LF_BN / 16)                  /* k-steps of the PV product     */
+// LDS row strides (elements).  LF_PAD: rows are padded instead of XOR-swizzled, so
+// every fragment address is one per-lane base plus a compile-time offset (no
+// per-fragment address arithmetic): +16 bytes per K row spreads 16 consecutive
+// rows over all 64 banks for ds_read_b128, +64 bytes per V row does the same for
+// the 4 rows x 64 bytes a transposed read touches.
+#ifndef LF_PAD
+#define LF_PAD 0
+#endif
+#if LF_PAD
+#define LF_KS (LF_D + 8)
+#define LF_VS (LF_D + 32)
+#else
+#define LF_KS LF_D
+#define LF_VS LF_D
+#endif
 
 // Physical 16-byte chunk of logical chunk `ch` in row `row` of the K tile: rows
 // that a ds_read_b128 touches together (16 consecutive rows, same logical chunk)
 // land in 16 different chunks, i.e. on all 64 banks.
 __device__ __forceinline__ int lf_k_phys(int row, int ch) {
+#if LF_PAD
+  return ch;
+#else
   return ch ^ ((row / LF_RPS) & (LF_CPR - 1));
+#endif
 }
 // Same for the V tile, where a transposed read touches 4 consecutive rows x 64
 // contiguous bytes per 32 lanes: permute the 64-byte groups by the row.
 __device__ __forceinline__ int lf_v_phys(int row, int ch) {
+#if LF_PAD
+  return ch;
+#else
   return ch ^ (4 * ((row / LF_RPS) & (LF_CPR / 4 - 1)));
+#endif
 }
 
 extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(const LfAttnParams p) {
-  __shared__ __attribute__((aligned(16))) lf_elem lds_k[2][LF_BN * LF_D];
-  __shared__ __attribute__((aligned(16))) lf_elem lds_v[2][LF_BN * LF_D];
+  __shared__ __attribute__((aligned(16))) lf_elem lds_k[2][LF_BN * LF_KS];
+  __shared__ __attribute__((aligned(16))) lf_elem lds_v[2][LF_BN * LF_VS];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -85,22 +111,27 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
   // to the 8 XCDs, so ids with equal id%8 share an L2: keep all q tiles of one
   // (batch, head) on one XCD, heaviest (latest) q tile first.
   const int nqt = (p.Sq + LF_BM - 1) / LF_BM;
+  const int npair = (nqt + 1) / 2;
   const int nbh = p.B * p.Hq;
   const int xcd = blockIdx.x & 7;
   const int slot = blockIdx.x >> 3;
   // within an XCD: groups of 4 (batch, head) pairs (their K/V fit the 4 MB L2
-  // together), each group dealt heaviest q tile first across its 4 members
-  const int grp = slot / (4 * nqt);
-  const int in_grp = slot % (4 * nqt);
+  // together); a workgroup takes q tile nqt-1-i and then q tile i of its (batch,
+  // head), so that under a causal mask every workgroup walks the same number of
+  // KV tiles (2(i+1) + 2(nqt-i) of them) and the grid has no long tail
+  const int grp = slot / (4 * npair);
+  const int in_grp = slot % (4 * npair);
   const int bh = (grp * 4 + (in_grp & 3)) * 8 + xcd;
   if (bh >= nbh) return;
-  const int qt = nqt - 1 - (in_grp >> 2);
+  const int pair = in_grp >> 2;
   const int b = bh / p.Hq;
   const int h = bh % p.Hq;
   const int hkv = h / (p.Hq / p.Hkv);
+  const int nkt = (p.Sk + LF_BN - 1) / LF_BN;
+
+  auto run_q_tile = [&](const int qt) {
   const int q0 = qt * LF_BM;
   const int qlast = min(q0 + LF_BM, p.Sq) - 1;
-  const int nkt = (p.Sk + LF_BN - 1) / LF_BN;
 
   // ---- block skip: KV tiles [kt_begin, kt_end) are those with at least one
   // unmasked (i, j) for rows q0..qlast.
@@ -188,8 +219,8 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
 #pragma unroll
     for (int ps = 0; ps < LF_NPASS; ++ps) {
       const int row = srow + kRowsPerPass * ps;
-      *reinterpret_cast<lf_u32x4*>(&lds_k[buf][row * LF_D + 8 * lf_k_phys(row, sch)]) = kst[ps];
-      *reinterpret_cast<lf_u32x4*>(&lds_v[buf][row * LF_D + 8 * lf_v_phys(row, sch)]) = vst[ps];
+      *reinterpret_cast<lf_u32x4*>(&lds_k[buf][row * LF_KS + 8 * lf_k_phys(row, sch)]) = kst[ps];
+      *reinterpret_cast<lf_u32x4*>(&lds_v[buf][row * LF_VS + 8 * lf_v_phys(row, sch)]) = vst[ps];
     }
   };
 
@@ -199,6 +230,13 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
   store_tile(0);
   __syncthreads();
 
+#if LF_TIMING
+  unsigned long long tacc[6] = {0, 0, 0, 0, 0, 0};
+#define LF_T(i) { unsigned long long now_ = __builtin_amdgcn_s_memtime(); tacc[i] += now_ - tprev; tprev = now_; }
+  unsigned long long tprev = __builtin_amdgcn_s_memtime();
+#else
+#define LF_T(i)
+#endif
   for (int kt = kt_begin; kt < kt_end; ++kt) {
     const int cur = (kt - kt_begin) & 1;
     const bool have_next = kt + 1 < kt_end;
@@ -218,6 +256,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
     full = full && (wq0 + 31 - k0 < p.window);
 #endif
 
+    LF_T(0)
     if (need) {
       const lf_elem* kbuf = lds_k[cur];
       const lf_elem* vbuf = lds_v[cur];
@@ -240,7 +279,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
         auto k_frag = [&](int f) {
           const int ks = f / LF_NKB, kb = f % LF_NKB;
           const int row = 32 * kb + l32;
-          return *reinterpret_cast<const lf_u32x4*>(&kbuf[row * LF_D + 8 * lf_k_phys(row, 2 * ks + g)]);
+          return *reinterpret_cast<const lf_u32x4*>(&kbuf[row * LF_KS + 8 * lf_k_phys(row, 2 * ks + g)]);
         };
 #pragma unroll
         for (int f = 0; f < LF_KPF && f < kNF; ++f) kf[f] = k_frag(f);
@@ -264,6 +303,10 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
       __builtin_amdgcn_s_setprio(0);
 #endif
 
+#if LF_TIMING
+      asm volatile("" :: "v"(s[0][0]), "v"(s[LF_NKB - 1][15]));   // results needed here
+#endif
+      LF_T(1)
       // ---- score modifications and mask; element i of block kb is kv index
       // j = k0 + 32*kb + 8*(i/4) + 4*g + i%4, query my_q.
 #if LF_SOFTCAP
@@ -336,6 +379,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
         }
       l_run += rs;
 
+      LF_T(2)
 #if LF_SETPRIO
       __builtin_amdgcn_s_setprio(2);
 #endif
@@ -357,7 +401,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
 #pragma unroll
           for (int half = 0; half < 2; ++half) {
             const int row = 16 * kk + 8 * half + 4 * g + (j16 >> 2);
-            const lf_elem* src = &vbuf[row * LF_D + 8 * lf_v_phys(row, col / 8) + (col % 8)];
+            const lf_elem* src = &vbuf[row * LF_VS + 8 * lf_v_phys(row, col / 8) + (col % 8)];
             lf_s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                 (__attribute__((address_space(3))) lf_s16x4*)(src));
             lf_elem4 te = __builtin_bit_cast(lf_elem4, t);
@@ -371,7 +415,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
 #pragma unroll
           for (int sl = 0; sl < 8; ++sl) {
             const int row = 16 * kk + 8 * (sl / 4) + 4 * g + (sl % 4);
-            a[sl] = vbuf[row * LF_D + 8 * lf_v_phys(row, col / 8) + (col % 8)];
+            a[sl] = vbuf[row * LF_VS + 8 * lf_v_phys(row, col / 8) + (col % 8)];
           }
 #endif
           return a;
@@ -398,11 +442,23 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
 #endif
     }
 
+#if LF_TIMING
+    asm volatile("" :: "v"(o[0][0]), "v"(o[LF_NDB - 1][15]));
+#endif
+    LF_T(3)
 #if !(LF_ABLATE & 2)
     if (have_next) store_tile(cur ^ 1);
+    LF_T(4)
     __syncthreads();
+    LF_T(5)
 #endif
   }
+#if LF_TIMING
+  if (blockIdx.x == 8 * 5 && tid == 0 && p.part_acc != nullptr) {
+    for (int i = 0; i < 6; ++i) p.part_acc[i] += (float)tacc[i];
+    p.part_acc[6] += (float)(kt_end - kt_begin);
+  }
+#endif
 
   // ---- epilogue: O[q][d] = O^T[d][q] / l.  Element i of block db is
   // d = 32*db + 8*(i/4) + 4*g + i%4.
@@ -420,4 +476,8 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
         *reinterpret_cast<lf_elem4*>(orow + 32 * db + 8 * i4 + 4 * g) = w;
       }
   }
+  };   // run_q_tile
+
+  run_q_tile(nqt - 1 - pair);
+  if (pair != nqt - 1 - pair) run_q_tile(pair);
 }

@@ -125,6 +125,11 @@ def compile_spec(spec: KernelSpec, arch: str = runtime.DEFAULT_ARCH) -> Compiled
     """hipRTC-compile (or fetch from the on-disk cache) one specialisation.  Needs no GPU."""
     with _lock:
         ck = _compiled.get(spec)
+        override = os.environ.get("LOOPFUSE_HSACO_" + spec.family.upper())   # tuning aid: prebuilt code object
+        if ck is None and override:
+            with open(override, "rb") as fh:
+                ck = CompiledKernel(spec, fh.read(), False, "override " + override)
+            _compiled[spec] = ck
         if ck is None:
             code, hit, log = runtime.compile_source(spec.source(), spec.name(), spec.options(), arch)
             ck = CompiledKernel(spec, code, hit, log)
@@ -209,12 +214,14 @@ def _get_scratch(device: torch.device, nfloats: int) -> torch.Tensor:
 
 
 def decode_split(units: int, Sk: int, cus: int = 256) -> int:
-    """Number of KV splits across workgroups: enough workgroups for ~4 per CU,
-    but at least 256 tokens per split."""
+    """Number of KV splits across workgroups.  One workgroup (4 waves) per unit is
+    enough once there are two workgroups per CU (8 resident waves, each with 32 KB
+    of loads in flight); below that the KV range is split, down to 256 tokens per
+    split, and a second kernel merges the partial results."""
     env = os.environ.get("LOOPFUSE_DECODE_SPLITS")
     if env:
         return max(1, int(env))
-    want = max(1, (4 * cus + units - 1) // units)
+    want = max(1, (2 * cus + units - 1) // units)
     most = max(1, Sk // 256)
     return max(1, min(want, most))
 
@@ -327,6 +334,9 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         spec = KernelSpec(family, _DTYPE_CODE[dtype], D, mask, plan.softcap is not None, paged,
                           page_size, table_i64, v_tr=v_tr if family == "prefill" else True,
                           extra=tuple(os.environ.get("LOOPFUSE_KOPTS", "").split()))
+        if os.environ.get("LOOPFUSE_TIMING"):       # profiling aid, see LF_TIMING in the kernel
+            attention.timing = torch.zeros(16, dtype=torch.float32, device=q.device)
+            P.part_acc = attention.timing.data_ptr()
         bm, bn = TILE_SHAPES[family]
         nqt = (Sq + bm - 1) // bm
         nkt = (Sk + bn - 1) // bn
@@ -336,7 +346,9 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
             P.visits = visits.data_ptr()
         # 8 XCD classes x (batch*head pairs per class, padded to the kernel's groups of 4) x q tiles
         per_xcd = (B * Hq + 7) // 8
-        grid = 8 * ((per_xcd + 3) // 4 * 4) * nqt
+        # lf_attn_prefill takes two q tiles (heavy + light) per workgroup
+        per_bh = (nqt + 1) // 2 if family == "prefill" else nqt
+        grid = 8 * ((per_xcd + 3) // 4 * 4) * per_bh
         get_kernel(spec, spec.entry()).launch((grid, 1, 1), (256, 1, 1), P)
         return (out, visits) if record_visits else out
 

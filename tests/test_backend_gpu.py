@@ -1,0 +1,191 @@
+"""torch.compile(backend=loopfuse_backend) on the GPU: the graphs of the reference's
+own accuracy tests (tests/test_accuracy.py:125-311) and of its benchmark
+(tests/benchmark.py:78-84, 141-147, 216-226, 400-406) must take the fused HIP
+path (checked through interface.stats, so an eager fallback cannot pass) and match
+the CPU fp32 oracle within the bf16 tolerance.  Graphs the backend does not lower
+(the reference's add / matmul+add / biased attention cases) must still be right.
+"""
+import pytest
+import torch
+
+import loopfuse_amd
+from loopfuse_amd import loopfuse_backend
+from loopfuse_amd.torch_backend import interface
+from oracle import attention_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+TOL = 2e-2
+
+
+def rand(shape, dtype=torch.bfloat16, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(shape, generator=g, dtype=torch.float32).to(dtype)
+
+
+def run_fused(fn, inputs, mode=None):
+    torch._dynamo.reset()
+    before = dict(interface.stats)
+    out = torch.compile(fn, backend=loopfuse_backend, dynamic=True, mode=mode)(*[t.to(DEV) for t in inputs])
+    torch.cuda.synchronize()
+    assert interface.stats["fused"] == before["fused"] + 1, "the fused HIP path was not taken"
+    assert interface.stats["eager_graph"] == before["eager_graph"]
+    assert interface.stats["eager_runtime"] == before["eager_runtime"]
+    return out.float().cpu()
+
+
+@pytest.mark.parametrize("S", [256, 593])
+def test_standard_attn(S):
+    def fn(Q, K, V):
+        QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        return torch.softmax(torch.ops.loopfuse.causal_mask(QK), dim=-1) @ V
+
+    Q, K, V = (rand((4, 8, S, 64), seed=s) for s in (1, 2, 3))
+    torch._dynamo.mark_static(Q, 3)
+    torch._dynamo.mark_dynamic(Q, 2)
+    got = run_fused(fn, (Q, K, V))
+    assert (got - O.attention_reference(Q, K, V, mask="causal")).abs().max() <= TOL
+
+
+def test_gqa_attn():
+    def fn(Q, K, V):
+        g = Q.shape[1] // K.shape[1]
+        K = K.repeat_interleave(g, dim=1)
+        V = V.repeat_interleave(g, dim=1)
+        QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        return torch.softmax(torch.ops.loopfuse.causal_mask(QK), dim=-1) @ V
+
+    Q = rand((4, 8, 1024, 64), seed=1)
+    K, V = (rand((4, 4, 1024, 64), seed=s) for s in (2, 3))
+    got = run_fused(fn, (Q, K, V))
+    assert (got - O.attention_reference(Q, K, V, mask="causal")).abs().max() <= TOL
+
+
+def test_sliding_mask_softcap_gqa():
+    def fn(Q, K, V):
+        g = Q.shape[1] // K.shape[1]
+        K = K.repeat_interleave(g, dim=1)
+        V = V.repeat_interleave(g, dim=1)
+        QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        QK = torch.tanh(QK / 30) * 30
+        return torch.softmax(torch.ops.loopfuse.sliding_mask(QK, 256), dim=-1) @ V
+
+    Q = rand((2, 32, 1024, 128), seed=1)
+    K, V = (rand((2, 8, 1024, 128), seed=s) for s in (2, 3))
+    got = run_fused(fn, (Q, K, V), mode="max-autotune")
+    want = O.attention_reference(Q, K, V, mask="sliding", window=256, softcap=30.0)
+    assert (got - want).abs().max() <= TOL
+
+
+def test_paged_attention_k_only():
+    def fn(Q, K_cache, K_block_table, V):
+        K = torch.ops.loopfuse.paged_load(K_cache, K_block_table).transpose(1, 2)
+        QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        return torch.softmax(torch.ops.loopfuse.causal_mask(QK), dim=-1) @ V
+
+    B, H, S, D = 4, 8, 1024, 64
+    n = B * S * 2
+    Kc = rand((n, H, D), seed=1)
+    tab = torch.randint(0, n, (B, S), generator=torch.Generator().manual_seed(5), dtype=torch.int32)
+    Q, V = rand((B, H, S, D), seed=2), rand((B, H, S, D), seed=3)
+    got = run_fused(fn, (Q, Kc, tab, V))
+    want = O.attention_reference(Q, Kc, V, mask="causal", k_table=tab)
+    assert (got - want).abs().max() <= TOL
+
+
+def test_paged_decode_gqa_reference_format():
+    # tests/benchmark.py:400-443: one-token pages, Q viewed [B, Hkv, group, D]
+    def fn(Q, Kc, kt, Vc, vt):
+        K = torch.ops.loopfuse.paged_load(Kc, kt).transpose(-3, -2)
+        V = torch.ops.loopfuse.paged_load(Vc, vt).transpose(-3, -2)
+        QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        return torch.softmax(QK, dim=-1) @ V
+
+    B, Hkv, grp, S, D = 8, 4, 8, 2048, 128
+    n = B * S * 2
+    Kc, Vc = rand((n, Hkv, D), seed=1), rand((n, Hkv, D), seed=2)
+    g = torch.Generator().manual_seed(5)
+    kt = torch.randint(0, n, (B, S), generator=g, dtype=torch.int32)
+    vt = torch.randint(0, n, (B, S), generator=g, dtype=torch.int32)
+    Q = rand((B, Hkv, grp, D), seed=3)
+    got = run_fused(fn, (Q, Kc, kt, Vc, vt))
+    want = O.attention_reference(Q, Kc, Vc, k_table=kt, v_table=vt)
+    assert (got - want).abs().max() <= TOL
+
+
+def test_paged_decode_page16_config5_shape():
+    def fn(Q, Kc, kt, Vc, vt):
+        B, pages = kt.shape
+        P, H, D = Kc.shape[1:]
+        K = torch.ops.loopfuse.paged_load(Kc, kt).reshape(B, pages * P, H, D).transpose(1, 2)
+        V = torch.ops.loopfuse.paged_load(Vc, vt).reshape(B, pages * P, H, D).transpose(1, 2)
+        g = Q.shape[1] // H
+        K = K.repeat_interleave(g, dim=1)
+        V = V.repeat_interleave(g, dim=1)
+        QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        return torch.softmax(QK, dim=-1) @ V
+
+    from loopfuse_amd import workloads
+    w = workloads.make("c5", seed=4, B=8, S=1024)
+    got = run_fused(fn, (w.q, w.k, w.k_table, w.v, w.v_table))
+    want = O.attention_reference(w.q, w.k, w.v, k_table=w.k_table, v_table=w.v_table)
+    assert (got - want).abs().max() <= TOL
+
+
+def test_decode_contiguous():
+    def fn(Q, K, V):
+        QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        return torch.softmax(QK, dim=-1) @ V
+
+    Q = rand((8, 32, 1, 128), seed=1)
+    K, V = (rand((8, 32, 2048, 128), seed=s) for s in (2, 3))
+    got = run_fused(fn, (Q, K, V))
+    assert (got - O.attention_reference(Q, K, V)).abs().max() <= TOL
+
+
+def test_recompile_free_new_sequence_length():
+    """Sequence length is a kernel argument: a second length reuses the code object."""
+    from loopfuse_amd import lowering
+
+    def fn(Q, K, V):
+        QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        return torch.softmax(torch.ops.loopfuse.causal_mask(QK), dim=-1) @ V
+
+    torch._dynamo.reset()
+    cf = torch.compile(fn, backend=loopfuse_backend, dynamic=True)
+    outs = []
+    for S in (384, 640):
+        Q, K, V = (rand((2, 4, S, 128), seed=s) for s in (1, 2, 3))
+        torch._dynamo.mark_dynamic(Q, 2)
+        n_before = len(lowering._compiled)
+        o = cf(Q.to(DEV), K.to(DEV), V.to(DEV)).float().cpu()
+        assert (o - O.attention_reference(Q, K, V, mask="causal")).abs().max() <= TOL
+        outs.append(len(lowering._compiled) - n_before)
+    assert outs[1] == 0
+
+
+@pytest.mark.parametrize("which", ["add", "matmul_add", "modified_attn", "softmax_matmul"])
+def test_unlowered_graphs_still_correct(which):
+    """Reference tests/test_accuracy.py:29-82, 172-211: not attention-shaped for this
+    backend; they run unfused and must still be numerically right."""
+    if which == "add":
+        fn = lambda a, b: a + b
+        ins = (rand((4, 1024, 128), torch.float32, 1), rand((4, 1024, 128), torch.float32, 2))
+    elif which == "matmul_add":
+        fn = lambda a, b, c: a @ b + c
+        ins = (rand((256, 128), torch.float32, 1), rand((128, 128), torch.float32, 2), rand((256, 128), torch.float32, 3))
+    elif which == "modified_attn":
+        def fn(Q, K, V, qb, sb, ob):
+            QK = (Q + qb) @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+            QK = QK * 3.5 + sb
+            return torch.softmax(torch.ops.loopfuse.causal_mask(QK), dim=-1) @ V + ob
+        ins = tuple(rand((2, 2, 128, 64), torch.float32, s) for s in (1, 2, 3, 4)) + \
+            (rand((2, 2, 128, 128), torch.float32, 5), rand((2, 2, 128, 64), torch.float32, 6))
+    else:
+        fn = lambda x, y: torch.softmax(x, dim=-1) @ y
+        ins = (rand((2, 4, 128, 64), torch.float32, 1), rand((2, 4, 64, 128), torch.float32, 2))
+    torch._dynamo.reset()
+    dev_ins = [t.to(DEV) for t in ins]
+    want = fn(*dev_ins)
+    got = torch.compile(fn, backend=loopfuse_backend, dynamic=True)(*dev_ins)
+    torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-4)
