@@ -27,6 +27,9 @@ if ROOT not in sys.path:
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16/fp16, published
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, published
+# HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by a plain copy of known
+# size (profiles/*_hbm_traffic.md); counters cannot be read from inside this process
+TRAFFIC_BYTES = {"c2": (449 + 128) * (1 << 20), "c5": (514 + 1) * (1 << 20)}
 
 
 def time_gpu(fn, steps: int, warmup: int):
@@ -162,14 +165,15 @@ def main() -> int:
             "value": tflops, "unit": "TFLOP/s",
         })
         out["roofline"] = {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                           "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                           "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": TRAFFIC_BYTES.get(args.workload),
                            "kernel": "lf_attn_prefill", "us_per_launch": pre["sec"] * 1e6}
     if dec is not None:
         gbs = dec["bytes"] / dec["sec"] / 1e9
         d = {"workload": dec["workload"], "value": gbs, "unit": "GB/s", "us_per_launch": dec["sec"] * 1e6,
              "host_us_per_launch": dec["wall_sec"] * 1e6, "kv_pool_rotation": dec["rotation"],
              "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                          "frac": gbs / HBM_PEAK_GBS, "traffic": None, "kernel": "lf_attn_decode(+combine)"}}
+                          "frac": gbs / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES.get(args.decode_workload),
+                          "kernel": "lf_attn_decode"}}
         if pre is None:
             out.update({"metric": "prefill TFLOP/s + decode HBM GB/s on 1 MI355X (% of roofline)",
                         "value": gbs, "unit": "GB/s", "roofline": d["roofline"]})

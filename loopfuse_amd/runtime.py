@@ -182,9 +182,17 @@ def device_count() -> int:
 
 
 def read_kernel_source(*files: str) -> str:
-    """Concatenate building-block files from csrc/kernels into one hipRTC translation unit."""
+    """Concatenate building-block files from csrc/kernels into one hipRTC translation unit.
+
+    With ``USE_HARDCODE_KERNEL=1`` a file ``hardcode_kernel.hip`` in the current
+    directory replaces the last (kernel) file -- the debugging hook the reference
+    offers with ``hardcode_kernel.py`` (``loopfuse/torch_backend/interface.py:606-613``).
+    """
     parts = []
-    for f in files:
-        with open(os.path.join(KERNEL_DIR, f), "r") as fh:
-            parts.append(f"// ---- {f}\n" + fh.read())
+    hard = os.path.join(os.getcwd(), "hardcode_kernel.hip")
+    use_hard = os.environ.get("USE_HARDCODE_KERNEL", "0") == "1" and os.path.exists(hard)
+    for i, f in enumerate(files):
+        path = hard if (use_hard and i == len(files) - 1) else os.path.join(KERNEL_DIR, f)
+        with open(path, "r") as fh:
+            parts.append(f"// ---- {os.path.basename(path)}\n" + fh.read())
     return "\n".join(parts)
