@@ -34,6 +34,9 @@
 #ifndef LF_SCHED
 #define LF_SCHED 1       /* pin read/MFMA interleaving with sched_group_barrier */
 #endif
+#ifndef LF_KVBUF
+#define LF_KVBUF 1       /* dense K/V staged with range-checked buffer loads (needs < 2 GiB per (batch, head) span) */
+#endif
 #ifndef LF_TIMING
 #define LF_TIMING 0      /* profiling aid: per-phase s_memtime totals of one wave into part_acc */
 #endif
@@ -44,15 +47,17 @@
 #define LF_LAZY_LOG2 8   /* slack of the softmax exponent offset, log2 units */
 #endif
 
-#define LF_BM 128
 #ifndef LF_BN
 #define LF_BN 64
 #endif
 #ifndef LF_OCC
 #define LF_OCC 2    /* waves per SIMD the register budget is set for */
 #endif
-#define LF_NW 4
+#ifndef LF_NW
+#define LF_NW 4     /* waves per workgroup (4 or 8) */
+#endif
 #define LF_NT (LF_NW * 64)
+#define LF_BM (32 * LF_NW)
 #define LF_D LF_HEAD_DIM
 #define LF_CPR (LF_D / 8)                    /* 16-byte chunks per K/V row    */
 #define LF_RPS (256 / (LF_D * 2))            /* rows per 256-byte bank span   */
@@ -183,35 +188,47 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
   float mc_ref = LF_NEG_INF;  // exponent offset of this query in log2 units (a lagging running max)
   float l_run = 0.0f;         // this lane's share of the running sum
 
-  // ---- staging: thread handles chunk (row0 + 16*ps*LF_RPS.., ch) of every pass.
-  // Dense K/V: address = wave-uniform base (batch, head, tile, pass) + a fixed
-  // 32-bit per-thread offset, so the loop carries no 64-bit address arithmetic.
+  // ---- staging: thread handles chunk (srow + kRowsPerPass*ps, sch) of every pass.
+  // Dense K/V go through buffer loads: one resource per tensor covering rows
+  // 0..Sk-1 of this (batch, kv head); the byte offset (a fixed per-thread part plus
+  // a uniform tile/pass part) is range-checked by the hardware, so rows past Sk read
+  // as zeros (their scores are masked, their probabilities exactly 0) and the loop
+  // carries one 32-bit add per load instead of 64-bit address arithmetic.
+  // Paged K/V: plain global loads through the page table, rows clamped to Sk-1.
   lf_u32x4 kst[LF_NPASS], vst[LF_NPASS];
   constexpr int kRowsPerPass = LF_NT / LF_CPR;
   const int srow = tid / LF_CPR;
   const int sch = tid % LF_CPR;
   const lf_elem* k_uni = p.k + (long long)b * p.k_sb + (long long)hkv * p.k_sh;
   const lf_elem* v_uni = p.v + (long long)b * p.v_sb + (long long)hkv * p.v_sh;
-  const unsigned k_toff = (unsigned)(srow * p.k_ss) + 8u * sch;
-  const unsigned v_toff = (unsigned)(srow * p.v_ss) + 8u * sch;
+#if LF_KVBUF
+  const unsigned k_bytes = (unsigned)(((long long)(p.Sk - 1) * p.k_ss + LF_D) * 2);
+  const unsigned v_bytes = (unsigned)(((long long)(p.Sk - 1) * p.v_ss + LF_D) * 2);
+  const __amdgpu_buffer_rsrc_t k_rs = __builtin_amdgcn_make_buffer_rsrc((void*)k_uni, 0, (int)k_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc((void*)v_uni, 0, (int)v_bytes, 0x00020000);
+  const unsigned k_toff = ((unsigned)(srow * p.k_ss) + 8u * sch) * 2u;      // bytes
+  const unsigned v_toff = ((unsigned)(srow * p.v_ss) + 8u * sch) * 2u;
+  const unsigned k_rowb = (unsigned)p.k_ss * 2u, v_rowb = (unsigned)p.v_ss * 2u;
+#endif
   auto load_tile = [&](int kt) {
-    const bool tail = (kt + 1) * LF_BN > p.Sk;          // uniform
 #pragma unroll
     for (int ps = 0; ps < LF_NPASS; ++ps) {
       const int r0 = kt * LF_BN + kRowsPerPass * ps;    // uniform
-      if ((LF_PAGED & 1) || tail) {
-        // rows past the end re-read the last row: their scores are masked (j >= Sk)
-        // and their probabilities are exactly 0, so any finite data will do
+      if ((LF_PAGED & 1) || !LF_KVBUF) {
         const int tok = min(r0 + srow, p.Sk - 1);
         kst[ps] = *reinterpret_cast<const lf_u32x4*>(lf_kv_row(p, 0, b, hkv, tok) + 8 * sch);
       } else {
-        kst[ps] = *reinterpret_cast<const lf_u32x4*>(k_uni + (long long)r0 * p.k_ss + k_toff);
+#if LF_KVBUF
+        kst[ps] = __builtin_amdgcn_raw_buffer_load_b128(k_rs, k_toff + (unsigned)r0 * k_rowb, 0, 0);
+#endif
       }
-      if ((LF_PAGED & 2) || tail) {
+      if ((LF_PAGED & 2) || !LF_KVBUF) {
         const int tok = min(r0 + srow, p.Sk - 1);
         vst[ps] = *reinterpret_cast<const lf_u32x4*>(lf_kv_row(p, 1, b, hkv, tok) + 8 * sch);
       } else {
-        vst[ps] = *reinterpret_cast<const lf_u32x4*>(v_uni + (long long)r0 * p.v_ss + v_toff);
+#if LF_KVBUF
+        vst[ps] = __builtin_amdgcn_raw_buffer_load_b128(v_rs, v_toff + (unsigned)r0 * v_rowb, 0, 0);
+#endif
       }
     }
   };

@@ -331,13 +331,22 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     if family in ("prefill", "prefill_pipe"):
         P.q_sb, P.q_sh, P.q_ss = q.stride(0), q.stride(1), q.stride(2)
         P.o_sb, P.o_sh, P.o_ss = out.stride(0), out.stride(1), out.stride(2)
+        extra = tuple(os.environ.get("LOOPFUSE_KOPTS", "").split())
+        # buffer loads address a (batch, kv head) span with 32-bit byte offsets
+        span = max((Sk - 1) * abs(P.k_ss), (Sk - 1) * abs(P.v_ss)) * 2 + 2 * D
+        if family == "prefill" and span >= (1 << 31):
+            extra += ("-DLF_KVBUF=0",)
         spec = KernelSpec(family, _DTYPE_CODE[dtype], D, mask, plan.softcap is not None, paged,
-                          page_size, table_i64, v_tr=v_tr if family == "prefill" else True,
-                          extra=tuple(os.environ.get("LOOPFUSE_KOPTS", "").split()))
+                          page_size, table_i64, v_tr=v_tr if family == "prefill" else True, extra=extra)
         if os.environ.get("LOOPFUSE_TIMING"):       # profiling aid, see LF_TIMING in the kernel
             attention.timing = torch.zeros(16, dtype=torch.float32, device=q.device)
             P.part_acc = attention.timing.data_ptr()
         bm, bn = TILE_SHAPES[family]
+        nw = 4
+        for e in spec.extra:                    # tuning: -DLF_NW=8 doubles the q tile
+            if e.startswith("-DLF_NW="):
+                nw = int(e.split("=")[1])
+                bm = 32 * nw
         nqt = (Sq + bm - 1) // bm
         nkt = (Sk + bn - 1) // bn
         visits = None
@@ -349,7 +358,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         # lf_attn_prefill takes two q tiles (heavy + light) per workgroup
         per_bh = (nqt + 1) // 2 if family == "prefill" else nqt
         grid = 8 * ((per_xcd + 3) // 4 * 4) * per_bh
-        get_kernel(spec, spec.entry()).launch((grid, 1, 1), (256, 1, 1), P)
+        get_kernel(spec, spec.entry()).launch((grid, 1, 1), (64 * nw, 1, 1), P)
         return (out, visits) if record_visits else out
 
     if family != "decode":
