@@ -32,11 +32,18 @@
 #define LF_VPF 4         /* V fragments (two transposed reads each) in flight */
 #endif
 #ifndef LF_SCHED
-#define LF_SCHED 1       /* pin read/MFMA interleaving with sched_group_barrier */
+#define LF_SCHED 0       /* 1: pin read/MFMA interleaving with sched_group_barrier (measured slower) */
 #endif
 #ifndef LF_KVBUF
 #define LF_KVBUF 1       /* dense K/V staged with range-checked buffer loads (needs < 2 GiB per (batch, head) span) */
 #endif
+#ifndef LF_DMA
+#define LF_DMA 0   /* 1 (needs LF_KVBUF, no LF_PAD): dense K/V tiles go global -> LDS directly
+                      (buffer_load ... lds through inline asm); parity-clean, no faster than the
+                      register path on the measured shapes, so off by default */
+#endif
+#define LF_DMA_K (LF_DMA && !(LF_PAGED & 1))
+#define LF_DMA_V (LF_DMA && !(LF_PAGED & 2))
 #ifndef LF_TIMING
 #define LF_TIMING 0      /* profiling aid: per-phase s_memtime totals of one wave into part_acc */
 #endif
@@ -210,10 +217,42 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
   const unsigned v_toff = ((unsigned)(srow * p.v_ss) + 8u * sch) * 2u;
   const unsigned k_rowb = (unsigned)p.k_ss * 2u, v_rowb = (unsigned)p.v_ss * 2u;
 #endif
-  auto load_tile = [&](int kt) {
+#if LF_DMA
+  // Direct global -> LDS staging: a wave-level buffer_load_dwordx4 ... lds writes
+  // 64 lanes x 16 B to LDS at M0 + 16*lane, i.e. 64/LF_CPR whole rows of the
+  // (unpadded, row-major) tile; the XOR swizzle is applied on the global side: the
+  // lane that lands on physical chunk `sch` fetches logical chunk sch ^ swizzle(row).
+  // No staging registers, no ds_write, and rows past Sk arrive as zeros.
+  lf_u32x4 k_rsq, v_rsq;
+  {
+    const unsigned long long ka = (unsigned long long)k_uni, va = (unsigned long long)v_uni;
+    k_rsq[0] = __builtin_amdgcn_readfirstlane((unsigned)ka);
+    k_rsq[1] = __builtin_amdgcn_readfirstlane((unsigned)(ka >> 32) & 0xffffu);
+    k_rsq[2] = __builtin_amdgcn_readfirstlane(k_bytes);
+    k_rsq[3] = 0x00020000u;
+    v_rsq[0] = __builtin_amdgcn_readfirstlane((unsigned)va);
+    v_rsq[1] = __builtin_amdgcn_readfirstlane((unsigned)(va >> 32) & 0xffffu);
+    v_rsq[2] = __builtin_amdgcn_readfirstlane(v_bytes);
+    v_rsq[3] = 0x00020000u;
+  }
+  const unsigned k_doff = (unsigned)srow * k_rowb + 16u * (unsigned)lf_k_phys(srow, sch);
+  const unsigned v_doff = (unsigned)srow * v_rowb + 16u * (unsigned)lf_v_phys(srow, sch);
+  constexpr int kRowsPerWave = 64 / LF_CPR;
+  auto dma = [&](const lf_u32x4& rs, unsigned voff, const lf_elem* lds_row0) {
+    const unsigned m0v = __builtin_amdgcn_readfirstlane(
+        (unsigned)(size_t)(__attribute__((address_space(3))) const void*)lds_row0);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :: "s"(m0v), "v"(voff), "s"(rs) : "memory");
+  };
+#endif
+  auto load_tile = [&](int kt, int buf) {
 #pragma unroll
     for (int ps = 0; ps < LF_NPASS; ++ps) {
       const int r0 = kt * LF_BN + kRowsPerPass * ps;    // uniform
+      (void)buf;
+#if LF_DMA_K
+      dma(k_rsq, k_doff + (unsigned)r0 * k_rowb, &lds_k[buf][(kRowsPerPass * ps + kRowsPerWave * wave) * LF_KS]);
+#else
       if ((LF_PAGED & 1) || !LF_KVBUF) {
         const int tok = min(r0 + srow, p.Sk - 1);
         kst[ps] = *reinterpret_cast<const lf_u32x4*>(lf_kv_row(p, 0, b, hkv, tok) + 8 * sch);
@@ -222,6 +261,10 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
         kst[ps] = __builtin_amdgcn_raw_buffer_load_b128(k_rs, k_toff + (unsigned)r0 * k_rowb, 0, 0);
 #endif
       }
+#endif
+#if LF_DMA_V
+      dma(v_rsq, v_doff + (unsigned)r0 * v_rowb, &lds_v[buf][(kRowsPerPass * ps + kRowsPerWave * wave) * LF_VS]);
+#else
       if ((LF_PAGED & 2) || !LF_KVBUF) {
         const int tok = min(r0 + srow, p.Sk - 1);
         vst[ps] = *reinterpret_cast<const lf_u32x4*>(lf_kv_row(p, 1, b, hkv, tok) + 8 * sch);
@@ -230,20 +273,29 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
         vst[ps] = __builtin_amdgcn_raw_buffer_load_b128(v_rs, v_toff + (unsigned)r0 * v_rowb, 0, 0);
 #endif
       }
+#endif
     }
   };
   auto store_tile = [&](int buf) {
 #pragma unroll
     for (int ps = 0; ps < LF_NPASS; ++ps) {
       const int row = srow + kRowsPerPass * ps;
+      (void)row;
+#if !LF_DMA_K
       *reinterpret_cast<lf_u32x4*>(&lds_k[buf][row * LF_KS + 8 * lf_k_phys(row, sch)]) = kst[ps];
+#endif
+#if !LF_DMA_V
       *reinterpret_cast<lf_u32x4*>(&lds_v[buf][row * LF_VS + 8 * lf_v_phys(row, sch)]) = vst[ps];
+#endif
     }
+#if LF_DMA_K || LF_DMA_V
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's direct-to-LDS loads have landed
+#endif
   };
 
   // every valid q tile has at least one KV tile (kt_end >= 1 > kt_begin is not
   // guaranteed only for Sk == 0, which the host rejects)
-  load_tile(kt_begin);
+  load_tile(kt_begin, 0);
   store_tile(0);
   __syncthreads();
 
@@ -258,7 +310,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
     const int cur = (kt - kt_begin) & 1;
     const bool have_next = kt + 1 < kt_end;
 #if !(LF_ABLATE & 2)
-    if (have_next) load_tile(kt + 1);
+    if (have_next) load_tile(kt + 1, cur ^ 1);
 #endif
 
     const int k0 = kt * LF_BN;
@@ -299,10 +351,10 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
           return *reinterpret_cast<const lf_u32x4*>(&kbuf[row * LF_KS + 8 * lf_k_phys(row, 2 * ks + g)]);
         };
 #pragma unroll
-        for (int f = 0; f < LF_KPF && f < kNF; ++f) kf[f] = k_frag(f);
+        for (int f = 0; f < LF_KPF && f < kNF; ++f) kf[f] = (LF_ABLATE & 16) ? __builtin_bit_cast(lf_u32x4, qf[f % LF_NKS]) : k_frag(f);
 #pragma unroll
         for (int f = 0; f < kNF; ++f) {
-          if (f + LF_KPF < kNF) kf[f + LF_KPF] = k_frag(f + LF_KPF);
+          if (f + LF_KPF < kNF) kf[f + LF_KPF] = (LF_ABLATE & 16) ? __builtin_bit_cast(lf_u32x4, qf[f % LF_NKS]) : k_frag(f + LF_KPF);
           s[f % LF_NKB] = lf_mfma32(__builtin_bit_cast(lf_elem8, kf[f]), qf[f / LF_NKB], s[f % LF_NKB]);
         }
 #if LF_SCHED
@@ -438,10 +490,10 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
           return a;
         };
 #pragma unroll
-        for (int f = 0; f < LF_VPF && f < kNF; ++f) vf[f] = v_frag(f);
+        for (int f = 0; f < LF_VPF && f < kNF; ++f) vf[f] = (LF_ABLATE & 32) ? qf[f % LF_NKS] : v_frag(f);
 #pragma unroll
         for (int f = 0; f < kNF; ++f) {
-          if (f + LF_VPF < kNF) vf[f + LF_VPF] = v_frag(f + LF_VPF);
+          if (f + LF_VPF < kNF) vf[f + LF_VPF] = (LF_ABLATE & 32) ? qf[f % LF_NKS] : v_frag(f + LF_VPF);
           o[f % LF_NDB] = lf_mfma32(vf[f], pf[f / LF_NDB], o[f % LF_NDB]);
         }
 #if LF_SCHED && LF_V_TR

@@ -110,9 +110,16 @@ __device__ __forceinline__ lf_f32x4 lf_mfma16(lf_elem8 a, lf_elem8 b, lf_f32x4 c
 #endif
 }
 
-// Value held by the lane 32 positions away (lane l <-> lane l ^ 32).
+// Value held by the lane 32 positions away (lane l <-> lane l ^ 32): one
+// v_permlane32_swap (VALU) instead of a round trip through the LDS crossbar.
 __device__ __forceinline__ float lf_swap32(float x) {
-  return __shfl_xor(x, 32, 64);
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  // swaps the upper half of the first operand with the lower half of the second:
+  // with both operands = x, result[0] holds x of lane^32 in lanes 32..63 and
+  // result[1] holds it in lanes 0..31
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const unsigned other = (__lane_id() < 32) ? r[1] : r[0];
+  return __builtin_bit_cast(float, other);
 }
 
 __device__ __forceinline__ float lf_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
