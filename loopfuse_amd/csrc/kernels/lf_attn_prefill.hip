@@ -40,8 +40,11 @@
 #ifndef LF_DMA
 #define LF_DMA 0   /* 1 (needs LF_KVBUF, no LF_PAD): dense K/V tiles go global -> LDS directly
                       (buffer_load ... lds through inline asm); parity-clean, no faster than the
-                      register path on the measured shapes, so off by default */
+                      register path on the measured shapes, so off by default.
+                      2: the same, with the loads of the next tile issued one pass at a time
+                      between the MFMAs of the current tile instead of in a burst at the top */
 #endif
+#define LF_DMA_SPREAD (LF_DMA == 2 && !LF_PAGED)
 #define LF_DMA_K (LF_DMA && !(LF_PAGED & 1))
 #define LF_DMA_V (LF_DMA && !(LF_PAGED & 2))
 #ifndef LF_TIMING
@@ -244,6 +247,16 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                  :: "s"(m0v), "v"(voff), "s"(rs) : "memory");
   };
+  // one staging pass (LF_BN / LF_NPASS rows) of tile kt into buffer buf; rows past
+  // Sk arrive as zeros, so a tile index past the last tile is harmless
+  auto dma_k_pass = [&](int kt, int buf, int ps) {
+    dma(k_rsq, k_doff + (unsigned)(kt * LF_BN + kRowsPerPass * ps) * k_rowb,
+        &lds_k[buf][(kRowsPerPass * ps + kRowsPerWave * wave) * LF_KS]);
+  };
+  auto dma_v_pass = [&](int kt, int buf, int ps) {
+    dma(v_rsq, v_doff + (unsigned)(kt * LF_BN + kRowsPerPass * ps) * v_rowb,
+        &lds_v[buf][(kRowsPerPass * ps + kRowsPerWave * wave) * LF_VS]);
+  };
 #endif
   auto load_tile = [&](int kt, int buf) {
 #pragma unroll
@@ -309,7 +322,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
   for (int kt = kt_begin; kt < kt_end; ++kt) {
     const int cur = (kt - kt_begin) & 1;
     const bool have_next = kt + 1 < kt_end;
-#if !(LF_ABLATE & 2)
+#if !(LF_ABLATE & 2) && !LF_DMA_SPREAD
     if (have_next) load_tile(kt + 1, cur ^ 1);
 #endif
 
@@ -356,6 +369,9 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
         for (int f = 0; f < kNF; ++f) {
           if (f + LF_KPF < kNF) kf[f + LF_KPF] = (LF_ABLATE & 16) ? __builtin_bit_cast(lf_u32x4, qf[f % LF_NKS]) : k_frag(f + LF_KPF);
           s[f % LF_NKB] = lf_mfma32(__builtin_bit_cast(lf_elem8, kf[f]), qf[f / LF_NKB], s[f % LF_NKB]);
+#if LF_DMA_SPREAD
+          if (f % (kNF / LF_NPASS) == 1) dma_k_pass(kt + 1, cur ^ 1, f / (kNF / LF_NPASS));
+#endif
         }
 #if LF_SCHED
         // pin the order: LF_KPF reads, then (MFMA, read) pairs, then the last MFMAs
@@ -495,6 +511,9 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
         for (int f = 0; f < kNF; ++f) {
           if (f + LF_VPF < kNF) vf[f + LF_VPF] = (LF_ABLATE & 32) ? qf[f % LF_NKS] : v_frag(f + LF_VPF);
           o[f % LF_NDB] = lf_mfma32(vf[f], pf[f / LF_NDB], o[f % LF_NDB]);
+#if LF_DMA_SPREAD
+          if (f % (kNF / LF_NPASS) == 1) dma_v_pass(kt + 1, cur ^ 1, f / (kNF / LF_NPASS));
+#endif
         }
 #if LF_SCHED && LF_V_TR
         __builtin_amdgcn_sched_group_barrier(0x100, 2 * LF_VPF, 0);
@@ -510,13 +529,22 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
       __builtin_amdgcn_s_setprio(0);
 #endif
     }
+#if LF_DMA_SPREAD
+    else {
+#pragma unroll
+      for (int ps = 0; ps < LF_NPASS; ++ps) {
+        dma_k_pass(kt + 1, cur ^ 1, ps);
+        dma_v_pass(kt + 1, cur ^ 1, ps);
+      }
+    }
+#endif
 
 #if LF_TIMING
     asm volatile("" :: "v"(o[0][0]), "v"(o[LF_NDB - 1][15]));
 #endif
     LF_T(3)
 #if !(LF_ABLATE & 2)
-    if (have_next) store_tile(cur ^ 1);
+    if (have_next || LF_DMA_SPREAD) store_tile(cur ^ 1);
     LF_T(4)
     __syncthreads();
     LF_T(5)

@@ -1,0 +1,424 @@
+// lf_attn_prefill_swp.hip — fused attention forward for gfx950 (prefill shapes),
+// software-pipelined variant of lf_attn_prefill.hip for dense K/V.
+//
+// Same math, layouts and operand orders as lf_attn_prefill.hip (4 waves x 32 query
+// rows, KV tiles of 64 rows, transposed problem S^T = K Q^T, O^T += V^T P^T,
+// XOR-swizzled LDS tiles, transposed V reads, lagging softmax offset, closed-form
+// tile bounds; reference loopfuse/compiler/passes/factor_acc.py:23-109,
+// loopfuse/compiler/passes/skip_loop_iterations.py:343-376).  What differs is when
+// memory operations are issued, so that a wave never waits for a memory round trip
+// at the head of an MFMA sequence and never stalls on a burst of loads:
+//
+//   * K/V tiles go global -> LDS directly (buffer_load_dwordx4 ... lds, range-checked,
+//     rows past Sk arrive as zeros).  The loads of K(i+2) and V(i+1) are issued one
+//     at a time BETWEEN the MFMAs of S^T(i); no staging registers, no LDS writes.
+//   * K lives in three LDS slots, V in two (80 KB, two workgroups per CU): K(i+1) is
+//     already resident while tile i is processed, so its first fragments are read
+//     during the last MFMAs of O^T(i), across the workgroup barrier.
+//   * the first V fragments of tile i are read during the last MFMAs of S^T(i), i.e.
+//     before the softmax that separates the two products.
+//   * the order of reads, loads and MFMAs is pinned with scheduling barriers.
+//
+// One workgroup barrier per tile; before it each wave waits for its own direct
+// loads (issued a full softmax + product earlier).
+
+#ifndef LF_LAZY_LOG2
+#define LF_LAZY_LOG2 8
+#endif
+#ifndef LF_KPF
+#define LF_KPF 6         /* K fragments in flight ahead of the MFMA consuming them */
+#endif
+#ifndef LF_VPF
+#define LF_VPF 4         /* V fragments (two transposed reads each) in flight */
+#endif
+#ifndef LF_SETPRIO
+#define LF_SETPRIO 1
+#endif
+#ifndef LF_ABLATE
+#define LF_ABLATE 0      /* profiling aid (wrong results): 1 no exp, 2 no direct loads, 16 no K reads,
+                            32 V fragments by one plain 16-byte read, 64 no V reads */
+#endif
+
+#define LF_NW 4
+#define LF_NT (LF_NW * 64)
+#define LF_BM (32 * LF_NW)
+#define LF_BN 64
+#define LF_KSLOTS 3
+#define LF_VSLOTS 2
+#define LF_D LF_HEAD_DIM
+#define LF_CPR (LF_D / 8)
+#define LF_RPS (256 / (LF_D * 2))
+#define LF_NPASS (LF_BN * LF_CPR / LF_NT)
+#define LF_NKB (LF_BN / 32)
+#define LF_NKS (LF_D / 16)
+#define LF_NDB (LF_D / 32)
+#define LF_NKK (LF_BN / 16)
+#define LF_NFK (LF_NKS * LF_NKB)      /* MFMAs (= K fragments) of S^T per tile */
+#define LF_NFV (LF_NKK * LF_NDB)      /* MFMAs (= V fragments) of O^T per tile */
+
+__device__ __forceinline__ int lf_k_phys(int row, int ch) {
+  return ch ^ ((row / LF_RPS) & (LF_CPR - 1));
+}
+__device__ __forceinline__ int lf_v_phys(int row, int ch) {
+  return ch ^ (4 * ((row / LF_RPS) & (LF_CPR / 4 - 1)));
+}
+
+// workgroup barrier that waits for this wave's direct-to-LDS loads but leaves LDS
+// reads in flight (the compiler's own barrier would wait for those too)
+#define LF_BARRIER_VM0() asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory")
+
+extern "C" __global__ void __launch_bounds__(LF_NT, 2) lf_attn_prefill_swp(const LfAttnParams p) {
+  __shared__ __attribute__((aligned(16))) lf_elem lds_k[LF_KSLOTS][LF_BN * LF_D];
+  __shared__ __attribute__((aligned(16))) lf_elem lds_v[LF_VSLOTS][LF_BN * LF_D];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int l32 = lane & 31;
+  const int g = lane >> 5;
+
+  // ---- workgroup -> (batch*head, pair of q tiles), as in lf_attn_prefill.hip
+  const int nqt = (p.Sq + LF_BM - 1) / LF_BM;
+  const int npair = (nqt + 1) / 2;
+  const int nbh = p.B * p.Hq;
+  const int xcd = blockIdx.x & 7;
+  const int slot = blockIdx.x >> 3;
+  const int grp = slot / (4 * npair);
+  const int in_grp = slot % (4 * npair);
+  const int bh = (grp * 4 + (in_grp & 3)) * 8 + xcd;
+  if (bh >= nbh) return;
+  const int pair = in_grp >> 2;
+  const int b = bh / p.Hq;
+  const int h = bh % p.Hq;
+  const int hkv = h / (p.Hq / p.Hkv);
+  const int nkt = (p.Sk + LF_BN - 1) / LF_BN;
+
+  // ---- direct-to-LDS staging: a wave-level load writes 64 lanes x 16 B at
+  // M0 + 16*lane, i.e. 64/LF_CPR whole rows of the row-major tile; the XOR swizzle
+  // is applied on the global side (the lane that lands on physical chunk c of row r
+  // fetches the logical chunk that lives there).
+  constexpr int kRowsPerPass = LF_NT / LF_CPR;
+  constexpr int kRowsPerWave = 64 / LF_CPR;
+  const int srow = tid / LF_CPR;
+  const int sch = tid % LF_CPR;
+  const lf_elem* k_uni = p.k + (long long)b * p.k_sb + (long long)hkv * p.k_sh;
+  const lf_elem* v_uni = p.v + (long long)b * p.v_sb + (long long)hkv * p.v_sh;
+  const unsigned k_bytes = (unsigned)(((long long)(p.Sk - 1) * p.k_ss + LF_D) * 2);
+  const unsigned v_bytes = (unsigned)(((long long)(p.Sk - 1) * p.v_ss + LF_D) * 2);
+  const unsigned k_rowb = (unsigned)p.k_ss * 2u, v_rowb = (unsigned)p.v_ss * 2u;
+  lf_u32x4 k_rsq, v_rsq;
+  {
+    const unsigned long long ka = (unsigned long long)k_uni, va = (unsigned long long)v_uni;
+    k_rsq[0] = __builtin_amdgcn_readfirstlane((unsigned)ka);
+    k_rsq[1] = __builtin_amdgcn_readfirstlane((unsigned)(ka >> 32) & 0xffffu);
+    k_rsq[2] = __builtin_amdgcn_readfirstlane(k_bytes);
+    k_rsq[3] = 0x00020000u;
+    v_rsq[0] = __builtin_amdgcn_readfirstlane((unsigned)va);
+    v_rsq[1] = __builtin_amdgcn_readfirstlane((unsigned)(va >> 32) & 0xffffu);
+    v_rsq[2] = __builtin_amdgcn_readfirstlane(v_bytes);
+    v_rsq[3] = 0x00020000u;
+  }
+  const unsigned k_doff = (unsigned)srow * k_rowb + 16u * (unsigned)lf_k_phys(srow, sch);
+  const unsigned v_doff = (unsigned)srow * v_rowb + 16u * (unsigned)lf_v_phys(srow, sch);
+  bool dma_on = true;
+  auto dma = [&](const lf_u32x4& rs, unsigned voff, const lf_elem* lds_row0) {
+    const unsigned m0v = __builtin_amdgcn_readfirstlane(
+        (unsigned)(size_t)(__attribute__((address_space(3))) const void*)lds_row0);
+#if LF_ABLATE & 2
+    if (dma_on)
+#endif
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :: "s"(m0v), "v"(voff), "s"(rs) : "memory");
+  };
+  auto dma_k_pass = [&](int kt, int sl, int ps) {
+    dma(k_rsq, k_doff + (unsigned)(kt * LF_BN + kRowsPerPass * ps) * k_rowb,
+        &lds_k[sl][(kRowsPerPass * ps + kRowsPerWave * wave) * LF_D]);
+  };
+  auto dma_v_pass = [&](int kt, int sl, int ps) {
+    dma(v_rsq, v_doff + (unsigned)(kt * LF_BN + kRowsPerPass * ps) * v_rowb,
+        &lds_v[sl][(kRowsPerPass * ps + kRowsPerWave * wave) * LF_D]);
+  };
+
+#if LF_SOFTCAP
+  const float sc_in = p.scale / p.softcap;
+  const float cexp = LF_LOG2E;
+#else
+  const float cexp = p.scale * LF_LOG2E;
+#endif
+
+  // per-lane fragment offsets (elements) inside a tile
+  auto k_off = [&](int f) {
+    const int ks = f / LF_NKB, kb = f % LF_NKB;
+    const int row = 32 * kb + l32;
+    return row * LF_D + 8 * lf_k_phys(row, 2 * ks + g);
+  };
+  auto k_frag = [&](const lf_elem* kbuf, int f) {
+#if LF_ABLATE & 16
+    lf_u32x4 z = {(unsigned)f, 1u, 2u, 3u};
+    return z;
+#else
+    return *reinterpret_cast<const lf_u32x4*>(&kbuf[k_off(f)]);
+#endif
+  };
+  // 16-lane group (2g + dh) asks for rows r0..r0+3, columns 32db+16dh..+15: lane j
+  // of the group supplies the 8-byte piece (row r0 + j/4, cols +4*(j%4)) and
+  // receives column j of the 4 rows.
+  auto v_frag = [&](const lf_elem* vbuf, int f) {
+    const int kk = f / LF_NDB, db = f % LF_NDB;
+    lf_elem8 a;
+#if LF_ABLATE & 64
+    for (int e = 0; e < 8; ++e) a[e] = (lf_elem)(float)(f + e);
+    return a;
+#elif LF_ABLATE & 32
+    return __builtin_bit_cast(lf_elem8, *reinterpret_cast<const lf_u32x4*>(&vbuf[k_off(f)]));
+#endif
+    const int j16 = lane & 15;
+    const int dh = (lane >> 4) & 1;
+    const int col = 32 * db + 16 * dh + 4 * (j16 & 3);
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int row = 16 * kk + 8 * half + 4 * g + (j16 >> 2);
+      const lf_elem* src = &vbuf[row * LF_D + 8 * lf_v_phys(row, col / 8) + (col % 8)];
+      lf_s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_s16x4*)(src));
+      lf_elem4 te = __builtin_bit_cast(lf_elem4, t);
+      a[4 * half + 0] = te[0];
+      a[4 * half + 1] = te[1];
+      a[4 * half + 2] = te[2];
+      a[4 * half + 3] = te[3];
+    }
+    return a;
+  };
+
+  auto run_q_tile = [&](const int qt) {
+    const int q0 = qt * LF_BM;
+    const int qlast = min(q0 + LF_BM, p.Sq) - 1;
+    // ---- block skip: KV tiles [kt_begin, kt_end) hold an unmasked (i, j) for rows q0..qlast
+    int kt_begin = 0, kt_end = nkt;
+#if LF_MASK >= 1
+    kt_end = min(nkt, qlast / LF_BN + 1);
+#endif
+#if LF_MASK == 2
+    {
+      int lo = q0 - p.window + 1;
+      if (lo > 0) kt_begin = lo / LF_BN;
+    }
+#endif
+    if (p.visits != nullptr && tid == 0) {
+      for (int kt = kt_begin; kt < kt_end; ++kt)
+        p.visits[((long long)bh * nqt + qt) * nkt + kt] = 1;
+    }
+
+    const int wq0 = q0 + 32 * wave;
+    const int wqlast = min(wq0 + 31, p.Sq - 1);
+    const bool wave_has_rows = wq0 < p.Sq;
+    const int my_q = wq0 + l32;
+
+    // Q^T fragments (B operand): lane holds row my_q, d = 16*ks + 8*g .. +7.
+    lf_elem8 qf[LF_NKS];
+    {
+      const lf_elem* qrow = p.q + (long long)b * p.q_sb + (long long)h * p.q_sh +
+                            (long long)min(my_q, p.Sq - 1) * p.q_ss;
+#pragma unroll
+      for (int ks = 0; ks < LF_NKS; ++ks)
+        qf[ks] = __builtin_bit_cast(lf_elem8, *reinterpret_cast<const lf_u32x4*>(qrow + 16 * ks + 8 * g));
+    }
+    // the compiler waits for the Q loads here (a use it can see) and all older vector
+    // memory operations are drained, so its bookkeeping is clear before the direct
+    // loads, which it does not track, start
+#pragma unroll
+    for (int ks = 0; ks < LF_NKS; ++ks) asm volatile("" :: "v"(qf[ks]));
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    lf_f32x16 o[LF_NDB];
+#pragma unroll
+    for (int db = 0; db < LF_NDB; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[db][i] = 0.0f;
+    float mc_ref = LF_NEG_INF;   // exponent offset of this query, log2 units (a lagging running max)
+    float l_run = 0.0f;          // this lane's share of the running sum
+
+    // ---- prologue: K(begin), K(begin+1), V(begin) resident; first K fragments in flight
+#pragma unroll
+    for (int ps = 0; ps < LF_NPASS; ++ps) {
+      dma_k_pass(kt_begin, 0, ps);
+      dma_k_pass(kt_begin + 1, 1, ps);
+      dma_v_pass(kt_begin, 0, ps);
+#if LF_ABLATE & 2
+      dma_k_pass(kt_begin, 2, ps);
+      dma_v_pass(kt_begin, 1, ps);
+#endif
+    }
+#if LF_ABLATE & 2
+    dma_on = false;
+#endif
+    LF_BARRIER_VM0();
+    lf_u32x4 kpre[LF_KPF];
+#pragma unroll
+    for (int f = 0; f < LF_KPF; ++f) kpre[f] = k_frag(lds_k[0], f);
+
+    int ks_cur = 0;   // K slot of tile kt
+    for (int kt = kt_begin; kt < kt_end; ++kt) {
+      const int rel = kt - kt_begin;
+      const int ks_nxt = (ks_cur == LF_KSLOTS - 1) ? 0 : ks_cur + 1;   // slot of K(kt+1)
+      const int ks_ld = (ks_nxt == LF_KSLOTS - 1) ? 0 : ks_nxt + 1;    // slot K(kt+2) is loaded into
+      const lf_elem* kbuf = lds_k[ks_cur];
+      const lf_elem* knext = lds_k[ks_nxt];
+      const lf_elem* vbuf = lds_v[rel & 1];
+      const int vs_ld = (rel + 1) & 1;                                 // slot V(kt+1) is loaded into
+      // direct load number d of this tile: K(kt+2) passes, then V(kt+1) passes
+      auto dma_step = [&](int d) {
+        if (d < LF_NPASS) dma_k_pass(kt + 2, ks_ld, d);
+        else dma_v_pass(kt + 1, vs_ld, d - LF_NPASS);
+      };
+
+      const int k0 = kt * LF_BN;
+      bool need = wave_has_rows;
+      bool full = (k0 + LF_BN <= p.Sk);
+#if LF_MASK >= 1
+      need = need && (k0 <= wqlast);
+      full = full && (k0 + LF_BN - 1 <= wq0);
+#endif
+#if LF_MASK == 2
+      need = need && (min(k0 + LF_BN, p.Sk) - 1 >= wq0 - p.window + 1);
+      full = full && (wq0 + 31 - k0 < p.window);
+#endif
+
+      if (need) {
+        // ---- S^T = K Q^T; the two accumulator chains alternate
+        lf_f32x16 s[LF_NKB];
+#pragma unroll
+        for (int kb = 0; kb < LF_NKB; ++kb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) s[kb][i] = 0.0f;
+        lf_u32x4 kf[LF_NFK];
+        lf_elem8 vf[LF_NFV];
+#pragma unroll
+        for (int f = 0; f < LF_KPF; ++f) kf[f] = kpre[f];
+#if LF_SETPRIO
+        __builtin_amdgcn_s_setprio(2);
+#endif
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int f = 0; f < LF_NFK; ++f) {
+          if (f + LF_KPF < LF_NFK) kf[f + LF_KPF] = k_frag(kbuf, f + LF_KPF);
+          if (f >= LF_NFK - LF_VPF) vf[f - (LF_NFK - LF_VPF)] = v_frag(vbuf, f - (LF_NFK - LF_VPF));
+          if (f % (LF_NFK / (2 * LF_NPASS)) == 1) dma_step(f / (LF_NFK / (2 * LF_NPASS)));
+          s[f % LF_NKB] = lf_mfma32(__builtin_bit_cast(lf_elem8, kf[f]), qf[f / LF_NKB], s[f % LF_NKB]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+#if LF_SETPRIO
+        __builtin_amdgcn_s_setprio(0);
+#endif
+
+        // ---- score modifications and mask; element i of block kb is kv index
+        // j = k0 + 32*kb + 8*(i/4) + 4*g + i%4, query my_q.
+#if LF_SOFTCAP
+#pragma unroll
+        for (int kb = 0; kb < LF_NKB; ++kb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) s[kb][i] = p.softcap * lf_tanh(s[kb][i] * sc_in);
+#endif
+        if (!full) {
+#pragma unroll
+          for (int kb = 0; kb < LF_NKB; ++kb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              const int j = k0 + 32 * kb + 8 * (i / 4) + 4 * g + (i % 4);
+              bool ok = j < p.Sk;
+#if LF_MASK >= 1
+              ok = ok && (j <= my_q);
+#endif
+#if LF_MASK == 2
+              ok = ok && (my_q - j < p.window);
+#endif
+              s[kb][i] = ok ? s[kb][i] : LF_NEG_INF;
+            }
+        }
+
+        // ---- online softmax with a lagging offset (see lf_attn_prefill.hip)
+        float mx = LF_NEG_INF;
+#pragma unroll
+        for (int kb = 0; kb < LF_NKB; ++kb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kb][i]);
+        mx = fmaxf(mx, lf_swap32(mx));
+        const float mxc = mx * cexp;
+        if (__builtin_amdgcn_ballot_w64(mxc > mc_ref + (float)LF_LAZY_LOG2) != 0ull) {
+          const float mc_new = fmaxf(mc_ref, mxc);
+          const float r = (mc_new == LF_NEG_INF) ? 1.0f : lf_exp2(mc_ref - mc_new);
+          mc_ref = mc_new;
+          l_run *= r;
+#pragma unroll
+          for (int db = 0; db < LF_NDB; ++db)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o[db][i] *= r;
+        }
+        const float mc_sub = (mc_ref == LF_NEG_INF) ? 0.0f : mc_ref;
+        float rs = 0.0f;
+        lf_elem8 pf[LF_NKK];
+#pragma unroll
+        for (int kb = 0; kb < LF_NKB; ++kb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+#if LF_ABLATE & 1
+            const float e = s[kb][i] * cexp - mc_sub;
+#else
+            const float e = lf_exp2(s[kb][i] * cexp - mc_sub);
+#endif
+            rs += e;
+            pf[2 * kb + i / 8][i % 8] = lf_from_float(e);
+          }
+        l_run += rs;
+
+        // ---- O^T += V^T P^T; the last steps also read the first fragments of K(kt+1)
+#if LF_SETPRIO
+        __builtin_amdgcn_s_setprio(2);
+#endif
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int f = 0; f < LF_NFV; ++f) {
+          if (f + LF_VPF < LF_NFV) vf[f + LF_VPF] = v_frag(vbuf, f + LF_VPF);
+          if (f >= LF_NFV - LF_KPF) kpre[f - (LF_NFV - LF_KPF)] = k_frag(knext, f - (LF_NFV - LF_KPF));
+          o[f % LF_NDB] = lf_mfma32(vf[f], pf[f / LF_NDB], o[f % LF_NDB]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+#if LF_SETPRIO
+        __builtin_amdgcn_s_setprio(0);
+#endif
+      } else {
+        // this wave's rows see nothing of tile kt: it only stages and reads ahead
+#pragma unroll
+        for (int d = 0; d < 2 * LF_NPASS; ++d) dma_step(d);
+#pragma unroll
+        for (int f = 0; f < LF_KPF; ++f) kpre[f] = k_frag(knext, f);
+      }
+      LF_BARRIER_VM0();
+      ks_cur = ks_nxt;
+    }
+
+    // ---- epilogue: O[q][d] = O^T[d][q] / l.  Element i of block db is
+    // d = 32*db + 8*(i/4) + 4*g + i%4.
+#if LF_ABLATE & 2
+    dma_on = true;
+#endif
+    const float l_tot = l_run + lf_swap32(l_run);
+    if (my_q < p.Sq) {
+      const float inv = 1.0f / l_tot;
+      lf_elem* orow = p.o + (long long)b * p.o_sb + (long long)h * p.o_sh + (long long)my_q * p.o_ss;
+#pragma unroll
+      for (int db = 0; db < LF_NDB; ++db)
+#pragma unroll
+        for (int i4 = 0; i4 < 4; ++i4) {
+          lf_elem4 w;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) w[e] = lf_from_float(o[db][4 * i4 + e] * inv);
+          *reinterpret_cast<lf_elem4*>(orow + 32 * db + 8 * i4 + 4 * g) = w;
+        }
+    }
+    // the next q tile's prologue overwrites slots other waves may still read ahead from
+    __syncthreads();
+  };
+
+  run_q_tile(nqt - 1 - pair);
+  if (pair != nqt - 1 - pair) run_q_tile(pair);
+}

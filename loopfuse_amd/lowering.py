@@ -85,11 +85,11 @@ class KernelSpec:
 
     def files(self) -> tuple[str, ...]:
         return ("lf_common.hip.h", {"prefill": "lf_attn_prefill.hip", "prefill_pipe": "lf_attn_prefill_pipe.hip",
-                                    "decode": "lf_attn_decode.hip"}[self.family])
+                                    "prefill_swp": "lf_attn_prefill_swp.hip", "decode": "lf_attn_decode.hip"}[self.family])
 
     def entry(self) -> str:
         return {"prefill": "lf_attn_prefill", "prefill_pipe": "lf_attn_prefill_pipe",
-                "decode": "lf_attn_decode"}[self.family]
+                "prefill_swp": "lf_attn_prefill_swp", "decode": "lf_attn_decode"}[self.family]
 
     def name(self) -> str:
         return (f"lf_{self.family}_t{self.dtype}_d{self.head_dim}_m{self.mask}_c{int(self.softcap)}"
@@ -227,13 +227,16 @@ def decode_split(units: int, Sk: int, cus: int = 256) -> int:
 
 
 def prefill_variant(Sq: int, v_tr: bool = True) -> str:
-    """Which prefill kernel serves a call.  The two-waves-per-SIMD kernel
-    (``prefill``) is the measured-faster default; LOOPFUSE_PREFILL=pipe selects the
-    one-wave-per-SIMD software-pipelined kernel for comparison."""
-    env = os.environ.get("LOOPFUSE_PREFILL")
-    if env == "pipe" and v_tr:
+    """Which prefill kernel serves a call.  Default: the software-pipelined kernel
+    with direct-to-LDS staging (``prefill_swp``; dense K/V only, ``attention`` falls
+    back to ``prefill`` for paged operands).  LOOPFUSE_PREFILL=w32 selects the
+    register-staged kernel, =pipe the one-wave-per-SIMD kernel, for comparison."""
+    env = os.environ.get("LOOPFUSE_PREFILL", "swp")
+    if not v_tr or env == "w32":
+        return "prefill"
+    if env == "pipe":
         return "prefill_pipe"
-    return "prefill"
+    return "prefill_swp"
 
 
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
@@ -328,7 +331,17 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
 
     if family == "prefill":
         family = prefill_variant(Sq, v_tr)
-    if family in ("prefill", "prefill_pipe"):
+    if family == "prefill_swp":
+        # direct-to-LDS staging: dense K/V only, 32-bit byte offsets per (batch, kv head)
+        # span; the kernel also addresses up to three tiles past Sk (those reads are
+        # range-checked to zeros, but their offsets must not wrap)
+        reach = max(abs(P.k_ss), abs(P.v_ss)) * 2 * (Sk + 3 * 64) + 2 * D
+        if paged or reach >= (1 << 32) or P.k_ss < 0 or P.v_ss < 0:
+            family = "prefill"
+        span = max((Sk - 1) * abs(P.k_ss), (Sk - 1) * abs(P.v_ss)) * 2 + 2 * D
+        if span >= (1 << 31):
+            family = "prefill"
+    if family in ("prefill", "prefill_pipe", "prefill_swp"):
         P.q_sb, P.q_sh, P.q_ss = q.stride(0), q.stride(1), q.stride(2)
         P.o_sb, P.o_sh, P.o_ss = out.stride(0), out.stride(1), out.stride(2)
         extra = tuple(os.environ.get("LOOPFUSE_KOPTS", "").split())
@@ -356,7 +369,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         # 8 XCD classes x (batch*head pairs per class, padded to the kernel's groups of 4) x q tiles
         per_xcd = (B * Hq + 7) // 8
         # lf_attn_prefill takes two q tiles (heavy + light) per workgroup
-        per_bh = (nqt + 1) // 2 if family == "prefill" else nqt
+        per_bh = nqt if family == "prefill_pipe" else (nqt + 1) // 2
         grid = 8 * ((per_xcd + 3) // 4 * 4) * per_bh
         get_kernel(spec, spec.entry()).launch((grid, 1, 1), (64 * nw, 1, 1), P)
         return (out, visits) if record_visits else out

@@ -18,6 +18,7 @@ from __future__ import annotations
 TILE_SHAPES = {
     "prefill": (128, 64),        # lf_attn_prefill: 4 waves x 32 rows, two waves per SIMD
     "prefill_pipe": (256, 32),   # lf_attn_prefill_pipe: 4 waves x 64 rows, software-pipelined
+    "prefill_swp": (128, 64),    # lf_attn_prefill_swp: 4 waves x 32 rows, direct-to-LDS staging, reads issued ahead
 }
 PREFILL_BM, PREFILL_BN = TILE_SHAPES["prefill"]
 

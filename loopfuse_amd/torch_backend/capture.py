@@ -228,7 +228,8 @@ class AttentionMatch:
             ps = k.shape[1] if k.dim() == 4 else 1
             i64 = args[self.k.table_index].dtype == torch.int64
         mask = lowering._MASK_NAMES[plan.mask]
-        return [lowering.KernelSpec("prefill", dt, D, mask, plan.softcap is not None, paged, ps, i64)]
+        family = "prefill" if paged else lowering.prefill_variant(q.shape[-2])
+        return [lowering.KernelSpec(family, dt, D, mask, plan.softcap is not None, paged, ps, i64)]
 
 
 # ----------------------------------------------------------------------------
