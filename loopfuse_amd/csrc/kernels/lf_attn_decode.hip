@@ -26,7 +26,11 @@
 // O^T lives in 4*D/16 accumulator registers per lane whatever the number of rows.
 // At the end the LF_DW waves are merged through LDS with the (offset, sum, acc)
 // log-sum-exp combine; with nsplit > 1 the workgroup writes its partial to
-// scratch and lf_attn_decode_combine merges the splits.
+// scratch and lf_attn_decode_combine merges the splits.  With LF_HEADWAVE the
+// waves do not share a head: each writes its own result or partial.  (Merging the
+// splits inside the same launch, by the last split to arrive, was measured slower
+// than the second launch: the device-scope fences or write-through stores it needs
+// between XCDs cost more than the launch.)
 
 #ifndef LF_DW
 #define LF_DW 4              /* waves per workgroup */
@@ -34,6 +38,14 @@
 #ifndef LF_LAZY_LOG2
 #define LF_LAZY_LOG2 8       /* slack of the softmax exponent offset, log2 units */
 #endif
+#ifndef LF_HEADWAVE
+#define LF_HEADWAVE 0        /* 1: the waves of a workgroup take LF_DW consecutive kv heads of one batch
+                                element (same tokens) instead of sharing one head: with a token-major
+                                page pool, where the heads of a token lie side by side, the workgroup
+                                then reads whole pages front to back.  No merge between waves; every
+                                wave writes its own result (nsplit == 1) or partial. */
+#endif
+#define LF_PSTRIDE (LF_HEADWAVE ? 1 : LF_DW)   /* distance between the pairs of steps of one wave */
 #define LF_DT (LF_DW * 64)
 #define LF_D LF_HEAD_DIM
 #define LF_NJ (LF_D / 32)    /* 16-byte pieces of a row held by one lane = k-steps of QK^T */
@@ -49,15 +61,17 @@ struct LfDecIds {            // page ids of one step
   long long k, v;
 };
 
-extern "C" __global__ void __launch_bounds__(LF_DT, 2) lf_attn_decode(const LfAttnParams p) {
+extern "C" __global__ void __launch_bounds__(LF_DT, 8 / LF_DW) lf_attn_decode(const LfAttnParams p) {
   // One buffer, two lives: wave-private V tiles of the pair being consumed
   // ([LF_DW][2][16*D] elements) during the loop, merge buffer
   // ([LF_DW][16][LF_OSTRIDE] floats) after it.
   constexpr int kVBytes = LF_DW * 2 * 16 * LF_D * 2;
   constexpr int kOBytes = LF_DW * LF_QROWS * LF_OSTRIDE * 4;
   __shared__ __attribute__((aligned(16))) unsigned char smem[kVBytes > kOBytes ? kVBytes : kOBytes];
+#if !LF_HEADWAVE
   __shared__ float red_m[LF_DW][LF_QROWS];
   __shared__ float red_l[LF_DW][LF_QROWS];
+#endif
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -65,13 +79,22 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 2) lf_attn_decode(const LfAt
   const int c = lane & 15;      // token of a step (loads) / query column (MFMA results)
   const int g = lane >> 4;
 
-  const int unit = blockIdx.x;
   const int z = blockIdx.y;
   const int chunks = (p.rows + LF_QROWS - 1) / LF_QROWS;   // row chunks per (b, kv head)
+  const int unit = blockIdx.x;
   const int rc = unit % chunks;
+#if LF_HEADWAVE
+  // grid.x = B * ceil(Hkv / LF_DW) * chunks; wave w serves head LF_DW*hc + w
+  const int hchunks = (p.Hkv + LF_DW - 1) / LF_DW;
+  const int hkv = ((unit / chunks) % hchunks) * LF_DW + wave;
+  const int b = unit / (chunks * hchunks);
+  if (hkv >= p.Hkv) return;          // no workgroup barrier in this mode
+  const int bh = b * p.Hkv + hkv;
+#else
   const int bh = unit / chunks;
   const int hkv = bh % p.Hkv;
   const int b = bh / p.Hkv;
+#endif
   const int row0 = rc * LF_QROWS;
   const int nrows = min(p.rows - row0, LF_QROWS);          // query rows of this unit
 
@@ -219,47 +242,48 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 2) lf_attn_decode(const LfAt
     }
   };
 
-  // ---- streaming loop: this wave's pairs are wave, wave + LF_DW, ...; four register
+  // ---- streaming loop: this wave's pairs are wave, wave + LF_DW, ... (all pairs of the
+  // split when each wave has its own head); four register
   // stages (two pairs) rotate, two trips of the pipeline per loop iteration so every
   // stage has a static name
   {
     LfDecStage s0, s1, s2, s3;
     LfDecIds i0, i1, i2, i3;
-    int pr = wave;
+    int pr = LF_HEADWAVE ? 0 : wave;
     i0 = fetch_ids(2 * pr);
     i1 = fetch_ids(2 * pr + 1);
-    i2 = fetch_ids(2 * (pr + LF_DW));
-    i3 = fetch_ids(2 * (pr + LF_DW) + 1);
+    i2 = fetch_ids(2 * (pr + LF_PSTRIDE));
+    i3 = fetch_ids(2 * (pr + LF_PSTRIDE) + 1);
     if (pr < npairs) {
       issue(s0, 2 * pr, i0);
       issue(s1, 2 * pr + 1, i1);
-      i0 = fetch_ids(2 * (pr + 2 * LF_DW));
-      i1 = fetch_ids(2 * (pr + 2 * LF_DW) + 1);
+      i0 = fetch_ids(2 * (pr + 2 * LF_PSTRIDE));
+      i1 = fetch_ids(2 * (pr + 2 * LF_PSTRIDE) + 1);
     }
-    if (pr + LF_DW < npairs) {
-      issue(s2, 2 * (pr + LF_DW), i2);
-      issue(s3, 2 * (pr + LF_DW) + 1, i3);
-      i2 = fetch_ids(2 * (pr + 3 * LF_DW));
-      i3 = fetch_ids(2 * (pr + 3 * LF_DW) + 1);
+    if (pr + LF_PSTRIDE < npairs) {
+      issue(s2, 2 * (pr + LF_PSTRIDE), i2);
+      issue(s3, 2 * (pr + LF_PSTRIDE) + 1, i3);
+      i2 = fetch_ids(2 * (pr + 3 * LF_PSTRIDE));
+      i3 = fetch_ids(2 * (pr + 3 * LF_PSTRIDE) + 1);
     }
-    for (; pr < npairs; pr += 2 * LF_DW) {
+    for (; pr < npairs; pr += 2 * LF_PSTRIDE) {
       consume(s0, s1, pr);
-      const int pa = pr + 2 * LF_DW;
+      const int pa = pr + 2 * LF_PSTRIDE;
       if (pa < npairs) {
         issue(s0, 2 * pa, i0);
         issue(s1, 2 * pa + 1, i1);
-        i0 = fetch_ids(2 * (pa + 2 * LF_DW));
-        i1 = fetch_ids(2 * (pa + 2 * LF_DW) + 1);
+        i0 = fetch_ids(2 * (pa + 2 * LF_PSTRIDE));
+        i1 = fetch_ids(2 * (pa + 2 * LF_PSTRIDE) + 1);
       }
-      const int pb2 = pr + LF_DW;
+      const int pb2 = pr + LF_PSTRIDE;
       if (pb2 < npairs) {
         consume(s2, s3, pb2);
-        const int pc = pb2 + 2 * LF_DW;
+        const int pc = pb2 + 2 * LF_PSTRIDE;
         if (pc < npairs) {
           issue(s2, 2 * pc, i2);
           issue(s3, 2 * pc + 1, i3);
-          i2 = fetch_ids(2 * (pc + 2 * LF_DW));
-          i3 = fetch_ids(2 * (pc + 2 * LF_DW) + 1);
+          i2 = fetch_ids(2 * (pc + 2 * LF_PSTRIDE));
+          i3 = fetch_ids(2 * (pc + 2 * LF_PSTRIDE) + 1);
         }
       }
     }
@@ -268,6 +292,32 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 2) lf_attn_decode(const LfAt
   // ---- merge: lane groups (sum), then the LF_DW waves
   float l_wave = l_part + __shfl_xor(l_part, 16, 64);
   l_wave += __shfl_xor(l_wave, 32, 64);
+#if LF_HEADWAVE
+  // each wave owns its (batch, head): lane (q = c, g) writes d = 16*db + 4*g .. +3 of row q
+  if (c < nrows) {
+    const int qr = row0 + c;
+    if (p.nsplit == 1) {
+      lf_elem* orow = p.o + (long long)b * p.o_sb + (long long)hkv * p.o_sh + (long long)qr * p.o_ss;
+      const float inv = 1.0f / l_wave;
+#pragma unroll
+      for (int db = 0; db < LF_NDB; ++db) {
+        lf_elem4 w4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w4[e] = lf_from_float(o[db][e] * inv);
+        *reinterpret_cast<lf_elem4*>(orow + 16 * db + 4 * g) = w4;
+      }
+    } else {
+      const long long slot = ((long long)bh * p.rows + qr) * p.nsplit + z;
+#pragma unroll
+      for (int db = 0; db < LF_NDB; ++db)
+        *reinterpret_cast<lf_f32x4*>(&p.part_acc[slot * LF_D + 16 * db + 4 * g]) = o[db];
+      if (g == 0) {
+        p.part_ml[slot * 2 + 0] = mc;            // exponent offset, log2 units
+        p.part_ml[slot * 2 + 1] = l_wave;
+      }
+    }
+  }
+#else
   if (g == 0) {
     red_m[wave][c] = mc;
     red_l[wave][c] = l_wave;
@@ -322,6 +372,7 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 2) lf_attn_decode(const LfAt
       }
     }
   }
+#endif   // LF_HEADWAVE
 }
 
 // Merge nsplit partial results per query row: grid = (B*Hkv*rows), block = LF_D.

@@ -32,14 +32,19 @@
 #define LF_VPF 4         /* V fragments (two transposed reads each) in flight */
 #endif
 #ifndef LF_SETPRIO
-#define LF_SETPRIO 1
+#define LF_SETPRIO 1     /* 1: raise the wave priority while it issues MFMAs; 2: static, by workgroup:
+                            the workgroup whose LDS allocation starts at 0 runs at low priority, the
+                            one above it at high priority, which keeps the two workgroups of a CU out
+                            of phase (one in its MFMAs while the other is in its softmax) */
 #endif
 #ifndef LF_ABLATE
 #define LF_ABLATE 0      /* profiling aid (wrong results): 1 no exp, 2 no direct loads, 16 no K reads,
                             32 V fragments by one plain 16-byte read, 64 no V reads */
 #endif
 
-#define LF_NW 4
+#ifndef LF_NW
+#define LF_NW 4     /* waves per workgroup: 4 (two workgroups per CU) or 8 (one) */
+#endif
 #define LF_NT (LF_NW * 64)
 #define LF_BM (32 * LF_NW)
 #define LF_BN 64
@@ -67,7 +72,7 @@ __device__ __forceinline__ int lf_v_phys(int row, int ch) {
 // reads in flight (the compiler's own barrier would wait for those too)
 #define LF_BARRIER_VM0() asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory")
 
-extern "C" __global__ void __launch_bounds__(LF_NT, 2) lf_attn_prefill_swp(const LfAttnParams p) {
+extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_swp(const LfAttnParams p) {
   __shared__ __attribute__((aligned(16))) lf_elem lds_k[LF_KSLOTS][LF_BN * LF_D];
   __shared__ __attribute__((aligned(16))) lf_elem lds_v[LF_VSLOTS][LF_BN * LF_D];
 
@@ -76,6 +81,11 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 2) lf_attn_prefill_swp(const
   const int wave = tid >> 6;
   const int l32 = lane & 31;
   const int g = lane >> 5;
+#if LF_SETPRIO == 2
+  // hardware register LDS_ALLOC (id 6), field LDS_BASE (low 12 bits read here)
+  if ((__builtin_amdgcn_s_getreg((11 << 11) | 6) & 0xfff) != 0) __builtin_amdgcn_s_setprio(3);
+  else __builtin_amdgcn_s_setprio(0);
+#endif
 
   // ---- workgroup -> (batch*head, pair of q tiles), as in lf_attn_prefill.hip
   const int nqt = (p.Sq + LF_BM - 1) / LF_BM;
@@ -294,7 +304,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 2) lf_attn_prefill_swp(const
         lf_elem8 vf[LF_NFV];
 #pragma unroll
         for (int f = 0; f < LF_KPF; ++f) kf[f] = kpre[f];
-#if LF_SETPRIO
+#if LF_SETPRIO == 1
         __builtin_amdgcn_s_setprio(2);
 #endif
         __builtin_amdgcn_sched_barrier(0);
@@ -306,7 +316,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 2) lf_attn_prefill_swp(const
           s[f % LF_NKB] = lf_mfma32(__builtin_bit_cast(lf_elem8, kf[f]), qf[f / LF_NKB], s[f % LF_NKB]);
           __builtin_amdgcn_sched_barrier(0);
         }
-#if LF_SETPRIO
+#if LF_SETPRIO == 1
         __builtin_amdgcn_s_setprio(0);
 #endif
 
@@ -371,7 +381,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 2) lf_attn_prefill_swp(const
         l_run += rs;
 
         // ---- O^T += V^T P^T; the last steps also read the first fragments of K(kt+1)
-#if LF_SETPRIO
+#if LF_SETPRIO == 1
         __builtin_amdgcn_s_setprio(2);
 #endif
         __builtin_amdgcn_sched_barrier(0);
@@ -382,7 +392,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 2) lf_attn_prefill_swp(const
           o[f % LF_NDB] = lf_mfma32(vf[f], pf[f / LF_NDB], o[f % LF_NDB]);
           __builtin_amdgcn_sched_barrier(0);
         }
-#if LF_SETPRIO
+#if LF_SETPRIO == 1
         __builtin_amdgcn_s_setprio(0);
 #endif
       } else {

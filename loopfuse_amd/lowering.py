@@ -65,6 +65,7 @@ class KernelSpec:
     rows: int = 1          # decode: query rows a unit can hold (fixed, the MFMA N dimension)
     waves: int = 4         # decode: waves per workgroup
     v_tr: bool = True      # prefill: transposed LDS reads for V
+    headwave: bool = False  # decode: one kv head per wave (8 waves) instead of 4 waves sharing a head
     extra: tuple = ()      # further -D options (tuning experiments)
 
     def options(self) -> list[str]:
@@ -78,7 +79,7 @@ class KernelSpec:
             f"-DLF_TABLE_I64={int(self.table_i64)}",
         ]
         if self.family == "decode":
-            o += [f"-DLF_DW={self.waves}"]
+            o += [f"-DLF_DW={self.waves}", f"-DLF_HEADWAVE={int(self.headwave)}"]
         elif self.family == "prefill":
             o += [f"-DLF_V_TR={int(self.v_tr)}"]
         return o + list(self.extra)
@@ -93,7 +94,7 @@ class KernelSpec:
 
     def name(self) -> str:
         return (f"lf_{self.family}_t{self.dtype}_d{self.head_dim}_m{self.mask}_c{int(self.softcap)}"
-                f"_p{self.paged}x{self.page_size}i{int(self.table_i64)}_r{self.rows}w{self.waves}v{int(self.v_tr)}"
+                f"_p{self.paged}x{self.page_size}i{int(self.table_i64)}_r{self.rows}w{self.waves}v{int(self.v_tr)}h{int(self.headwave)}"
                 + "".join("_" + e.replace("-D", "").replace("=", "") for e in self.extra))
 
     def source(self) -> str:
@@ -213,17 +214,28 @@ def _get_scratch(device: torch.device, nfloats: int) -> torch.Tensor:
     return t
 
 
-def decode_split(units: int, Sk: int, cus: int = 256) -> int:
-    """Number of KV splits across workgroups.  One workgroup (4 waves) per unit is
-    enough once there are two workgroups per CU (8 resident waves, each with 32 KB
-    of loads in flight); below that the KV range is split, down to 256 tokens per
-    split, and a second kernel merges the partial results."""
+def decode_split(units: int, Sk: int, cus: int = 256, per_cu: int = 2) -> int:
+    """Number of KV splits across workgroups.  One workgroup per unit is enough once
+    there are ``per_cu`` workgroups per CU (8 resident waves, each with 32 KB of loads
+    in flight: two workgroups of 4 waves, or one of 8); below that the KV range is
+    split, down to 256 tokens per split, and a second kernel merges the partial
+    results."""
     env = os.environ.get("LOOPFUSE_DECODE_SPLITS")
     if env:
         return max(1, int(env))
-    want = max(1, (2 * cus + units - 1) // units)
+    want = max(1, (per_cu * cus + units - 1) // units)
     most = max(1, Sk // 256)
     return max(1, min(want, most))
+
+
+def _decode_headwave(paged: int, page_size: int, Hkv: int, D: int, P: "AttnParams") -> bool:
+    """One kv head per wave pays when K and V are paged, token-major (head stride D,
+    token stride Hkv*D) and there are at least 8 heads to fill the 8 waves."""
+    env = os.environ.get("LOOPFUSE_DECODE_HEADWAVE")
+    if env is not None:
+        return env == "1"
+    return (paged == 3 and Hkv % 8 == 0 and P.k_sh == D and P.v_sh == D
+            and P.k_ss == Hkv * D and P.v_ss == Hkv * D)
 
 
 def prefill_variant(Sq: int, v_tr: bool = True) -> str:
@@ -391,13 +403,19 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         raise UnsupportedPlan("decode needs Sq == 1 or group == 1")
     chunks = (rows + DECODE_QROWS - 1) // DECODE_QROWS
     units = B * Hkv * chunks
-    nsplit = num_splits if num_splits else decode_split(units, Sk)
+    waves = int(os.environ.get("LOOPFUSE_DECODE_WAVES", "4"))
+    # Token-major page pools ([pages, page, Hkv, D]: the heads of a token side by side)
+    # are read whole-page-wise when the 8 waves of a workgroup take 8 consecutive heads.
+    headwave = _decode_headwave(paged, page_size, Hkv, D, P)
+    if headwave:
+        waves = 8
+        units = B * ((Hkv + waves - 1) // waves) * chunks
+    nsplit = num_splits if num_splits else decode_split(units, Sk, per_cu=1 if headwave else 2)
     split_len = ((Sk + nsplit - 1) // nsplit + 31) // 32 * 32     # whole pairs of 16-token steps
     nsplit = (Sk + split_len - 1) // split_len
     P.rows, P.nsplit, P.split_len = rows, nsplit, split_len
     spec = KernelSpec("decode", _DTYPE_CODE[dtype], D, MASK_NONE, plan.softcap is not None, paged,
-                      page_size, table_i64, rows=DECODE_QROWS,
-                      waves=int(os.environ.get("LOOPFUSE_DECODE_WAVES", "4")),
+                      page_size, table_i64, rows=DECODE_QROWS, waves=waves, headwave=headwave,
                       extra=tuple(os.environ.get("LOOPFUSE_KOPTS", "").split()))
     if nsplit > 1:
         nrow = B * Hkv * rows * nsplit
