@@ -120,7 +120,7 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
         return 3
-    from loopfuse_amd import workloads
+    from loopfuse_amd import lowering, workloads
 
     dev = torch.device("cuda:0")
     out: dict = {}
@@ -140,7 +140,8 @@ def main() -> int:
         o = workloads.run(w)     # first call compiles / loads the code object
         torch.cuda.synchronize()
         t, wall = time_gpu(lambda i: workloads.run(w, out=o), args.steps, args.warmup)
-        pre = {"workload": args.workload, "sec": t, "wall_sec": wall, "flops": w.flops()}
+        pre = {"workload": args.workload, "sec": t, "wall_sec": wall, "flops": w.flops(),
+               "kernels": lowering.attention.last_launch["kernels"]}
 
     dec = None
     if args.only in (None, "decode"):
@@ -155,7 +156,8 @@ def main() -> int:
         o = workloads.run(ws[0])
         torch.cuda.synchronize()
         t, wall = time_gpu(lambda i: workloads.run(ws[i % nrot], out=o), args.steps, args.warmup)
-        dec = {"workload": args.decode_workload, "sec": t, "wall_sec": wall, "bytes": base.kv_bytes(), "rotation": nrot}
+        dec = {"workload": args.decode_workload, "sec": t, "wall_sec": wall, "bytes": base.kv_bytes(), "rotation": nrot,
+               "kernels": lowering.attention.last_launch["kernels"]}
 
     primary = pre if pre is not None else dec
     if pre is not None:
@@ -166,14 +168,14 @@ def main() -> int:
         })
         out["roofline"] = {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                            "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": TRAFFIC_BYTES.get(args.workload),
-                           "kernel": "lf_attn_prefill", "us_per_launch": pre["sec"] * 1e6}
+                           "kernel": "+".join(pre["kernels"]), "us_per_launch": pre["sec"] * 1e6}
     if dec is not None:
         gbs = dec["bytes"] / dec["sec"] / 1e9
         d = {"workload": dec["workload"], "value": gbs, "unit": "GB/s", "us_per_launch": dec["sec"] * 1e6,
              "host_us_per_launch": dec["wall_sec"] * 1e6, "kv_pool_rotation": dec["rotation"],
              "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                           "frac": gbs / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES.get(args.decode_workload),
-                          "kernel": "lf_attn_decode"}}
+                          "kernel": "+".join(dec["kernels"])}}
         if pre is None:
             out.update({"metric": "prefill TFLOP/s + decode HBM GB/s on 1 MI355X (% of roofline)",
                         "value": gbs, "unit": "GB/s", "roofline": d["roofline"]})

@@ -251,7 +251,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
 #pragma unroll
     for (int ps = 0; ps < LF_NPASS; ++ps) {
       dma_k_pass(kt_begin, 0, ps);
-      dma_k_pass(kt_begin + 1, 1, ps);
+      if (kt_begin + 1 < kt_end) dma_k_pass(kt_begin + 1, 1, ps);
       dma_v_pass(kt_begin, 0, ps);
 #if LF_ABLATE & 2
       dma_k_pass(kt_begin, 2, ps);
@@ -276,9 +276,13 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
       const lf_elem* vbuf = lds_v[rel & 1];
       const int vs_ld = (rel + 1) & 1;                                 // slot V(kt+1) is loaded into
       // direct load number d of this tile: K(kt+2) passes, then V(kt+1) passes
+      // (tiles past the last one are not fetched: wave-uniform tests)
       auto dma_step = [&](int d) {
-        if (d < LF_NPASS) dma_k_pass(kt + 2, ks_ld, d);
-        else dma_v_pass(kt + 1, vs_ld, d - LF_NPASS);
+        if (d < LF_NPASS) {
+          if (kt + 2 < kt_end) dma_k_pass(kt + 2, ks_ld, d);
+        } else if (kt + 1 < kt_end) {
+          dma_v_pass(kt + 1, vs_ld, d - LF_NPASS);
+        }
       };
 
       const int k0 = kt * LF_BN;

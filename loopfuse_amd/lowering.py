@@ -384,6 +384,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         per_bh = nqt if family == "prefill_pipe" else (nqt + 1) // 2
         grid = 8 * ((per_xcd + 3) // 4 * 4) * per_bh
         get_kernel(spec, spec.entry()).launch((grid, 1, 1), (64 * nw, 1, 1), P)
+        attention.last_launch = {"kernels": [spec.entry()], "grid": grid, "block": 64 * nw}
         return (out, visits) if record_visits else out
 
     if family != "decode":
@@ -425,4 +426,6 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     get_kernel(spec, "lf_attn_decode").launch((units, nsplit, 1), (64 * spec.waves, 1, 1), P)
     if nsplit > 1:
         get_kernel(spec, "lf_attn_decode_combine").launch((B * Hkv * rows, 1, 1), (D, 1, 1), P)
+    attention.last_launch = {"kernels": ["lf_attn_decode"] + (["lf_attn_decode_combine"] if nsplit > 1 else []),
+                             "grid": (units, nsplit), "block": 64 * spec.waves, "head_per_wave": headwave}
     return out
