@@ -38,7 +38,7 @@
                             of phase (one in its MFMAs while the other is in its softmax) */
 #endif
 #ifndef LF_ABLATE
-#define LF_ABLATE 0      /* profiling aid (wrong results): 1 no exp, 2 no direct loads, 16 no K reads,
+#define LF_ABLATE 0      /* profiling aid (wrong results): 1 no exp, 2 no direct loads, 4 no O store, 8 no Q load, 16 no K reads,
                             32 V fragments by one plain 16-byte read, 64 no V reads */
 #endif
 
@@ -230,7 +230,11 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
                             (long long)min(my_q, p.Sq - 1) * p.q_ss;
 #pragma unroll
       for (int ks = 0; ks < LF_NKS; ++ks)
+#if LF_ABLATE & 8
+        qf[ks] = __builtin_bit_cast(lf_elem8, lf_u32x4{0x3e803f00u + lane * 65537u * ks, 0xbe803e00u, 0x3f000000u + lane, 0xbf003d80u});
+#else
         qf[ks] = __builtin_bit_cast(lf_elem8, *reinterpret_cast<const lf_u32x4*>(qrow + 16 * ks + 8 * g));
+#endif
     }
     // the compiler waits for the Q loads here (a use it can see) and all older vector
     // memory operations are drained, so its bookkeeping is clear before the direct
@@ -426,6 +430,9 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
           lf_elem4 w;
 #pragma unroll
           for (int e = 0; e < 4; ++e) w[e] = lf_from_float(o[db][4 * i4 + e] * inv);
+#if LF_ABLATE & 4
+          if (w[0] == (lf_elem)123.25f)
+#endif
           *reinterpret_cast<lf_elem4*>(orow + 32 * db + 8 * i4 + 4 * g) = w;
         }
     }

@@ -93,6 +93,28 @@ def test_paged_attention_k_only():
     assert (got - want).abs().max() <= TOL
 
 
+def test_paged_attention_gqa():
+    # reference tests/test_accuracy.py:281-311: paged K (one-token pages) + GQA, causal prefill
+    def fn(Q, K_cache, K_block_table, V):
+        K = torch.ops.loopfuse.paged_load(K_cache, K_block_table).transpose(1, 2)
+        g = Q.shape[1] // K.shape[1]
+        K = K.repeat_interleave(g, dim=1)
+        V = V.repeat_interleave(g, dim=1)
+        QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        return torch.softmax(torch.ops.loopfuse.causal_mask(QK), dim=-1) @ V
+
+    B, Hq, Hk, S, D = 4, 8, 4, 256, 64
+    n = B * S * 2
+    Kc = rand((n, Hk, D), seed=1)
+    tab = torch.randint(0, n, (B, S), generator=torch.Generator().manual_seed(5), dtype=torch.int32)
+    Q, V = rand((B, Hq, S, D), seed=2), rand((B, Hk, S, D), seed=3)
+    torch._dynamo.mark_static(Q, 3)
+    torch._dynamo.mark_dynamic(Q, 2)
+    got = run_fused(fn, (Q, Kc, tab, V))
+    want = O.attention_reference(Q, Kc, V, mask="causal", k_table=tab)
+    assert (got - want).abs().max() <= TOL
+
+
 def test_paged_decode_gqa_reference_format():
     # tests/benchmark.py:400-443: one-token pages, Q viewed [B, Hkv, group, D]
     def fn(Q, Kc, kt, Vc, vt):
@@ -164,7 +186,7 @@ def test_recompile_free_new_sequence_length():
     assert outs[1] == 0
 
 
-@pytest.mark.parametrize("which", ["add", "matmul_add", "modified_attn", "softmax_matmul"])
+@pytest.mark.parametrize("which", ["add", "matmul_add", "modified_attn", "softmax_matmul", "paged_add"])
 def test_unlowered_graphs_still_correct(which):
     """Reference tests/test_accuracy.py:29-82, 172-211: not attention-shaped for this
     backend; they run unfused and must still be numerically right."""
@@ -181,6 +203,10 @@ def test_unlowered_graphs_still_correct(which):
             return torch.softmax(torch.ops.loopfuse.causal_mask(QK), dim=-1) @ V + ob
         ins = tuple(rand((2, 2, 128, 64), torch.float32, s) for s in (1, 2, 3, 4)) + \
             (rand((2, 2, 128, 128), torch.float32, 5), rand((2, 2, 128, 64), torch.float32, 6))
+    elif which == "paged_add":       # reference tests/test_accuracy.py:233-250
+        fn = lambda buf, tab: torch.ops.loopfuse.paged_load(buf, tab) + 1
+        ins = (rand((64, 4, 32), torch.float32, 1),
+               torch.randint(0, 64, (3, 20), generator=torch.Generator().manual_seed(2), dtype=torch.int32))
     else:
         fn = lambda x, y: torch.softmax(x, dim=-1) @ y
         ins = (rand((2, 4, 128, 64), torch.float32, 1), rand((2, 4, 64, 128), torch.float32, 2))
