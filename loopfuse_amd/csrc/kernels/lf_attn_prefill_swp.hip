@@ -72,6 +72,9 @@ __device__ __forceinline__ int lf_v_phys(int row, int ch) {
 // reads in flight (the compiler's own barrier would wait for those too)
 #define LF_BARRIER_VM0() asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory")
 
+// slots per XCD class: (batch, head) pairs of the class, padded to groups of 4, times q-tile pairs
+#define LF_NSLOTS(p, npair) ((((p.B * p.Hq + 7) / 8 + 3) / 4 * 4) * (npair))
+
 extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_swp(const LfAttnParams p) {
   __shared__ __attribute__((aligned(16))) lf_elem lds_k[LF_KSLOTS][LF_BN * LF_D];
   __shared__ __attribute__((aligned(16))) lf_elem lds_v[LF_VSLOTS][LF_BN * LF_D];
@@ -92,11 +95,13 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
   const int npair = (nqt + 1) / 2;
   const int nbh = p.B * p.Hq;
   const int xcd = blockIdx.x & 7;
-  const int slot = blockIdx.x >> 3;
+  // a workgroup takes slots blockIdx.x/8, + gridDim.x/8, ... of its XCD class (the host
+  // may launch fewer workgroups than slots: the resident set, which then stays)
+  for (int slot = blockIdx.x >> 3; slot < LF_NSLOTS(p, npair); slot += (int)(gridDim.x >> 3)) {
   const int grp = slot / (4 * npair);
   const int in_grp = slot % (4 * npair);
   const int bh = (grp * 4 + (in_grp & 3)) * 8 + xcd;
-  if (bh >= nbh) return;
+  if (bh >= nbh) continue;
   const int pair = in_grp >> 2;
   const int b = bh / p.Hq;
   const int h = bh % p.Hq;
@@ -420,21 +425,37 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
     dma_on = true;
 #endif
     const float l_tot = l_run + lf_swap32(l_run);
-    if (my_q < p.Sq) {
+    {
+      // Lane (q, g) holds, per block db, four 4-value chunks d = 32*db + 8*i4 + 4*g + 0..3.
+      // One v_permlane32_swap per register pair trades chunks with the lane that holds
+      // the other half of the same row, so that each lane owns 8 consecutive d's and
+      // writes them with one 16-byte store (32 contiguous bytes per row and instruction).
       const float inv = 1.0f / l_tot;
-      lf_elem* orow = p.o + (long long)b * p.o_sb + (long long)h * p.o_sh + (long long)my_q * p.o_ss;
+      lf_elem* orow = p.o + (long long)b * p.o_sb + (long long)h * p.o_sh +
+                      (long long)min(my_q, p.Sq - 1) * p.o_ss;
 #pragma unroll
-      for (int db = 0; db < LF_NDB; ++db)
+      for (int db = 0; db < LF_NDB; ++db) {
+        unsigned ch[4][2];
 #pragma unroll
         for (int i4 = 0; i4 < 4; ++i4) {
           lf_elem4 w;
 #pragma unroll
           for (int e = 0; e < 4; ++e) w[e] = lf_from_float(o[db][4 * i4 + e] * inv);
-#if LF_ABLATE & 4
-          if (w[0] == (lf_elem)123.25f)
-#endif
-          *reinterpret_cast<lf_elem4*>(orow + 32 * db + 8 * i4 + 4 * g) = w;
+          const lf_u32x2 wu = __builtin_bit_cast(lf_u32x2, w);
+          ch[i4][0] = wu[0];
+          ch[i4][1] = wu[1];
         }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          auto r0 = __builtin_amdgcn_permlane32_swap(ch[2 * j][0], ch[2 * j + 1][0], false, false);
+          auto r1 = __builtin_amdgcn_permlane32_swap(ch[2 * j][1], ch[2 * j + 1][1], false, false);
+          const lf_u32x4 out = {r0[0], r1[0], r0[1], r1[1]};
+#if LF_ABLATE & 4
+          if (out[0] == 0x12345678u)
+#endif
+          if (my_q < p.Sq) *reinterpret_cast<lf_u32x4*>(orow + 32 * db + 16 * j + 8 * g) = out;
+        }
+      }
     }
     // the next q tile's prologue overwrites slots other waves may still read ahead from
     __syncthreads();
@@ -442,4 +463,5 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
 
   run_q_tile(nqt - 1 - pair);
   if (pair != nqt - 1 - pair) run_q_tile(pair);
+  }   // slot
 }

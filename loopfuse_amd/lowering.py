@@ -383,6 +383,9 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         # lf_attn_prefill takes two q tiles (heavy + light) per workgroup
         per_bh = nqt if family == "prefill_pipe" else (nqt + 1) // 2
         grid = 8 * ((per_xcd + 3) // 4 * 4) * per_bh
+        persist = os.environ.get("LOOPFUSE_PREFILL_PERSIST")
+        if family == "prefill_swp" and persist:
+            grid = min(grid, 8 * int(persist))
         get_kernel(spec, spec.entry()).launch((grid, 1, 1), (64 * nw, 1, 1), P)
         attention.last_launch = {"kernels": [spec.entry()], "grid": grid, "block": 64 * nw}
         return (out, visits) if record_visits else out
