@@ -186,6 +186,8 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
 #if LF_SOFTCAP
   const float sc_in = p.scale / p.softcap;   // tanh argument multiplier
   const float cexp = LF_LOG2E;               // scores are final before exp
+#elif LF_BIAS & 1
+  const float cexp = LF_LOG2E;               // scores are scaled explicitly, then biased
 #else
   const float cexp = p.scale * LF_LOG2E;     // scale folded into the exponent
 #endif
@@ -400,6 +402,36 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
 #pragma unroll
         for (int i = 0; i < 16; ++i) s[kb][i] = p.softcap * lf_tanh(s[kb][i] * sc_in);
 #endif
+#if LF_BIAS & 1
+      // additive score bias (reference tests/test_accuracy.py:172-196 "modified attention"):
+      // x = scale * s (or the capped score) + bias[b, h, my_q, j]; four consecutive keys
+      // per 8-byte load, element-wise with clamped indices where the group crosses Sk
+      {
+        const lf_elem* brow = p.bias + (long long)b * p.bias_sb + (long long)h * p.bias_sh +
+                              (long long)min(my_q, p.Sq - 1) * p.bias_sq;
+#pragma unroll
+        for (int kb = 0; kb < LF_NKB; ++kb)
+#pragma unroll
+          for (int i4 = 0; i4 < 4; ++i4) {
+            const int j0 = k0 + 32 * kb + 8 * i4 + 4 * g;
+            lf_elem4 bv;
+            if (!(LF_BIAS & 4) && j0 + 3 < p.Sk) {
+              bv = *reinterpret_cast<const lf_elem4*>(brow + j0);
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) bv[e] = brow[min(j0 + e, p.Sk - 1)];
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+#if LF_SOFTCAP
+              s[kb][4 * i4 + e] += lf_to_float(bv[e]);
+#else
+              s[kb][4 * i4 + e] = s[kb][4 * i4 + e] * p.scale + lf_to_float(bv[e]);
+#endif
+            }
+          }
+      }
+#endif
       if (!full) {
 #pragma unroll
         for (int kb = 0; kb < LF_NKB; ++kb)
@@ -568,8 +600,22 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
         lf_elem4 w;
+#if LF_BIAS & 2
+        const lf_elem* obp = p.obias + (long long)b * p.ob_sb + (long long)h * p.ob_sh +
+                             (long long)my_q * p.ob_sq + 32 * db + 8 * i4 + 4 * g;
+        lf_elem4 ob;
+        if (LF_BIAS & 4) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) ob[e] = obp[e];
+        } else {
+          ob = *reinterpret_cast<const lf_elem4*>(obp);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[e] = lf_from_float(o[db][4 * i4 + e] * inv + lf_to_float(ob[e]));
+#else
 #pragma unroll
         for (int e = 0; e < 4; ++e) w[e] = lf_from_float(o[db][4 * i4 + e] * inv);
+#endif
         *reinterpret_cast<lf_elem4*>(orow + 32 * db + 8 * i4 + 4 * g) = w;
       }
   }

@@ -29,6 +29,10 @@
 #ifndef LF_MASK
 #define LF_MASK 0
 #endif
+#ifndef LF_BIAS
+#define LF_BIAS 0     /* bit 0: score bias tensor, bit 1: output bias tensor, bit 2: their rows are not
+                         8-byte aligned (element loads); lf_attn_prefill only */
+#endif
 #ifndef LF_SOFTCAP
 #define LF_SOFTCAP 0
 #endif
@@ -79,11 +83,16 @@ struct LfAttnParams {
   float* part_acc;           // split-K scratch: [units, nsplit, rows, D]
   float* part_ml;            // split-K scratch: [units, nsplit, rows, 2] (max, sum)
   unsigned char* visits;     // optional [B*Hq*nqt, nkt] visited-tile record
+  const lf_elem* bias;       // LF_BIAS & 1: additive score bias [B, Hq, Sq, Sk] (key stride 1),
+                             // added after scale / softcap and before the mask
+  const lf_elem* obias;      // LF_BIAS & 2: additive output bias [B, Hq, Sq, D] (d stride 1)
   long long q_sb, q_sh, q_ss;  // element strides of Q [B, Hq, Sq, D] (d stride 1)
   long long k_sb, k_sh, k_ss;  // K [B, Hkv, Sk, D]; paged: k_sb = page stride,
                                // k_ss = stride between tokens inside a page
   long long v_sb, v_sh, v_ss;
   long long o_sb, o_sh, o_ss;
+  long long bias_sb, bias_sh, bias_sq;   // element strides of bias (0 = broadcast)
+  long long ob_sb, ob_sh, ob_sq;         // element strides of obias (0 = broadcast)
   int B, Hq, Hkv, Sq, Sk;
   int window;                // sliding-window width (LF_MASK == 2)
   int kt_stride, vt_stride;  // row strides (elements) of k_table / v_table

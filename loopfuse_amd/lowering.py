@@ -41,9 +41,10 @@ class AttnParams(ctypes.Structure):
     """Mirror of ``struct LfAttnParams`` in csrc/kernels/lf_common.hip.h."""
 
     _fields_ = (
-        [(n, ctypes.c_void_p) for n in ("q", "k", "v", "o", "k_table", "v_table", "part_acc", "part_ml", "visits")]
+        [(n, ctypes.c_void_p) for n in ("q", "k", "v", "o", "k_table", "v_table", "part_acc", "part_ml", "visits", "bias", "obias")]
         + [(n, ctypes.c_longlong) for n in (
-            "q_sb", "q_sh", "q_ss", "k_sb", "k_sh", "k_ss", "v_sb", "v_sh", "v_ss", "o_sb", "o_sh", "o_ss")]
+            "q_sb", "q_sh", "q_ss", "k_sb", "k_sh", "k_ss", "v_sb", "v_sh", "v_ss", "o_sb", "o_sh", "o_ss",
+            "bias_sb", "bias_sh", "bias_sq", "ob_sb", "ob_sh", "ob_sq")]
         + [(n, ctypes.c_int) for n in (
             "B", "Hq", "Hkv", "Sq", "Sk", "window", "kt_stride", "vt_stride", "nsplit", "rows", "split_len")]
         + [("scale", ctypes.c_float), ("softcap", ctypes.c_float)]
@@ -66,6 +67,7 @@ class KernelSpec:
     waves: int = 4         # decode: waves per workgroup
     v_tr: bool = True      # prefill: transposed LDS reads for V
     headwave: bool = False  # decode: one kv head per wave (8 waves) instead of 4 waves sharing a head
+    bias: int = 0          # prefill: bit 0 additive score bias tensor, bit 1 additive output bias tensor, bit 2 unaligned rows
     extra: tuple = ()      # further -D options (tuning experiments)
 
     def options(self) -> list[str]:
@@ -81,7 +83,7 @@ class KernelSpec:
         if self.family == "decode":
             o += [f"-DLF_DW={self.waves}", f"-DLF_HEADWAVE={int(self.headwave)}"]
         elif self.family == "prefill":
-            o += [f"-DLF_V_TR={int(self.v_tr)}"]
+            o += [f"-DLF_V_TR={int(self.v_tr)}", f"-DLF_BIAS={self.bias}"]
         return o + list(self.extra)
 
     def files(self) -> tuple[str, ...]:
@@ -94,7 +96,7 @@ class KernelSpec:
 
     def name(self) -> str:
         return (f"lf_{self.family}_t{self.dtype}_d{self.head_dim}_m{self.mask}_c{int(self.softcap)}"
-                f"_p{self.paged}x{self.page_size}i{int(self.table_i64)}_r{self.rows}w{self.waves}v{int(self.v_tr)}h{int(self.headwave)}"
+                f"_p{self.paged}x{self.page_size}i{int(self.table_i64)}_r{self.rows}w{self.waves}v{int(self.v_tr)}h{int(self.headwave)}b{self.bias}"
                 + "".join("_" + e.replace("-D", "").replace("=", "") for e in self.extra))
 
     def source(self) -> str:
@@ -254,11 +256,16 @@ def prefill_variant(Sq: int, v_tr: bool = True) -> str:
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
               k_table: Optional[torch.Tensor] = None, v_table: Optional[torch.Tensor] = None,
               *, out: Optional[torch.Tensor] = None, record_visits: bool = False,
-              force_family: str | None = None, num_splits: int | None = None, v_tr: bool = True):
+              force_family: str | None = None, num_splits: int | None = None, v_tr: bool = True,
+              score_bias: Optional[torch.Tensor] = None, out_bias: Optional[torch.Tensor] = None):
     """Run fused attention on the GPU.
 
     q : [B, Hq, Sq, D];  k, v : [B, Hkv, Sk, D], or page pools [N, P, Hkv, D]
     ([N, Hkv, D] for one-token pages) with ``k_table``/``v_table`` [B, Sk/P].
+    ``score_bias`` (broadcastable to [B, Hq, Sq, Sk], key stride 1) is added to the
+    scaled / capped scores before the mask, ``out_bias`` (broadcastable to
+    [B, Hq, Sq, D]) to the result -- the reference's "modified attention" graph
+    (tests/test_accuracy.py:172-196).  Both are served by ``lf_attn_prefill`` only.
     Returns O [B, Hq, Sq, D] (and the visited-tile record if asked).
     """
     dtype = q.dtype
@@ -334,14 +341,46 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     P.softcap = float(plan.softcap) if plan.softcap else 0.0
     P.nsplit, P.rows, P.split_len = 1, 1, 0
 
+    # ---- additive biases: [B, Hq, Sq, X] views with broadcast (stride 0) batch/head/row dims
+    bias_bits = 0
+
+    def bias_layout(t: torch.Tensor, what: str, last: int):
+        nonlocal bias_bits
+        if t.dtype != dtype or not t.is_cuda:
+            raise UnsupportedPlan(f"{what} must be a {dtype} GPU tensor")
+        if t.dim() > 4:
+            raise UnsupportedPlan(f"{what} has more than 4 dims")
+        try:
+            t = t.expand(B, Hq, Sq, last)
+        except RuntimeError:
+            raise UnsupportedPlan(f"{what} does not broadcast to [{B}, {Hq}, {Sq}, {last}]")
+        if t.stride(3) != 1:
+            raise UnsupportedPlan(f"{what} needs last-dim stride 1")
+        if t.data_ptr() % 8 or any(st % 4 for st in t.stride()[:3]):
+            bias_bits |= 4          # rows not 8-byte aligned: element loads
+        return t
+
+    if score_bias is not None:
+        score_bias = bias_layout(score_bias, "score bias", Sk)
+        P.bias = score_bias.data_ptr()
+        P.bias_sb, P.bias_sh, P.bias_sq = score_bias.stride(0), score_bias.stride(1), score_bias.stride(2)
+        bias_bits |= 1
+    if out_bias is not None:
+        out_bias = bias_layout(out_bias, "output bias", D)
+        P.obias = out_bias.data_ptr()
+        P.ob_sb, P.ob_sh, P.ob_sq = out_bias.stride(0), out_bias.stride(1), out_bias.stride(2)
+        bias_bits |= 2
+    if bias_bits & 3:
+        force_family = "prefill"
+
     # ---- family: decode when there is no mask and few query rows share a KV head
     family = force_family
     if family is None:
         few = (Sq == 1 and group <= 64) or (group == 1 and Sq <= 16)
         family = "decode" if (mask == MASK_NONE and few and Sk >= 16) else "prefill"
-    keep = (q, k, v, out, kt, vt)  # noqa: F841  (tensors stay alive until the launch is queued)
+    keep = (q, k, v, out, kt, vt, score_bias, out_bias)  # noqa: F841  (tensors stay alive until the launch is queued)
 
-    if family == "prefill":
+    if family == "prefill" and not bias_bits:
         family = prefill_variant(Sq, v_tr)
     if family == "prefill_swp":
         # direct-to-LDS staging: dense K/V only, 32-bit byte offsets per (batch, kv head)
@@ -361,8 +400,10 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         span = max((Sk - 1) * abs(P.k_ss), (Sk - 1) * abs(P.v_ss)) * 2 + 2 * D
         if family == "prefill" and span >= (1 << 31):
             extra += ("-DLF_KVBUF=0",)
+        elif family == "prefill" and bias_bits and not paged:
+            extra += ("-DLF_DMA=1",)     # frees the staging registers the bias values need
         spec = KernelSpec(family, _DTYPE_CODE[dtype], D, mask, plan.softcap is not None, paged,
-                          page_size, table_i64, v_tr=v_tr if family == "prefill" else True, extra=extra)
+                          page_size, table_i64, v_tr=v_tr if family == "prefill" else True, bias=bias_bits, extra=extra)
         if os.environ.get("LOOPFUSE_TIMING"):       # profiling aid, see LF_TIMING in the kernel
             attention.timing = torch.zeros(16, dtype=torch.float32, device=q.device)
             P.part_acc = attention.timing.data_ptr()

@@ -50,11 +50,13 @@ class NoMatch(Exception):
 class Source:
     """Where an ``Ids`` tensor's elements come from."""
 
-    kind: str                      # "input" | "paged"
-    index: int                     # placeholder position (pool, for paged)
+    kind: str                      # "input" | "paged" | "computed"
+    index: int                     # placeholder position (pool, for paged; -1 for computed)
     table_index: int = -1          # placeholder position of the page table
     shape: tuple[int, ...] = ()    # stand-in shape the ids enumerate (row-major)
     table_rank: int = 0            # paged: leading dims that come from the table
+    node: Any = None               # computed: the fx node whose value (an elementwise combination of
+                                   # inputs, e.g. Q + q_bias) is evaluated eagerly at call time
 
 
 @dataclasses.dataclass
@@ -81,6 +83,8 @@ class Stage:
     has_tanh: bool = False
     mask: Optional[str] = None
     window: Any = 0                # int or fx.Node (SymInt)
+    bias: Optional[tuple] = None       # (Ids, stage shape when added): additive score bias, before the mask
+    out_bias: Optional[tuple] = None   # (Ids, stage shape when added): additive output bias
 
 
 _VIEW_OPS = {
@@ -93,6 +97,7 @@ _SHAPE_ONLY_VIEW_OPS = {aten.view.default, aten._unsafe_view.default, aten.resha
                         aten.expand.default, aten.clone.default, aten.alias.default,
                         aten.detach.default, aten.contiguous.default}
 _CAST_OPS = {prims.convert_element_type.default, aten._to_copy.default}
+_ELEMENTWISE_OPS = {aten.add.Tensor, aten.sub.Tensor, aten.mul.Tensor, aten.div.Tensor}
 _SCALAR_OPS = {aten.scalar_tensor.default, aten.pow.Tensor_Tensor, aten.pow.Tensor_Scalar,
                aten.pow.Scalar, aten.mul.Tensor, aten.div.Tensor, aten.reciprocal.default,
                aten.sqrt.default, aten.rsqrt.default, aten.neg.default,
@@ -137,6 +142,16 @@ class Operand:
     paged: bool = False
     table_index: int = -1
     group: int = 1                 # head repeat factor seen in the graph (stand-in value)
+    node: Any = None               # computed operand: fx node evaluated eagerly at call time
+
+
+@dataclasses.dataclass
+class BiasOperand:
+    """An additive bias as a strided [B, Hq, Sq, X] view of a graph input (or computed value)."""
+
+    index: int
+    node: Any
+    dims: tuple                    # per logical dim (b, h, row, col): source dim it walks, or None (broadcast)
 
 
 @dataclasses.dataclass
@@ -152,13 +167,16 @@ class AttentionMatch:
     mask: Optional[str]
     window: Any
     out_rank: int
+    bias: Optional[BiasOperand] = None
+    out_bias: Optional[BiasOperand] = None
 
     def describe(self) -> str:
         return (f"attention: Q=arg{self.q.index}{self.q.perm} K=arg{self.k.index}"
                 f"{'[paged by arg%d]' % self.k.table_index if self.k.paged else self.k.perm} "
                 f"V=arg{self.v.index}{'[paged by arg%d]' % self.v.table_index if self.v.paged else self.v.perm} "
                 f"mask={self.mask} window={self.window} tanh={self.has_tanh} "
-                f"factors={self.factors} post={self.post_factors}")
+                f"factors={self.factors} post={self.post_factors}"
+                f"{' +score_bias' if self.bias else ''}{' +out_bias' if self.out_bias else ''}")
 
     # -- call-time evaluation of shape-derived scalars
     def _eval(self, x, env: dict) -> Any:
@@ -195,11 +213,27 @@ class AttentionMatch:
         return lowering.AttnPlan(mask=self.mask, window=int(window), scale=scale, softcap=softcap,
                                  k_paged=self.k.paged, v_paged=self.v.paged)
 
+    def _source(self, index: int, node, args):
+        if node is None:
+            return args[index]
+        env = {p: a for p, a in zip(self.placeholders, args)}
+        return self._eval(node, env)      # e.g. Q + q_bias: run those graph nodes as they are
+
     def _operand(self, op: Operand, args):
-        t = args[op.index]
+        t = self._source(op.index, op.node, args)
         if op.paged:
             return t, args[op.table_index]
         return t.permute(op.perm), None
+
+    def _bias_view(self, bo: Optional[BiasOperand], args, shape):
+        if bo is None:
+            return None
+        t = self._source(bo.index, bo.node, args)
+        strides = tuple(0 if d is None else t.stride(d) for d in bo.dims)
+        for size, d in zip(shape, bo.dims):
+            if d is not None and t.shape[d] != size:
+                raise lowering.UnsupportedPlan("bias does not have the shape seen at trace time")
+        return torch.as_strided(t, tuple(shape), strides, t.storage_offset())
 
     def run(self, args) -> torch.Tensor:
         q, _ = self._operand(self.q, args)
@@ -207,7 +241,11 @@ class AttentionMatch:
             raise lowering.UnsupportedPlan("tensors are not on the GPU")
         k, kt = self._operand(self.k, args)
         v, vt = self._operand(self.v, args)
-        out = lowering.attention(q, k, v, self.plan_for(args), kt, vt)
+        B, Hq, Sq, D = q.shape
+        Sk = kt.shape[1] * (k.shape[1] if k.dim() == 4 else 1) if kt is not None else k.shape[2]
+        out = lowering.attention(q, k, v, self.plan_for(args), kt, vt,
+                                 score_bias=self._bias_view(self.bias, args, (B, Hq, Sq, Sk)),
+                                 out_bias=self._bias_view(self.out_bias, args, (B, Hq, Sq, D)))
         if self.out_rank == 3:
             out = out.view(out.shape[0] * out.shape[1], out.shape[2], out.shape[3])
         return out
@@ -228,8 +266,10 @@ class AttentionMatch:
             ps = k.shape[1] if k.dim() == 4 else 1
             i64 = args[self.k.table_index].dtype == torch.int64
         mask = lowering._MASK_NAMES[plan.mask]
-        family = "prefill" if paged else lowering.prefill_variant(q.shape[-2])
-        return [lowering.KernelSpec(family, dt, D, mask, plan.softcap is not None, paged, ps, i64)]
+        bias = (1 if self.bias else 0) | (2 if self.out_bias else 0)
+        family = "prefill" if (paged or bias) else lowering.prefill_variant(q.shape[-2])
+        extra = ("-DLF_DMA=1",) if (bias and not paged) else ()
+        return [lowering.KernelSpec(family, dt, D, mask, plan.softcap is not None, paged, ps, i64, bias=bias, extra=extra)]
 
 
 # ----------------------------------------------------------------------------
@@ -272,6 +312,48 @@ def _fit_operand(x: torch.Tensor, src: Source, rows_are_d: bool) -> tuple[tuple[
             out = (db, dh, dc, dr) if rows_are_d else (db, dh, dr, dc)
             return out, g
     raise NoMatch("operand is not a (head-repeated) permuted view of one input")
+
+
+def _fit_bias(entry: tuple, logical: tuple) -> BiasOperand:
+    """Express a bias (ids broadcast against the stage it was added to) as a strided
+    [B, Hq, Sq, X] view of its source: per logical dim, the source dim it walks."""
+    ids, stage_shape = entry
+    src = ids.src
+    if src.kind not in ("input", "computed"):
+        raise NoMatch("bias must be a graph input or an elementwise combination of inputs")
+    try:
+        x = torch.broadcast_to(ids.t, stage_shape).reshape(logical)
+    except RuntimeError as e:
+        raise NoMatch(f"bias does not broadcast to the scores/output: {e}")
+    shape = list(src.shape)
+    cstride = [math.prod(shape[i + 1:]) for i in range(len(shape))]
+    zero = (0,) * len(logical)
+    if int(x[zero]) != 0:
+        raise NoMatch("bias view does not start at the first element of its source")
+    dims = []
+    recon = torch.zeros(logical, dtype=torch.int64)
+    for d, n in enumerate(logical):
+        if n == 1:
+            dims.append(None)
+            continue
+        idx = list(zero)
+        idx[d] = 1
+        step = int(x[tuple(idx)])
+        if step == 0:
+            dims.append(None)
+            continue
+        cand = [k for k in range(len(shape)) if cstride[k] == step and shape[k] == n]
+        if not cand:
+            raise NoMatch("bias is not a permuted / broadcast view of one tensor")
+        dims.append(cand[0])
+        view = [1] * len(logical)
+        view[d] = n
+        recon = recon + (torch.arange(n) * step).view(view)
+    if not torch.equal(recon, x):
+        raise NoMatch("bias is not an affine view of its source")
+    if dims[3] is None and logical[3] > 1:
+        raise NoMatch("bias is broadcast along its last dim")
+    return BiasOperand(src.index, src.node, tuple(dims))
 
 
 def match_attention(gm: torch.fx.GraphModule) -> AttentionMatch:
@@ -378,7 +460,14 @@ def _match_attention(gm: torch.fx.GraphModule) -> AttentionMatch:
             env[node] = tgt(*a)
             continue
         if tgt in (aten.sym_size.int,):
-            raise NoMatch("sym_size on intermediate")
+            # size of an intermediate (duck-sized batch == heads makes dynamo re-read it)
+            if isinstance(first, Stage):
+                env[node] = int(first.shape[a[1]])
+            elif isinstance(first, Ids):
+                env[node] = int(first.t.shape[a[1]])
+            else:
+                raise NoMatch("sym_size on an unsupported value")
+            continue
 
         # -- scalars derived from sizes
         if tgt is aten.scalar_tensor.default:
@@ -389,8 +478,27 @@ def _match_attention(gm: torch.fx.GraphModule) -> AttentionMatch:
             env[node] = Scalar(node, 1.0)
             continue
 
+        # -- tensor + scores / tensor + output with the tensor written first
+        if tgt is aten.add.Tensor and isinstance(first, Ids) and len(a) > 1 and isinstance(a[1], Stage) \
+                and not kw.get("alpha", 1) != 1:
+            a = (a[1], a[0]) + tuple(a[2:])
+            first = a[0]
+
         # -- views of inputs
         if isinstance(first, Ids):
+            if tgt in _ELEMENTWISE_OPS and len(a) == 2 and isinstance(a[1], (Ids, int, float)) \
+                    and not isinstance(a[1], bool) and not kw:
+                # an elementwise combination of inputs (the reference's Q + q_bias,
+                # tests/test_accuracy.py:176): a new source, computed eagerly per call
+                other_shape = tuple(a[1].t.shape) if isinstance(a[1], Ids) else ()
+                try:
+                    shape = tuple(torch.broadcast_shapes(tuple(first.t.shape), other_shape))
+                except RuntimeError as e:
+                    raise NoMatch(f"elementwise operands do not broadcast: {e}")
+                n = math.prod(shape)
+                src = Source("computed", -1, shape=shape, node=node)
+                env[node] = Ids(src, torch.arange(n, dtype=torch.int64).reshape(shape))
+                continue
             if tgt in _VIEW_OPS:
                 try:
                     env[node] = Ids(first.src, tgt(first.t, *a[1:], **kw))
@@ -436,6 +544,16 @@ def _match_attention(gm: torch.fx.GraphModule) -> AttentionMatch:
             if tgt in _CAST_OPS:
                 env[node] = st
                 continue
+            if st.kind == "scores" and tgt is aten.add.Tensor and isinstance(a[1], Ids) and st.mask is None \
+                    and st.bias is None and kw.get("alpha", 1) == 1:
+                env[node] = dataclasses.replace(st, bias=(a[1], st.shape))
+                continue
+            if st.kind == "out" and tgt is aten.add.Tensor and isinstance(a[1], Ids) and st.out_bias is None \
+                    and kw.get("alpha", 1) == 1:
+                env[node] = dataclasses.replace(st, out_bias=(a[1], st.shape))
+                continue
+            if st.kind == "scores" and st.bias is not None and tgt in (aten.mul.Tensor, aten.div.Tensor, aten.tanh.default):
+                raise NoMatch("score modification after the additive bias")
             if st.kind == "scores":
                 if tgt in (aten.mul.Tensor, aten.div.Tensor) and st.mask is None:
                     other = a[1]
@@ -491,8 +609,8 @@ def _match_attention(gm: torch.fx.GraphModule) -> AttentionMatch:
     qperm, qg = _fit_operand(st.q.t, st.q.src, rows_are_d=False)
     kperm, kg = _fit_operand(st.kt.t, st.kt.src, rows_are_d=True)
     vperm, vg = _fit_operand(st.v.t, st.v.src, rows_are_d=False)
-    if st.q.src.kind != "input" or qg != 1:
-        raise NoMatch("Q must be a plain graph input")
+    if st.q.src.kind not in ("input", "computed") or qg != 1:
+        raise NoMatch("Q must be a graph input or an elementwise combination of inputs")
     if kg != vg:
         raise NoMatch("K and V head repeat factors differ")
 
@@ -501,7 +619,7 @@ def _match_attention(gm: torch.fx.GraphModule) -> AttentionMatch:
             if perm != (0, 2, 1, 3) or ids.src.table_rank != 2:
                 raise NoMatch("paged operand must be pool[N,(P,)H,D] gathered by table[B,pages]")
             return Operand(ids.src.index, (), True, ids.src.table_index, g)
-        return Operand(ids.src.index, perm, False, -1, g)
+        return Operand(ids.src.index, perm, False, -1, g, node=ids.src.node)
 
     q_op = operand(st.q, qperm, qg)
     k_op = operand(st.kt, kperm, kg)
@@ -519,6 +637,9 @@ def _match_attention(gm: torch.fx.GraphModule) -> AttentionMatch:
     else:
         raise NoMatch("unsupported output rank")
 
+    sk = st.kt.t.shape[-1]
+    bias_op = _fit_bias(st.bias, (qshape[0], qshape[1], qshape[2], sk)) if st.bias is not None else None
+    obias_op = _fit_bias(st.out_bias, qshape) if st.out_bias is not None else None
     m = AttentionMatch(gm, placeholders, q_op, k_op, v_op, list(st.factors), list(st.post_factors),
-                       st.has_tanh, st.mask, st.window, out_rank)
+                       st.has_tanh, st.mask, st.window, out_rank, bias_op, obias_op)
     return m

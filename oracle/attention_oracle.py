@@ -63,8 +63,11 @@ def gather_paged(pool: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
 
 def attention_reference(q, k, v, *, mask: Optional[str] = None, window: int = 0,
                         scale: Optional[float] = None, softcap: Optional[float] = None,
-                        k_table=None, v_table=None) -> torch.Tensor:
-    """fp32 eager attention.  q [B,Hq,Sq,D]; k, v [B,Hkv,Sk,D] or page pools + tables."""
+                        k_table=None, v_table=None, score_bias=None, out_bias=None) -> torch.Tensor:
+    """fp32 eager attention.  q [B,Hq,Sq,D]; k, v [B,Hkv,Sk,D] or page pools + tables.
+    ``score_bias`` (broadcastable to [B,Hq,Sq,Sk]) is added to the scaled / capped scores
+    before the mask and ``out_bias`` ([B,Hq,Sq,D]) to the result, as in the reference's
+    modified-attention graph (tests/test_accuracy.py:172-196)."""
     q = q.float()
     k = gather_paged(k.float(), k_table) if k_table is not None else k.float()
     v = gather_paged(v.float(), v_table) if v_table is not None else v.float()
@@ -78,10 +81,15 @@ def attention_reference(q, k, v, *, mask: Optional[str] = None, window: int = 0,
     s = torch.matmul(q, k.transpose(-2, -1)) * scale
     if softcap is not None:
         s = torch.tanh(s / softcap) * softcap
+    if score_bias is not None:
+        s = s + score_bias.float()
     keep = dense_mask(mask, Sq, Sk, window).to(s.device)
     s = s.masked_fill(~keep, float("-inf"))
     p = torch.softmax(s, dim=-1)
-    return torch.matmul(p, v)
+    out = torch.matmul(p, v)
+    if out_bias is not None:
+        out = out + out_bias.float()
+    return out
 
 
 def online_tiled_reference(q, k, v, *, mask=None, window=0, scale=None, softcap=None,

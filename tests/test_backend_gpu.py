@@ -115,6 +115,45 @@ def test_paged_attention_gqa():
     assert (got - want).abs().max() <= TOL
 
 
+def test_modified_attn():
+    # reference tests/test_accuracy.py:172-196: query bias, score scale and bias, output bias
+    def fn(Q, K, V, q_bias, scores_bias, out_bias):
+        QK = (Q + q_bias) @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        QK = QK * 3.5 + scores_bias
+        return torch.softmax(torch.ops.loopfuse.causal_mask(QK), dim=-1) @ V + out_bias
+
+    B, H, S, D = 4, 8, 1024, 64
+    Q, K, V, qb = (rand((B, H, S, D), seed=s) for s in (1, 2, 3, 4))
+    sb, ob = rand((B, H, S, S), seed=5), rand((B, H, S, D), seed=6)
+    torch._dynamo.mark_static(Q, 3)
+    torch._dynamo.mark_dynamic(Q, 2)
+    got = run_fused(fn, (Q, K, V, qb, sb, ob))
+    # the graph adds the query bias in bf16 before the first product; so does the oracle input
+    want = O.attention_reference(Q + qb, K, V, mask="causal", scale=3.5 * D ** -0.5, score_bias=sb, out_bias=ob)
+    excess = ((got - want).abs() - 2.0 ** -8 * want.abs()).max()     # bf16 rounding of the shifted output
+    assert excess <= TOL
+
+
+def test_broadcast_score_bias_gqa():
+    # an ALiBi-like bias shared by the batch, one slope per head, with grouped K/V
+    def fn(Q, K, V, bias):
+        g = Q.shape[1] // K.shape[1]
+        K = K.repeat_interleave(g, dim=1)
+        V = V.repeat_interleave(g, dim=1)
+        QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5) + bias
+        return torch.softmax(torch.ops.loopfuse.causal_mask(QK), dim=-1) @ V
+
+    B, Hq, Hkv, S, D = 2, 8, 2, 512, 128
+    Q = rand((B, Hq, S, D), seed=1)
+    K, V = (rand((B, Hkv, S, D), seed=s) for s in (2, 3))
+    pos = torch.arange(S)
+    slopes = 2.0 ** -(torch.arange(1, Hq + 1).float())
+    bias = (-(pos[:, None] - pos[None, :]).abs().float() * slopes[:, None, None]).to(torch.bfloat16)[None]
+    got = run_fused(fn, (Q, K, V, bias))
+    want = O.attention_reference(Q, K, V, mask="causal", score_bias=bias)
+    assert (got - want).abs().max() <= TOL
+
+
 def test_paged_decode_gqa_reference_format():
     # tests/benchmark.py:400-443: one-token pages, Q viewed [B, Hkv, group, D]
     def fn(Q, Kc, kt, Vc, vt):

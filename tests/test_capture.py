@@ -50,6 +50,13 @@ def bf(*shape, seed=0):
     return torch.randn(*shape, generator=torch.Generator().manual_seed(seed)).to(torch.bfloat16)
 
 
+def _flat_args(m, tensors):
+    """The flat placeholder list of a call: ints for SymInt placeholders, tensors otherwise."""
+    it = iter(tensors)
+    return [next(it) if isinstance(p.meta["val"], torch.Tensor) else int(p.meta["val"].node.hint)
+            for p in m.placeholders]
+
+
 def test_capture_causal_static_head_dim():
     def fn(q, k, v):
         s = q @ k.transpose(-2, -1) * (q.shape[-1] ** -0.5)
@@ -83,6 +90,50 @@ def test_capture_gqa_softcap_sliding_and_plan_values():
     plan = m.plan_for(args)
     assert plan.mask == "sliding" and plan.window == 256
     assert plan.softcap == pytest.approx(30.0) and plan.scale == pytest.approx(64 ** -0.5, rel=1e-6)
+
+
+def test_capture_modified_attention_biases():
+    # reference tests/test_accuracy.py:172-196
+    def fn(Q, qb, K, sb, V, ob):       # parameters in order of first use = placeholder order
+        QK = (Q + qb) @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        QK = QK * 3.5 + sb
+        return torch.softmax(torch.ops.loopfuse.causal_mask(QK), dim=-1) @ V + ob
+
+    q, k, v, qb = (bf(2, 4, 48, 64, seed=s) for s in range(4))
+    sb, ob = bf(2, 4, 48, 48, seed=5), bf(2, 4, 48, 64, seed=6)
+    m = capture_graph(fn, (q, qb, k, sb, v, ob))["match"]
+    assert m.mask == "causal" and m.q.node is not None          # Q is computed (Q + q_bias)
+    assert m.bias is not None and m.bias.dims == (0, 1, 2, 3) and m.bias.node is None
+    assert m.out_bias is not None and m.out_bias.dims == (0, 1, 2, 3)
+    args = _flat_args(m, (q, qb, k, sb, v, ob))
+    plan = m.plan_for(args)
+    assert plan.scale == pytest.approx(3.5 * 64 ** -0.5, rel=1e-6)
+    # views handed to the kernels: the inputs themselves, Q replaced by the eager sum
+    assert torch.equal(m._operand(m.q, args)[0], q + qb)
+    assert m._bias_view(m.bias, args, (2, 4, 48, 48)).data_ptr() == sb.data_ptr()
+
+
+def test_capture_broadcast_and_transposed_bias():
+    def fn(Q, K, bias, V):
+        s = Q @ K.transpose(-2, -1) * 0.125 + bias.transpose(0, 1)      # stored [H, 1, Sq, Sk]
+        return torch.softmax(s, dim=-1) @ V
+
+    q, k, v = (bf(3, 4, 40, 64, seed=s) for s in range(3))
+    bias = bf(4, 1, 40, 40, seed=4)
+    m = capture_graph(fn, (q, k, bias, v))["match"]
+    assert m.bias.dims == (None, 0, 2, 3)                # batch broadcast, heads walk source dim 0
+    view = m._bias_view(m.bias, _flat_args(m, (q, k, bias, v)), (3, 4, 40, 40))
+    assert torch.equal(view, bias.transpose(0, 1).expand(3, 4, 40, 40))
+
+
+def test_bias_after_mask_or_scaled_afterwards_is_not_matched():
+    def scaled_after(Q, K, V, bias):
+        s = (Q @ K.transpose(-2, -1) + bias) * 0.125
+        return torch.softmax(s, dim=-1) @ V
+
+    q, k, v = (bf(2, 2, 40, 64, seed=s) for s in range(3))
+    box = capture_graph(scaled_after, (q, k, v, bf(2, 2, 40, 40, seed=4)))
+    assert "match" not in box and "nomatch" in box
 
 
 def test_capture_paged_decode():
@@ -125,12 +176,12 @@ def test_capture_paged_page16_reshape():
     assert box["match"].k.paged and box["match"].v.paged
 
 
-@pytest.mark.parametrize("which", ["bias", "add", "softmax_matmul", "two_outputs"])
+@pytest.mark.parametrize("which", ["gated_probs", "add", "softmax_matmul", "two_outputs"])
 def test_unrecognised_graphs_do_not_match(which):
-    if which == "bias":
+    if which == "gated_probs":
         def fn(q, k, v, b):
-            s = q @ k.transpose(-2, -1) * 0.125 + b
-            return torch.softmax(torch.ops.loopfuse.causal_mask(s), dim=-1) @ v
+            s = q @ k.transpose(-2, -1) * 0.125
+            return (torch.softmax(torch.ops.loopfuse.causal_mask(s), dim=-1) * b) @ v
         ins = (bf(1, 2, 32, 64), bf(1, 2, 32, 64, seed=1), bf(1, 2, 32, 64, seed=2), bf(1, 2, 32, 32, seed=3))
     elif which == "add":
         def fn(a, b):

@@ -12,7 +12,7 @@ import torch
 from oracle import attention_oracle as O
 
 
-def brute_force(q, k, v, mask, window, scale, softcap):
+def brute_force(q, k, v, mask, window, scale, softcap, score_bias=None, out_bias=None):
     """float64 loops straight from the definition; no shared code with the oracle."""
     B, Hq, Sq, D = q.shape
     Hkv, Sk = k.shape[1], k.shape[2]
@@ -35,12 +35,16 @@ def brute_force(q, k, v, mask, window, scale, softcap):
                     dot = sum(float(q[b, h, i, d]) * float(k[b, hk, j, d]) for d in range(D)) * scale
                     if softcap is not None:
                         dot = softcap * math.tanh(dot / softcap)
+                    if score_bias is not None:
+                        dot += float(score_bias[b, h, i, j])
                     sc.append(dot)
                 mx = max(x for x in sc if x is not None)
                 w = [0.0 if x is None else math.exp(x - mx) for x in sc]
                 tot = sum(w)
                 for d in range(D):
                     out[b][h][i][d] = sum(w[j] * float(v[b, hk, j, d]) for j in range(Sk)) / tot
+                    if out_bias is not None:
+                        out[b][h][i][d] += float(out_bias[b, h, i, d])
     return torch.tensor(out, dtype=torch.float64)
 
 
@@ -57,6 +61,41 @@ def test_reference_matches_float64_loops(mask, window, softcap, hq, hkv):
     got = O.attention_reference(q, k, v, mask=mask, window=window, scale=scale, softcap=softcap)
     want = brute_force(q, k, v, mask, window, scale, softcap)
     assert torch.allclose(got.double(), want, atol=2e-6, rtol=1e-5)
+
+
+@pytest.mark.parametrize("mask", [None, "causal"])
+@pytest.mark.parametrize("softcap", [None, 2.5])
+def test_biases_match_float64_loops(mask, softcap):
+    g = torch.Generator().manual_seed(11)
+    B, H, S, D = 2, 2, 7, 4
+    q, k, v = (torch.randn(B, H, S, D, generator=g) for _ in range(3))
+    sb = torch.randn(B, H, S, S, generator=g)
+    ob = torch.randn(B, H, S, D, generator=g)
+    got = O.attention_reference(q, k, v, mask=mask, scale=0.6, softcap=softcap, score_bias=sb, out_bias=ob)
+    want = brute_force(q, k, v, mask, 0, 0.6, softcap, sb, ob)
+    assert torch.allclose(got.double(), want, atol=2e-6, rtol=1e-5)
+
+
+def test_bias_closed_forms():
+    g = torch.Generator().manual_seed(12)
+    q, k, v = (torch.randn(1, 2, 6, 8, generator=g) for _ in range(3))
+    base = O.attention_reference(q, k, v, mask="causal")
+    # a bias constant along the key axis cancels in the softmax
+    row_const = torch.randn(1, 2, 6, 1, generator=g).expand(1, 2, 6, 6)
+    assert torch.allclose(O.attention_reference(q, k, v, mask="causal", score_bias=row_const), base, atol=1e-6)
+    # a -inf-like bias on every key but one selects that key's V row (the bias comes before the mask:
+    # a masked key stays masked whatever its bias)
+    pick = torch.full((1, 2, 6, 6), -1e4)
+    pick[..., 0] = 0.0
+    sel = O.attention_reference(q, k, v, mask="causal", score_bias=pick)
+    assert torch.allclose(sel, v[:, :, :1].expand(1, 2, 6, 8), atol=1e-5)
+    unmask = torch.zeros(1, 2, 6, 6)
+    unmask[..., 5] = 1e4           # key 5 is masked for rows 0..4 under the causal mask
+    got = O.attention_reference(q, k, v, mask="causal", score_bias=unmask)
+    assert torch.allclose(got[:, :, :5], base[:, :, :5], atol=1e-6)
+    # the output bias is a plain shift
+    ob = torch.randn(1, 2, 6, 8, generator=g)
+    assert torch.allclose(O.attention_reference(q, k, v, mask="causal", out_bias=ob), base + ob, atol=1e-6)
 
 
 def test_default_scale_is_rsqrt_head_dim():

@@ -24,20 +24,29 @@ def rand(shape, dtype, seed):
     return torch.randn(shape, generator=g, dtype=torch.float32).to(dtype)
 
 
-def check(q, k, v, *, mask=None, window=0, softcap=None, k_table=None, v_table=None, scale=None, **kw):
+def check(q, k, v, *, mask=None, window=0, softcap=None, k_table=None, v_table=None, scale=None,
+          score_bias=None, out_bias=None, **kw):
     dtype = q.dtype
     scale = q.shape[-1] ** -0.5 if scale is None else scale
     plan = lowering.AttnPlan(mask=mask, window=window, scale=scale, softcap=softcap,
                              k_paged=k_table is not None, v_paged=v_table is not None)
     mv = lambda t: None if t is None else t.to(dev())
-    got = lowering.attention(mv(q), mv(k), mv(v), plan, mv(k_table), mv(v_table), **kw)
+    got = lowering.attention(mv(q), mv(k), mv(v), plan, mv(k_table), mv(v_table),
+                             score_bias=mv(score_bias), out_bias=mv(out_bias), **kw)
     if isinstance(got, tuple):
         got = got[0]
     torch.cuda.synchronize()
     want = O.attention_reference(q, k, v, mask=mask, window=window, softcap=softcap, scale=scale,
-                                 k_table=k_table, v_table=v_table)
+                                 k_table=k_table, v_table=v_table, score_bias=score_bias, out_bias=out_bias)
     got = got.float().cpu()
     assert torch.isfinite(got).all()
+    if out_bias is not None:
+        # the bias moves the result away from O(1): add the storage format's half-ulp
+        # (2^-8 relative for bf16, 2^-11 for fp16) of the expected value to the budget
+        rel = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+        excess = ((got - want).abs() - rel * want.abs()).max().item()
+        assert excess <= TOL[dtype], f"max abs err beyond output rounding {excess} > {TOL[dtype]}"
+        return excess
     err = (got - want).abs().max().item()
     assert err <= TOL[dtype], f"max abs err {err} > {TOL[dtype]}"
     return err
@@ -124,6 +133,56 @@ def test_paged_kv_prefill_page16_int64():
     table = torch.randperm(n, generator=g).view(B, S // P)
     q = rand((B, 2 * H, S, D), torch.bfloat16, 3)
     check(q, kp, vp, mask="causal", k_table=table, v_table=table)
+
+
+# ---------------------------------------------------------------- additive biases
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("which", ["score", "out", "both"])
+@pytest.mark.parametrize("S", [333, 336])
+def test_biased_attention(dtype, which, S):
+    # reference tests/test_accuracy.py:172-196 (scores * 3.5 + bias, causal, + output bias);
+    # S = 333: bias rows start at odd offsets (element loads), S = 336: 8-byte loads
+    B, H, D = 2, 4, 64
+    q, k, v = (rand((B, H, S, D), dtype, s) for s in (1, 2, 3))
+    sb = rand((B, H, S, S), dtype, 4) if which != "out" else None
+    ob = rand((B, H, S, D), dtype, 5) if which != "score" else None
+    check(q, k, v, mask="causal", scale=3.5 * D ** -0.5, score_bias=sb, out_bias=ob)
+
+
+def test_biased_attention_broadcast_and_softcap_gqa():
+    B, Hq, Hkv, S, D = 2, 8, 2, 200, 128
+    q = rand((B, Hq, S, D), torch.bfloat16, 1)
+    k, v = (rand((B, Hkv, S, D), torch.bfloat16, s) for s in (2, 3))
+    sb = rand((1, 1, S, S), torch.bfloat16, 4)            # one bias shared by batch and heads
+    ob = rand((1, Hq, 1, D), torch.bfloat16, 5)
+    check(q, k, v, mask="sliding", window=64, softcap=20.0, score_bias=sb, out_bias=ob)
+    check(q[:, :, :1], k, v, score_bias=sb[:, :, :1], out_bias=ob)      # a single query row, no mask
+
+
+def test_biased_attention_paged_kv():
+    B, H, S, D, P = 2, 2, 256, 128, 16
+    n = B * S // P
+    kp, vp = rand((n, P, H, D), torch.bfloat16, 1), rand((n, P, H, D), torch.bfloat16, 2)
+    table = torch.randperm(n, generator=torch.Generator().manual_seed(9)).view(B, S // P).to(torch.int32)
+    q = rand((B, H, S, D), torch.bfloat16, 3)
+    sb = rand((B, H, S, S), torch.bfloat16, 4)
+    check(q, kp, vp, mask="causal", k_table=table, v_table=table, score_bias=sb)
+
+
+def test_unaligned_bias_rows():
+    # contiguous [.., 333, 333] bias: rows start at odd element offsets -> element loads
+    B, H, S, D = 1, 2, 333, 64
+    q, k, v = (rand((B, H, S, D), torch.bfloat16, s) for s in (1, 2, 3))
+    sb = rand((B, H, S, S), torch.bfloat16, 4)
+    ob = rand((B, H, S, D + 2), torch.bfloat16, 5)[..., 1:D + 1]
+    check(q, k, v, mask="causal", score_bias=sb, out_bias=ob)
+
+
+def test_bias_with_wrong_dtype_is_refused():
+    q, k, v = (rand((1, 1, 64, 64), torch.bfloat16, s).to(dev()) for s in (1, 2, 3))
+    sb = rand((1, 1, 64, 64), torch.float16, 4).to(dev())
+    with pytest.raises(lowering.UnsupportedPlan):
+        lowering.attention(q, k, v, lowering.AttnPlan(mask="causal", scale=0.125), score_bias=sb)
 
 
 # ---------------------------------------------------------------- block skip

@@ -67,8 +67,8 @@ def test_launch_geometry_checks(shim_built):
 def test_params_struct_layout():
     from loopfuse_amd.lowering import AttnParams
 
-    # 9 pointers, 12 int64 strides, 11 ints, 2 floats; no implicit padding before the tail
-    assert AttnParams.q.offset == 0 and AttnParams.q_sb.offset == 72
-    assert AttnParams.B.offset == 72 + 96
-    assert AttnParams.scale.offset == 72 + 96 + 44
-    assert ctypes.sizeof(AttnParams) == 224
+    # 11 pointers, 18 int64 strides, 11 ints, 2 floats; no implicit padding before the tail
+    assert AttnParams.q.offset == 0 and AttnParams.q_sb.offset == 88
+    assert AttnParams.B.offset == 88 + 144
+    assert AttnParams.scale.offset == 88 + 144 + 44
+    assert ctypes.sizeof(AttnParams) == 288
