@@ -1,4 +1,4 @@
-"""Graph capture: recognise ``softmax(mask(mods(Q K^T))) V`` in an ATen graph.
+"""Graph capture: find ``softmax(mask(mods(Q K^T) [+ bias])) V [+ bias]`` sub-graphs in an ATen graph.
 
 The reference turns every ATen node into a tiled loop nest and lets its
 optimiser discover the fused form (``loopfuse/torch_backend/interface.py:
@@ -16,6 +16,12 @@ with three kinds of abstract values
                 dynamic D), re-evaluated on every call;
   * ``Stage``   scores / probabilities / output of the attention pipeline,
                 with the score-modification chain seen so far.
+
+Every other node is left to run as it is: its result is an ``Ids`` over a fresh
+"computed" source, so an attention whose operands are produced by other ops
+(``Q + q_bias``, projections, a second attention ...) is still recognised, and a graph
+may hold several attentions.  The caller (``interface.py``) replaces each matched
+output node by one fused call and lets dead-code elimination drop the unfused chain.
 
 Shapes are symbolic under ``dynamic=True``; the interpretation runs on small
 concrete stand-in sizes that keep the divisibility relations of the traced
@@ -50,13 +56,11 @@ class NoMatch(Exception):
 class Source:
     """Where an ``Ids`` tensor's elements come from."""
 
-    kind: str                      # "input" | "paged" | "computed"
-    index: int                     # placeholder position (pool, for paged; -1 for computed)
-    table_index: int = -1          # placeholder position of the page table
+    kind: str                      # "node" (a placeholder or any eagerly computed node) | "paged"
+    node: Any                      # fx node holding the tensor (the pool, for paged)
+    table_node: Any = None         # paged: fx node holding the page table
     shape: tuple[int, ...] = ()    # stand-in shape the ids enumerate (row-major)
     table_rank: int = 0            # paged: leading dims that come from the table
-    node: Any = None               # computed: the fx node whose value (an elementwise combination of
-                                   # inputs, e.g. Q + q_bias) is evaluated eagerly at call time
 
 
 @dataclasses.dataclass
@@ -97,11 +101,6 @@ _SHAPE_ONLY_VIEW_OPS = {aten.view.default, aten._unsafe_view.default, aten.resha
                         aten.expand.default, aten.clone.default, aten.alias.default,
                         aten.detach.default, aten.contiguous.default}
 _CAST_OPS = {prims.convert_element_type.default, aten._to_copy.default}
-_ELEMENTWISE_OPS = {aten.add.Tensor, aten.sub.Tensor, aten.mul.Tensor, aten.div.Tensor}
-_SCALAR_OPS = {aten.scalar_tensor.default, aten.pow.Tensor_Tensor, aten.pow.Tensor_Scalar,
-               aten.pow.Scalar, aten.mul.Tensor, aten.div.Tensor, aten.reciprocal.default,
-               aten.sqrt.default, aten.rsqrt.default, aten.neg.default,
-               prims.convert_element_type.default, aten._to_copy.default}
 
 
 def _hint(sym) -> int:
@@ -135,126 +134,140 @@ def _stand_in_sizes(hints: dict) -> dict:
 
 @dataclasses.dataclass
 class Operand:
-    """How to obtain a [B, H, S, D] strided view of Q/K/V from the call's arguments."""
+    """How to obtain a [B, H, S, D] strided view of Q/K/V from the fused call's inputs."""
 
-    index: int                     # placeholder position of the tensor (pool when paged)
+    index: int                     # position in AttentionMatch.inputs (the pool when paged)
     perm: tuple[int, ...] = ()     # dense: permutation giving [B, H, S, D]
     paged: bool = False
     table_index: int = -1
     group: int = 1                 # head repeat factor seen in the graph (stand-in value)
-    node: Any = None               # computed operand: fx node evaluated eagerly at call time
 
 
 @dataclasses.dataclass
 class BiasOperand:
-    """An additive bias as a strided [B, Hq, Sq, X] view of a graph input (or computed value)."""
+    """An additive bias as a strided [B, Hq, Sq, X] view of one of the fused call's inputs."""
 
     index: int
-    node: Any
     dims: tuple                    # per logical dim (b, h, row, col): source dim it walks, or None (broadcast)
 
 
 @dataclasses.dataclass
 class AttentionMatch:
-    gm: torch.fx.GraphModule
-    placeholders: list[torch.fx.Node]
+    """One attention sub-graph.  ``inputs`` are the graph nodes (placeholders or nodes
+    that keep running unfused) whose run-time values the fused call receives, in
+    order; operands, factors and the window refer to them by position."""
+
+    out_node: torch.fx.Node        # node whose value the fused call replaces
+    inputs: list
     q: Operand
     k: Operand
     v: Operand
-    factors: list                  # floats / fx.Nodes, multiplied together
+    factors: list                  # float | ("arg", i) | ("recip", x), multiplied together
     post_factors: list
     has_tanh: bool
     mask: Optional[str]
-    window: Any
+    window: Any                    # int | ("arg", i)
     out_rank: int
     bias: Optional[BiasOperand] = None
     out_bias: Optional[BiasOperand] = None
 
     def describe(self) -> str:
-        return (f"attention: Q=arg{self.q.index}{self.q.perm} K=arg{self.k.index}"
-                f"{'[paged by arg%d]' % self.k.table_index if self.k.paged else self.k.perm} "
-                f"V=arg{self.v.index}{'[paged by arg%d]' % self.v.table_index if self.v.paged else self.v.perm} "
+        nm = lambda i: self.inputs[i].name
+        return (f"attention -> {self.out_node.name}: Q={nm(self.q.index)}{self.q.perm} K={nm(self.k.index)}"
+                f"{'[paged by %s]' % nm(self.k.table_index) if self.k.paged else self.k.perm} "
+                f"V={nm(self.v.index)}{'[paged by %s]' % nm(self.v.table_index) if self.v.paged else self.v.perm} "
                 f"mask={self.mask} window={self.window} tanh={self.has_tanh} "
                 f"factors={self.factors} post={self.post_factors}"
-                f"{' +score_bias' if self.bias else ''}{' +out_bias' if self.out_bias else ''}")
+                f"{' +score_bias(%s)' % nm(self.bias.index) if self.bias else ''}"
+                f"{' +out_bias(%s)' % nm(self.out_bias.index) if self.out_bias else ''}")
 
     # -- call-time evaluation of shape-derived scalars
-    def _eval(self, x, env: dict) -> Any:
-        if isinstance(x, tuple) and len(x) == 2 and x[0] == "recip":   # from aten.div
-            val = self._eval(x[1], env)
-            return 1.0 / float(val.item() if isinstance(val, torch.Tensor) else val)
-        if isinstance(x, torch.fx.Node):
-            if x in env:
-                return env[x]
-            args = torch.fx.node.map_arg(x.args, lambda n: self._eval(n, env))
-            kwargs = torch.fx.node.map_arg(x.kwargs, lambda n: self._eval(n, env))
-            kwargs = {k: v for k, v in kwargs.items() if k != "device"}
-            val = x.target(*args, **kwargs)
-            env[x] = val
-            return val
-        return x
+    @staticmethod
+    def _number(x, vals) -> float:
+        if isinstance(x, tuple) and x[0] == "recip":
+            return 1.0 / AttentionMatch._number(x[1], vals)
+        if isinstance(x, tuple) and x[0] == "arg":
+            x = vals[x[1]]
+        return float(x.item() if isinstance(x, torch.Tensor) else x)
 
-    def _product(self, items, env) -> float:
+    def _product(self, items, vals) -> float:
         r = 1.0
         for f in items:
-            val = self._eval(f, env)
-            r *= float(val.item() if isinstance(val, torch.Tensor) else val)
+            r *= self._number(f, vals)
         return r
 
-    def plan_for(self, args) -> lowering.AttnPlan:
-        env = {p: a for p, a in zip(self.placeholders, args)}
-        pre = self._product(self.factors, env)
+    def plan_for(self, vals) -> lowering.AttnPlan:
+        pre = self._product(self.factors, vals)
         if self.has_tanh:
-            cap = self._product(self.post_factors, env)
+            cap = self._product(self.post_factors, vals)
             scale, softcap = pre * cap, cap
         else:
             scale, softcap = pre, None
-        window = self._eval(self.window, env) if self.mask == "sliding" else 0
+        window = self._number(self.window, vals) if self.mask == "sliding" else 0
         return lowering.AttnPlan(mask=self.mask, window=int(window), scale=scale, softcap=softcap,
                                  k_paged=self.k.paged, v_paged=self.v.paged)
 
-    def _source(self, index: int, node, args):
-        if node is None:
-            return args[index]
-        env = {p: a for p, a in zip(self.placeholders, args)}
-        return self._eval(node, env)      # e.g. Q + q_bias: run those graph nodes as they are
-
-    def _operand(self, op: Operand, args):
-        t = self._source(op.index, op.node, args)
+    def _operand(self, op: Operand, vals):
+        t = vals[op.index]
         if op.paged:
-            return t, args[op.table_index]
+            return t, vals[op.table_index]
         return t.permute(op.perm), None
 
-    def _bias_view(self, bo: Optional[BiasOperand], args, shape):
+    def _bias_view(self, bo: Optional[BiasOperand], vals, shape):
         if bo is None:
             return None
-        t = self._source(bo.index, bo.node, args)
+        t = vals[bo.index]
         strides = tuple(0 if d is None else t.stride(d) for d in bo.dims)
         for size, d in zip(shape, bo.dims):
             if d is not None and t.shape[d] != size:
                 raise lowering.UnsupportedPlan("bias does not have the shape seen at trace time")
         return torch.as_strided(t, tuple(shape), strides, t.storage_offset())
 
-    def run(self, args) -> torch.Tensor:
-        q, _ = self._operand(self.q, args)
-        if not q.is_cuda:
-            raise lowering.UnsupportedPlan("tensors are not on the GPU")
-        k, kt = self._operand(self.k, args)
-        v, vt = self._operand(self.v, args)
+    def _shapes(self, vals):
+        q, _ = self._operand(self.q, vals)
+        k, kt = self._operand(self.k, vals)
         B, Hq, Sq, D = q.shape
         Sk = kt.shape[1] * (k.shape[1] if k.dim() == 4 else 1) if kt is not None else k.shape[2]
-        out = lowering.attention(q, k, v, self.plan_for(args), kt, vt,
-                                 score_bias=self._bias_view(self.bias, args, (B, Hq, Sq, Sk)),
-                                 out_bias=self._bias_view(self.out_bias, args, (B, Hq, Sq, D)))
+        return B, Hq, Sq, Sk, D
+
+    def out_shape(self, vals) -> tuple:
+        B, Hq, Sq, _, D = self._shapes(vals)
+        return (B * Hq, Sq, D) if self.out_rank == 3 else (B, Hq, Sq, D)
+
+    def input_values(self, gm: torch.fx.GraphModule, flat_args) -> list:
+        """Run-time values of ``inputs`` for a call of the ORIGINAL graph with
+        ``flat_args`` (runs the graph node by node; for tests and debugging)."""
+        class Rec(torch.fx.Interpreter):
+            def run_node(inner, n):
+                r = super().run_node(n)
+                if n in self.inputs:
+                    got[n] = r
+                return r
+
+        got: dict = {}
+        Rec(gm).run(*flat_args)
+        return [got[n] for n in self.inputs]
+
+    def run(self, vals) -> torch.Tensor:
+        """``vals``: run-time values of ``inputs``."""
+        q, _ = self._operand(self.q, vals)
+        if not q.is_cuda:
+            raise lowering.UnsupportedPlan("tensors are not on the GPU")
+        k, kt = self._operand(self.k, vals)
+        v, vt = self._operand(self.v, vals)
+        B, Hq, Sq, Sk, D = self._shapes(vals)
+        out = lowering.attention(q, k, v, self.plan_for(vals), kt, vt,
+                                 score_bias=self._bias_view(self.bias, vals, (B, Hq, Sq, Sk)),
+                                 out_bias=self._bias_view(self.out_bias, vals, (B, Hq, Sq, D)))
         if self.out_rank == 3:
             out = out.view(out.shape[0] * out.shape[1], out.shape[2], out.shape[3])
         return out
 
-    def kernel_specs_for(self, args):
+    def kernel_specs_for(self, vals):
         """Specialisations the call would use (for CODEGEN_ONLY; no GPU needed)."""
-        q, _ = self._operand(self.q, args)
-        plan = self.plan_for(args)
-        k = args[self.k.index]
+        q, _ = self._operand(self.q, vals)
+        plan = self.plan_for(vals)
+        k = vals[self.k.index]
         D = q.shape[-1]
         dt = lowering._DTYPE_CODE.get(q.dtype)
         if dt is None or D not in (64, 128):
@@ -264,7 +277,7 @@ class AttentionMatch:
         i64 = False
         if self.k.paged:
             ps = k.shape[1] if k.dim() == 4 else 1
-            i64 = args[self.k.table_index].dtype == torch.int64
+            i64 = vals[self.k.table_index].dtype == torch.int64
         mask = lowering._MASK_NAMES[plan.mask]
         bias = (1 if self.bias else 0) | (2 if self.out_bias else 0)
         family = "prefill" if (paged or bias) else lowering.prefill_variant(q.shape[-2])
@@ -314,13 +327,14 @@ def _fit_operand(x: torch.Tensor, src: Source, rows_are_d: bool) -> tuple[tuple[
     raise NoMatch("operand is not a (head-repeated) permuted view of one input")
 
 
-def _fit_bias(entry: tuple, logical: tuple) -> BiasOperand:
+def _fit_bias(entry: tuple, logical: tuple):
     """Express a bias (ids broadcast against the stage it was added to) as a strided
-    [B, Hq, Sq, X] view of its source: per logical dim, the source dim it walks."""
+    [B, Hq, Sq, X] view of its source: per logical dim, the source dim it walks.
+    Returns (source node, dims)."""
     ids, stage_shape = entry
     src = ids.src
-    if src.kind not in ("input", "computed"):
-        raise NoMatch("bias must be a graph input or an elementwise combination of inputs")
+    if src.kind != "node":
+        raise NoMatch("bias must be a plain tensor")
     try:
         x = torch.broadcast_to(ids.t, stage_shape).reshape(logical)
     except RuntimeError as e:
@@ -353,11 +367,12 @@ def _fit_bias(entry: tuple, logical: tuple) -> BiasOperand:
         raise NoMatch("bias is not an affine view of its source")
     if dims[3] is None and logical[3] > 1:
         raise NoMatch("bias is broadcast along its last dim")
-    return BiasOperand(src.index, src.node, tuple(dims))
+    return src.node, tuple(dims)
 
 
-def match_attention(gm: torch.fx.GraphModule) -> AttentionMatch:
-    """Interpret ``gm`` abstractly; return the match or raise ``NoMatch``.
+def match_attention(gm: torch.fx.GraphModule) -> list:
+    """Interpret ``gm`` abstractly; return its attention sub-graphs (``AttentionMatch``
+    list, possibly several) or raise ``NoMatch`` with the reason none was found.
 
     The fw_compiler runs under AOTAutograd's fake-tensor mode; the stand-in id
     tensors must be real, so dispatch modes are switched off for the duration.
@@ -368,15 +383,16 @@ def match_attention(gm: torch.fx.GraphModule) -> AttentionMatch:
         return _match_attention(gm)
 
 
-def _match_attention(gm: torch.fx.GraphModule) -> AttentionMatch:
+class _Skip(Exception):
+    """This node does not continue an attention pattern: treat it as an ordinary op."""
+
+
+def _match_attention(gm: torch.fx.GraphModule) -> list:
     graph = gm.graph
     placeholders = [n for n in graph.nodes if n.op == "placeholder"]
     outputs = [n for n in graph.nodes if n.op == "output"]
     if len(outputs) != 1:
         raise NoMatch("no single output node")
-    out_args = outputs[0].args[0]
-    if not isinstance(out_args, (tuple, list)) or len(out_args) != 1 or not isinstance(out_args[0], torch.fx.Node):
-        raise NoMatch("graph does not return exactly one tensor")
 
     # ---- stand-in sizes for every free symbol
     import sympy
@@ -415,15 +431,19 @@ def _match_attention(gm: torch.fx.GraphModule) -> AttentionMatch:
             return int(d.node.expr.subs(sizes))
         return int(d)
 
+    def fresh_ids(node: torch.fx.Node, val) -> Any:
+        """A tensor-valued node that simply runs: ids over its own (stand-in) shape."""
+        shape = tuple(concrete(d) for d in val.shape)
+        n = math.prod(shape)
+        if n > (1 << 22):
+            raise NoMatch("stand-in tensor too large")
+        return Ids(Source("node", node, shape=shape), torch.arange(n, dtype=torch.int64).reshape(shape))
+
     env: dict[torch.fx.Node, Any] = {}
-    for i, p in enumerate(placeholders):
+    for p in placeholders:
         val = p.meta.get("val")
         if isinstance(val, torch.Tensor):
-            shape = tuple(concrete(d) for d in val.shape)
-            n = math.prod(shape)
-            if n > (1 << 22):
-                raise NoMatch("stand-in tensor too large")
-            env[p] = Ids(Source("input", i, shape=shape), torch.arange(n, dtype=torch.int64).reshape(shape))
+            env[p] = fresh_ids(p, val)
         elif isinstance(val, (torch.SymInt, int)):
             env[p] = concrete(val)
         elif isinstance(val, (torch.SymFloat, float)):
@@ -441,92 +461,83 @@ def _match_attention(gm: torch.fx.GraphModule) -> AttentionMatch:
         m = torch.empty(shape, device="meta")
         return tuple(target(m, *args, **kwargs).shape)
 
-    for node in graph.nodes:
-        if node.op in ("placeholder", "output"):
-            continue
-        if node.op == "get_attr":
-            raise NoMatch("graph has constant tensors")
-        if node.op != "call_function":
-            raise NoMatch(f"unsupported node kind {node.op}")
-        tgt = node.target
-        a = arg(node.args)
-        kw = arg(node.kwargs)
-        first = a[0] if a else None
+    matches: list = []
+    reasons: list = []
+    finalised: dict = {}
 
+    def finalise(node: torch.fx.Node) -> None:
+        """``node`` holds a finished attention that something outside the pattern reads."""
+        if node in finalised:
+            return
+        finalised[node] = None
+        try:
+            finalised[node] = _build_match(node, env[node])
+            matches.append(finalised[node])
+        except NoMatch as e:
+            reasons.append(str(e))
+
+    def consume(values) -> None:
+        for x in values:
+            if isinstance(x, torch.fx.Node) and isinstance(env.get(x), Stage) and env[x].kind == "out":
+                finalise(x)
+
+    def pattern_step(node, tgt, a, kw, first):
+        """The abstract value of ``node`` if it continues a pattern; raises _Skip otherwise."""
         # -- integer / float arithmetic on sizes
         if all(is_number(x) for x in a) and tgt in (
                 operator.mul, operator.floordiv, operator.add, operator.sub, operator.truediv,
                 operator.pow, operator.neg, operator.mod):
-            env[node] = tgt(*a)
-            continue
-        if tgt in (aten.sym_size.int,):
+            return tgt(*a)
+        if tgt is aten.sym_size.int:
             # size of an intermediate (duck-sized batch == heads makes dynamo re-read it)
             if isinstance(first, Stage):
-                env[node] = int(first.shape[a[1]])
-            elif isinstance(first, Ids):
-                env[node] = int(first.t.shape[a[1]])
-            else:
-                raise NoMatch("sym_size on an unsupported value")
-            continue
+                return int(first.shape[a[1]])
+            if isinstance(first, Ids):
+                return int(first.t.shape[a[1]])
+            raise _Skip("sym_size on an unsupported value")
 
         # -- scalars derived from sizes
-        if tgt is aten.scalar_tensor.default:
-            env[node] = Scalar(node, float(a[0]))
-            continue
-        if isinstance(first, Scalar) and tgt in _SCALAR_OPS and all(
-                isinstance(x, (Scalar, int, float, torch.dtype)) for x in a):
-            env[node] = Scalar(node, 1.0)
-            continue
+        if tgt is aten.scalar_tensor.default and is_number(a[0]):
+            return Scalar(node, float(a[0]))
+        val = node.meta.get("val")
+        if isinstance(first, Scalar) and isinstance(val, torch.Tensor) and val.dim() == 0 and all(
+                isinstance(x, (Scalar, int, float, bool, str, torch.dtype, type(None)))
+                for x in list(a) + list(kw.values())):
+            return Scalar(node, 1.0)       # any arithmetic among shape-derived 0-dim values
 
         # -- tensor + scores / tensor + output with the tensor written first
         if tgt is aten.add.Tensor and isinstance(first, Ids) and len(a) > 1 and isinstance(a[1], Stage) \
-                and not kw.get("alpha", 1) != 1:
+                and kw.get("alpha", 1) == 1:
             a = (a[1], a[0]) + tuple(a[2:])
             first = a[0]
 
-        # -- views of inputs
+        # -- views of tensors
         if isinstance(first, Ids):
-            if tgt in _ELEMENTWISE_OPS and len(a) == 2 and isinstance(a[1], (Ids, int, float)) \
-                    and not isinstance(a[1], bool) and not kw:
-                # an elementwise combination of inputs (the reference's Q + q_bias,
-                # tests/test_accuracy.py:176): a new source, computed eagerly per call
-                other_shape = tuple(a[1].t.shape) if isinstance(a[1], Ids) else ()
-                try:
-                    shape = tuple(torch.broadcast_shapes(tuple(first.t.shape), other_shape))
-                except RuntimeError as e:
-                    raise NoMatch(f"elementwise operands do not broadcast: {e}")
-                n = math.prod(shape)
-                src = Source("computed", -1, shape=shape, node=node)
-                env[node] = Ids(src, torch.arange(n, dtype=torch.int64).reshape(shape))
-                continue
             if tgt in _VIEW_OPS:
                 try:
-                    env[node] = Ids(first.src, tgt(first.t, *a[1:], **kw))
+                    return Ids(first.src, tgt(first.t, *a[1:], **kw))
                 except Exception as e:  # invalid for the stand-in sizes
-                    raise NoMatch(f"view chain not reproducible on stand-in sizes: {e}")
-                continue
+                    raise _Skip(f"view chain not reproducible on stand-in sizes: {e}")
             if tgt is torch.ops.loopfuse.paged_load.default:
                 pool, table = a[0], a[1]
-                if not (isinstance(table, Ids) and pool.src.kind == "input" and table.src.kind == "input"):
-                    raise NoMatch("paged_load operands must be graph inputs")
+                if not (isinstance(table, Ids) and pool.src.kind == "node" and table.src.kind == "node"):
+                    raise _Skip("paged_load operands must be plain tensors")
                 if pool.t.shape != pool.src.shape or table.t.shape != table.src.shape or \
                         not torch.equal(pool.t.reshape(-1), torch.arange(pool.t.numel())) or \
                         not torch.equal(table.t.reshape(-1), torch.arange(table.t.numel())):
-                    raise NoMatch("paged_load operands must be untouched graph inputs")
+                    raise _Skip("paged_load operands must be whole tensors, not views")
                 shape = tuple(table.src.shape) + tuple(pool.src.shape[1:])
-                src = Source("paged", pool.src.index, table.src.index, shape, len(table.src.shape))
-                env[node] = Ids(src, torch.arange(math.prod(shape), dtype=torch.int64).reshape(shape))
-                continue
+                src = Source("paged", pool.src.node, table.src.node, shape, len(table.src.shape))
+                return Ids(src, torch.arange(math.prod(shape), dtype=torch.int64).reshape(shape))
             if tgt in (aten.bmm.default, aten.mm.default, aten.matmul.default) and isinstance(a[1], Ids):
                 qi, ki = a[0], a[1]
                 if qi.t.dim() < 3 or ki.t.dim() != qi.t.dim():
-                    raise NoMatch("QK^T is not a batched matmul")
+                    raise _Skip("QK^T is not a batched matmul")
                 if qi.t.shape[:-2] != ki.t.shape[:-2] or qi.t.shape[-1] != ki.t.shape[-2]:
-                    raise NoMatch("QK^T shapes disagree")
+                    raise _Skip("QK^T shapes disagree")
                 shape = tuple(qi.t.shape[:-1]) + (ki.t.shape[-1],)
-                env[node] = Stage("scores", shape, qi, ki)
-                continue
-            raise NoMatch(f"unsupported op on an input view: {tgt}")
+                return Stage("scores", shape, qi, ki)
+            raise _Skip(f"op on a tensor view: {tgt}")
 
         # -- the attention pipeline
         if isinstance(first, Stage):
@@ -536,24 +547,20 @@ def _match_attention(gm: torch.fx.GraphModule) -> AttentionMatch:
                 try:
                     new_shape = meta_view(tgt, st.shape, a[1:], kw2)
                 except Exception as e:
-                    raise NoMatch(f"reshape of scores not reproducible: {e}")
+                    raise _Skip(f"reshape of scores not reproducible: {e}")
                 if new_shape[-2:] != st.shape[-2:] or math.prod(new_shape) != math.prod(st.shape):
-                    raise NoMatch("reshape changes the matrix dims of the scores")
-                env[node] = dataclasses.replace(st, shape=new_shape)
-                continue
+                    raise _Skip("reshape changes the matrix dims of the scores")
+                return dataclasses.replace(st, shape=new_shape)
             if tgt in _CAST_OPS:
-                env[node] = st
-                continue
+                return st
             if st.kind == "scores" and tgt is aten.add.Tensor and isinstance(a[1], Ids) and st.mask is None \
                     and st.bias is None and kw.get("alpha", 1) == 1:
-                env[node] = dataclasses.replace(st, bias=(a[1], st.shape))
-                continue
+                return dataclasses.replace(st, bias=(a[1], st.shape))
             if st.kind == "out" and tgt is aten.add.Tensor and isinstance(a[1], Ids) and st.out_bias is None \
                     and kw.get("alpha", 1) == 1:
-                env[node] = dataclasses.replace(st, out_bias=(a[1], st.shape))
-                continue
+                return dataclasses.replace(st, out_bias=(a[1], st.shape))
             if st.kind == "scores" and st.bias is not None and tgt in (aten.mul.Tensor, aten.div.Tensor, aten.tanh.default):
-                raise NoMatch("score modification after the additive bias")
+                raise _Skip("score modification after the additive bias")
             if st.kind == "scores":
                 if tgt in (aten.mul.Tensor, aten.div.Tensor) and st.mask is None:
                     other = a[1]
@@ -563,7 +570,7 @@ def _match_attention(gm: torch.fx.GraphModule) -> AttentionMatch:
                     elif is_number(other):
                         f = raw if isinstance(raw, torch.fx.Node) else float(other)
                     else:
-                        raise NoMatch("scores multiplied by a tensor (bias/modified attention)")
+                        raise _Skip("scores multiplied by a tensor")
                     if tgt is aten.div.Tensor:
                         f = ("recip", f)
                     new = dataclasses.replace(st)
@@ -571,46 +578,83 @@ def _match_attention(gm: torch.fx.GraphModule) -> AttentionMatch:
                         new.post_factors = st.post_factors + [f]
                     else:
                         new.factors = st.factors + [f]
-                    env[node] = new
-                    continue
+                    return new
                 if tgt is aten.tanh.default and not st.has_tanh and st.mask is None:
-                    env[node] = dataclasses.replace(st, has_tanh=True)
-                    continue
+                    return dataclasses.replace(st, has_tanh=True)
                 if tgt is torch.ops.loopfuse.causal_mask.default and st.mask is None:
-                    env[node] = dataclasses.replace(st, mask="causal")
-                    continue
+                    return dataclasses.replace(st, mask="causal")
                 if tgt is torch.ops.loopfuse.sliding_mask.default and st.mask is None:
                     w = node.args[1]
-                    env[node] = dataclasses.replace(st, mask="sliding", window=w if isinstance(w, torch.fx.Node) else int(a[1]))
-                    continue
+                    return dataclasses.replace(st, mask="sliding", window=w if isinstance(w, torch.fx.Node) else int(a[1]))
                 if tgt is aten._softmax.default:
                     dim = a[1]
                     if dim not in (-1, len(st.shape) - 1) or a[2]:
-                        raise NoMatch("softmax not over the key dimension")
-                    env[node] = dataclasses.replace(st, kind="probs")
-                    continue
-                raise NoMatch(f"unsupported score modification: {tgt}")
+                        raise _Skip("softmax not over the key dimension")
+                    return dataclasses.replace(st, kind="probs")
+                raise _Skip(f"unsupported score modification: {tgt}")
             if st.kind == "probs":
                 if tgt in (aten.bmm.default, aten.mm.default, aten.matmul.default) and isinstance(a[1], Ids):
                     vi = a[1]
                     if vi.t.dim() != len(st.shape) or vi.t.shape[:-2] != st.shape[:-2] or vi.t.shape[-2] != st.shape[-1]:
-                        raise NoMatch("PV shapes disagree")
-                    env[node] = dataclasses.replace(st, kind="out", v=vi, shape=tuple(st.shape[:-1]) + (vi.t.shape[-1],))
-                    continue
-                raise NoMatch(f"unsupported op on probabilities: {tgt}")
-            raise NoMatch(f"unsupported op on the attention output: {tgt}")
+                        raise _Skip("PV shapes disagree")
+                    return dataclasses.replace(st, kind="out", v=vi, shape=tuple(st.shape[:-1]) + (vi.t.shape[-1],))
+                raise _Skip(f"unsupported op on probabilities: {tgt}")
+            raise _Skip(f"op on the attention output: {tgt}")
 
-        raise NoMatch(f"unsupported node {node.format_node()}")
+        raise _Skip(f"ordinary node {node.name}")
 
-    result = env.get(out_args[0])
-    if not isinstance(result, Stage) or result.kind != "out":
-        raise NoMatch("output is not an attention result")
-    st = result
+    for node in graph.nodes:
+        if node.op == "placeholder":
+            continue
+        if node.op == "output":
+            consume(node.all_input_nodes)
+            continue
+        if node.op == "get_attr":
+            raise NoMatch("graph has constant tensors")
+        if node.op != "call_function":
+            raise NoMatch(f"unsupported node kind {node.op}")
+        a = arg(node.args)
+        kw = arg(node.kwargs)
+        first = a[0] if a else None
+        try:
+            env[node] = pattern_step(node, node.target, a, kw, first)
+            continue
+        except _Skip as e:
+            if any(isinstance(x, Stage) for x in list(a) + list(kw.values())):
+                reasons.append(str(e))
+        # an ordinary op: it keeps running as it is; finished attentions it reads are fused
+        consume(node.all_input_nodes)
+        val = node.meta.get("val")
+        if isinstance(val, torch.Tensor):
+            env[node] = fresh_ids(node, val)
+        elif isinstance(val, (tuple, list)):
+            env[node] = None      # its elements are reached through getitem nodes, each a source of its own
+        elif isinstance(val, (torch.SymInt, int)) and not isinstance(val, bool):
+            env[node] = concrete(val)
+        elif isinstance(val, (torch.SymFloat, float)):
+            env[node] = Scalar(node, 1.0)
+        else:
+            env[node] = None
+
+    if not matches:
+        raise NoMatch(reasons[0] if reasons else "no attention pattern in the graph")
+    return matches
+
+
+def _build_match(out_node: torch.fx.Node, st: Stage) -> AttentionMatch:
+    """Operands, factors and biases of a finished attention in terms of graph nodes."""
+    inputs: list = []
+
+    def slot(n: torch.fx.Node) -> int:
+        if n not in inputs:
+            inputs.append(n)
+        return inputs.index(n)
+
     qperm, qg = _fit_operand(st.q.t, st.q.src, rows_are_d=False)
     kperm, kg = _fit_operand(st.kt.t, st.kt.src, rows_are_d=True)
     vperm, vg = _fit_operand(st.v.t, st.v.src, rows_are_d=False)
-    if st.q.src.kind not in ("input", "computed") or qg != 1:
-        raise NoMatch("Q must be a graph input or an elementwise combination of inputs")
+    if st.q.src.kind != "node" or qg != 1:
+        raise NoMatch("Q must be a plain tensor")
     if kg != vg:
         raise NoMatch("K and V head repeat factors differ")
 
@@ -618,8 +662,8 @@ def _match_attention(gm: torch.fx.GraphModule) -> AttentionMatch:
         if ids.src.kind == "paged":
             if perm != (0, 2, 1, 3) or ids.src.table_rank != 2:
                 raise NoMatch("paged operand must be pool[N,(P,)H,D] gathered by table[B,pages]")
-            return Operand(ids.src.index, (), True, ids.src.table_index, g)
-        return Operand(ids.src.index, perm, False, -1, g, node=ids.src.node)
+            return Operand(slot(ids.src.node), (), True, slot(ids.src.table_node), g)
+        return Operand(slot(ids.src.node), perm, False, -1, g)
 
     q_op = operand(st.q, qperm, qg)
     k_op = operand(st.kt, kperm, kg)
@@ -637,9 +681,22 @@ def _match_attention(gm: torch.fx.GraphModule) -> AttentionMatch:
     else:
         raise NoMatch("unsupported output rank")
 
+    def scalar(f):
+        if isinstance(f, tuple) and f[0] == "recip":
+            return ("recip", scalar(f[1]))
+        if isinstance(f, torch.fx.Node):
+            return ("arg", slot(f))
+        return f
+
     sk = st.kt.t.shape[-1]
-    bias_op = _fit_bias(st.bias, (qshape[0], qshape[1], qshape[2], sk)) if st.bias is not None else None
-    obias_op = _fit_bias(st.out_bias, qshape) if st.out_bias is not None else None
-    m = AttentionMatch(gm, placeholders, q_op, k_op, v_op, list(st.factors), list(st.post_factors),
-                       st.has_tanh, st.mask, st.window, out_rank, bias_op, obias_op)
-    return m
+    bias_op = obias_op = None
+    if st.bias is not None:
+        n, dims = _fit_bias(st.bias, (qshape[0], qshape[1], qshape[2], sk))
+        bias_op = BiasOperand(slot(n), dims)
+    if st.out_bias is not None:
+        n, dims = _fit_bias(st.out_bias, qshape)
+        obias_op = BiasOperand(slot(n), dims)
+    window = scalar(st.window) if st.mask == "sliding" else 0
+    return AttentionMatch(out_node, inputs, q_op, k_op, v_op, [scalar(f) for f in st.factors],
+                          [scalar(f) for f in st.post_factors], st.has_tanh, st.mask, window, out_rank,
+                          bias_op, obias_op)

@@ -14,11 +14,12 @@ and the same environment switches ``DEBUG``, ``CODEGEN_ONLY`` and
 Where the reference parses the ATen graph into per-op loop nests, fuses them and
 prints Triton (``interface.py:387-400``, ``optimize.py:34-60``,
 ``codegen.py:100-126``), this front end recognises the fused result directly: it
-abstract-interprets the graph (``capture.py``) and, when the graph is
-``softmax(mask(mods(Q K^T))) V``, produces an ``AttnPlan`` that
-``lowering.attention`` runs on the hand-written HIP kernels.
+abstract-interprets the graph (``capture.py``), finds every sub-graph of the form
+``softmax(mask(mods(Q K^T) [+ bias])) V [+ bias]`` and replaces it by one call that
+``lowering.attention`` runs on the hand-written HIP kernels; the rest of the graph
+keeps running as it is.
 
-Graphs that are not of that form, and calls on CPU tensors, run the captured
+Graphs without such a sub-graph, and calls on CPU tensors, run the captured
 graph unchanged (the reference raises ``ValueError``/``NotImplementedError``
 there, ``interface.py:157-161``).  Set ``LOOPFUSE_STRICT=1`` to raise instead;
 ``stats`` counts which route each call took so tests can insist on the fused one.
@@ -69,23 +70,58 @@ def loopfuse_backend(gm: torch.fx.GraphModule, sample_inputs, mode="max-autotune
     return aot_module_simplified(gm, sample_inputs, fw_compiler=compiler)
 
 
+# attention sub-graphs of the graphs compiled so far; the rewritten graphs call
+# ``_fused_call(id, *inputs)`` where the unfused chain used to end
+_MATCHES: list = []
+_codegen_sink: list | None = None     # CODEGEN_ONLY: compiled specialisations are collected here
+
+
+def _fused_call(match_id: int, *vals):
+    """Stand-in for one attention sub-graph inside a rewritten graph."""
+    match = _MATCHES[match_id]
+    if _codegen_sink is not None:
+        _codegen_sink.extend(lowering.compile_spec(s) for s in match.kernel_specs_for(vals))
+        q = vals[match.q.index]
+        return torch.empty(match.out_shape(vals), dtype=q.dtype, device=q.device)
+    return match.run(vals)
+
+
+def rewrite_graph(gm: torch.fx.GraphModule, matches: list) -> torch.fx.GraphModule:
+    """A copy of ``gm`` in which every matched attention output is produced by one
+    ``_fused_call`` node; what only fed the unfused chain is dropped."""
+    new_graph = torch.fx.Graph()
+    val_map: dict = {}
+    out = new_graph.graph_copy(gm.graph, val_map)
+    new_graph.output(out)
+    for m in matches:
+        _MATCHES.append(m)
+        old = val_map[m.out_node]
+        with new_graph.inserting_after(old):
+            call = new_graph.call_function(_fused_call, (len(_MATCHES) - 1, *[val_map[n] for n in m.inputs]))
+        old.replace_all_uses_with(call)
+    new_graph.eliminate_dead_code()
+    new_graph.lint()
+    return torch.fx.GraphModule(gm, new_graph)
+
+
 def loopfuse_compiler(gm: torch.fx.GraphModule, sample_inputs, input_names: list[str] | None = None,
                       symint_names: dict[str, str] | None = None, mode: str | None = None) -> Callable:
     """fw_compiler: ATen graph -> callable over the flat placeholder list."""
+    global _codegen_sink
     stats["compiled_graphs"] += 1
     if DEBUG:
         print("---- loopfuse_amd: ATen graph ----")
         print(gm.code)
     try:
-        match = capture.match_attention(gm)
+        matches = capture.match_attention(gm)
     except capture.NoMatch as e:
-        match = None
+        matches = []
         reason = str(e)
     else:
         reason = ""
-    if match is None:
+    if not matches:
         if _strict():
-            raise NotImplementedError(f"loopfuse_amd: graph is not a fused-attention pattern: {reason}")
+            raise NotImplementedError(f"loopfuse_amd: no fused-attention pattern in the graph: {reason}")
         log.info("graph not recognised (%s); running it unfused", reason)
         if DEBUG:
             print(f"---- loopfuse_amd: no match ({reason}); eager graph ----")
@@ -97,22 +133,30 @@ def loopfuse_compiler(gm: torch.fx.GraphModule, sample_inputs, input_names: list
         return eager_fn
 
     stats["matched_graphs"] += 1
+    fused_gm = rewrite_graph(gm, matches)
     if DEBUG:
         print("---- loopfuse_amd: matched ----")
-        print(match.describe())
+        for m in matches:
+            print(m.describe())
+        print(fused_gm.code)
 
     if CODEGEN_ONLY:
         # no launch: hand back what would be compiled, as the reference hands back
         # KernelData under CODEGEN_ONLY (interface.py:615-622)
         def codegen_fn(*args):
-            specs = match.kernel_specs_for(args)
-            return [lowering.compile_spec(s) for s in specs]
+            global _codegen_sink
+            _codegen_sink = []
+            try:
+                fused_gm(*args)
+                return list(_codegen_sink)
+            finally:
+                _codegen_sink = None
 
         return codegen_fn
 
     def optimized_fn(*args):
         try:
-            out = match.run(args)
+            out = fused_gm(*args)
         except lowering.UnsupportedPlan as e:
             if _strict():
                 raise
@@ -120,6 +164,6 @@ def loopfuse_compiler(gm: torch.fx.GraphModule, sample_inputs, input_names: list
             stats["eager_runtime"] += 1
             return gm(*args)
         stats["fused"] += 1
-        return (out,)
+        return out
 
     return optimized_fn

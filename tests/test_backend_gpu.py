@@ -154,6 +154,43 @@ def test_broadcast_score_bias_gqa():
     assert (got - want).abs().max() <= TOL
 
 
+def test_prefix_attention_two_fused_calls():
+    # reference tests/test_attention.py:339-362: a shared prefix (batch 1, broadcast) attended without
+    # a mask plus the causal suffix, each with its own softmax, summed
+    def fn(Q, Kp, Vp, Ks, Vs):
+        QKp = Q @ Kp.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        QKs = Q @ Ks.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        return torch.softmax(QKp, dim=-1) @ Vp + torch.softmax(torch.ops.loopfuse.causal_mask(QKs), dim=-1) @ Vs
+
+    B, H, Sq, Sp, D = 3, 4, 320, 512, 128
+    Q, Ks, Vs = (rand((B, H, Sq, D), seed=s) for s in (1, 2, 3))
+    Kp, Vp = (rand((B, H, Sp, D), seed=s) for s in (4, 5))
+    n0 = len(interface._MATCHES)
+    got = run_fused(fn, (Q, Kp, Vp, Ks, Vs))
+    assert len(interface._MATCHES) == n0 + 2
+    want = O.attention_reference(Q, Kp, Vp) + O.attention_reference(Q, Ks, Vs, mask="causal")
+    assert (got - want).abs().max() <= 2 * TOL      # two bf16 results added in bf16
+
+
+def test_attention_inside_a_transformer_block():
+    # the attention is found inside projections and a residual; everything else runs as it is
+    def fn(x, wq, wk, wv, wo):
+        B, S, E = x.shape
+        H = 8
+        q = (x @ wq).view(B, S, H, E // H).transpose(1, 2)
+        k = (x @ wk).view(B, S, H, E // H).transpose(1, 2)
+        v = (x @ wv).view(B, S, H, E // H).transpose(1, 2)
+        a = torch.softmax(torch.ops.loopfuse.causal_mask(q @ k.transpose(-2, -1) * (E // H) ** -0.5), dim=-1) @ v
+        return a.transpose(1, 2).reshape(B, S, E) @ wo + x
+
+    x = rand((2, 384, 1024), seed=1)
+    ws = [rand((1024, 1024), seed=s) * 0.03 for s in (2, 3, 4, 5)]
+    ws = [w.to(torch.bfloat16) for w in ws]
+    got = run_fused(fn, (x, *ws))
+    want = fn(*[t.to(DEV) for t in (x, *ws)]).float().cpu()       # the same graph, eager, on the GPU
+    assert (got - want).abs().max() <= 4 * TOL and (got - want).abs().mean() <= 4e-3
+
+
 def test_paged_decode_gqa_reference_format():
     # tests/benchmark.py:400-443: one-token pages, Q viewed [B, Hkv, group, D]
     def fn(Q, Kc, kt, Vc, vt):

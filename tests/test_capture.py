@@ -30,7 +30,8 @@ def capture_graph(fn, inputs, marks=()):
     def backend(gm, sample):
         def fw(g, _):
             try:
-                box["match"] = capture.match_attention(g)
+                box["matches"] = capture.match_attention(g)
+                box["match"] = box["matches"][0]
             except capture.NoMatch as e:
                 box["nomatch"] = e
             box["gm"] = g
@@ -50,11 +51,17 @@ def bf(*shape, seed=0):
     return torch.randn(*shape, generator=torch.Generator().manual_seed(seed)).to(torch.bfloat16)
 
 
-def _flat_args(m, tensors):
-    """The flat placeholder list of a call: ints for SymInt placeholders, tensors otherwise."""
+def _flat_args(box, tensors):
+    """The flat placeholder list of a call: ints for SymInt placeholders, tensors (in
+    order of first use) otherwise."""
     it = iter(tensors)
     return [next(it) if isinstance(p.meta["val"], torch.Tensor) else int(p.meta["val"].node.hint)
-            for p in m.placeholders]
+            for p in box["gm"].graph.nodes if p.op == "placeholder"]
+
+
+def _vals(box, m, tensors):
+    """Run-time values of the fused call's inputs for a call with these tensors."""
+    return m.input_values(box["gm"], _flat_args(box, tensors))
 
 
 def test_capture_causal_static_head_dim():
@@ -81,13 +88,7 @@ def test_capture_gqa_softcap_sliding_and_plan_values():
     box = capture_graph(fn, (q, k, v))
     m = box["match"]
     assert m.mask == "sliding" and m.has_tanh
-    args = [None] * len(m.placeholders)
-    # rebuild the flat argument list: ints for SymInt placeholders, tensors otherwise
-    tensors = iter((q, k, v))
-    for i, p in enumerate(m.placeholders):
-        val = p.meta["val"]
-        args[i] = next(tensors) if isinstance(val, torch.Tensor) else int(val.node.hint)
-    plan = m.plan_for(args)
+    plan = m.plan_for(_vals(box, m, (q, k, v)))
     assert plan.mask == "sliding" and plan.window == 256
     assert plan.softcap == pytest.approx(30.0) and plan.scale == pytest.approx(64 ** -0.5, rel=1e-6)
 
@@ -101,16 +102,17 @@ def test_capture_modified_attention_biases():
 
     q, k, v, qb = (bf(2, 4, 48, 64, seed=s) for s in range(4))
     sb, ob = bf(2, 4, 48, 48, seed=5), bf(2, 4, 48, 64, seed=6)
-    m = capture_graph(fn, (q, qb, k, sb, v, ob))["match"]
-    assert m.mask == "causal" and m.q.node is not None          # Q is computed (Q + q_bias)
-    assert m.bias is not None and m.bias.dims == (0, 1, 2, 3) and m.bias.node is None
+    box = capture_graph(fn, (q, qb, k, sb, v, ob))
+    m = box["match"]
+    assert m.mask == "causal" and m.inputs[m.q.index].op == "call_function"   # Q is the node Q + q_bias
+    assert m.bias is not None and m.bias.dims == (0, 1, 2, 3) and m.inputs[m.bias.index].op == "placeholder"
     assert m.out_bias is not None and m.out_bias.dims == (0, 1, 2, 3)
-    args = _flat_args(m, (q, qb, k, sb, v, ob))
-    plan = m.plan_for(args)
+    vals = _vals(box, m, (q, qb, k, sb, v, ob))
+    plan = m.plan_for(vals)
     assert plan.scale == pytest.approx(3.5 * 64 ** -0.5, rel=1e-6)
     # views handed to the kernels: the inputs themselves, Q replaced by the eager sum
-    assert torch.equal(m._operand(m.q, args)[0], q + qb)
-    assert m._bias_view(m.bias, args, (2, 4, 48, 48)).data_ptr() == sb.data_ptr()
+    assert torch.equal(m._operand(m.q, vals)[0], q + qb)
+    assert m._bias_view(m.bias, vals, (2, 4, 48, 48)).data_ptr() == sb.data_ptr()
 
 
 def test_capture_broadcast_and_transposed_bias():
@@ -120,9 +122,10 @@ def test_capture_broadcast_and_transposed_bias():
 
     q, k, v = (bf(3, 4, 40, 64, seed=s) for s in range(3))
     bias = bf(4, 1, 40, 40, seed=4)
-    m = capture_graph(fn, (q, k, bias, v))["match"]
+    box = capture_graph(fn, (q, k, bias, v))
+    m = box["match"]
     assert m.bias.dims == (None, 0, 2, 3)                # batch broadcast, heads walk source dim 0
-    view = m._bias_view(m.bias, _flat_args(m, (q, k, bias, v)), (3, 4, 40, 40))
+    view = m._bias_view(m.bias, _vals(box, m, (q, k, bias, v)), (3, 4, 40, 40))
     assert torch.equal(view, bias.transpose(0, 1).expand(3, 4, 40, 40))
 
 
@@ -176,7 +179,7 @@ def test_capture_paged_page16_reshape():
     assert box["match"].k.paged and box["match"].v.paged
 
 
-@pytest.mark.parametrize("which", ["gated_probs", "add", "softmax_matmul", "two_outputs"])
+@pytest.mark.parametrize("which", ["gated_probs", "add", "softmax_matmul"])
 def test_unrecognised_graphs_do_not_match(which):
     if which == "gated_probs":
         def fn(q, k, v, b):
@@ -187,18 +190,76 @@ def test_unrecognised_graphs_do_not_match(which):
         def fn(a, b):
             return a + b
         ins = (bf(4, 8), bf(4, 8, seed=1))
-    elif which == "softmax_matmul":
+    else:
         def fn(x, y):
             return torch.softmax(x, dim=-1) @ y
         ins = (bf(2, 2, 16, 8), bf(2, 2, 8, 16, seed=1))
-    else:
-        def fn(q, k, v):
-            s = q @ k.transpose(-2, -1)
-            p = torch.softmax(s, dim=-1)
-            return p @ v, p
-        ins = (bf(1, 2, 32, 64), bf(1, 2, 32, 64, seed=1), bf(1, 2, 32, 64, seed=2))
     box = capture_graph(fn, ins)
     assert "match" not in box and "nomatch" in box
+
+
+def _oracle_run(self, vals):
+    """Stand-in for AttentionMatch.run on the CPU: same operand plumbing, oracle arithmetic."""
+    q, _ = self._operand(self.q, vals)
+    k, kt = self._operand(self.k, vals)
+    v, vt = self._operand(self.v, vals)
+    B, Hq, Sq, Sk, D = self._shapes(vals)
+    plan = self.plan_for(vals)
+    out = O.attention_reference(q, k, v, mask=plan.mask, window=plan.window, scale=plan.scale, softcap=plan.softcap,
+                                k_table=kt, v_table=vt,
+                                score_bias=self._bias_view(self.bias, vals, (B, Hq, Sq, Sk)),
+                                out_bias=self._bias_view(self.out_bias, vals, (B, Hq, Sq, D))).to(q.dtype)
+    return out.reshape(self.out_shape(vals))
+
+
+@pytest.mark.parametrize("which", ["two_outputs", "prefix", "inside_block", "modified"])
+def test_rewritten_graphs_compute_the_same(which, monkeypatch):
+    """Sub-graph fusion: the attention(s) inside a larger graph are replaced by fused
+    calls and the rest keeps running.  Here the fused call is the oracle (no GPU), so
+    the test pins the rewrite and the operand plumbing (reference graphs:
+    tests/test_attention.py:72-92, 339-362)."""
+    monkeypatch.setattr(capture.AttentionMatch, "run", _oracle_run)
+    f32 = lambda *shape, seed=0: torch.randn(*shape, generator=torch.Generator().manual_seed(seed))
+    if which == "two_outputs":
+        def fn(q, k, v):
+            p = torch.softmax(q @ k.transpose(-2, -1), dim=-1)
+            return p @ v, p
+        ins, n_attn = (f32(1, 2, 32, 64), f32(1, 2, 32, 64, seed=1), f32(1, 2, 32, 64, seed=2)), 1
+    elif which == "prefix":
+        def fn(Q, Kp, Vp, Ks, Vs):
+            QKp = Q @ Kp.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+            QKs = Q @ Ks.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+            return torch.softmax(QKp, dim=-1) @ Vp + torch.softmax(torch.ops.loopfuse.causal_mask(QKs), dim=-1) @ Vs
+        ins = (f32(3, 2, 24, 64), f32(3, 2, 40, 64, seed=1), f32(3, 2, 40, 64, seed=2),
+               f32(3, 2, 24, 64, seed=3), f32(3, 2, 24, 64, seed=4))
+        n_attn = 2
+    elif which == "inside_block":
+        def fn(x, wq, wk, wv, wo):
+            B, S, E = x.shape
+            H = 4
+            q = (x @ wq).view(B, S, H, E // H).transpose(1, 2)
+            k = (x @ wk).view(B, S, H, E // H).transpose(1, 2)
+            v = (x @ wv).view(B, S, H, E // H).transpose(1, 2)
+            a = torch.softmax(torch.ops.loopfuse.causal_mask(q @ k.transpose(-2, -1) * 0.125), dim=-1) @ v
+            return a.transpose(1, 2).reshape(B, S, E) @ wo + x
+        ins = (f32(2, 24, 256),) + tuple(f32(256, 256, seed=s) * 0.06 for s in (1, 2, 3, 4))
+        n_attn = 1
+    else:
+        def fn(Q, qb, K, sb, V, ob):
+            QK = (Q + qb) @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+            return torch.softmax(torch.ops.loopfuse.causal_mask(QK * 3.5 + sb), dim=-1) @ V + ob
+        ins = (f32(2, 3, 24, 64), f32(2, 3, 24, 64, seed=1), f32(2, 3, 24, 64, seed=2), f32(2, 3, 24, 24, seed=3),
+               f32(2, 3, 24, 64, seed=4), f32(2, 3, 24, 64, seed=5))
+        n_attn = 1
+    torch._dynamo.reset()
+    before = dict(interface.stats)
+    n_before = len(interface._MATCHES)
+    got = torch.compile(fn, backend=loopfuse_amd.loopfuse_backend, dynamic=True)(*ins)
+    assert interface.stats["fused"] == before["fused"] + 1
+    assert len(interface._MATCHES) == n_before + n_attn
+    want = fn(*ins)
+    for g, w in zip(got if isinstance(got, tuple) else (got,), want if isinstance(want, tuple) else (want,)):
+        torch.testing.assert_close(g, w, rtol=2e-4, atol=2e-4)
 
 
 def test_backend_on_cpu_tensors_runs_graph_unfused():
