@@ -377,3 +377,69 @@ def test_c1_on_gpu_vs_cpu_eager():
     want_r = O.attention_reference(q, k, v, mask="causal")
     assert (got.float().cpu() - want_r).abs().max().item() <= 2e-2
     assert (got.float().cpu() - want).abs().max().item() <= 6e-2
+
+
+# ---------------------------------------------------------------- seeded sweep
+def _sweep_case(i):
+    """Case i of a seeded sweep over shapes, masks, head groupings, paging and biases."""
+    g = torch.Generator().manual_seed(1000 + i)
+    ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    pick = lambda xs: xs[ri(0, len(xs) - 1)]
+    dtype = pick([torch.bfloat16, torch.float16])
+    D = pick([64, 128])
+    B = ri(1, 3)
+    Hkv = pick([1, 2, 3, 8])
+    group = pick([1, 1, 2, 4])
+    kind = pick(["prefill", "prefill", "decode", "rect"])
+    if kind == "prefill":
+        Sq = Sk = ri(1, 700)
+        mask = pick([None, "causal", "causal", "sliding"])
+    elif kind == "rect":
+        Sq, Sk = ri(1, 300), ri(1, 900)
+        mask = pick([None, "causal", "sliding"])
+    else:
+        Sq, Sk = 1, ri(16, 3000)
+        mask = None
+    window = ri(1, 400) if mask == "sliding" else 0
+    softcap = pick([None, None, 15.0, 50.0])
+    paged = pick([0, 0, 1, 3]) if kind != "rect" else 0
+    page = pick([1, 16, 32]) if paged else 1
+    bias = pick([0, 0, 0, 1, 2, 3]) if kind != "decode" else 0
+    return dict(dtype=dtype, D=D, B=B, Hkv=Hkv, group=group, Sq=Sq, Sk=Sk, mask=mask, window=window,
+                softcap=softcap, paged=paged, page=page, bias=bias, seed=2000 + i)
+
+
+@pytest.mark.parametrize("i", range(40))
+def test_seeded_sweep(i):
+    c = _sweep_case(i)
+    dt, D, B, Hkv, Sq, Sk = c["dtype"], c["D"], c["B"], c["Hkv"], c["Sq"], c["Sk"]
+    Hq = Hkv * c["group"]
+    if c["mask"] is not None and Sq > Sk:
+        Sq = Sk             # keep every query row with at least one visible key
+    q = rand((B, Hq, Sq, D), dt, c["seed"])
+    kt = vt = None
+    if c["paged"]:
+        P = c["page"]
+        Skp = (Sk + P - 1) // P * P
+        Sk = Skp
+        if c["mask"] is not None:
+            Sq = min(Sq, Sk)
+            q = q[:, :, :Sq].contiguous()
+        n = B * Skp // P * 2
+        pool_shape = (n, Hkv, D) if P == 1 else (n, P, Hkv, D)
+        gen = torch.Generator().manual_seed(c["seed"] + 7)
+        k = rand(pool_shape, dt, c["seed"] + 1)
+        kt = torch.randint(0, n, (B, Skp // P), generator=gen, dtype=torch.int32 if c["seed"] % 2 else torch.int64)
+        if c["paged"] & 2:
+            v = rand(pool_shape, dt, c["seed"] + 2)
+            vt = torch.randint(0, n, (B, Skp // P), generator=gen, dtype=kt.dtype)
+        else:
+            v = rand((B, Hkv, Sk, D), dt, c["seed"] + 2)
+    else:
+        k = rand((B, Hkv, Sk, D), dt, c["seed"] + 1)
+        v = rand((B, Hkv, Sk, D), dt, c["seed"] + 2)
+    sb = rand((B, Hq, Sq, Sk), dt, c["seed"] + 3) if c["bias"] & 1 else None
+    ob = rand((B, Hq, Sq, D), dt, c["seed"] + 4) if c["bias"] & 2 else None
+    print("sweep case", i, {**c, "Sq": Sq, "Sk": Sk}, flush=True)
+    check(q, k, v, mask=c["mask"], window=c["window"], softcap=c["softcap"], k_table=kt, v_table=vt,
+          score_bias=sb, out_bias=ob)
