@@ -253,11 +253,96 @@ def prefill_variant(Sq: int, v_tr: bool = True) -> str:
     return "prefill_swp"
 
 
+# ---------------------------------------------------------------------------
+# launch-heuristic tuning (the reference autotunes tile sizes with triton.autotune,
+# loopfuse/codegen.py:355-404; the HIP kernels have fixed tiles, what varies here is
+# which kernel variant and which work split serve a shape)
+# ---------------------------------------------------------------------------
+_tuned: dict = {}
+_TUNE_FILE = os.path.join(runtime.CACHE_DIR, "autotune.json")
+
+
+def _tune_key(q, k, plan: AttnPlan, k_table, bias_bits: int) -> str:
+    B, Hq, Sq, D = q.shape
+    if plan.k_paged:
+        Hkv = k.shape[-2]
+        Sk = k_table.shape[1] * (k.shape[1] if k.dim() == 4 else 1)
+        ps = k.shape[1] if k.dim() == 4 else 1
+    else:
+        Hkv, Sk, ps = k.shape[1], k.shape[2], 0
+    bucket = lambda n: 1 << max(0, (int(n) - 1)).bit_length()       # next power of two
+    return (f"{q.dtype}|D{D}|m{plan.mask}|c{int(plan.softcap is not None)}|p{int(plan.k_paged)}{int(plan.v_paged)}x{ps}"
+            f"|B{bucket(B * Hkv)}|g{Hq // Hkv}|q{bucket(Sq)}|k{bucket(Sk)}|b{bias_bits}")
+
+
+def _load_tuned() -> None:
+    if not _tuned and os.path.exists(_TUNE_FILE):
+        try:
+            import json
+            with open(_TUNE_FILE) as fh:
+                _tuned.update(json.load(fh))
+        except (OSError, ValueError):
+            pass
+
+
+def tuned_attention(q, k, v, plan: AttnPlan, k_table=None, v_table=None, **kw):
+    """``attention`` with the launch heuristics chosen by measurement: on the first call
+    of a shape class each candidate is timed on the call's own tensors (HIP events, a few
+    launches), the winner is remembered in the process and in ``autotune.json`` beside
+    the code-object cache.  Used by the backend under ``mode="max-autotune"``."""
+    if kw.get("score_bias") is not None or kw.get("out_bias") is not None or kw.get("record_visits") \
+            or kw.get("force_family") or kw.get("num_splits") or kw.get("choice"):
+        return attention(q, k, v, plan, k_table, v_table, **kw)
+    _load_tuned()
+    key = _tune_key(q, k, plan, k_table, 0)
+    if key not in _tuned:
+        B, Hq, Sq, D = q.shape
+        Hkv = k.shape[-2] if plan.k_paged else k.shape[1]
+        group = Hq // max(Hkv, 1)
+        decode = plan.mask is None and ((Sq == 1 and group <= 64) or (group == 1 and Sq <= 16))
+        if decode:
+            cands = [{"head_per_wave": hw, "splits": sp} for hw in ((False, True) if plan.k_paged and plan.v_paged else (False,))
+                     for sp in (None, 1, 2, 4, 8)]
+        elif not (plan.k_paged or plan.v_paged):
+            cands = [{"prefill": "swp"}, {"prefill": "w32"}]
+        else:
+            cands = [{}]
+        best, best_t = cands[0], float("inf")
+        if len(cands) > 1:
+            out = kw.get("out")
+            for c in cands:
+                c = {a: b for a, b in c.items() if b is not None}
+                try:
+                    for _ in range(2):
+                        out = attention(q, k, v, plan, k_table, v_table, **{**kw, "out": out, "choice": c})
+                    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    a.record()
+                    for _ in range(5):
+                        attention(q, k, v, plan, k_table, v_table, **{**kw, "out": out, "choice": c})
+                    b.record()
+                    b.synchronize()
+                    t = a.elapsed_time(b)
+                except UnsupportedPlan:
+                    continue
+                if t < best_t:
+                    best, best_t = c, t
+        _tuned[key] = best
+        try:
+            import json
+            os.makedirs(os.path.dirname(_TUNE_FILE), exist_ok=True)
+            with open(_TUNE_FILE, "w") as fh:
+                json.dump(_tuned, fh, indent=0, sort_keys=True)
+        except OSError:
+            pass
+    return attention(q, k, v, plan, k_table, v_table, **{**kw, "choice": _tuned[key]})
+
+
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
               k_table: Optional[torch.Tensor] = None, v_table: Optional[torch.Tensor] = None,
               *, out: Optional[torch.Tensor] = None, record_visits: bool = False,
               force_family: str | None = None, num_splits: int | None = None, v_tr: bool = True,
-              score_bias: Optional[torch.Tensor] = None, out_bias: Optional[torch.Tensor] = None):
+              score_bias: Optional[torch.Tensor] = None, out_bias: Optional[torch.Tensor] = None,
+              choice: Optional[dict] = None):
     """Run fused attention on the GPU.
 
     q : [B, Hq, Sq, D];  k, v : [B, Hkv, Sk, D], or page pools [N, P, Hkv, D]
@@ -266,8 +351,11 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     scaled / capped scores before the mask, ``out_bias`` (broadcastable to
     [B, Hq, Sq, D]) to the result -- the reference's "modified attention" graph
     (tests/test_accuracy.py:172-196).  Both are served by ``lf_attn_prefill`` only.
+    ``choice`` overrides the launch heuristics (what ``tuned_attention`` searches over):
+    ``{"prefill": "swp" | "w32"}``, ``{"head_per_wave": bool, "splits": n}``.
     Returns O [B, Hq, Sq, D] (and the visited-tile record if asked).
     """
+    choice = choice or {}
     dtype = q.dtype
     if dtype not in _DTYPE_CODE:
         raise UnsupportedPlan(f"dtype {dtype} not supported by the MFMA kernels (bf16/fp16 only)")
@@ -381,7 +469,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     keep = (q, k, v, out, kt, vt, score_bias, out_bias)  # noqa: F841  (tensors stay alive until the launch is queued)
 
     if family == "prefill" and not bias_bits:
-        family = prefill_variant(Sq, v_tr)
+        family = {"swp": "prefill_swp", "w32": "prefill"}.get(choice.get("prefill"), None) or prefill_variant(Sq, v_tr)
     if family == "prefill_swp":
         # direct-to-LDS staging: dense K/V only, 32-bit byte offsets per (batch, kv head)
         # span; the kernel also addresses up to three tiles past Sk (those reads are
@@ -452,9 +540,12 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     # Token-major page pools ([pages, page, Hkv, D]: the heads of a token side by side)
     # are read whole-page-wise when the 8 waves of a workgroup take 8 consecutive heads.
     headwave = _decode_headwave(paged, page_size, Hkv, D, P)
+    if "head_per_wave" in choice:
+        headwave = bool(choice["head_per_wave"]) and paged == 3 and Hkv % 8 == 0
     if headwave:
         waves = 8
         units = B * ((Hkv + waves - 1) // waves) * chunks
+    num_splits = num_splits or choice.get("splits")
     nsplit = num_splits if num_splits else decode_split(units, Sk, per_cu=1 if headwave else 2)
     split_len = ((Sk + nsplit - 1) // nsplit + 31) // 32 * 32     # whole pairs of 16-token steps
     nsplit = (Sk + split_len - 1) // split_len

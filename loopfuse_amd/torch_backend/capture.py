@@ -170,6 +170,7 @@ class AttentionMatch:
     out_rank: int
     bias: Optional[BiasOperand] = None
     out_bias: Optional[BiasOperand] = None
+    tune: bool = False             # mode="max-autotune": measure the launch heuristics per shape class
 
     def describe(self) -> str:
         nm = lambda i: self.inputs[i].name
@@ -256,7 +257,8 @@ class AttentionMatch:
         k, kt = self._operand(self.k, vals)
         v, vt = self._operand(self.v, vals)
         B, Hq, Sq, Sk, D = self._shapes(vals)
-        out = lowering.attention(q, k, v, self.plan_for(vals), kt, vt,
+        run = lowering.tuned_attention if self.tune else lowering.attention
+        out = run(q, k, v, self.plan_for(vals), kt, vt,
                                  score_bias=self._bias_view(self.bias, vals, (B, Hq, Sq, Sk)),
                                  out_bias=self._bias_view(self.out_bias, vals, (B, Hq, Sq, D)))
         if self.out_rank == 3:

@@ -61,8 +61,9 @@ def get_input_names(gm: torch.fx.GraphModule) -> list[str]:
 def loopfuse_backend(gm: torch.fx.GraphModule, sample_inputs, mode="max-autotune", **kwargs):
     """``torch.compile`` backend entry point (reference ``interface.py:77-86``).
 
-    ``mode`` is accepted for compatibility: the reference uses it to pick the
-    Triton autotune space; the HIP kernels have fixed tile shapes.
+    ``mode="max-autotune"`` (the default, as in the reference) makes the first call of
+    each shape class time the candidate kernel variants / work splits and keep the
+    fastest (``lowering.tuned_attention``); ``mode=None`` uses the fixed heuristics.
     """
     if mode:
         kwargs["mode"] = mode
@@ -133,6 +134,10 @@ def loopfuse_compiler(gm: torch.fx.GraphModule, sample_inputs, input_names: list
         return eager_fn
 
     stats["matched_graphs"] += 1
+    for m in matches:
+        # the reference's "max-autotune" searches Triton tile sizes (codegen.py:355-404);
+        # here it measures which kernel variant / work split serves each shape class
+        m.tune = (mode == "max-autotune") and os.environ.get("LOOPFUSE_AUTOTUNE", "1") == "1"
     fused_gm = rewrite_graph(gm, matches)
     if DEBUG:
         print("---- loopfuse_amd: matched ----")

@@ -443,3 +443,24 @@ def test_seeded_sweep(i):
     print("sweep case", i, {**c, "Sq": Sq, "Sk": Sk}, flush=True)
     check(q, k, v, mask=c["mask"], window=c["window"], softcap=c["softcap"], k_table=kt, v_table=vt,
           score_bias=sb, out_bias=ob)
+
+
+# ---------------------------------------------------------------- measured launch heuristics
+@pytest.mark.parametrize("name", ["c2", "c5"])
+def test_tuned_attention_matches_and_remembers(name, monkeypatch, tmp_path):
+    monkeypatch.setattr(lowering, "_TUNE_FILE", str(tmp_path / "autotune.json"))
+    monkeypatch.setattr(lowering, "_tuned", {})
+    w = workloads.make(name, seed=5, B=2, S=512)
+    plan = lowering.AttnPlan(mask=w.mask, window=w.window, scale=w.scale, softcap=w.softcap,
+                             k_paged=w.k_table is not None, v_paged=w.v_table is not None)
+    mv = lambda t: None if t is None else t.to(dev())
+    args = (mv(w.q), mv(w.k), mv(w.v), plan, mv(w.k_table), mv(w.v_table))
+    got = lowering.tuned_attention(*args)
+    assert len(lowering._tuned) == 1
+    key, choice = next(iter(lowering._tuned.items()))
+    again = lowering.tuned_attention(*args)            # no second search
+    assert len(lowering._tuned) == 1 and torch.equal(got, again)
+    import json
+    assert json.load(open(lowering._TUNE_FILE)) == {key: choice}
+    want = O.attention_reference(w.q, w.k, w.v, mask=w.mask, k_table=w.k_table, v_table=w.v_table)
+    assert (got.float().cpu() - want).abs().max().item() <= TOL[torch.bfloat16]

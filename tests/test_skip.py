@@ -35,3 +35,16 @@ def test_baseline_counts():
     assert sum(e - b for b, e in skip.visited_tiles("causal", 2048, 2048)) == 272
     # executed vs algorithmic flops for C2 = 272/256
     assert skip.executed_flops("causal", 8, 32, 2048, 2048, 128) * 256 == 2 * 8 * 32 * 2048 * 2048 * 128 * 272
+
+
+def test_tuning_key_buckets_sizes():
+    import torch
+    from loopfuse_amd import lowering
+
+    plan = lowering.AttnPlan(mask="causal", scale=0.1)
+    mk = lambda B, H, S: torch.empty(B, H, S, 64, dtype=torch.bfloat16, device="meta")
+    a = lowering._tune_key(mk(2, 4, 1000), mk(2, 4, 1000), plan, None, 0)
+    b = lowering._tune_key(mk(2, 4, 1024), mk(2, 4, 1024), plan, None, 0)
+    c = lowering._tune_key(mk(2, 4, 1025), mk(2, 4, 1025), plan, None, 0)
+    assert a == b != c
+    assert lowering._tune_key(mk(2, 8, 1000), mk(2, 4, 1000), plan, None, 0) != a       # GQA group differs
