@@ -198,6 +198,9 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
 #pragma unroll
     for (int i = 0; i < 16; ++i) o[db][i] = 0.0f;
   float mc_ref = LF_NEG_INF;  // exponent offset of this query in log2 units (a lagging running max)
+#if LF_DENOM
+  float mc_true = LF_NEG_INF; // the running max itself (the extra denominator term is relative to it)
+#endif
   float l_run = 0.0f;         // this lane's share of the running sum
 
   // ---- staging: thread handles chunk (srow + kRowsPerPass*ps, sch) of every pass.
@@ -465,6 +468,9 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
       mx = fmaxf(mx, lf_swap32(mx));
 #endif
       const float mxc = mx * cexp;
+#if LF_DENOM
+      mc_true = fmaxf(mc_true, mxc);
+#endif
       if (__builtin_amdgcn_ballot_w64(mxc > mc_ref + (float)LF_LAZY_LOG2) != 0ull) {
         const float mc_new = fmaxf(mc_ref, mxc);          // finite wherever mxc is
         // 0 on a query's first update (its O and l are still 0); 1 for a query
@@ -592,7 +598,11 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
   // ---- epilogue: O[q][d] = O^T[d][q] / l.  Element i of block db is
   // d = 32*db + 8*(i/4) + 4*g + i%4.
   if (my_q < p.Sq) {
-    const float l_tot = l_run + lf_swap32(l_run);
+    float l_tot = l_run + lf_swap32(l_run);
+#if LF_DENOM
+    // sum and extra term in the same units: l is relative to the lagging offset
+    l_tot += p.denom_add * lf_exp2(mc_true - mc_ref);
+#endif
     const float inv = 1.0f / l_tot;
     lf_elem* orow = p.o + (long long)b * p.o_sb + (long long)h * p.o_sh + (long long)my_q * p.o_ss;
 #pragma unroll

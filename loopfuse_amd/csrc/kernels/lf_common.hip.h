@@ -33,6 +33,10 @@
 #define LF_BIAS 0     /* bit 0: score bias tensor, bit 1: output bias tensor, bit 2: their rows are not
                          8-byte aligned (element loads); lf_attn_prefill only */
 #endif
+#ifndef LF_DENOM
+#define LF_DENOM 0    /* 1: softmax denominator is (sum + denom_add) in units where the row maximum
+                         contributes 1 (reference tests/test_attention.py:95-125); lf_attn_prefill only */
+#endif
 #ifndef LF_SOFTCAP
 #define LF_SOFTCAP 0
 #endif
@@ -101,6 +105,7 @@ struct LfAttnParams {
   int split_len;             // decode: tokens per split (multiple of 16)
   float scale;               // multiplies QK^T (D^-0.5 in the reference graphs)
   float softcap;             // cap of cap*tanh(s/cap) (LF_SOFTCAP)
+  float denom_add;           // LF_DENOM: probabilities are e^(x - max) / (sum e^(x - max) + denom_add)
 };
 
 __device__ __forceinline__ lf_f32x16 lf_mfma32(lf_elem8 a, lf_elem8 b, lf_f32x16 c) {

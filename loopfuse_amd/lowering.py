@@ -47,7 +47,7 @@ class AttnParams(ctypes.Structure):
             "bias_sb", "bias_sh", "bias_sq", "ob_sb", "ob_sh", "ob_sq")]
         + [(n, ctypes.c_int) for n in (
             "B", "Hq", "Hkv", "Sq", "Sk", "window", "kt_stride", "vt_stride", "nsplit", "rows", "split_len")]
-        + [("scale", ctypes.c_float), ("softcap", ctypes.c_float)]
+        + [("scale", ctypes.c_float), ("softcap", ctypes.c_float), ("denom_add", ctypes.c_float)]
     )
 
 
@@ -67,6 +67,7 @@ class KernelSpec:
     waves: int = 4         # decode: waves per workgroup
     v_tr: bool = True      # prefill: transposed LDS reads for V
     headwave: bool = False  # decode: one kv head per wave (8 waves) instead of 4 waves sharing a head
+    denom: bool = False    # prefill: softmax denominator sum + c (c a run-time parameter)
     bias: int = 0          # prefill: bit 0 additive score bias tensor, bit 1 additive output bias tensor, bit 2 unaligned rows
     extra: tuple = ()      # further -D options (tuning experiments)
 
@@ -83,7 +84,7 @@ class KernelSpec:
         if self.family == "decode":
             o += [f"-DLF_DW={self.waves}", f"-DLF_HEADWAVE={int(self.headwave)}"]
         elif self.family == "prefill":
-            o += [f"-DLF_V_TR={int(self.v_tr)}", f"-DLF_BIAS={self.bias}"]
+            o += [f"-DLF_V_TR={int(self.v_tr)}", f"-DLF_BIAS={self.bias}", f"-DLF_DENOM={int(self.denom)}"]
         return o + list(self.extra)
 
     def files(self) -> tuple[str, ...]:
@@ -96,7 +97,7 @@ class KernelSpec:
 
     def name(self) -> str:
         return (f"lf_{self.family}_t{self.dtype}_d{self.head_dim}_m{self.mask}_c{int(self.softcap)}"
-                f"_p{self.paged}x{self.page_size}i{int(self.table_i64)}_r{self.rows}w{self.waves}v{int(self.v_tr)}h{int(self.headwave)}b{self.bias}"
+                f"_p{self.paged}x{self.page_size}i{int(self.table_i64)}_r{self.rows}w{self.waves}v{int(self.v_tr)}h{int(self.headwave)}b{self.bias}n{int(self.denom)}"
                 + "".join("_" + e.replace("-D", "").replace("=", "") for e in self.extra))
 
     def source(self) -> str:
@@ -184,6 +185,7 @@ class AttnPlan:
     softcap: float | None = None
     k_paged: bool = False
     v_paged: bool = False
+    denom_add: float = 0.0             # probabilities are e^(x-max) / (sum e^(x-max) + denom_add)
 
 
 class UnsupportedPlan(ValueError):
@@ -291,7 +293,7 @@ def tuned_attention(q, k, v, plan: AttnPlan, k_table=None, v_table=None, **kw):
     launches), the winner is remembered in the process and in ``autotune.json`` beside
     the code-object cache.  Used by the backend under ``mode="max-autotune"``."""
     if kw.get("score_bias") is not None or kw.get("out_bias") is not None or kw.get("record_visits") \
-            or kw.get("force_family") or kw.get("num_splits") or kw.get("choice"):
+            or kw.get("force_family") or kw.get("num_splits") or kw.get("choice") or plan.denom_add != 0.0:
         return attention(q, k, v, plan, k_table, v_table, **kw)
     _load_tuned()
     key = _tune_key(q, k, plan, k_table, 0)
@@ -427,6 +429,9 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     P.window = int(plan.window)
     P.scale = float(plan.scale)
     P.softcap = float(plan.softcap) if plan.softcap else 0.0
+    P.denom_add = float(plan.denom_add)
+    if plan.denom_add < 0.0 or not math.isfinite(plan.denom_add):
+        raise UnsupportedPlan("the denominator offset must be finite and >= 0")
     P.nsplit, P.rows, P.split_len = 1, 1, 0
 
     # ---- additive biases: [B, Hq, Sq, X] views with broadcast (stride 0) batch/head/row dims
@@ -458,7 +463,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         P.obias = out_bias.data_ptr()
         P.ob_sb, P.ob_sh, P.ob_sq = out_bias.stride(0), out_bias.stride(1), out_bias.stride(2)
         bias_bits |= 2
-    if bias_bits & 3:
+    if bias_bits & 3 or plan.denom_add != 0.0:
         force_family = "prefill"
 
     # ---- family: decode when there is no mask and few query rows share a KV head
@@ -468,7 +473,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         family = "decode" if (mask == MASK_NONE and few and Sk >= 16) else "prefill"
     keep = (q, k, v, out, kt, vt, score_bias, out_bias)  # noqa: F841  (tensors stay alive until the launch is queued)
 
-    if family == "prefill" and not bias_bits:
+    if family == "prefill" and not bias_bits and plan.denom_add == 0.0:
         family = {"swp": "prefill_swp", "w32": "prefill"}.get(choice.get("prefill"), None) or prefill_variant(Sq, v_tr)
     if family == "prefill_swp":
         # direct-to-LDS staging: dense K/V only, 32-bit byte offsets per (batch, kv head)
@@ -491,7 +496,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         elif family == "prefill" and bias_bits and not paged:
             extra += ("-DLF_DMA=1",)     # frees the staging registers the bias values need
         spec = KernelSpec(family, _DTYPE_CODE[dtype], D, mask, plan.softcap is not None, paged,
-                          page_size, table_i64, v_tr=v_tr if family == "prefill" else True, bias=bias_bits, extra=extra)
+                          page_size, table_i64, v_tr=v_tr if family == "prefill" else True, bias=bias_bits,
+                          denom=plan.denom_add != 0.0, extra=extra)
         if os.environ.get("LOOPFUSE_TIMING"):       # profiling aid, see LF_TIMING in the kernel
             attention.timing = torch.zeros(16, dtype=torch.float32, device=q.device)
             P.part_acc = attention.timing.data_ptr()

@@ -89,6 +89,21 @@ class Stage:
     window: Any = 0                # int or fx.Node (SymInt)
     bias: Optional[tuple] = None       # (Ids, stage shape when added): additive score bias, before the mask
     out_bias: Optional[tuple] = None   # (Ids, stage shape when added): additive output bias
+    # explicit softmax written with loopfuse.scan_max (reference tests/test_attention.py:95-125):
+    uid: int = 0                       # set when scan_max is applied to this value
+    sm: str = ""                       # "" | "minus_run" (x - running max) | "exp_run" | "num" (b^(x - max))
+    base2: bool = False                # the exponentials are exp2
+    denom_add: tuple = ()              # probabilities = num / (sum num + these terms)
+
+
+@dataclasses.dataclass
+class Aux:
+    """By-products of an explicit softmax on the scores with id ``uid``."""
+
+    kind: str                          # "run" | "fin" (scan_max results) | "gap" (run - fin) | "expgap" | "den"
+    uid: int
+    c: tuple = ()                      # den: terms (numbers or Scalar nodes) added to the sum so far
+    base2: bool = False
 
 
 _VIEW_OPS = {
@@ -171,6 +186,8 @@ class AttentionMatch:
     bias: Optional[BiasOperand] = None
     out_bias: Optional[BiasOperand] = None
     tune: bool = False             # mode="max-autotune": measure the launch heuristics per shape class
+    denom_add: tuple = ()          # explicit softmax with denominator (sum + these terms): floats | ("arg", i)
+    base2: bool = False            # explicit softmax written with exp2: scores are in log2 units
 
     def describe(self) -> str:
         nm = lambda i: self.inputs[i].name
@@ -179,6 +196,7 @@ class AttentionMatch:
                 f"V={nm(self.v.index)}{'[paged by %s]' % nm(self.v.table_index) if self.v.paged else self.v.perm} "
                 f"mask={self.mask} window={self.window} tanh={self.has_tanh} "
                 f"factors={self.factors} post={self.post_factors}"
+                f"{' denom+%s' % (self.denom_add,) if self.denom_add else ''}{' exp2' if self.base2 else ''}"
                 f"{' +score_bias(%s)' % nm(self.bias.index) if self.bias else ''}"
                 f"{' +out_bias(%s)' % nm(self.out_bias.index) if self.out_bias else ''}")
 
@@ -205,8 +223,13 @@ class AttentionMatch:
         else:
             scale, softcap = pre, None
         window = self._number(self.window, vals) if self.mask == "sliding" else 0
+        if self.base2:              # 2^x = e^(x ln 2): the kernels take natural-exponent scores
+            if softcap is not None:
+                raise lowering.UnsupportedPlan("softcap inside an exp2-based explicit softmax")
+            scale *= math.log(2.0)
         return lowering.AttnPlan(mask=self.mask, window=int(window), scale=scale, softcap=softcap,
-                                 k_paged=self.k.paged, v_paged=self.v.paged)
+                                 k_paged=self.k.paged, v_paged=self.v.paged,
+                                 denom_add=sum(self._number(t, vals) for t in self.denom_add))
 
     def _operand(self, op: Operand, vals):
         t = vals[op.index]
@@ -435,6 +458,8 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
 
     def fresh_ids(node: torch.fx.Node, val) -> Any:
         """A tensor-valued node that simply runs: ids over its own (stand-in) shape."""
+        if val.dim() == 0:
+            return Scalar(node, 1.0)       # e.g. a Python float that dynamo passes as a 0-dim tensor
         shape = tuple(concrete(d) for d in val.shape)
         n = math.prod(shape)
         if n > (1 << 22):
@@ -466,6 +491,7 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
     matches: list = []
     reasons: list = []
     finalised: dict = {}
+    uid_box = [0]
 
     def finalise(node: torch.fx.Node) -> None:
         """``node`` holds a finished attention that something outside the pattern reads."""
@@ -506,6 +532,27 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
                 isinstance(x, (Scalar, int, float, bool, str, torch.dtype, type(None)))
                 for x in list(a) + list(kw.values())):
             return Scalar(node, 1.0)       # any arithmetic among shape-derived 0-dim values
+
+        # -- explicit softmax by-products (running / final max, their gap, the denominator)
+        if tgt is operator.getitem and isinstance(first, list) and isinstance(a[1], int):
+            return first[a[1]]
+        if isinstance(first, Aux):
+            x = first
+            if tgt is aten.sub.Tensor and x.kind == "run" and isinstance(a[1], Aux) and a[1].kind == "fin" \
+                    and a[1].uid == x.uid and kw.get("alpha", 1) == 1:
+                return Aux("gap", x.uid)
+            if tgt in (aten.exp2.default, aten.exp.default) and x.kind == "gap":
+                return Aux("expgap", x.uid, base2=tgt is aten.exp2.default)
+            if tgt is aten.add.Tensor and x.kind == "den" and kw.get("alpha", 1) == 1 and (
+                    (is_number(a[1]) and a[1] >= 0) or isinstance(a[1], Scalar)):
+                raw = node.args[1]
+                term = a[1].node if isinstance(a[1], Scalar) else (raw if isinstance(raw, torch.fx.Node) else float(a[1]))
+                return Aux("den", x.uid, c=x.c + (term,))
+            if tgt is aten.mul.Tensor and x.kind == "expgap" and isinstance(a[1], Stage):
+                a = (a[1], a[0])            # handled below with the stage first
+                first = a[0]
+            else:
+                raise _Skip(f"op on a softmax by-product: {tgt}")
 
         # -- tensor + scores / tensor + output with the tensor written first
         if tgt is aten.add.Tensor and isinstance(first, Ids) and len(a) > 1 and isinstance(a[1], Stage) \
@@ -555,6 +602,38 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
                 return dataclasses.replace(st, shape=new_shape)
             if tgt in _CAST_OPS:
                 return st
+            if st.kind == "scores":
+                # the explicit softmax: x - run_max, exp, * exp(run_max - max), / (sum + c)
+                if tgt is torch.ops.loopfuse.scan_max.default and st.sm == "" and st.uid == 0:
+                    uid_box[0] += 1
+                    st.uid = uid_box[0]
+                    return [Aux("run", st.uid), Aux("fin", st.uid)]
+                if tgt is aten.sub.Tensor and st.sm == "" and st.uid and isinstance(a[1], Aux) and a[1].kind == "run" \
+                        and a[1].uid == st.uid and kw.get("alpha", 1) == 1:
+                    return dataclasses.replace(st, sm="minus_run")
+                if tgt in (aten.exp2.default, aten.exp.default) and st.sm == "minus_run":
+                    return dataclasses.replace(st, sm="exp_run", base2=tgt is aten.exp2.default)
+                if tgt is aten.mul.Tensor and st.sm == "exp_run" and isinstance(a[1], Aux) and a[1].kind == "expgap" \
+                        and a[1].uid == st.uid and a[1].base2 == st.base2:
+                    return dataclasses.replace(st, sm="num")
+                if tgt is aten.sum.dim_IntList and st.sm == "num" and list(a[1]) in ([-1], [len(st.shape) - 1]) \
+                        and len(a) > 2 and a[2] is True:
+                    return Aux("den", st.uid)
+                if tgt is aten.div.Tensor and st.sm == "num" and isinstance(a[1], Aux) and a[1].kind == "den" \
+                        and a[1].uid == st.uid:
+                    return dataclasses.replace(st, kind="probs", sm="", denom_add=a[1].c)
+                if st.sm != "":
+                    raise _Skip(f"op inside an explicit softmax: {tgt}")
+                # a positive constant factor commutes with the mask (-inf stays -inf)
+                if tgt in (aten.mul.Tensor, aten.div.Tensor) and st.mask is not None and st.bias is None \
+                        and is_number(a[1]) and a[1] > 0 and not isinstance(node.args[1], torch.fx.Node) and st.uid == 0:
+                    f = float(a[1]) if tgt is aten.mul.Tensor else 1.0 / float(a[1])
+                    new = dataclasses.replace(st)
+                    if st.has_tanh:
+                        new.post_factors = st.post_factors + [f]
+                    else:
+                        new.factors = st.factors + [f]
+                    return new
             if st.kind == "scores" and tgt is aten.add.Tensor and isinstance(a[1], Ids) and st.mask is None \
                     and st.bias is None and kw.get("alpha", 1) == 1:
                 return dataclasses.replace(st, bias=(a[1], st.shape))
@@ -701,4 +780,4 @@ def _build_match(out_node: torch.fx.Node, st: Stage) -> AttentionMatch:
     window = scalar(st.window) if st.mask == "sliding" else 0
     return AttentionMatch(out_node, inputs, q_op, k_op, v_op, [scalar(f) for f in st.factors],
                           [scalar(f) for f in st.post_factors], st.has_tanh, st.mask, window, out_rank,
-                          bias_op, obias_op)
+                          bias_op, obias_op, denom_add=tuple(scalar(t) for t in st.denom_add), base2=st.base2)

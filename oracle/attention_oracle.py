@@ -63,11 +63,14 @@ def gather_paged(pool: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
 
 def attention_reference(q, k, v, *, mask: Optional[str] = None, window: int = 0,
                         scale: Optional[float] = None, softcap: Optional[float] = None,
-                        k_table=None, v_table=None, score_bias=None, out_bias=None) -> torch.Tensor:
+                        k_table=None, v_table=None, score_bias=None, out_bias=None,
+                        denom_add: float = 0.0) -> torch.Tensor:
     """fp32 eager attention.  q [B,Hq,Sq,D]; k, v [B,Hkv,Sk,D] or page pools + tables.
     ``score_bias`` (broadcastable to [B,Hq,Sq,Sk]) is added to the scaled / capped scores
     before the mask and ``out_bias`` ([B,Hq,Sq,D]) to the result, as in the reference's
-    modified-attention graph (tests/test_accuracy.py:172-196)."""
+    modified-attention graph (tests/test_accuracy.py:172-196).  ``denom_add`` = c gives the
+    probabilities e^(s - m) / (sum_j e^(s_j - m) + c) with m the row maximum, the explicit
+    softmax of the reference's tests/test_attention.py:95-125 (c = 1 there)."""
     q = q.float()
     k = gather_paged(k.float(), k_table) if k_table is not None else k.float()
     v = gather_paged(v.float(), v_table) if v_table is not None else v.float()
@@ -85,7 +88,11 @@ def attention_reference(q, k, v, *, mask: Optional[str] = None, window: int = 0,
         s = s + score_bias.float()
     keep = dense_mask(mask, Sq, Sk, window).to(s.device)
     s = s.masked_fill(~keep, float("-inf"))
-    p = torch.softmax(s, dim=-1)
+    if denom_add:
+        e = torch.exp(s - s.max(dim=-1, keepdim=True).values)
+        p = e / (e.sum(dim=-1, keepdim=True) + denom_add)
+    else:
+        p = torch.softmax(s, dim=-1)
     out = torch.matmul(p, v)
     if out_bias is not None:
         out = out + out_bias.float()

@@ -154,6 +154,28 @@ def test_broadcast_score_bias_gqa():
     assert (got - want).abs().max() <= TOL
 
 
+def test_explicit_softmax_shifted_denominator():
+    # reference tests/test_attention.py:95-125: online-softmax hint with scan_max, out = e / (S + 1)
+    import math
+
+    def _softmax(X):
+        Xf = X.to(torch.float32)
+        Xf_scaled = Xf * 1 / math.log(2)
+        X_mik, X_mi = torch.ops.loopfuse.scan_max(Xf_scaled)
+        expX = torch.exp2(Xf_scaled - X_mik) * torch.exp2(X_mik - X_mi)
+        return expX / (torch.sum(expX, dim=-1, keepdim=True) + 1)
+
+    def fn(Q, K, V):
+        QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        return _softmax(torch.ops.loopfuse.causal_mask(QK)).to(Q.dtype) @ V
+
+    Q, K, V = (rand((2, 8, 700, 128), seed=s) for s in (1, 2, 3))
+    torch._dynamo.mark_static(Q, 3)
+    torch._dynamo.mark_dynamic(Q, 2)
+    got = run_fused(fn, (Q, K, V))
+    assert (got - O.attention_reference(Q, K, V, mask="causal", denom_add=1.0)).abs().max() <= TOL
+
+
 def test_prefix_attention_two_fused_calls():
     # reference tests/test_attention.py:339-362: a shared prefix (batch 1, broadcast) attended without
     # a mask plus the causal suffix, each with its own softmax, summed

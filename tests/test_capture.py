@@ -1,5 +1,7 @@
 """Front end on the CPU: custom-op semantics, graph capture -> plan, CODEGEN_ONLY-style
 compilation of the matched kernels, and eager fallback for everything else."""
+import math
+
 import pytest
 import torch
 
@@ -206,13 +208,37 @@ def _oracle_run(self, vals):
     B, Hq, Sq, Sk, D = self._shapes(vals)
     plan = self.plan_for(vals)
     out = O.attention_reference(q, k, v, mask=plan.mask, window=plan.window, scale=plan.scale, softcap=plan.softcap,
-                                k_table=kt, v_table=vt,
+                                k_table=kt, v_table=vt, denom_add=plan.denom_add,
                                 score_bias=self._bias_view(self.bias, vals, (B, Hq, Sq, Sk)),
                                 out_bias=self._bias_view(self.out_bias, vals, (B, Hq, Sq, D))).to(q.dtype)
     return out.reshape(self.out_shape(vals))
 
 
-@pytest.mark.parametrize("which", ["two_outputs", "prefix", "inside_block", "modified"])
+def _explicit_softmax(X, base2=True, c=1.0):
+    """The reference's hand-written online-softmax hint (tests/test_attention.py:95-107)."""
+    Xf = X.to(torch.float32)
+    if base2:
+        Xf = Xf * 1 / math.log(2)
+    run, fin = torch.ops.loopfuse.scan_max(Xf)
+    ex = torch.exp2 if base2 else torch.exp
+    e = ex(Xf - run) * ex(run - fin)
+    return e / (torch.sum(e, dim=-1, keepdim=True) + c)
+
+
+def test_capture_explicit_softmax_with_shifted_denominator():
+    def fn(Q, K, V):
+        QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        return _explicit_softmax(torch.ops.loopfuse.causal_mask(QK)).to(Q.dtype) @ V
+
+    q, k, v = (bf(2, 4, 48, 64, seed=s) for s in range(3))
+    box = capture_graph(fn, (q, k, v), [(q, 3, "static"), (q, 2, "dynamic")])
+    m = box["match"]
+    assert m.mask == "causal" and m.denom_add == (1.0,) and m.base2
+    plan = m.plan_for(_vals(box, m, (q, k, v)))
+    assert plan.denom_add == 1.0 and plan.scale == pytest.approx(64 ** -0.5, rel=1e-6)   # 1/ln2 and ln2 cancel
+
+
+@pytest.mark.parametrize("which", ["two_outputs", "prefix", "inside_block", "modified", "softmax1", "softmax_e"])
 def test_rewritten_graphs_compute_the_same(which, monkeypatch):
     """Sub-graph fusion: the attention(s) inside a larger graph are replaced by fused
     calls and the rest keeps running.  Here the fused call is the oracle (no GPU), so
@@ -244,6 +270,13 @@ def test_rewritten_graphs_compute_the_same(which, monkeypatch):
             return a.transpose(1, 2).reshape(B, S, E) @ wo + x
         ins = (f32(2, 24, 256),) + tuple(f32(256, 256, seed=s) * 0.06 for s in (1, 2, 3, 4))
         n_attn = 1
+    elif which in ("softmax1", "softmax_e"):
+        base2, c = (True, 1.0) if which == "softmax1" else (False, 0.25)
+
+        def fn(Q, K, V):
+            QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+            return _explicit_softmax(torch.ops.loopfuse.causal_mask(QK), base2, c).to(Q.dtype) @ V
+        ins, n_attn = (f32(2, 3, 40, 64), f32(2, 3, 40, 64, seed=1), f32(2, 3, 40, 64, seed=2)), 1
     else:
         def fn(Q, qb, K, sb, V, ob):
             QK = (Q + qb) @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)

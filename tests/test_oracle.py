@@ -12,7 +12,7 @@ import torch
 from oracle import attention_oracle as O
 
 
-def brute_force(q, k, v, mask, window, scale, softcap, score_bias=None, out_bias=None):
+def brute_force(q, k, v, mask, window, scale, softcap, score_bias=None, out_bias=None, denom_add=0.0):
     """float64 loops straight from the definition; no shared code with the oracle."""
     B, Hq, Sq, D = q.shape
     Hkv, Sk = k.shape[1], k.shape[2]
@@ -40,7 +40,7 @@ def brute_force(q, k, v, mask, window, scale, softcap, score_bias=None, out_bias
                     sc.append(dot)
                 mx = max(x for x in sc if x is not None)
                 w = [0.0 if x is None else math.exp(x - mx) for x in sc]
-                tot = sum(w)
+                tot = sum(w) + denom_add
                 for d in range(D):
                     out[b][h][i][d] = sum(w[j] * float(v[b, hk, j, d]) for j in range(Sk)) / tot
                     if out_bias is not None:
@@ -74,6 +74,26 @@ def test_biases_match_float64_loops(mask, softcap):
     got = O.attention_reference(q, k, v, mask=mask, scale=0.6, softcap=softcap, score_bias=sb, out_bias=ob)
     want = brute_force(q, k, v, mask, 0, 0.6, softcap, sb, ob)
     assert torch.allclose(got.double(), want, atol=2e-6, rtol=1e-5)
+
+
+def test_denominator_offset():
+    g = torch.Generator().manual_seed(13)
+    q, k, v = (torch.randn(1, 2, 6, 4, generator=g) for _ in range(3))
+    got = O.attention_reference(q, k, v, mask="causal", scale=0.5, denom_add=1.0)
+    want = brute_force(q, k, v, "causal", 0, 0.5, None, denom_add=1.0)
+    assert torch.allclose(got.double(), want, atol=2e-6, rtol=1e-5)
+    # row 0 sees one key: its probability is 1 / (1 + c)
+    assert torch.allclose(got[:, :, 0], v[:, :, 0] / 2.0, atol=1e-6)
+    # the offset is relative to the row maximum: shifting all scores of a row changes nothing
+    shift = torch.randn(1, 2, 6, 1, generator=g).expand(1, 2, 6, 6)
+    assert torch.allclose(O.attention_reference(q, k, v, mask="causal", scale=0.5, denom_add=1.0, score_bias=shift),
+                          got, atol=1e-6)
+    # c = 0 is the plain softmax; the output shrinks monotonically with c
+    assert torch.equal(O.attention_reference(q, k, v, denom_add=0.0), O.attention_reference(q, k, v))
+    plain = O.attention_reference(q, k, v, mask="causal", scale=0.5)
+    l = torch.exp((q @ k.transpose(-2, -1) * 0.5).masked_fill(~O.dense_mask("causal", 6, 6), float("-inf")))
+    l = (l / l.max(-1, keepdim=True).values).sum(-1, keepdim=True)
+    assert torch.allclose(got, plain * l / (l + 1.0), atol=1e-6)
 
 
 def test_bias_closed_forms():

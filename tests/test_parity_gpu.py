@@ -25,11 +25,11 @@ def rand(shape, dtype, seed):
 
 
 def check(q, k, v, *, mask=None, window=0, softcap=None, k_table=None, v_table=None, scale=None,
-          score_bias=None, out_bias=None, **kw):
+          score_bias=None, out_bias=None, denom_add=0.0, **kw):
     dtype = q.dtype
     scale = q.shape[-1] ** -0.5 if scale is None else scale
     plan = lowering.AttnPlan(mask=mask, window=window, scale=scale, softcap=softcap,
-                             k_paged=k_table is not None, v_paged=v_table is not None)
+                             k_paged=k_table is not None, v_paged=v_table is not None, denom_add=denom_add)
     mv = lambda t: None if t is None else t.to(dev())
     got = lowering.attention(mv(q), mv(k), mv(v), plan, mv(k_table), mv(v_table),
                              score_bias=mv(score_bias), out_bias=mv(out_bias), **kw)
@@ -37,7 +37,8 @@ def check(q, k, v, *, mask=None, window=0, softcap=None, k_table=None, v_table=N
         got = got[0]
     torch.cuda.synchronize()
     want = O.attention_reference(q, k, v, mask=mask, window=window, softcap=softcap, scale=scale,
-                                 k_table=k_table, v_table=v_table, score_bias=score_bias, out_bias=out_bias)
+                                 k_table=k_table, v_table=v_table, score_bias=score_bias, out_bias=out_bias,
+                                 denom_add=denom_add)
     got = got.float().cpu()
     assert torch.isfinite(got).all()
     if out_bias is not None:
@@ -183,6 +184,25 @@ def test_bias_with_wrong_dtype_is_refused():
     sb = rand((1, 1, 64, 64), torch.float16, 4).to(dev())
     with pytest.raises(lowering.UnsupportedPlan):
         lowering.attention(q, k, v, lowering.AttnPlan(mask="causal", scale=0.125), score_bias=sb)
+
+
+# ---------------------------------------------------------------- shifted softmax denominator
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("mask,S,c", [("causal", 593, 1.0), ("sliding", 300, 0.25), (None, 129, 3.0)])
+def test_shifted_denominator(dtype, mask, S, c):
+    # probabilities e^(s-m) / (sum e^(s-m) + c), reference tests/test_attention.py:95-125
+    q, k, v = (rand((2, 4, S, 128), dtype, s) for s in (1, 2, 3))
+    check(q, k, v, mask=mask, window=77, denom_add=c)
+    check(q * 6, k, v, mask=mask, window=77, denom_add=c)          # sharp rows: the max dominates the sum
+
+
+def test_shifted_denominator_single_row_and_gqa_paged():
+    B, Hq, Hkv, S, D, P = 2, 8, 2, 256, 64, 16
+    n = B * S // P
+    kp, vp = rand((n, P, Hkv, D), torch.bfloat16, 1), rand((n, P, Hkv, D), torch.bfloat16, 2)
+    table = torch.randperm(n, generator=torch.Generator().manual_seed(9)).view(B, S // P).to(torch.int32)
+    check(rand((B, Hq, 1, D), torch.bfloat16, 3), kp, vp, k_table=table, v_table=table, denom_add=1.0)
+    check(rand((B, Hq, S, D), torch.bfloat16, 3), kp, vp, mask="causal", k_table=table, v_table=table, denom_add=1.0)
 
 
 # ---------------------------------------------------------------- block skip
