@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A step is one pass of the hot path over one batch of synthetic input.  The
-headline workload is BASELINE config 2 (bf16 causal prefill, B8 H32 S2048 D128):
+headline workload is config 2 (bf16 causal prefill, B8 H32 S2048 D128):
 ``value`` is its algorithmic TFLOP/s with the reference's flop convention
 (2*B*H*S^2*D, reference tests/benchmark.py:110).  The same run also times the
 memory-bound half of the metric, config 5 (paged GQA decode, B64 K_len 2048, page
@@ -28,7 +28,7 @@ if ROOT not in sys.path:
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16/fp16, published
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, published
 # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by a plain copy of known
-# size (profiles/*_hbm_traffic.md); counters cannot be read from inside this process
+# size (the rocprofv3 summaries under profiles/); counters cannot be read from inside this process
 TRAFFIC_BYTES = {"c2": (558 + 128) * (1 << 20), "c5": (513 + 4) * (1 << 20)}
 
 

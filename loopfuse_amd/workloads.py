@@ -3,7 +3,7 @@
 Generated on the CPU generator in fp32 and cast, so a CPU checker and the GPU
 kernel see identical bits whatever the device.  Shapes follow the reference's
 benchmark harness (``tests/benchmark.py:68-76, 207-217, 380-398, 510-520``) with
-the sizes of this repository's BASELINE configs.
+the sizes of the five benchmark configurations.
 """
 from __future__ import annotations
 

@@ -1,7 +1,7 @@
 """GPU parity: HIP kernels (through the C-ABI shim) vs the CPU fp32 oracle on the
-same seeded inputs.  Tolerances are the north-star ones: max-abs <= 2e-2 for bf16,
+same seeded inputs.  Tolerances: max-abs <= 2e-2 for bf16,
 <= 5e-3 for fp16.  Mirrors the reference's tests/test_accuracy.py cases (causal
-S in {256, 593}, GQA, sliding window 256, paged K, paged GQA) plus the BASELINE
+S in {256, 593}, GQA, sliding window 256, paged K, paged GQA) plus the benchmark
 configs.
 """
 import pytest
@@ -345,7 +345,7 @@ def test_decode_equals_last_prefill_row():
     assert (full[:, :, -1:].float() - last.float()).abs().max().item() <= 1e-2
 
 
-# ---------------------------------------------------------------- BASELINE configs at full size
+# ---------------------------------------------------------------- benchmark configs at full size
 def _full_size_check(w, rows=64):
     """Full-size run; oracle on a sample of (batch, head) pairs to stay within seconds."""
     wd = w.to(dev())
