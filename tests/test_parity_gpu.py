@@ -484,3 +484,33 @@ def test_tuned_attention_matches_and_remembers(name, monkeypatch, tmp_path):
     assert json.load(open(lowering._TUNE_FILE)) == {key: choice}
     want = O.attention_reference(w.q, w.k, w.v, mask=w.mask, k_table=w.k_table, v_table=w.v_table)
     assert (got.float().cpu() - want).abs().max().item() <= TOL[torch.bfloat16]
+
+
+# ---------------------------------------------------------------- HIP graph capture
+@pytest.mark.parametrize("name", ["c5", "c2"])
+def test_launches_can_be_captured_in_a_hip_graph(name):
+    """A serving loop captures the decode step once and replays it: the launches go to
+    the capturing stream, allocate nothing during capture (output and split scratch
+    exist beforehand) and read their inputs by address, so refreshed inputs are seen.
+    Every replay is checked against the eager launch, with eager work in between."""
+    w = workloads.make(name, seed=11, B=2, S=512).to(dev())
+    plan = lowering.AttnPlan(mask=w.mask, window=w.window, scale=w.scale, softcap=w.softcap,
+                             k_paged=w.k_table is not None, v_paged=w.v_table is not None)
+    q = w.q.clone()
+    out = lowering.attention(q, w.k, w.v, plan, w.k_table, w.v_table)      # warm: code objects, scratch
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        lowering.attention(q, w.k, w.v, plan, w.k_table, w.v_table, out=out)
+        stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            lowering.attention(q, w.k, w.v, plan, w.k_table, w.v_table, out=out)
+    for rep in range(3):
+        q.copy_(rand(tuple(q.shape), torch.bfloat16, 100 + rep).to(dev()))
+        want = lowering.attention(q, w.k, w.v, plan, w.k_table, w.v_table).clone()    # eager, other buffer
+        torch.cuda.synchronize()
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), f"replay {rep} differs from the eager launch"
