@@ -29,7 +29,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16/fp16, published
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, published
 # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by a plain copy of known
 # size (the rocprofv3 summaries under profiles/); counters cannot be read from inside this process
-TRAFFIC_BYTES = {"c2": (558 + 128) * (1 << 20), "c5": (513 + 4) * (1 << 20)}
+TRAFFIC_BYTES = {"c2": (548 + 128) * (1 << 20), "c5": (513 + 4) * (1 << 20)}
 
 
 def time_gpu(fn, steps: int, warmup: int):
@@ -100,8 +100,8 @@ def cpu_baseline(seconds: float = 12.0) -> dict:
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="time only one of the two kernels (profiling aid)")
