@@ -88,11 +88,11 @@ class KernelSpec:
         return o + list(self.extra)
 
     def files(self) -> tuple[str, ...]:
-        return ("lf_common.hip.h", {"prefill": "lf_attn_prefill.hip", "prefill_pipe": "lf_attn_prefill_pipe.hip",
+        return ("lf_common.hip.h", {"prefill": "lf_attn_prefill.hip",
                                     "prefill_swp": "lf_attn_prefill_swp.hip", "decode": "lf_attn_decode.hip"}[self.family])
 
     def entry(self) -> str:
-        return {"prefill": "lf_attn_prefill", "prefill_pipe": "lf_attn_prefill_pipe",
+        return {"prefill": "lf_attn_prefill",
                 "prefill_swp": "lf_attn_prefill_swp", "decode": "lf_attn_decode"}[self.family]
 
     def name(self) -> str:
@@ -246,12 +246,10 @@ def prefill_variant(Sq: int, v_tr: bool = True) -> str:
     """Which prefill kernel serves a call.  Default: the software-pipelined kernel
     with direct-to-LDS staging (``prefill_swp``; dense K/V only, ``attention`` falls
     back to ``prefill`` for paged operands).  LOOPFUSE_PREFILL=w32 selects the
-    register-staged kernel, =pipe the one-wave-per-SIMD kernel, for comparison."""
+    register-staged kernel for comparison."""
     env = os.environ.get("LOOPFUSE_PREFILL", "swp")
     if not v_tr or env == "w32":
         return "prefill"
-    if env == "pipe":
-        return "prefill_pipe"
     return "prefill_swp"
 
 
@@ -485,7 +483,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         span = max((Sk - 1) * abs(P.k_ss), (Sk - 1) * abs(P.v_ss)) * 2 + 2 * D
         if span >= (1 << 31):
             family = "prefill"
-    if family in ("prefill", "prefill_pipe", "prefill_swp"):
+    if family in ("prefill", "prefill_swp"):
         P.q_sb, P.q_sh, P.q_ss = q.stride(0), q.stride(1), q.stride(2)
         P.o_sb, P.o_sh, P.o_ss = out.stride(0), out.stride(1), out.stride(2)
         extra = tuple(os.environ.get("LOOPFUSE_KOPTS", "").split())
@@ -516,7 +514,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         # 8 XCD classes x (batch*head pairs per class, padded to the kernel's groups of 4) x q tiles
         per_xcd = (B * Hq + 7) // 8
         # lf_attn_prefill takes two q tiles (heavy + light) per workgroup
-        per_bh = nqt if family == "prefill_pipe" else (nqt + 1) // 2
+        per_bh = (nqt + 1) // 2
         grid = 8 * ((per_xcd + 3) // 4 * 4) * per_bh
         persist = os.environ.get("LOOPFUSE_PREFILL_PERSIST")
         if family == "prefill_swp" and persist:
