@@ -222,24 +222,28 @@ def decode_split(units: int, Sk: int, cus: int = 256, per_cu: int = 2) -> int:
     """Number of KV splits across workgroups.  One workgroup per unit is enough once
     there are ``per_cu`` workgroups per CU (8 resident waves, each with 32 KB of loads
     in flight: two workgroups of 4 waves, or one of 8); below that the KV range is
-    split, down to 256 tokens per split, and a second kernel merges the partial
-    results."""
+    split, down to 512 tokens per split and 16 splits, and a second kernel merges the
+    partial results."""
     env = os.environ.get("LOOPFUSE_DECODE_SPLITS")
     if env:
         return max(1, int(env))
     want = max(1, (per_cu * cus + units - 1) // units)
-    most = max(1, Sk // 256)
+    most = max(1, min(16, Sk // 512))      # measured: >= 512 tokens per split, at most 16 splits
     return max(1, min(want, most))
 
 
-def _decode_headwave(paged: int, page_size: int, Hkv: int, D: int, P: "AttnParams") -> bool:
+def _decode_headwave(paged: int, page_size: int, Hkv: int, D: int, P: "AttnParams", units_hw: int = 1 << 30,
+                     Sk: int = 1 << 30, cus: int = 256) -> bool:
     """One kv head per wave pays when K and V are paged, token-major (head stride D,
-    token stride Hkv*D) and there are at least 8 heads to fill the 8 waves."""
+    token stride Hkv*D), there are at least 8 heads to fill the 8 waves, and the
+    (batch, head-chunk) units times at most 8 KV splits of >= 256 tokens still give one
+    workgroup per CU (measured: below that, 4 waves per head with more splits win)."""
     env = os.environ.get("LOOPFUSE_DECODE_HEADWAVE")
     if env is not None:
         return env == "1"
     return (paged == 3 and Hkv % 8 == 0 and P.k_sh == D and P.v_sh == D
-            and P.k_ss == Hkv * D and P.v_ss == Hkv * D)
+            and P.k_ss == Hkv * D and P.v_ss == Hkv * D
+            and units_hw * max(1, min(8, Sk // 512)) >= cus)
 
 
 def prefill_variant(Sq: int, v_tr: bool = True) -> str:
@@ -543,7 +547,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     waves = int(os.environ.get("LOOPFUSE_DECODE_WAVES", "4"))
     # Token-major page pools ([pages, page, Hkv, D]: the heads of a token side by side)
     # are read whole-page-wise when the 8 waves of a workgroup take 8 consecutive heads.
-    headwave = _decode_headwave(paged, page_size, Hkv, D, P)
+    headwave = _decode_headwave(paged, page_size, Hkv, D, P, B * ((Hkv + 7) // 8) * chunks, Sk)
     if "head_per_wave" in choice:
         headwave = bool(choice["head_per_wave"]) and paged == 3 and Hkv % 8 == 0
     if headwave:
