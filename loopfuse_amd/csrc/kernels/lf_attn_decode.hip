@@ -375,10 +375,15 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 8 / LF_DW) lf_attn_decode(co
 #endif   // LF_HEADWAVE
 }
 
-// Merge nsplit partial results per query row: grid = (B*Hkv*rows), block = LF_D.
-extern "C" __global__ void __launch_bounds__(LF_HEAD_DIM) lf_attn_decode_combine(const LfAttnParams p) {
-  const int d = threadIdx.x;
-  const long long rowid = blockIdx.x;               // (bh * rows + qr)
+// Merge nsplit partial results per query row.  A thread owns 4 consecutive d of one row;
+// block = 256 threads = 1024 / LF_HEAD_DIM rows, grid = ceil(B*Hkv*rows / rows per block).
+extern "C" __global__ void __launch_bounds__(256) lf_attn_decode_combine(const LfAttnParams p) {
+  constexpr int kTPR = LF_HEAD_DIM / 4;              // threads per row
+  constexpr int kRPB = 256 / kTPR;                   // rows per block
+  const long long rowid = (long long)blockIdx.x * kRPB + threadIdx.x / kTPR;   // (bh * rows + qr)
+  const long long nrows = (long long)p.B * p.Hkv * p.rows;
+  if (rowid >= nrows) return;
+  const int d0 = 4 * (threadIdx.x % kTPR);
   const int qr = (int)(rowid % p.rows);
   const int bh = (int)(rowid / p.rows);
   const int hkv = bh % p.Hkv;
@@ -386,13 +391,18 @@ extern "C" __global__ void __launch_bounds__(LF_HEAD_DIM) lf_attn_decode_combine
   float m = LF_NEG_INF;
   for (int z = 0; z < p.nsplit; ++z) m = fmaxf(m, p.part_ml[(rowid * p.nsplit + z) * 2]);
   const float m_sub = (m == LF_NEG_INF) ? 0.0f : m;
-  float l = 0.0f, a = 0.0f;
+  float l = 0.0f;
+  lf_f32x4 a = {0.0f, 0.0f, 0.0f, 0.0f};
   for (int z = 0; z < p.nsplit; ++z) {
     const long long slot = rowid * p.nsplit + z;
     const float f = lf_exp2(p.part_ml[slot * 2] - m_sub);
     l += p.part_ml[slot * 2 + 1] * f;
-    a += p.part_acc[slot * LF_HEAD_DIM + d] * f;
+    a += *reinterpret_cast<const lf_f32x4*>(&p.part_acc[slot * LF_HEAD_DIM + d0]) * f;
   }
   lf_elem* orow = p.o + (long long)b * p.o_sb + (long long)hkv * p.o_sh + (long long)qr * p.o_ss;
-  orow[d] = lf_from_float(a / l);
+  const float inv = 1.0f / l;
+  lf_elem4 w;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) w[e] = lf_from_float(a[e] * inv);
+  *reinterpret_cast<lf_elem4*>(orow + d0) = w;
 }

@@ -568,7 +568,9 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         P.part_ml = scratch.data_ptr() + 4 * nrow * D
     get_kernel(spec, "lf_attn_decode").launch((units, nsplit, 1), (64 * spec.waves, 1, 1), P)
     if nsplit > 1:
-        get_kernel(spec, "lf_attn_decode_combine").launch((B * Hkv * rows, 1, 1), (D, 1, 1), P)
+        rows_per_block = 1024 // D       # 256 threads, 4 consecutive d each
+        get_kernel(spec, "lf_attn_decode_combine").launch(
+            ((B * Hkv * rows + rows_per_block - 1) // rows_per_block, 1, 1), (256, 1, 1), P)
     attention.last_launch = {"kernels": ["lf_attn_decode"] + (["lf_attn_decode_combine"] if nsplit > 1 else []),
                              "grid": (units, nsplit), "block": 64 * spec.waves, "head_per_wave": headwave}
     return out
