@@ -346,7 +346,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
               *, out: Optional[torch.Tensor] = None, record_visits: bool = False,
               force_family: str | None = None, num_splits: int | None = None, v_tr: bool = True,
               score_bias: Optional[torch.Tensor] = None, out_bias: Optional[torch.Tensor] = None,
-              choice: Optional[dict] = None):
+              choice: Optional[dict] = None, merge_splits: bool = True):
     """Run fused attention on the GPU.
 
     q : [B, Hq, Sq, D];  k, v : [B, Hkv, Sk, D], or page pools [N, P, Hkv, D]
@@ -355,6 +355,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     scaled / capped scores before the mask, ``out_bias`` (broadcastable to
     [B, Hq, Sq, D]) to the result -- the reference's "modified attention" graph
     (tests/test_accuracy.py:172-196).  Both are served by ``lf_attn_prefill`` only.
+    ``merge_splits=False`` leaves the partial results of a split decode unmerged (the
+    output is then not written): for timing the streaming kernel alone.
     ``choice`` overrides the launch heuristics (what ``tuned_attention`` searches over):
     ``{"prefill": "swp" | "w32"}``, ``{"head_per_wave": bool, "splits": n}``.
     Returns O [B, Hq, Sq, D] (and the visited-tile record if asked).
@@ -567,10 +569,10 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         P.part_acc = scratch.data_ptr()
         P.part_ml = scratch.data_ptr() + 4 * nrow * D
     get_kernel(spec, "lf_attn_decode").launch((units, nsplit, 1), (64 * spec.waves, 1, 1), P)
-    if nsplit > 1:
+    if nsplit > 1 and merge_splits:
         rows_per_block = 1024 // D       # 256 threads, 4 consecutive d each
         get_kernel(spec, "lf_attn_decode_combine").launch(
             ((B * Hkv * rows + rows_per_block - 1) // rows_per_block, 1, 1), (256, 1, 1), P)
-    attention.last_launch = {"kernels": ["lf_attn_decode"] + (["lf_attn_decode_combine"] if nsplit > 1 else []),
+    attention.last_launch = {"kernels": ["lf_attn_decode"] + (["lf_attn_decode_combine"] if nsplit > 1 and merge_splits else []),
                              "grid": (units, nsplit), "block": 64 * spec.waves, "head_per_wave": headwave}
     return out
