@@ -57,6 +57,13 @@
 #define LF_LAZY_LOG2 8   /* slack of the softmax exponent offset, log2 units */
 #endif
 
+#ifndef LF_D2
+#define LF_D2 0     /* depth of a second score product: S = Q K^T + Q2 K2^T (16, 32 or 64; 0 = none) */
+#endif
+#if LF_D2 && LF_DMA == 2
+#error "the second score product is staged through registers: LF_DMA 0 or 1"
+#endif
+
 #ifndef LF_BN
 #define LF_BN 64
 #endif
@@ -76,6 +83,10 @@
 #define LF_NKS (LF_D / 16)                   /* k-steps of the QK^T product   */
 #define LF_NDB (LF_D / 32)                   /* 32-row blocks of O^T          */
 #define LF_NKK (LF_BN / 16)                  /* k-steps of the PV product     */
+#define LF_CPR2 (LF_D2 / 8)                  /* 16-byte chunks per K2 row      */
+#define LF_NKS2 (LF_D2 / 16)                 /* k-steps of the Q2 K2^T product */
+#define LF_RPS2 (LF_D2 ? 256 / (LF_D2 * 2) : 1)
+#define LF_NP2 ((LF_BN * LF_CPR2 + LF_NT - 1) / LF_NT)   /* staging passes of a K2 tile */
 // LDS row strides (elements).  LF_PAD: rows are padded instead of XOR-swizzled, so
 // every fragment address is one per-lane base plus a compile-time offset (no
 // per-fragment address arithmetic): +16 bytes per K row spreads 16 consecutive
@@ -102,6 +113,13 @@ __device__ __forceinline__ int lf_k_phys(int row, int ch) {
   return ch ^ ((row / LF_RPS) & (LF_CPR - 1));
 #endif
 }
+#if LF_D2
+// The K2 tile (rows of LF_D2 elements, several rows per 256-byte bank span): the same
+// permutation with its own row length.
+__device__ __forceinline__ int lf_k2_phys(int row, int ch) {
+  return ch ^ ((row / LF_RPS2) & (LF_CPR2 - 1));
+}
+#endif
 // Same for the V tile, where a transposed read touches 4 consecutive rows x 64
 // contiguous bytes per 32 lanes: permute the 64-byte groups by the row.
 __device__ __forceinline__ int lf_v_phys(int row, int ch) {
@@ -115,6 +133,9 @@ __device__ __forceinline__ int lf_v_phys(int row, int ch) {
 extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(const LfAttnParams p) {
   __shared__ __attribute__((aligned(16))) lf_elem lds_k[2][LF_BN * LF_KS];
   __shared__ __attribute__((aligned(16))) lf_elem lds_v[2][LF_BN * LF_VS];
+#if LF_D2
+  __shared__ __attribute__((aligned(16))) lf_elem lds_k2[2][LF_BN * LF_D2];
+#endif
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -182,6 +203,22 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
       qf[ks] = __builtin_bit_cast(lf_elem8, raw);
     }
   }
+
+#if LF_D2
+  lf_elem8 qf2[LF_NKS2];
+  {
+    const lf_elem* qrow = p.q2 + (long long)b * p.q2_sb + (long long)h * p.q2_sh + (long long)my_q * p.q2_ss;
+#pragma unroll
+    for (int ks = 0; ks < LF_NKS2; ++ks) {
+      lf_u32x4 raw = {0u, 0u, 0u, 0u};
+      if (my_q < p.Sq) raw = *reinterpret_cast<const lf_u32x4*>(qrow + 16 * ks + 8 * g);
+      qf2[ks] = __builtin_bit_cast(lf_elem8, raw);
+    }
+  }
+  // K2 tile: plain loads with the row clamped to Sk-1 (scores of rows past Sk are masked)
+  lf_u32x4 k2st[LF_NP2];
+  const lf_elem* k2_uni = p.k2 + (long long)b * p.k2_sb + (long long)(h / p.k2_group) * p.k2_sh;
+#endif
 
 #if LF_SOFTCAP
   const float sc_in = p.scale / p.softcap;   // tanh argument multiplier
@@ -293,6 +330,16 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
       }
 #endif
     }
+#if LF_D2
+#pragma unroll
+    for (int ps = 0; ps < LF_NP2; ++ps) {
+      const int c = tid + LF_NT * ps;
+      if (c < LF_BN * LF_CPR2) {
+        const int tok = min(kt * LF_BN + c / LF_CPR2, p.Sk - 1);
+        k2st[ps] = *reinterpret_cast<const lf_u32x4*>(k2_uni + (long long)tok * p.k2_ss + 8 * (c % LF_CPR2));
+      }
+    }
+#endif
   };
   auto store_tile = [&](int buf) {
 #pragma unroll
@@ -306,6 +353,16 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
       *reinterpret_cast<lf_u32x4*>(&lds_v[buf][row * LF_VS + 8 * lf_v_phys(row, sch)]) = vst[ps];
 #endif
     }
+#if LF_D2
+#pragma unroll
+    for (int ps = 0; ps < LF_NP2; ++ps) {
+      const int c = tid + LF_NT * ps;
+      if (c < LF_BN * LF_CPR2) {
+        const int row = c / LF_CPR2;
+        *reinterpret_cast<lf_u32x4*>(&lds_k2[buf][row * LF_D2 + 8 * lf_k2_phys(row, c % LF_CPR2)]) = k2st[ps];
+      }
+    }
+#endif
 #if LF_DMA_K || LF_DMA_V
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's direct-to-LDS loads have landed
 #endif
@@ -378,6 +435,19 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
           if (f % (kNF / LF_NPASS) == 1) dma_k_pass(kt + 1, cur ^ 1, f / (kNF / LF_NPASS));
 #endif
         }
+#if LF_D2
+        // + Q2 K2^T into the same accumulators
+        {
+          const lf_elem* k2buf = lds_k2[cur];
+#pragma unroll
+          for (int f = 0; f < LF_NKS2 * LF_NKB; ++f) {
+            const int ks = f / LF_NKB, kb = f % LF_NKB;
+            const int row = 32 * kb + l32;
+            const lf_u32x4 kv = *reinterpret_cast<const lf_u32x4*>(&k2buf[row * LF_D2 + 8 * lf_k2_phys(row, 2 * ks + g)]);
+            s[kb] = lf_mfma32(__builtin_bit_cast(lf_elem8, kv), qf2[ks], s[kb]);
+          }
+        }
+#endif
 #if LF_SCHED
         // pin the order: LF_KPF reads, then (MFMA, read) pairs, then the last MFMAs
         __builtin_amdgcn_sched_group_barrier(0x100, LF_KPF, 0);

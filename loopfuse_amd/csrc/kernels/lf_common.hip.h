@@ -90,6 +90,8 @@ struct LfAttnParams {
   const lf_elem* bias;       // LF_BIAS & 1: additive score bias [B, Hq, Sq, Sk] (key stride 1),
                              // added after scale / softcap and before the mask
   const lf_elem* obias;      // LF_BIAS & 2: additive output bias [B, Hq, Sq, D] (d stride 1)
+  const lf_elem* q2;         // LF_D2: second score product, scores = Q K^T + Q2 K2^T (the two-part
+  const lf_elem* k2;         // scores of reference tests/test_attention.py:126-151); dense, depth LF_D2
   long long q_sb, q_sh, q_ss;  // element strides of Q [B, Hq, Sq, D] (d stride 1)
   long long k_sb, k_sh, k_ss;  // K [B, Hkv, Sk, D]; paged: k_sb = page stride,
                                // k_ss = stride between tokens inside a page
@@ -97,12 +99,15 @@ struct LfAttnParams {
   long long o_sb, o_sh, o_ss;
   long long bias_sb, bias_sh, bias_sq;   // element strides of bias (0 = broadcast)
   long long ob_sb, ob_sh, ob_sq;         // element strides of obias (0 = broadcast)
+  long long q2_sb, q2_sh, q2_ss;         // Q2 [B, Hq, Sq, LF_D2] (d stride 1)
+  long long k2_sb, k2_sh, k2_ss;         // K2 [B, Hq / k2_group, Sk, LF_D2] (d stride 1)
   int B, Hq, Hkv, Sq, Sk;
   int window;                // sliding-window width (LF_MASK == 2)
   int kt_stride, vt_stride;  // row strides (elements) of k_table / v_table
   int nsplit;                // decode: number of KV splits across workgroups
   int rows;                  // decode: query rows per (batch, kv head) unit
   int split_len;             // decode: tokens per split (multiple of 16)
+  int k2_group;              // LF_D2: query heads per K2 head
   float scale;               // multiplies QK^T (D^-0.5 in the reference graphs)
   float softcap;             // cap of cap*tanh(s/cap) (LF_SOFTCAP)
   float denom_add;           // LF_DENOM: probabilities are e^(x - max) / (sum e^(x - max) + denom_add)

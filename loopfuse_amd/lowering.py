@@ -41,12 +41,14 @@ class AttnParams(ctypes.Structure):
     """Mirror of ``struct LfAttnParams`` in csrc/kernels/lf_common.hip.h."""
 
     _fields_ = (
-        [(n, ctypes.c_void_p) for n in ("q", "k", "v", "o", "k_table", "v_table", "part_acc", "part_ml", "visits", "bias", "obias")]
+        [(n, ctypes.c_void_p) for n in ("q", "k", "v", "o", "k_table", "v_table", "part_acc", "part_ml", "visits", "bias", "obias",
+                                        "q2", "k2")]
         + [(n, ctypes.c_longlong) for n in (
             "q_sb", "q_sh", "q_ss", "k_sb", "k_sh", "k_ss", "v_sb", "v_sh", "v_ss", "o_sb", "o_sh", "o_ss",
-            "bias_sb", "bias_sh", "bias_sq", "ob_sb", "ob_sh", "ob_sq")]
+            "bias_sb", "bias_sh", "bias_sq", "ob_sb", "ob_sh", "ob_sq",
+            "q2_sb", "q2_sh", "q2_ss", "k2_sb", "k2_sh", "k2_ss")]
         + [(n, ctypes.c_int) for n in (
-            "B", "Hq", "Hkv", "Sq", "Sk", "window", "kt_stride", "vt_stride", "nsplit", "rows", "split_len")]
+            "B", "Hq", "Hkv", "Sq", "Sk", "window", "kt_stride", "vt_stride", "nsplit", "rows", "split_len", "k2_group")]
         + [("scale", ctypes.c_float), ("softcap", ctypes.c_float), ("denom_add", ctypes.c_float)]
     )
 
@@ -69,6 +71,7 @@ class KernelSpec:
     headwave: bool = False  # decode: one kv head per wave (8 waves) instead of 4 waves sharing a head
     denom: bool = False    # prefill: softmax denominator sum + c (c a run-time parameter)
     bias: int = 0          # prefill: bit 0 additive score bias tensor, bit 1 additive output bias tensor, bit 2 unaligned rows
+    d2: int = 0            # prefill: depth of a second score product Q2 K2^T (0, 16, 32, 64)
     extra: tuple = ()      # further -D options (tuning experiments)
 
     def options(self) -> list[str]:
@@ -85,6 +88,8 @@ class KernelSpec:
             o += [f"-DLF_DW={self.waves}", f"-DLF_HEADWAVE={int(self.headwave)}"]
         elif self.family == "prefill":
             o += [f"-DLF_V_TR={int(self.v_tr)}", f"-DLF_BIAS={self.bias}", f"-DLF_DENOM={int(self.denom)}"]
+            if self.d2:
+                o += [f"-DLF_D2={self.d2}"]
         return o + list(self.extra)
 
     def files(self) -> tuple[str, ...]:
@@ -98,6 +103,7 @@ class KernelSpec:
     def name(self) -> str:
         return (f"lf_{self.family}_t{self.dtype}_d{self.head_dim}_m{self.mask}_c{int(self.softcap)}"
                 f"_p{self.paged}x{self.page_size}i{int(self.table_i64)}_r{self.rows}w{self.waves}v{int(self.v_tr)}h{int(self.headwave)}b{self.bias}n{int(self.denom)}"
+                + (f"_q{self.d2}" if self.d2 else "")
                 + "".join("_" + e.replace("-D", "").replace("=", "") for e in self.extra))
 
     def source(self) -> str:
@@ -295,7 +301,7 @@ def tuned_attention(q, k, v, plan: AttnPlan, k_table=None, v_table=None, **kw):
     launches), the winner is remembered in the process and in ``autotune.json`` beside
     the code-object cache.  Used by the backend under ``mode="max-autotune"``."""
     if kw.get("score_bias") is not None or kw.get("out_bias") is not None or kw.get("record_visits") \
-            or kw.get("force_family") or kw.get("num_splits") or kw.get("choice") or plan.denom_add != 0.0:
+            or kw.get("force_family") or kw.get("num_splits") or kw.get("choice") or plan.denom_add != 0.0 or kw.get("q2") is not None:
         return attention(q, k, v, plan, k_table, v_table, **kw)
     _load_tuned()
     key = _tune_key(q, k, plan, k_table, 0)
@@ -346,7 +352,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
               *, out: Optional[torch.Tensor] = None, record_visits: bool = False,
               force_family: str | None = None, num_splits: int | None = None, v_tr: bool = True,
               score_bias: Optional[torch.Tensor] = None, out_bias: Optional[torch.Tensor] = None,
-              choice: Optional[dict] = None, merge_splits: bool = True):
+              choice: Optional[dict] = None, merge_splits: bool = True,
+              q2: Optional[torch.Tensor] = None, k2: Optional[torch.Tensor] = None):
     """Run fused attention on the GPU.
 
     q : [B, Hq, Sq, D];  k, v : [B, Hkv, Sk, D], or page pools [N, P, Hkv, D]
@@ -355,6 +362,10 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     scaled / capped scores before the mask, ``out_bias`` (broadcastable to
     [B, Hq, Sq, D]) to the result -- the reference's "modified attention" graph
     (tests/test_accuracy.py:172-196).  Both are served by ``lf_attn_prefill`` only.
+    ``q2`` [B, Hq, Sq, D2] and ``k2`` [B, H2, Sk, D2] (H2 divides Hq; D2 in 16, 32, 64) add a
+    second product to the scores, ``Q K^T + Q2 K2^T`` before the scale -- the two-part scores
+    of multi-head latent attention (reference tests/test_attention.py:126-151); served by
+    ``lf_attn_prefill`` with dense K2.
     ``merge_splits=False`` leaves the partial results of a split decode unmerged (the
     output is then not written): for timing the streaming kernel alone.
     ``choice`` overrides the launch heuristics (what ``tuned_attention`` searches over):
@@ -467,7 +478,24 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         P.obias = out_bias.data_ptr()
         P.ob_sb, P.ob_sh, P.ob_sq = out_bias.stride(0), out_bias.stride(1), out_bias.stride(2)
         bias_bits |= 2
-    if bias_bits & 3 or plan.denom_add != 0.0:
+    d2 = 0
+    if (q2 is None) != (k2 is None):
+        raise UnsupportedPlan("q2 and k2 come together")
+    if q2 is not None:
+        if q2.dim() != 4 or k2.dim() != 4 or q2.shape[:3] != (B, Hq, Sq):
+            raise UnsupportedPlan(f"Q2 must be [{B}, {Hq}, {Sq}, D2]")
+        d2 = q2.shape[3]
+        if d2 not in (16, 32, 64):
+            raise UnsupportedPlan(f"depth {d2} of the second score product not supported (16, 32, 64)")
+        if k2.shape[0] != B or k2.shape[2] != Sk or k2.shape[3] != d2 or k2.shape[1] < 1 or Hq % k2.shape[1]:
+            raise UnsupportedPlan(f"K2 must be [{B}, H2 | {Hq}, {Sk}, {d2}]")
+        _check_tensor("Q2", q2, dtype)
+        _check_tensor("K2", k2, dtype)
+        P.q2, P.k2 = q2.data_ptr(), k2.data_ptr()
+        P.q2_sb, P.q2_sh, P.q2_ss = q2.stride(0), q2.stride(1), q2.stride(2)
+        P.k2_sb, P.k2_sh, P.k2_ss = k2.stride(0), k2.stride(1), k2.stride(2)
+        P.k2_group = Hq // k2.shape[1]
+    if bias_bits & 3 or plan.denom_add != 0.0 or d2:
         force_family = "prefill"
 
     # ---- family: decode when there is no mask and few query rows share a KV head
@@ -475,9 +503,9 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     if family is None:
         few = (Sq == 1 and group <= 64) or (group == 1 and Sq <= 16)
         family = "decode" if (mask == MASK_NONE and few and Sk >= 16) else "prefill"
-    keep = (q, k, v, out, kt, vt, score_bias, out_bias)  # noqa: F841  (tensors stay alive until the launch is queued)
+    keep = (q, k, v, out, kt, vt, score_bias, out_bias, q2, k2)  # noqa: F841  (tensors stay alive until the launch is queued)
 
-    if family == "prefill" and not bias_bits and plan.denom_add == 0.0:
+    if family == "prefill" and not bias_bits and plan.denom_add == 0.0 and not d2:
         family = {"swp": "prefill_swp", "w32": "prefill"}.get(choice.get("prefill"), None) or prefill_variant(Sq, v_tr)
     if family == "prefill_swp":
         # direct-to-LDS staging: dense K/V only, 32-bit byte offsets per (batch, kv head)
@@ -497,11 +525,11 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         span = max((Sk - 1) * abs(P.k_ss), (Sk - 1) * abs(P.v_ss)) * 2 + 2 * D
         if family == "prefill" and span >= (1 << 31):
             extra += ("-DLF_KVBUF=0",)
-        elif family == "prefill" and bias_bits and not paged:
-            extra += ("-DLF_DMA=1",)     # frees the staging registers the bias values need
+        elif family == "prefill" and (bias_bits or d2) and not paged:
+            extra += ("-DLF_DMA=1",)     # frees the staging registers the bias values / Q2 fragments need
         spec = KernelSpec(family, _DTYPE_CODE[dtype], D, mask, plan.softcap is not None, paged,
                           page_size, table_i64, v_tr=v_tr if family == "prefill" else True, bias=bias_bits,
-                          denom=plan.denom_add != 0.0, extra=extra)
+                          denom=plan.denom_add != 0.0, d2=d2, extra=extra)
         if os.environ.get("LOOPFUSE_TIMING"):       # profiling aid, see LF_TIMING in the kernel
             attention.timing = torch.zeros(16, dtype=torch.float32, device=q.device)
             P.part_acc = attention.timing.data_ptr()

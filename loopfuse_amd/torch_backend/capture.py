@@ -82,6 +82,8 @@ class Stage:
     q: Ids
     kt: Ids                        # K^T operand [.., D, Sk]
     v: Optional[Ids] = None
+    q2: Optional[Ids] = None       # second score product (scores = Q K^T + Q2 K2^T), reference
+    kt2: Optional[Ids] = None      # tests/test_attention.py:126-151
     factors: list = dataclasses.field(default_factory=list)       # multipliers before tanh
     post_factors: list = dataclasses.field(default_factory=list)  # multipliers after tanh
     has_tanh: bool = False
@@ -188,6 +190,8 @@ class AttentionMatch:
     tune: bool = False             # mode="max-autotune": measure the launch heuristics per shape class
     denom_add: tuple = ()          # explicit softmax with denominator (sum + these terms): floats | ("arg", i)
     base2: bool = False            # explicit softmax written with exp2: scores are in log2 units
+    q2: Optional[Operand] = None   # second score product: scores = Q K^T + Q2 K2^T
+    k2: Optional[Operand] = None
 
     def describe(self) -> str:
         nm = lambda i: self.inputs[i].name
@@ -197,6 +201,7 @@ class AttentionMatch:
                 f"mask={self.mask} window={self.window} tanh={self.has_tanh} "
                 f"factors={self.factors} post={self.post_factors}"
                 f"{' denom+%s' % (self.denom_add,) if self.denom_add else ''}{' exp2' if self.base2 else ''}"
+                f"{' +Q2=%s K2=%s' % (nm(self.q2.index), nm(self.k2.index)) if self.q2 else ''}"
                 f"{' +score_bias(%s)' % nm(self.bias.index) if self.bias else ''}"
                 f"{' +out_bias(%s)' % nm(self.out_bias.index) if self.out_bias else ''}")
 
@@ -247,6 +252,11 @@ class AttentionMatch:
                 raise lowering.UnsupportedPlan("bias does not have the shape seen at trace time")
         return torch.as_strided(t, tuple(shape), strides, t.storage_offset())
 
+    def _second_product(self, vals) -> dict:
+        if self.q2 is None:
+            return {}
+        return {"q2": self._operand(self.q2, vals)[0], "k2": self._operand(self.k2, vals)[0]}
+
     def _shapes(self, vals):
         q, _ = self._operand(self.q, vals)
         k, kt = self._operand(self.k, vals)
@@ -283,7 +293,8 @@ class AttentionMatch:
         run = lowering.tuned_attention if self.tune else lowering.attention
         out = run(q, k, v, self.plan_for(vals), kt, vt,
                                  score_bias=self._bias_view(self.bias, vals, (B, Hq, Sq, Sk)),
-                                 out_bias=self._bias_view(self.out_bias, vals, (B, Hq, Sq, D)))
+                                 out_bias=self._bias_view(self.out_bias, vals, (B, Hq, Sq, D)),
+                                 **self._second_product(vals))
         if self.out_rank == 3:
             out = out.view(out.shape[0] * out.shape[1], out.shape[2], out.shape[3])
         return out
@@ -305,9 +316,13 @@ class AttentionMatch:
             i64 = vals[self.k.table_index].dtype == torch.int64
         mask = lowering._MASK_NAMES[plan.mask]
         bias = (1 if self.bias else 0) | (2 if self.out_bias else 0)
-        family = "prefill" if (paged or bias) else lowering.prefill_variant(q.shape[-2])
-        extra = ("-DLF_DMA=1",) if (bias and not paged) else ()
-        return [lowering.KernelSpec(family, dt, D, mask, plan.softcap is not None, paged, ps, i64, bias=bias, extra=extra)]
+        d2 = self._operand(self.q2, vals)[0].shape[-1] if self.q2 is not None else 0
+        if d2 not in (0, 16, 32, 64):
+            raise lowering.UnsupportedPlan("depth of the second score product not served by the HIP kernels")
+        family = "prefill" if (paged or bias or d2) else lowering.prefill_variant(q.shape[-2])
+        extra = ("-DLF_DMA=1",) if ((bias or d2) and not paged) else ()
+        return [lowering.KernelSpec(family, dt, D, mask, plan.softcap is not None, paged, ps, i64, bias=bias, d2=d2,
+                                    extra=extra)]
 
 
 # ----------------------------------------------------------------------------
@@ -393,6 +408,21 @@ def _fit_bias(entry: tuple, logical: tuple):
     if dims[3] is None and logical[3] > 1:
         raise NoMatch("bias is broadcast along its last dim")
     return src.node, tuple(dims)
+
+
+def _same_scalar(x, y) -> bool:
+    """Two score factors (numbers, graph nodes, ("recip", f)) that are the same value by
+    construction: identical, or the same pure computation on the same inputs."""
+    if x is y:
+        return True
+    if isinstance(x, tuple) and isinstance(y, tuple):
+        return len(x) == len(y) and all(_same_scalar(a, b) for a, b in zip(x, y))
+    if isinstance(x, torch.fx.Node) and isinstance(y, torch.fx.Node):
+        return (x.op == y.op == "call_function" and x.target is y.target and len(x.args) == len(y.args)
+                and not x.kwargs and not y.kwargs and all(_same_scalar(a, b) for a, b in zip(x.args, y.args)))
+    if isinstance(x, (int, float, str)) and isinstance(y, (int, float, str)):
+        return type(x) is type(y) and x == y
+    return False
 
 
 def match_attention(gm: torch.fx.GraphModule) -> list:
@@ -634,6 +664,17 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
                     else:
                         new.factors = st.factors + [f]
                     return new
+            if st.kind == "scores" and tgt is aten.add.Tensor and isinstance(a[1], Stage):
+                # Q K^T + Q2 K2^T: two bare products (or two products with the same factors)
+                o = a[1]
+                plain = lambda x: (x.kind == "scores" and x.q2 is None and not x.has_tanh and x.mask is None
+                                   and x.bias is None and x.uid == 0 and x.sm == "" and not x.post_factors)
+                if not (plain(st) and plain(o)) or kw.get("alpha", 1) != 1 or tuple(st.shape) != tuple(o.shape):
+                    raise _Skip("sum of two score tensors that are not bare products of one shape")
+                same = len(st.factors) == len(o.factors) and all(_same_scalar(x, y) for x, y in zip(st.factors, o.factors))
+                if not same:
+                    raise _Skip("the two score products carry different factors")
+                return dataclasses.replace(st, q2=o.q, kt2=o.kt)
             if st.kind == "scores" and tgt is aten.add.Tensor and isinstance(a[1], Ids) and st.mask is None \
                     and st.bias is None and kw.get("alpha", 1) == 1:
                 return dataclasses.replace(st, bias=(a[1], st.shape))
@@ -731,6 +772,9 @@ def _build_match(out_node: torch.fx.Node, st: Stage) -> AttentionMatch:
             inputs.append(n)
         return inputs.index(n)
 
+    if st.q2 is not None and st.q.t.shape[-1] != st.v.t.shape[-1] and st.q2.t.shape[-1] == st.v.t.shape[-1]:
+        # the product whose depth is V's head dim is the kernel's main one
+        st = dataclasses.replace(st, q=st.q2, kt=st.kt2, q2=st.q, kt2=st.kt)
     qperm, qg = _fit_operand(st.q.t, st.q.src, rows_are_d=False)
     kperm, kg = _fit_operand(st.kt.t, st.kt.src, rows_are_d=True)
     vperm, vg = _fit_operand(st.v.t, st.v.src, rows_are_d=False)
@@ -749,6 +793,15 @@ def _build_match(out_node: torch.fx.Node, st: Stage) -> AttentionMatch:
     q_op = operand(st.q, qperm, qg)
     k_op = operand(st.kt, kperm, kg)
     v_op = operand(st.v, vperm, vg)
+
+    q2_op = k2_op = None
+    if st.q2 is not None:
+        q2perm, q2g = _fit_operand(st.q2.t, st.q2.src, rows_are_d=False)
+        k2perm, k2g = _fit_operand(st.kt2.t, st.kt2.src, rows_are_d=True)
+        if st.q2.src.kind != "node" or q2g != 1 or st.kt2.src.kind != "node":
+            raise NoMatch("the second score product needs plain (unpaged) tensors")
+        q2_op = operand(st.q2, q2perm, q2g)
+        k2_op = operand(st.kt2, k2perm, k2g)
 
     qshape = tuple(st.q.src.shape[i] for i in qperm)       # stand-in [B, Hq, Sq, D]
     if len(st.shape) == 4:
@@ -780,4 +833,5 @@ def _build_match(out_node: torch.fx.Node, st: Stage) -> AttentionMatch:
     window = scalar(st.window) if st.mask == "sliding" else 0
     return AttentionMatch(out_node, inputs, q_op, k_op, v_op, [scalar(f) for f in st.factors],
                           [scalar(f) for f in st.post_factors], st.has_tanh, st.mask, window, out_rank,
-                          bias_op, obias_op, denom_add=tuple(scalar(t) for t in st.denom_add), base2=st.base2)
+                          bias_op, obias_op, denom_add=tuple(scalar(t) for t in st.denom_add), base2=st.base2,
+                          q2=q2_op, k2=k2_op)

@@ -64,13 +64,17 @@ def gather_paged(pool: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
 def attention_reference(q, k, v, *, mask: Optional[str] = None, window: int = 0,
                         scale: Optional[float] = None, softcap: Optional[float] = None,
                         k_table=None, v_table=None, score_bias=None, out_bias=None,
-                        denom_add: float = 0.0) -> torch.Tensor:
+                        denom_add: float = 0.0, q2=None, k2=None) -> torch.Tensor:
     """fp32 eager attention.  q [B,Hq,Sq,D]; k, v [B,Hkv,Sk,D] or page pools + tables.
     ``score_bias`` (broadcastable to [B,Hq,Sq,Sk]) is added to the scaled / capped scores
     before the mask and ``out_bias`` ([B,Hq,Sq,D]) to the result, as in the reference's
     modified-attention graph (tests/test_accuracy.py:172-196).  ``denom_add`` = c gives the
     probabilities e^(s - m) / (sum_j e^(s_j - m) + c) with m the row maximum, the explicit
-    softmax of the reference's tests/test_attention.py:95-125 (c = 1 there)."""
+    softmax of the reference's tests/test_attention.py:95-125 (c = 1 there).  ``q2``
+    [B,Hq,Sq,D2] and ``k2`` [B,H2,Sk,D2] (heads repeated like K's) add a second product to
+    the raw scores, (Q K^T + Q2 K2^T) * scale, the two-part scores of the reference's
+    tests/test_attention.py:126-151 (``scale`` must then be given: that graph uses
+    (D + D2)^-0.5)."""
     q = q.float()
     k = gather_paged(k.float(), k_table) if k_table is not None else k.float()
     v = gather_paged(v.float(), v_table) if v_table is not None else v.float()
@@ -81,7 +85,13 @@ def attention_reference(q, k, v, *, mask: Optional[str] = None, window: int = 0,
     if Hq != Hkv:
         k = k.repeat_interleave(Hq // Hkv, dim=1)
         v = v.repeat_interleave(Hq // Hkv, dim=1)
-    s = torch.matmul(q, k.transpose(-2, -1)) * scale
+    s = torch.matmul(q, k.transpose(-2, -1))
+    if q2 is not None:
+        k2 = k2.float()
+        if k2.shape[1] != Hq:
+            k2 = k2.repeat_interleave(Hq // k2.shape[1], dim=1)
+        s = s + torch.matmul(q2.float(), k2.transpose(-2, -1))
+    s = s * scale
     if softcap is not None:
         s = torch.tanh(s / softcap) * softcap
     if score_bias is not None:

@@ -194,6 +194,29 @@ def test_prefix_attention_two_fused_calls():
     assert (got - want).abs().max() <= 2 * TOL      # two bf16 results added in bf16
 
 
+@pytest.mark.parametrize("shared_rope", [False, True])
+def test_mla_two_part_scores(shared_rope):
+    # reference tests/test_attention.py:126-151 (D_pe = D / 8); the second variant shares the
+    # positional key across heads, as latent-attention models do
+    def fn(Q_nope, Q_pe, K_nope, K_pe, V):
+        qk_nope = Q_nope @ K_nope.transpose(-2, -1)
+        qk_pe = Q_pe @ K_pe.expand(-1, Q_pe.shape[1], -1, -1).transpose(-2, -1)
+        qk = qk_nope + qk_pe
+        qk *= (Q_nope.shape[-1] + Q_pe.shape[-1]) ** (-0.5)
+        return torch.softmax(torch.ops.loopfuse.causal_mask(qk), dim=-1) @ V
+
+    B, H, S, D = 2, 8, 1024, 128
+    Dp = D // 8
+    Qn, Kn, V = (rand((B, H, S, D), seed=s) for s in (1, 2, 3))
+    Qp, Kp = rand((B, H, S, Dp), seed=4), rand((B, 1 if shared_rope else H, S, Dp), seed=5)
+    torch._dynamo.mark_static(Qn, 3)
+    torch._dynamo.mark_static(Qp, 3)
+    torch._dynamo.mark_dynamic(Qn, 2)
+    got = run_fused(fn, (Qn, Qp, Kn, Kp, V))
+    want = O.attention_reference(Qn, Kn, V, mask="causal", scale=(D + Dp) ** -0.5, q2=Qp, k2=Kp)
+    assert (got - want).abs().max() <= TOL
+
+
 def test_attention_inside_a_transformer_block():
     # the attention is found inside projections and a residual; everything else runs as it is
     def fn(x, wq, wk, wv, wo):

@@ -210,7 +210,8 @@ def _oracle_run(self, vals):
     out = O.attention_reference(q, k, v, mask=plan.mask, window=plan.window, scale=plan.scale, softcap=plan.softcap,
                                 k_table=kt, v_table=vt, denom_add=plan.denom_add,
                                 score_bias=self._bias_view(self.bias, vals, (B, Hq, Sq, Sk)),
-                                out_bias=self._bias_view(self.out_bias, vals, (B, Hq, Sq, D))).to(q.dtype)
+                                out_bias=self._bias_view(self.out_bias, vals, (B, Hq, Sq, D)),
+                                **self._second_product(vals)).to(q.dtype)
     return out.reshape(self.out_shape(vals))
 
 
@@ -238,7 +239,8 @@ def test_capture_explicit_softmax_with_shifted_denominator():
     assert plan.denom_add == 1.0 and plan.scale == pytest.approx(64 ** -0.5, rel=1e-6)   # 1/ln2 and ln2 cancel
 
 
-@pytest.mark.parametrize("which", ["two_outputs", "prefix", "inside_block", "modified", "softmax1", "softmax_e"])
+@pytest.mark.parametrize("which", ["two_outputs", "prefix", "inside_block", "modified", "softmax1", "softmax_e",
+                                   "mla", "mla_shared_rope", "double_k"])
 def test_rewritten_graphs_compute_the_same(which, monkeypatch):
     """Sub-graph fusion: the attention(s) inside a larger graph are replaced by fused
     calls and the rest keeps running.  Here the fused call is the oracle (no GPU), so
@@ -269,6 +271,29 @@ def test_rewritten_graphs_compute_the_same(which, monkeypatch):
             a = torch.softmax(torch.ops.loopfuse.causal_mask(q @ k.transpose(-2, -1) * 0.125), dim=-1) @ v
             return a.transpose(1, 2).reshape(B, S, E) @ wo + x
         ins = (f32(2, 24, 256),) + tuple(f32(256, 256, seed=s) * 0.06 for s in (1, 2, 3, 4))
+        n_attn = 1
+    elif which in ("mla", "mla_shared_rope"):
+        # two-part scores (reference tests/test_attention.py:126-151); the second variant
+        # writes the small product first and shares its key across heads
+        shared = which == "mla_shared_rope"
+
+        def fn(Q_nope, Q_pe, K_nope, K_pe, V):
+            if shared:
+                qk = Q_pe @ K_pe.expand(-1, Q_pe.shape[1], -1, -1).transpose(-2, -1) + Q_nope @ K_nope.transpose(-2, -1)
+            else:
+                qk = Q_nope @ K_nope.transpose(-2, -1) + Q_pe @ K_pe.transpose(-2, -1)
+            qk = qk * (Q_nope.shape[-1] + Q_pe.shape[-1]) ** (-0.5)
+            return torch.softmax(torch.ops.loopfuse.causal_mask(qk), dim=-1) @ V
+        ins = (f32(2, 3, 40, 64), f32(2, 3, 40, 16, seed=1), f32(2, 3, 40, 64, seed=2),
+               f32(2, 1 if shared else 3, 40, 16, seed=3), f32(2, 3, 40, 64, seed=4))
+        n_attn = 1
+    elif which == "double_k":
+        # reference tests/test_attention.py:441-462 with its commented-out tail restored
+        def fn(Q, K, K2, V):
+            QK1 = Q[..., :64] @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+            QK2 = Q[..., 64:] @ K2.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+            return torch.softmax(torch.ops.loopfuse.causal_mask(QK1 + QK2), dim=-1) @ V
+        ins = (f32(2, 3, 24, 96), f32(2, 3, 24, 64, seed=1), f32(2, 3, 24, 32, seed=2), f32(2, 3, 24, 64, seed=3))
         n_attn = 1
     elif which in ("softmax1", "softmax_e"):
         base2, c = (True, 1.0) if which == "softmax1" else (False, 0.25)

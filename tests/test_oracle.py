@@ -96,6 +96,41 @@ def test_denominator_offset():
     assert torch.allclose(got, plain * l / (l + 1.0), atol=1e-6)
 
 
+def test_two_part_scores():
+    """(Q K^T + Q2 K2^T) * scale: float64 loops, the concatenation identity, shared K2 heads."""
+    g = torch.Generator().manual_seed(17)
+    B, H, S, D, D2 = 2, 4, 6, 4, 3
+    q, k, v = (torch.randn(B, H, S, D, generator=g) for _ in range(3))
+    q2 = torch.randn(B, H, S, D2, generator=g)
+    k2 = torch.randn(B, 2, S, D2, generator=g)          # one K2 head per two query heads
+    scale = (D + D2) ** -0.5
+    got = O.attention_reference(q, k, v, mask="causal", scale=scale, q2=q2, k2=k2)
+    want = [[[[0.0] * D for _ in range(S)] for _ in range(H)] for _ in range(B)]
+    for b in range(B):
+        for h in range(H):
+            for i in range(S):
+                sc = [(sum(float(q[b, h, i, d]) * float(k[b, h, j, d]) for d in range(D))
+                       + sum(float(q2[b, h, i, d]) * float(k2[b, h // 2, j, d]) for d in range(D2))) * scale
+                      for j in range(i + 1)]
+                mx = max(sc)
+                w = [math.exp(x - mx) for x in sc]
+                for d in range(D):
+                    want[b][h][i][d] = sum(w[j] * float(v[b, h, j, d]) for j in range(i + 1)) / sum(w)
+    assert torch.allclose(got.double(), torch.tensor(want, dtype=torch.float64), atol=2e-6, rtol=1e-5)
+    # [Q | Q2] [K | K2]^T = Q K^T + Q2 K2^T: one product over the concatenated depth
+    k2r = k2.repeat_interleave(2, dim=1)
+    s_cat = torch.cat([q, q2], -1) @ torch.cat([k, k2r], -1).transpose(-2, -1) * scale
+    p = torch.softmax(s_cat.masked_fill(~O.dense_mask("causal", S, S), float("-inf")), -1)
+    assert torch.allclose(got, p @ v, atol=1e-6)
+    # a zero second part changes nothing; swapping the two parts' roles in the scores neither
+    assert torch.equal(O.attention_reference(q, k, v, mask="causal", scale=scale, q2=torch.zeros_like(q2), k2=k2),
+                       O.attention_reference(q, k, v, mask="causal", scale=scale))
+    vv = torch.randn(B, H, S, D2, generator=g)
+    a = O.attention_reference(q, k, vv, scale=scale, q2=q2, k2=k2r)
+    b_ = O.attention_reference(q2, k2r, vv, scale=scale, q2=q, k2=k)
+    assert torch.allclose(a, b_, atol=1e-6)
+
+
 def test_bias_closed_forms():
     g = torch.Generator().manual_seed(12)
     q, k, v = (torch.randn(1, 2, 6, 8, generator=g) for _ in range(3))

@@ -25,20 +25,20 @@ def rand(shape, dtype, seed):
 
 
 def check(q, k, v, *, mask=None, window=0, softcap=None, k_table=None, v_table=None, scale=None,
-          score_bias=None, out_bias=None, denom_add=0.0, **kw):
+          score_bias=None, out_bias=None, denom_add=0.0, q2=None, k2=None, **kw):
     dtype = q.dtype
     scale = q.shape[-1] ** -0.5 if scale is None else scale
     plan = lowering.AttnPlan(mask=mask, window=window, scale=scale, softcap=softcap,
                              k_paged=k_table is not None, v_paged=v_table is not None, denom_add=denom_add)
     mv = lambda t: None if t is None else t.to(dev())
     got = lowering.attention(mv(q), mv(k), mv(v), plan, mv(k_table), mv(v_table),
-                             score_bias=mv(score_bias), out_bias=mv(out_bias), **kw)
+                             score_bias=mv(score_bias), out_bias=mv(out_bias), q2=mv(q2), k2=mv(k2), **kw)
     if isinstance(got, tuple):
         got = got[0]
     torch.cuda.synchronize()
     want = O.attention_reference(q, k, v, mask=mask, window=window, softcap=softcap, scale=scale,
                                  k_table=k_table, v_table=v_table, score_bias=score_bias, out_bias=out_bias,
-                                 denom_add=denom_add)
+                                 denom_add=denom_add, q2=q2, k2=k2)
     got = got.float().cpu()
     assert torch.isfinite(got).all()
     if out_bias is not None:
@@ -203,6 +203,63 @@ def test_shifted_denominator_single_row_and_gqa_paged():
     table = torch.randperm(n, generator=torch.Generator().manual_seed(9)).view(B, S // P).to(torch.int32)
     check(rand((B, Hq, 1, D), torch.bfloat16, 3), kp, vp, k_table=table, v_table=table, denom_add=1.0)
     check(rand((B, Hq, S, D), torch.bfloat16, 3), kp, vp, mask="causal", k_table=table, v_table=table, denom_add=1.0)
+
+
+# ---------------------------------------------------------------- two-part scores
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("D,D2,S", [(128, 16, 593), (128, 64, 300), (64, 32, 129), (64, 16, 1024)])
+def test_two_part_scores(dtype, D, D2, S):
+    # scores (Q K^T + Q2 K2^T) (D + D2)^-0.5, reference tests/test_attention.py:126-151
+    q, k, v = (rand((2, 4, S, D), dtype, s) for s in (1, 2, 3))
+    q2, k2 = rand((2, 4, S, D2), dtype, 4), rand((2, 4, S, D2), dtype, 5)
+    check(q, k, v, mask="causal", scale=(D + D2) ** -0.5, q2=q2, k2=k2)
+    # the second part alone decides: zero Q makes the first product vanish
+    check(torch.zeros_like(q), k, v, mask="causal", scale=D2 ** -0.5, q2=q2, k2=k2)
+
+
+def test_two_part_scores_shared_key_gqa_window_softcap_bias():
+    B, Hq, Hkv, S, D, D2 = 2, 8, 2, 700, 128, 64
+    q, k, v = rand((B, Hq, S, D), torch.bfloat16, 1), rand((B, Hkv, S, D), torch.bfloat16, 2), rand((B, Hkv, S, D), torch.bfloat16, 3)
+    q2 = rand((B, Hq, S, D2), torch.bfloat16, 4)
+    k2 = rand((B, 1, S, D2), torch.bfloat16, 5)             # one positional key shared by all heads
+    sc = (D + D2) ** -0.5
+    check(q, k, v, mask="sliding", window=200, softcap=20.0, scale=sc, q2=q2, k2=k2)
+    check(q, k, v, scale=sc, q2=q2, k2=k2)                  # unmasked
+    check(q, k, v, mask="causal", scale=sc, q2=q2, k2=k2, score_bias=rand((B, Hq, S, S), torch.bfloat16, 6),
+          denom_add=1.0)
+    # strided operands: Q2 / K2 as slices of wider tensors
+    wide_q, wide_k = rand((B, Hq, S, D + D2), torch.bfloat16, 7), rand((B, Hkv, S, D + D2), torch.bfloat16, 8)
+    got = lowering.attention(wide_q.to(dev())[..., :D], wide_k.to(dev())[..., :D], v.to(dev()),
+                             lowering.AttnPlan(mask="causal", scale=sc),
+                             q2=wide_q.to(dev())[..., D:], k2=wide_k.to(dev())[..., D:])
+    want = O.attention_reference(wide_q[..., :D], wide_k[..., :D], v, mask="causal", scale=sc,
+                                 q2=wide_q[..., D:], k2=wide_k[..., D:])
+    assert (got.float().cpu() - want).abs().max().item() <= TOL[torch.bfloat16]
+
+
+def test_two_part_scores_few_rows_and_paged_kv():
+    B, Hq, Hkv, S, D, D2, P = 2, 4, 4, 256, 128, 64, 16
+    n = B * S // P
+    kp, vp = rand((n, P, Hkv, D), torch.bfloat16, 1), rand((n, P, Hkv, D), torch.bfloat16, 2)
+    table = torch.randperm(n, generator=torch.Generator().manual_seed(9)).view(B, S // P).to(torch.int32)
+    k2 = rand((B, Hkv, S, D2), torch.bfloat16, 5)
+    sc = (D + D2) ** -0.5
+    check(rand((B, Hq, S, D), torch.bfloat16, 3), kp, vp, mask="causal", k_table=table, v_table=table, scale=sc,
+          q2=rand((B, Hq, S, D2), torch.bfloat16, 4), k2=k2)
+    # a single query row without mask (decode shape) takes the same kernel
+    k, v = rand((B, Hkv, S, D), torch.bfloat16, 6), rand((B, Hkv, S, D), torch.bfloat16, 7)
+    check(rand((B, Hq, 1, D), torch.bfloat16, 3), k, v, scale=sc, q2=rand((B, Hq, 1, D2), torch.bfloat16, 4), k2=k2)
+
+
+def test_two_part_scores_rejects_what_it_cannot_serve():
+    q, k, v = (rand((1, 2, 64, 128), torch.bfloat16, s).to(dev()) for s in (1, 2, 3))
+    plan = lowering.AttnPlan(mask="causal", scale=0.1)
+    with pytest.raises(lowering.UnsupportedPlan):
+        lowering.attention(q, k, v, plan, q2=q[..., :24].contiguous(), k2=k[..., :24].contiguous())   # depth 24
+    with pytest.raises(lowering.UnsupportedPlan):
+        lowering.attention(q, k, v, plan, q2=q[..., :16].contiguous())                                 # no k2
+    with pytest.raises(lowering.UnsupportedPlan):
+        lowering.attention(q, k, v, plan, q2=q[..., :16].contiguous(), k2=k[:, :, :32, :16].contiguous())
 
 
 # ---------------------------------------------------------------- block skip

@@ -67,9 +67,11 @@ def test_launch_geometry_checks(shim_built):
 def test_params_struct_layout():
     from loopfuse_amd.lowering import AttnParams
 
-    # 11 pointers, 18 int64 strides, 11 ints, 3 floats (+4 bytes tail padding to the 8-byte alignment)
-    assert AttnParams.q.offset == 0 and AttnParams.q_sb.offset == 88
-    assert AttnParams.B.offset == 88 + 144
-    assert AttnParams.scale.offset == 88 + 144 + 44
-    assert AttnParams.denom_add.offset == 88 + 144 + 44 + 8
-    assert ctypes.sizeof(AttnParams) == 288
+    # 13 pointers, 24 int64 strides, 12 ints, 3 floats (+4 bytes tail padding to the 8-byte alignment)
+    assert AttnParams.q.offset == 0 and AttnParams.q2.offset == 88 and AttnParams.q_sb.offset == 104
+    assert AttnParams.q2_sb.offset == 104 + 144
+    assert AttnParams.B.offset == 104 + 192
+    assert AttnParams.k2_group.offset == 104 + 192 + 44
+    assert AttnParams.scale.offset == 104 + 192 + 48
+    assert AttnParams.denom_add.offset == 104 + 192 + 48 + 8
+    assert ctypes.sizeof(AttnParams) == 360
