@@ -240,7 +240,14 @@ class AttentionMatch:
         t = vals[op.index]
         if op.paged:
             return t, vals[op.table_index]
-        return t.permute(op.perm), None
+        t = t.permute(op.perm)
+        # the kernels read rows of D contiguous elements with 16-byte loads: a view that
+        # walks D with a stride (K given as [B, H, D, S], reference tests/test_attention.py:265-282)
+        # or sits on odd strides is copied once, O(S D) beside the O(S^2 D) attention
+        if t.is_cuda and (t.stride(-1) != 1 or t.data_ptr() % 16
+                          or any(n > 1 and st % 8 for n, st in zip(t.shape[:-1], t.stride()[:-1]))):
+            t = t.clone(memory_format=torch.contiguous_format)
+        return t, None
 
     def _bias_view(self, bo: Optional[BiasOperand], vals, shape):
         if bo is None:

@@ -217,6 +217,60 @@ def test_mla_two_part_scores(shared_rope):
     assert (got - want).abs().max() <= TOL
 
 
+def test_key_given_transposed():
+    # reference tests/test_attention.py:265-282: K arrives as [B, H, D, S] and the graph has no transpose
+    def fn(Q, K, V):
+        QK = Q @ K * (Q.shape[-1] ** -0.5)
+        return torch.softmax(torch.ops.loopfuse.causal_mask(QK), dim=-1) @ V
+
+    Q, V = rand((2, 4, 593, 128), seed=1), rand((2, 4, 593, 128), seed=3)
+    Kt = rand((2, 4, 128, 593), seed=2)
+    got = run_fused(fn, (Q, Kt, V))
+    assert (got - O.attention_reference(Q, Kt.transpose(-2, -1), V, mask="causal")).abs().max() <= TOL
+
+
+def test_operands_computed_in_the_graph():
+    # reference tests/test_attention.py:465-481: elementwise functions of Q, K, V feed the attention
+    def fn(Q, K, V):
+        QK = torch.sin(Q) @ torch.cos(K).transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        return torch.softmax(torch.ops.loopfuse.causal_mask(QK), dim=-1) @ torch.exp(V)
+
+    Q, K, V = (rand((2, 4, 320, 128), seed=s) for s in (1, 2, 3))
+    got = run_fused(fn, (Q, K, V))
+    sin, cos, ex = (f(t.float()).to(torch.bfloat16) for f, t in ((torch.sin, Q), (torch.cos, K), (torch.exp, V)))
+    assert (got - O.attention_reference(sin, cos, ex, mask="causal")).abs().max() <= 4 * TOL   # exp(V) reaches ~30
+
+
+def test_sliding_mask_with_one_query_row():
+    # reference tests/test_attention.py:365-381: top-left alignment leaves row 0 its first key only
+    def fn(Q, K, V):
+        QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        return torch.softmax(torch.ops.loopfuse.sliding_mask(QK, 256), dim=-1) @ V
+
+    Q = rand((2, 4, 1, 128), seed=1)
+    K, V = rand((2, 4, 512, 128), seed=2), rand((2, 4, 512, 128), seed=3)
+    torch._dynamo.mark_static(Q, 3)
+    got = run_fused(fn, (Q, K, V))
+    assert (got - O.attention_reference(Q, K, V, mask="sliding", window=256)).abs().max() <= TOL
+    assert (got - V[:, :, :1].float()).abs().max() <= TOL
+
+
+def test_gqa_decoding_with_repeat_interleave():
+    # reference tests/test_attention.py:172-189
+    def fn(Q, K, V):
+        g = Q.shape[1] // K.shape[1]
+        K = K.repeat_interleave(g, dim=1)
+        V = V.repeat_interleave(g, dim=1)
+        QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        return torch.softmax(QK, dim=-1) @ V
+
+    Q = rand((4, 32, 1, 128), seed=1)
+    K, V = rand((4, 4, 1024, 128), seed=2), rand((4, 4, 1024, 128), seed=3)
+    torch._dynamo.mark_static(Q, 3)
+    got = run_fused(fn, (Q, K, V))
+    assert (got - O.attention_reference(Q, K, V)).abs().max() <= TOL
+
+
 def test_attention_inside_a_transformer_block():
     # the attention is found inside projections and a residual; everything else runs as it is
     def fn(x, wq, wk, wv, wo):
