@@ -133,16 +133,15 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 8 / LF_DW) lf_attn_decode(co
   constexpr bool kPagedK = (LF_PAGED & 1) != 0;
   constexpr bool kPagedV = (LF_PAGED & 2) != 0;
   // pages of >= 16 tokens: a 16-token step lies inside one page, the id is wave-uniform
-  constexpr bool kUniformPage = (LF_PAGE_SIZE % 16) == 0;
+  constexpr bool kUniformPage = (!kPagedK || (LF_PAGE_SIZE % 16) == 0) && (!kPagedV || (LF_PAGE_SIZE_V % 16) == 0);
   auto step_tok0 = [&](int st) { return tok_begin + 16 * st; };
   auto fetch_ids = [&](int st) {
     LfDecIds id = {0, 0};
     if (kPagedK || kPagedV) {
       // clamp: steps past the end re-read the last page (their scores are masked)
       const int tok = min(step_tok0(st) + (kUniformPage ? 0 : c), p.Sk - 1);
-      const int pi = tok / LF_PAGE_SIZE;
-      if (kPagedK) id.k = reinterpret_cast<const lf_table_t*>(p.k_table)[(long long)b * p.kt_stride + pi];
-      if (kPagedV) id.v = reinterpret_cast<const lf_table_t*>(p.v_table)[(long long)b * p.vt_stride + pi];
+      if (kPagedK) id.k = reinterpret_cast<const lf_table_t*>(p.k_table)[(long long)b * p.kt_stride + tok / LF_PAGE_SIZE];
+      if (kPagedV) id.v = reinterpret_cast<const lf_table_t*>(p.v_table)[(long long)b * p.vt_stride + tok / LF_PAGE_SIZE_V];
     }
     return id;
   };
@@ -154,7 +153,7 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 8 / LF_DW) lf_attn_decode(co
     else
       kp = p.k + (long long)b * p.k_sb + (long long)hkv * p.k_sh + (long long)tok * p.k_ss + 8 * g;
     if (kPagedV)
-      vp = p.v + id.v * p.v_sb + (long long)(tok % LF_PAGE_SIZE) * p.v_ss + (long long)hkv * p.v_sh + 8 * g;
+      vp = p.v + id.v * p.v_sb + (long long)(tok % LF_PAGE_SIZE_V) * p.v_ss + (long long)hkv * p.v_sh + 8 * g;
     else
       vp = p.v + (long long)b * p.v_sb + (long long)hkv * p.v_sh + (long long)tok * p.v_ss + 8 * g;
 #pragma unroll

@@ -46,6 +46,9 @@
 #ifndef LF_PAGE_SIZE
 #define LF_PAGE_SIZE 16
 #endif
+#ifndef LF_PAGE_SIZE_V
+#define LF_PAGE_SIZE_V LF_PAGE_SIZE   /* tokens per page of the V pool (K and V pools may differ) */
+#endif
 #ifndef LF_TABLE_I64
 #define LF_TABLE_I64 0
 #endif
@@ -165,8 +168,9 @@ __device__ __forceinline__ const lf_elem* lf_kv_row(const LfAttnParams& p, int w
   const bool paged = which ? ((LF_PAGED & 2) != 0) : ((LF_PAGED & 1) != 0);
   if (paged) {
     const lf_table_t* table = reinterpret_cast<const lf_table_t*>(which ? p.v_table : p.k_table);
-    const long long page = table[(long long)b * (which ? p.vt_stride : p.kt_stride) + (tok / LF_PAGE_SIZE)];
-    return base + page * sb + (long long)(tok % LF_PAGE_SIZE) * ss + (long long)h * sh;
+    const int psz = which ? LF_PAGE_SIZE_V : LF_PAGE_SIZE;
+    const long long page = table[(long long)b * (which ? p.vt_stride : p.kt_stride) + (tok / psz)];
+    return base + page * sb + (long long)(tok % psz) * ss + (long long)h * sh;
   }
   return base + (long long)b * sb + (long long)h * sh + (long long)tok * ss;
 }

@@ -71,6 +71,7 @@ class KernelSpec:
     headwave: bool = False  # decode: one kv head per wave (8 waves) instead of 4 waves sharing a head
     denom: bool = False    # prefill: softmax denominator sum + c (c a run-time parameter)
     bias: int = 0          # prefill: bit 0 additive score bias tensor, bit 1 additive output bias tensor, bit 2 unaligned rows
+    page_size_v: int = 0   # tokens per page of the V pool when it differs from K's (0 = same)
     d2: int = 0            # prefill: depth of a second score product Q2 K2^T (0, 16, 32, 64)
     extra: tuple = ()      # further -D options (tuning experiments)
 
@@ -84,6 +85,8 @@ class KernelSpec:
             f"-DLF_PAGE_SIZE={self.page_size}",
             f"-DLF_TABLE_I64={int(self.table_i64)}",
         ]
+        if self.page_size_v:
+            o += [f"-DLF_PAGE_SIZE_V={self.page_size_v}"]
         if self.family == "decode":
             o += [f"-DLF_DW={self.waves}", f"-DLF_HEADWAVE={int(self.headwave)}"]
         elif self.family == "prefill":
@@ -103,7 +106,7 @@ class KernelSpec:
     def name(self) -> str:
         return (f"lf_{self.family}_t{self.dtype}_d{self.head_dim}_m{self.mask}_c{int(self.softcap)}"
                 f"_p{self.paged}x{self.page_size}i{int(self.table_i64)}_r{self.rows}w{self.waves}v{int(self.v_tr)}h{int(self.headwave)}b{self.bias}n{int(self.denom)}"
-                + (f"_q{self.d2}" if self.d2 else "")
+                + (f"_q{self.d2}" if self.d2 else "") + (f"_pv{self.page_size_v}" if self.page_size_v else "")
                 + "".join("_" + e.replace("-D", "").replace("=", "") for e in self.extra))
 
     def source(self) -> str:
@@ -389,11 +392,12 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
 
     P = AttnParams()
     paged = 0
-    page_size = 1
+    page_size = 1          # K pool (both pools when they agree)
+    page_size_v = 0        # V pool, when it differs from K's
     table_i64 = False
 
     def kv_layout(t: torch.Tensor, table: Optional[torch.Tensor], is_paged: bool, which: str):
-        nonlocal paged, page_size, table_i64
+        nonlocal paged, page_size, page_size_v, table_i64
         if not is_paged:
             if t.dim() != 4 or t.shape[0] != B or t.shape[3] != D:
                 raise UnsupportedPlan(f"{which} must be [B, Hkv, Sk, D]")
@@ -415,9 +419,13 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         if ps & (ps - 1):
             raise UnsupportedPlan("page size must be a power of two")
         i64 = table.dtype == torch.int64
-        if paged and (page_size != ps or table_i64 != i64):
-            raise UnsupportedPlan("K and V pools must share page size and table dtype")
-        page_size, table_i64 = ps, i64
+        if paged and table_i64 != i64:
+            raise UnsupportedPlan("K and V page tables must share their dtype")
+        if which == "V" and paged and ps != page_size:
+            page_size_v = ps               # pools with different page sizes
+        else:
+            page_size = ps
+        table_i64 = i64
         paged |= 1 if which == "K" else 2
         return hk, table.shape[1] * ps, sp, sh, st, table, table.stride(0)
 
@@ -529,7 +537,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
             extra += ("-DLF_DMA=1",)     # frees the staging registers the bias values / Q2 fragments need
         spec = KernelSpec(family, _DTYPE_CODE[dtype], D, mask, plan.softcap is not None, paged,
                           page_size, table_i64, v_tr=v_tr if family == "prefill" else True, bias=bias_bits,
-                          denom=plan.denom_add != 0.0, d2=d2, extra=extra)
+                          denom=plan.denom_add != 0.0, d2=d2, page_size_v=page_size_v, extra=extra)
         if os.environ.get("LOOPFUSE_TIMING"):       # profiling aid, see LF_TIMING in the kernel
             attention.timing = torch.zeros(16, dtype=torch.float32, device=q.device)
             P.part_acc = attention.timing.data_ptr()
@@ -577,7 +585,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     waves = int(os.environ.get("LOOPFUSE_DECODE_WAVES", "4"))
     # Token-major page pools ([pages, page, Hkv, D]: the heads of a token side by side)
     # are read whole-page-wise when the 8 waves of a workgroup take 8 consecutive heads.
-    headwave = _decode_headwave(paged, page_size, Hkv, D, P, B * ((Hkv + 7) // 8) * chunks, Sk)
+    headwave = _decode_headwave(paged, page_size, Hkv, D, P, B * ((Hkv + 7) // 8) * chunks, Sk) and not page_size_v
     if "head_per_wave" in choice:
         headwave = bool(choice["head_per_wave"]) and paged == 3 and Hkv % 8 == 0
     if headwave:
@@ -589,7 +597,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     nsplit = (Sk + split_len - 1) // split_len
     P.rows, P.nsplit, P.split_len = rows, nsplit, split_len
     spec = KernelSpec("decode", _DTYPE_CODE[dtype], D, MASK_NONE, plan.softcap is not None, paged,
-                      page_size, table_i64, rows=DECODE_QROWS, waves=waves, headwave=headwave,
+                      page_size, table_i64, rows=DECODE_QROWS, waves=waves, headwave=headwave, page_size_v=page_size_v,
                       extra=tuple(os.environ.get("LOOPFUSE_KOPTS", "").split()))
     if nsplit > 1:
         nrow = B * Hkv * rows * nsplit

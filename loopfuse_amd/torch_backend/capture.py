@@ -321,6 +321,14 @@ class AttentionMatch:
         if self.k.paged:
             ps = k.shape[1] if k.dim() == 4 else 1
             i64 = vals[self.k.table_index].dtype == torch.int64
+        psv = 0
+        if self.v.paged:
+            vp = vals[self.v.index]
+            pv = vp.shape[1] if vp.dim() == 4 else 1
+            if self.k.paged and pv != ps:
+                psv = pv
+            elif not self.k.paged:
+                ps, i64 = pv, vals[self.v.table_index].dtype == torch.int64
         mask = lowering._MASK_NAMES[plan.mask]
         bias = (1 if self.bias else 0) | (2 if self.out_bias else 0)
         d2 = self._operand(self.q2, vals)[0].shape[-1] if self.q2 is not None else 0
@@ -329,7 +337,7 @@ class AttentionMatch:
         family = "prefill" if (paged or bias or d2) else lowering.prefill_variant(q.shape[-2])
         extra = ("-DLF_DMA=1",) if ((bias or d2) and not paged) else ()
         return [lowering.KernelSpec(family, dt, D, mask, plan.softcap is not None, paged, ps, i64, bias=bias, d2=d2,
-                                    extra=extra)]
+                                    page_size_v=psv, extra=extra)]
 
 
 # ----------------------------------------------------------------------------
@@ -488,6 +496,30 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
             hints[s] = 8
     sizes = _stand_in_sizes(hints)
 
+    # Equalities the trace relies on without having solved them for one symbol (two page
+    # pools with pages_k * page_k == pages_v * page_v tokens): where the stand-ins break a
+    # matmul's contraction or batch dims, the symbols involved keep their traced values,
+    # which satisfy every such equality by construction.
+    def _expr(d):
+        return d.node.expr if isinstance(d, torch.SymInt) else sympy.Integer(int(d))
+
+    pairs = []
+    for n in graph.nodes:
+        if n.op == "call_function" and n.target in (aten.bmm.default, aten.mm.default, aten.matmul.default):
+            va, vb = (x.meta.get("val") if isinstance(x, torch.fx.Node) else None for x in n.args[:2])
+            if isinstance(va, torch.Tensor) and isinstance(vb, torch.Tensor) and va.dim() >= 2 and vb.dim() >= 2:
+                pairs.append((_expr(va.shape[-1]), _expr(vb.shape[-2])))
+                if va.dim() == vb.dim():
+                    pairs += [(_expr(x), _expr(y)) for x, y in zip(va.shape[:-2], vb.shape[:-2])
+                              if _expr(x) != 1 and _expr(y) != 1]          # 1 broadcasts
+    for _ in range(len(hints) + 1):
+        broken = [(x, y) for x, y in pairs if x.subs(sizes) != y.subs(sizes)]
+        if not broken:
+            break
+        for x, y in broken:
+            for sym in (x.free_symbols | y.free_symbols):
+                sizes[sym] = hints[sym]
+
     def concrete(d) -> int:
         if isinstance(d, torch.SymInt):
             return int(d.node.expr.subs(sizes))
@@ -601,9 +633,14 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
         if isinstance(first, Ids):
             if tgt in _VIEW_OPS:
                 try:
-                    return Ids(first.src, tgt(first.t, *a[1:], **kw))
+                    out = Ids(first.src, tgt(first.t, *a[1:], **kw))
                 except Exception as e:  # invalid for the stand-in sizes
                     raise _Skip(f"view chain not reproducible on stand-in sizes: {e}")
+                if first.src.kind == "node" and len(first.src.shape) != 4 and out.t.dim() == 4:
+                    # a projection output [B*S, E] viewed as [B, S, H, D]: operands are described
+                    # as permutations of a rank-4 tensor, so this view becomes the source
+                    raise _Skip("rank-4 view of a tensor of another rank: taken as a source of its own")
+                return out
             if tgt is torch.ops.loopfuse.paged_load.default:
                 pool, table = a[0], a[1]
                 if not (isinstance(table, Ids) and pool.src.kind == "node" and table.src.kind == "node"):

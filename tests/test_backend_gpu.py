@@ -229,6 +229,20 @@ def test_key_given_transposed():
     assert (got - O.attention_reference(Q, Kt.transpose(-2, -1), V, mask="causal")).abs().max() <= TOL
 
 
+def test_query_reshaped_from_merged_batch_and_heads():
+    # reference tests/test_attention.py:285-302 (marked broken there): Q arrives as [B*H, S, D]
+    def fn(Q, K, V):
+        Q = Q.reshape(*V.shape)
+        QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        return torch.softmax(torch.ops.loopfuse.causal_mask(QK), dim=-1) @ V
+
+    B, H, S, D = 2, 4, 384, 128
+    Q = rand((B * H, S, D), seed=1)
+    K, V = rand((B, H, S, D), seed=2), rand((B, H, S, D), seed=3)
+    got = run_fused(fn, (Q, K, V))
+    assert (got - O.attention_reference(Q.view(B, H, S, D), K, V, mask="causal")).abs().max() <= TOL
+
+
 def test_operands_computed_in_the_graph():
     # reference tests/test_attention.py:465-481: elementwise functions of Q, K, V feed the attention
     def fn(Q, K, V):
@@ -326,6 +340,27 @@ def test_paged_decode_page16_config5_shape():
     w = workloads.make("c5", seed=4, B=8, S=1024)
     got = run_fused(fn, (w.q, w.k, w.k_table, w.v, w.v_table))
     want = O.attention_reference(w.q, w.k, w.v, k_table=w.k_table, v_table=w.v_table)
+    assert (got - want).abs().max() <= TOL
+
+
+def test_paged_pools_with_different_page_sizes():
+    # K pool in pages of 16 tokens, V pool in pages of 4, each with its own table
+    def fn(Q, Kc, kt, Vc, vt):
+        B = kt.shape[0]
+        H, D = Kc.shape[2:]
+        K = torch.ops.loopfuse.paged_load(Kc, kt).reshape(B, -1, H, D).transpose(1, 2)
+        V = torch.ops.loopfuse.paged_load(Vc, vt).reshape(B, -1, H, D).transpose(1, 2)
+        QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        return torch.softmax(torch.ops.loopfuse.causal_mask(QK), dim=-1) @ V
+
+    B, H, S, D = 2, 4, 512, 128
+    g = torch.Generator().manual_seed(5)
+    Kc, Vc = rand((B * S // 16, 16, H, D), seed=1), rand((B * S // 4, 4, H, D), seed=2)
+    kt = torch.randperm(B * S // 16, generator=g).view(B, -1).to(torch.int32)
+    vt = torch.randperm(B * S // 4, generator=g).view(B, -1).to(torch.int32)
+    Q = rand((B, H, S, D), seed=3)
+    got = run_fused(fn, (Q, Kc, kt, Vc, vt))
+    want = O.attention_reference(Q, Kc, Vc, mask="causal", k_table=kt, v_table=vt)
     assert (got - want).abs().max() <= TOL
 
 

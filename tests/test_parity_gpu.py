@@ -359,6 +359,20 @@ def test_decode_paged_page16(dtype):
     check(w.q, w.k, w.v, k_table=w.k_table, v_table=w.v_table)
 
 
+@pytest.mark.parametrize("pk,pv", [(16, 64), (32, 16), (1, 16), (16, 4)])
+def test_mixed_page_sizes(pk, pv):
+    """K and V pools with different page sizes and their own tables (decode and prefill)."""
+    B, Hq, Hkv, S, D = 3, 8, 2, 320, 128
+    gen = torch.Generator().manual_seed(pk * 100 + pv)
+    nk, nv = B * S // pk, B * S // pv
+    kp = rand((nk, pk, Hkv, D), torch.bfloat16, 1) if pk > 1 else rand((nk, Hkv, D), torch.bfloat16, 1)
+    vp = rand((nv, pv, Hkv, D), torch.bfloat16, 2)
+    kt = torch.randperm(nk, generator=gen).view(B, S // pk).to(torch.int32)
+    vt = torch.randperm(nv, generator=gen).view(B, S // pv).to(torch.int32)
+    check(rand((B, Hq, 1, D), torch.bfloat16, 3), kp, vp, k_table=kt, v_table=vt)
+    check(rand((B, Hq, S, D), torch.bfloat16, 4), kp, vp, mask="causal", k_table=kt, v_table=vt)
+
+
 def test_decode_paged_identity_table_equals_contiguous(monkeypatch):
     w = workloads.make("c5", seed=2, B=2, S=256)
     n = w.k.shape[0]
