@@ -1,0 +1,64 @@
+/*
+ * lf_attn_params.h — the parameter block of the attention kernels, for C and C++
+ * hosts that launch them through lf_shim.h without Python.
+ *
+ * A kernel takes ONE argument, this struct by value; lf_launch receives
+ * `void* args[1] = { &params }`.  It is the device-side `struct LfAttnParams`
+ * (loopfuse_amd/csrc/kernels/lf_common.hip.h) restated with fixed-width host
+ * types, field for field; loopfuse_amd/lowering.py::AttnParams is the ctypes
+ * mirror.  It replaces the positional argument list of the reference's generated
+ * launch function — tensors, then one stride per dimension, then the dimensions
+ * (reference loopfuse/codegen.py:215-298, :241-242 for the strides).
+ *
+ * Strides are in ELEMENTS (bf16/fp16), the innermost dimension (head dim) has
+ * stride 1 everywhere.  Pointers are device pointers, 16-byte aligned.
+ */
+#ifndef LF_ATTN_PARAMS_H
+#define LF_ATTN_PARAMS_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct LfAttnParamsHost {
+  const void* q;        /* Q [B, Hq, Sq, D] */
+  const void* k;        /* K [B, Hkv, Sk, D], or the K page pool when the kernel is built with LF_PAGED & 1 */
+  const void* v;        /* V likewise (LF_PAGED & 2) */
+  void* o;              /* O [B, Hq, Sq, D] */
+  const void* k_table;  /* [B, pages] page ids, int32 or int64 (LF_TABLE_I64) */
+  const void* v_table;
+  float* part_acc;      /* decode split-K scratch: [units, nsplit, rows, D] floats */
+  float* part_ml;       /* decode split-K scratch: [units, nsplit, rows, 2] floats */
+  unsigned char* visits;/* optional [B*Hq*q_tiles, kv_tiles] visited-tile record, else NULL */
+  const void* bias;     /* LF_BIAS & 1: additive score bias [B, Hq, Sq, Sk] */
+  const void* obias;    /* LF_BIAS & 2: additive output bias [B, Hq, Sq, D] */
+  const void* q2;       /* LF_D2: second score product Q2 [B, Hq, Sq, D2] ... */
+  const void* k2;       /* ... K2 [B, Hq / k2_group, Sk, D2] */
+  int64_t q_sb, q_sh, q_ss;
+  int64_t k_sb, k_sh, k_ss;   /* paged: k_sb = page stride, k_ss = token stride inside a page */
+  int64_t v_sb, v_sh, v_ss;
+  int64_t o_sb, o_sh, o_ss;
+  int64_t bias_sb, bias_sh, bias_sq;   /* 0 = broadcast */
+  int64_t ob_sb, ob_sh, ob_sq;
+  int64_t q2_sb, q2_sh, q2_ss;
+  int64_t k2_sb, k2_sh, k2_ss;
+  int32_t B, Hq, Hkv, Sq, Sk;
+  int32_t window;             /* sliding-window width (LF_MASK == 2) */
+  int32_t kt_stride, vt_stride;
+  int32_t nsplit, rows, split_len;   /* decode */
+  int32_t k2_group;
+  float scale;                /* multiplies Q K^T */
+  float softcap;              /* LF_SOFTCAP: cap of cap * tanh(s / cap) */
+  float denom_add;            /* LF_DENOM: softmax denominator is sum + denom_add */
+} LfAttnParamsHost;
+
+#ifdef __cplusplus
+static_assert(sizeof(LfAttnParamsHost) == 360, "LfAttnParamsHost must match the device struct");
+}
+#else
+_Static_assert(sizeof(LfAttnParamsHost) == 360, "LfAttnParamsHost must match the device struct");
+#endif
+
+#endif /* LF_ATTN_PARAMS_H */

@@ -75,3 +75,35 @@ def test_params_struct_layout():
     assert AttnParams.scale.offset == 104 + 192 + 48
     assert AttnParams.denom_add.offset == 104 + 192 + 48 + 8
     assert ctypes.sizeof(AttnParams) == 360
+
+
+def test_c_header_matches_the_ctypes_mirror_and_the_device_struct(tmp_path):
+    """include/lf_attn_params.h (C hosts), lowering.AttnParams (ctypes) and struct
+    LfAttnParams (device) list the same fields at the same offsets."""
+    import subprocess
+
+    from loopfuse_amd.lowering import AttnParams
+
+    names = [n for n, _ in AttnParams._fields_]
+    prog = "#include <stdio.h>\n#include <stddef.h>\n#include \"lf_attn_params.h\"\nint main(void) {\n"
+    for n in names:
+        prog += f'  printf("{n} %zu\\n", offsetof(LfAttnParamsHost, {n}));\n'
+    prog += '  printf("sizeof %zu\\n", sizeof(LfAttnParamsHost));\n  return 0;\n}\n'
+    src = tmp_path / "off.c"
+    src.write_text(prog)
+    exe = tmp_path / "off"
+    subprocess.run(["gcc", "-std=c11", "-I" + os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    out = dict(line.split() for line in subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.splitlines())
+    for n in names:
+        assert int(out[n]) == getattr(AttnParams, n).offset, n
+    assert int(out["sizeof"]) == ctypes.sizeof(AttnParams)
+    # the device struct declares the same field names in the same order
+    dev = open(os.path.join(ROOT, "loopfuse_amd", "csrc", "kernels", "lf_common.hip.h")).read()
+    body = dev[dev.index("struct LfAttnParams {"):]
+    body = re.sub(r"//[^\n]*", "", body[:body.index("};")])
+    fields = []
+    for decl in body.split("{", 1)[1].split(";"):
+        decl = decl.strip()
+        if decl:
+            fields += [re.sub(r"[^A-Za-z0-9_]", "", x.split()[-1]) for x in decl.split(",")]
+    assert fields == names
