@@ -387,16 +387,36 @@ extern "C" __global__ void __launch_bounds__(256) lf_attn_decode_combine(const L
   const int bh = (int)(rowid / p.rows);
   const int hkv = bh % p.Hkv;
   const int b = bh / p.Hkv;
+  // four splits at a time: their eight loads are issued together (one memory round trip
+  // per group instead of one per split), then merged into the running (offset, sum, acc)
   float m = LF_NEG_INF;
-  for (int z = 0; z < p.nsplit; ++z) m = fmaxf(m, p.part_ml[(rowid * p.nsplit + z) * 2]);
-  const float m_sub = (m == LF_NEG_INF) ? 0.0f : m;
   float l = 0.0f;
   lf_f32x4 a = {0.0f, 0.0f, 0.0f, 0.0f};
-  for (int z = 0; z < p.nsplit; ++z) {
-    const long long slot = rowid * p.nsplit + z;
-    const float f = lf_exp2(p.part_ml[slot * 2] - m_sub);
-    l += p.part_ml[slot * 2 + 1] * f;
-    a += *reinterpret_cast<const lf_f32x4*>(&p.part_acc[slot * LF_HEAD_DIM + d0]) * f;
+  for (int z0 = 0; z0 < p.nsplit; z0 += 4) {
+    lf_f32x2 ml[4];
+    lf_f32x4 ac[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const long long slot = rowid * p.nsplit + min(z0 + u, p.nsplit - 1);
+      ml[u] = *reinterpret_cast<const lf_f32x2*>(&p.part_ml[slot * 2]);
+      ac[u] = *reinterpret_cast<const lf_f32x4*>(&p.part_acc[slot * LF_HEAD_DIM + d0]);
+    }
+    float mc = m;
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (z0 + u < p.nsplit) mc = fmaxf(mc, ml[u][0]);
+    const float m_sub = (mc == LF_NEG_INF) ? 0.0f : mc;
+    const float r = (m == LF_NEG_INF) ? 0.0f : lf_exp2(m - m_sub);   // nothing merged yet: l and a are 0
+    l *= r;
+    a *= r;
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (z0 + u < p.nsplit) {
+        const float f = lf_exp2(ml[u][0] - m_sub);
+        l += ml[u][1] * f;
+        a += ac[u] * f;
+      }
+    m = mc;
   }
   lf_elem* orow = p.o + (long long)b * p.o_sb + (long long)hkv * p.o_sh + (long long)qr * p.o_ss;
   const float inv = 1.0f / l;

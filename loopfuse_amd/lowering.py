@@ -440,10 +440,19 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     if mask == MASK_SLIDING and plan.window < 1:
         raise UnsupportedPlan("sliding mask needs window >= 1")
 
+    if Sk < 1:
+        # softmax over no keys is 0/0 in the eager graph: nothing a kernel should invent
+        raise UnsupportedPlan("attention over an empty key sequence")
     if out is None:
         out = torch.empty((B, Hq, Sq, D), dtype=dtype, device=q.device)
     else:
         _check_tensor("O", out, dtype)
+        if tuple(out.shape) != (B, Hq, Sq, D):
+            raise UnsupportedPlan(f"O must be [{B}, {Hq}, {Sq}, {D}]")
+    if B == 0 or Hq == 0 or Sq == 0:
+        # no query rows: the (empty) output is the whole result, nothing to launch
+        attention.last_launch = {"kernels": [], "grid": 0, "block": 0}
+        return (out, torch.zeros((0, 0), dtype=torch.uint8, device=q.device)) if record_visits else out
 
     P.q, P.k, P.v, P.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
     P.k_table = kt.data_ptr() if kt is not None else None

@@ -205,6 +205,21 @@ def test_shifted_denominator_single_row_and_gqa_paged():
     check(rand((B, Hq, S, D), torch.bfloat16, 3), kp, vp, mask="causal", k_table=table, v_table=table, denom_add=1.0)
 
 
+# ---------------------------------------------------------------- empty inputs
+def test_empty_inputs():
+    dt, d = torch.bfloat16, dev()
+    k, v = rand((2, 4, 64, 128), dt, 1).to(d), rand((2, 4, 64, 128), dt, 2).to(d)
+    plan = lowering.AttnPlan(mask="causal", scale=0.1)
+    # no query rows / no batch: an empty result and no launch
+    o = lowering.attention(torch.empty((2, 4, 0, 128), dtype=dt, device=d), k, v, plan)
+    assert o.shape == (2, 4, 0, 128) and lowering.attention.last_launch["kernels"] == []
+    e = torch.empty((0, 4, 64, 128), dtype=dt, device=d)
+    assert lowering.attention(e, e, e, plan).shape == (0, 4, 64, 128)
+    # no keys: softmax over nothing is undefined, the lowering refuses (torch.compile then runs the graph as it is)
+    with pytest.raises(lowering.UnsupportedPlan):
+        lowering.attention(rand((2, 4, 8, 128), dt, 3).to(d), k[:, :, :0], v[:, :, :0], lowering.AttnPlan(scale=0.1))
+
+
 # ---------------------------------------------------------------- two-part scores
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("D,D2,S", [(128, 16, 593), (128, 64, 300), (64, 32, 129), (64, 16, 1024)])
