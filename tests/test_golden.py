@@ -24,18 +24,23 @@ def load(path):
     case = dict(q=t(z["q"]), k=t(z["k"]), v=t(z["v"]), mask=MASKS[int(z["mask"])], window=int(z["window"]),
                 softcap=float(z["softcap"]) or None, expected=torch.from_numpy(z["expected"]),
                 table=torch.from_numpy(z["table"]) if "table" in z.files else None, dtype=dtype)
+    # optional inputs of the widened graphs
+    case["extra"] = {n: t(z[n]) for n in ("score_bias", "out_bias", "q2", "k2") if n in z.files}
+    case["denom_add"] = float(z["denom_add"]) if "denom_add" in z.files else 0.0
+    case["scale"] = float(z["scale"]) if "scale" in z.files else None
     return case
 
 
 def test_fixtures_exist():
-    assert len(FILES) >= 6
+    assert len(FILES) >= 9
 
 
 @pytest.mark.parametrize("path", FILES, ids=[os.path.basename(f)[:-4] for f in FILES])
 def test_oracle_reproduces_fixture(path):
     c = load(path)
     got = O.attention_reference(c["q"], c["k"], c["v"], mask=c["mask"], window=c["window"], softcap=c["softcap"],
-                                k_table=c["table"], v_table=c["table"])
+                                k_table=c["table"], v_table=c["table"], denom_add=c["denom_add"], scale=c["scale"],
+                                **c["extra"])
     assert torch.allclose(got, c["expected"], atol=1e-6, rtol=1e-6)
 
 
@@ -46,10 +51,15 @@ def test_kernel_reproduces_fixture(path):
 
     c = load(path)
     dev = torch.device("cuda:0")
-    plan = lowering.AttnPlan(mask=c["mask"], window=c["window"], scale=c["q"].shape[-1] ** -0.5, softcap=c["softcap"],
-                             k_paged=c["table"] is not None, v_paged=c["table"] is not None)
+    plan = lowering.AttnPlan(mask=c["mask"], window=c["window"], scale=c["scale"] or c["q"].shape[-1] ** -0.5,
+                             softcap=c["softcap"], k_paged=c["table"] is not None, v_paged=c["table"] is not None,
+                             denom_add=c["denom_add"])
     tab = None if c["table"] is None else c["table"].to(dev)
-    got = lowering.attention(c["q"].to(dev), c["k"].to(dev), c["v"].to(dev), plan, tab, tab)
+    got = lowering.attention(c["q"].to(dev), c["k"].to(dev), c["v"].to(dev), plan, tab, tab,
+                             **{n: t.to(dev) for n, t in c["extra"].items()})
     torch.cuda.synchronize()
     tol = 2e-2 if c["dtype"] == torch.bfloat16 else 5e-3
-    assert (got.float().cpu() - c["expected"]).abs().max().item() <= tol
+    err = (got.float().cpu() - c["expected"]).abs()
+    if "out_bias" in c["extra"]:     # the bias moves the result away from O(1): allow the storage format's half-ulp
+        err = err - (2.0 ** -8 if c["dtype"] == torch.bfloat16 else 2.0 ** -11) * c["expected"].abs()
+    assert err.max().item() <= tol
