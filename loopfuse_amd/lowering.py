@@ -219,7 +219,9 @@ _scratch: dict[tuple[int, int], torch.Tensor] = {}
 
 
 def _get_scratch(device: torch.device, nfloats: int) -> torch.Tensor:
-    key = (device.index or 0, 0)
+    """Split-K scratch, one buffer per (device, stream): launches on one stream are
+    ordered, so they can share it; launches on different streams must not."""
+    key = (device.index or 0, torch.cuda.current_stream(device).cuda_stream)
     t = _scratch.get(key)
     if t is None or t.numel() < nfloats:
         t = torch.empty(max(nfloats, 1 << 20), dtype=torch.float32, device=device)
@@ -308,6 +310,9 @@ def tuned_attention(q, k, v, plan: AttnPlan, k_table=None, v_table=None, **kw):
         return attention(q, k, v, plan, k_table, v_table, **kw)
     _load_tuned()
     key = _tune_key(q, k, plan, k_table, 0)
+    if key not in _tuned and q.is_cuda and torch.cuda.is_current_stream_capturing():
+        # timing needs a host synchronisation, which a stream capture forbids: fixed heuristics
+        return attention(q, k, v, plan, k_table, v_table, **kw)
     if key not in _tuned:
         B, Hq, Sq, D = q.shape
         Hkv = k.shape[-2] if plan.k_paged else k.shape[1]
