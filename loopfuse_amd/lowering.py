@@ -129,6 +129,16 @@ class CompiledKernel:
         return "// options: " + " ".join(self.spec.options()) + "\n" + self.spec.source()
 
 
+class CompiledKernels(list):
+    """What a ``CODEGEN_ONLY`` call returns: the ``CompiledKernel`` of every fused call in
+    the graph.  ``.code`` joins their sources, so the reference's usage
+    ``print(compiled_fn(Q, K, V).code)`` (``tests/test_attention.py:28-29``) works as is."""
+
+    @property
+    def code(self) -> str:
+        return "\n".join(k.code for k in self)
+
+
 _compiled: dict[KernelSpec, CompiledKernel] = {}
 _loaded: dict[tuple[KernelSpec, int], runtime.Module] = {}
 _lock = threading.Lock()

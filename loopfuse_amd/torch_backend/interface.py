@@ -148,12 +148,17 @@ def loopfuse_compiler(gm: torch.fx.GraphModule, sample_inputs, input_names: list
     if CODEGEN_ONLY:
         # no launch: hand back what would be compiled, as the reference hands back
         # KernelData under CODEGEN_ONLY (interface.py:615-622)
+        out_node = next(n for n in gm.graph.nodes if n.op == "output")
+        n_out = len(out_node.args[0]) if isinstance(out_node.args[0], (tuple, list)) else 1
+
         def codegen_fn(*args):
             global _codegen_sink
             _codegen_sink = []
             try:
                 fused_gm(*args)
-                return list(_codegen_sink)
+                # one object for the whole graph (its .code joins the kernels' sources), in
+                # the place of the first graph output; AOTAutograd hands it to the caller
+                return [lowering.CompiledKernels(_codegen_sink)] + [None] * (n_out - 1)
             finally:
                 _codegen_sink = None
 

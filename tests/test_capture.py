@@ -358,3 +358,27 @@ def test_cpu_tensors_fail_loudly_on_direct_call():
     q = torch.randn(1, 1, 16, 64).to(torch.bfloat16)
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         lowering.attention(q, q, q, lowering.AttnPlan(scale=0.125))
+
+
+def test_codegen_only_returns_kernel_objects_without_a_gpu(shim_built, monkeypatch):
+    """CODEGEN_ONLY=1 (reference interface.py:615-622, used as ``prg.code`` in
+    tests/test_attention.py:28-29): the compiled callable returns what would be launched."""
+    monkeypatch.setattr(interface, "CODEGEN_ONLY", True)
+
+    def fn(Q, K, V):
+        QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        return torch.softmax(torch.ops.loopfuse.causal_mask(QK), dim=-1) @ V
+
+    q, k, v = (bf(2, 4, 256, 128, seed=s) for s in range(3))
+    torch._dynamo.reset()
+    prg = torch.compile(fn, backend=loopfuse_amd.loopfuse_backend, dynamic=True)(q, k, v)
+    assert len(prg) == 1 and prg[0].code_object[:4] == b"\x7fELF"
+    assert "-DLF_MASK=1" in prg.code and "lf_attn_prefill" in prg.code and "-DLF_HEAD_DIM=128" in prg.code
+
+    def two(Q, Kp, Vp, Ks, Vs):      # two fused calls in one graph
+        a = torch.softmax(Q @ Kp.transpose(-2, -1) * 0.1, dim=-1) @ Vp
+        return a + torch.softmax(torch.ops.loopfuse.sliding_mask(Q @ Ks.transpose(-2, -1) * 0.1, 64), dim=-1) @ Vs
+
+    torch._dynamo.reset()
+    prg = torch.compile(two, backend=loopfuse_amd.loopfuse_backend, dynamic=True)(q, k, v, k, v)
+    assert len(prg) == 2 and "-DLF_MASK=0" in prg[0].code and "-DLF_MASK=2" in prg[1].code
