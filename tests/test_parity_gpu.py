@@ -470,6 +470,39 @@ def test_baseline_config_full_size(name, dtype):
         assert (o <= vmax + 1e-2).all() and (o >= vmin - 1e-2).all()
 
 
+@pytest.mark.parametrize("name", ["c2", "c3", "c5"])
+def test_full_size_linearity_and_scaling_in_v(name):
+    """Size-independent properties at the baseline sizes: the output is linear in V.
+    att(2 V) == 2 att(V) bit for bit (a power of two commutes with every rounding), and
+    att(V1) + att(V2) == att(V1 + V2) up to the bf16 rounding of the summed operand."""
+    w = workloads.make(name, seed=3).to(dev())
+    v1 = w.v
+    v2 = torch.randn(v1.shape, generator=torch.Generator().manual_seed(4)).to(torch.bfloat16).to(dev())
+    o1 = workloads.run(w).clone()
+    w.v = v1 * 2
+    assert torch.equal(workloads.run(w), o1 * 2)
+    w.v = v2
+    o2 = workloads.run(w).clone()
+    w.v = (v1.float() + v2.float()).to(torch.bfloat16)
+    o12 = workloads.run(w)
+    torch.cuda.synchronize()
+    want = o1.float() + o2.float()
+    # three bf16 roundings are involved (o1, o2, o12): allow an ulp of the result's magnitude
+    assert ((o12.float() - want).abs() - 2.0 ** -7 * want.abs()).max().item() <= 2e-2
+
+
+def test_full_size_causal_prefix_is_bit_equal():
+    """Causal attention over a prefix equals the first rows of causal attention over the
+    whole sequence, bit for bit: a q tile walks the same KV tiles either way."""
+    w = workloads.make("c2", seed=5).to(dev())
+    plan = lowering.AttnPlan(mask="causal", scale=w.scale)
+    whole = lowering.attention(w.q, w.k, w.v, plan)
+    for n in (1024, 593, 128):
+        part = lowering.attention(w.q[:, :, :n], w.k[:, :, :n], w.v[:, :, :n], plan)
+        torch.cuda.synchronize()
+        assert torch.equal(part, whole[:, :, :n]), n
+
+
 def test_c1_on_gpu_vs_cpu_eager():
     # config 1 (fp32, CPU-runnable): same tensors through the CPU eager graph and,
     # cast to bf16, through the GPU kernel
