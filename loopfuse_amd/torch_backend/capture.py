@@ -425,6 +425,55 @@ def _fit_bias(entry: tuple, logical: tuple):
     return src.node, tuple(dims)
 
 
+def _regroup(real_in, real_out, stand_in, stand_out_hint):
+    """Stand-in shape of a view/reshape: ``real_in -> real_out`` regroups contiguous dims;
+    the same regrouping is applied to ``stand_in``.  A target dim that merges source dims
+    is their stand-in product; where a source dim is split, the targets take
+    ``stand_out_hint`` (per target dim, may be None) and must multiply back to it.
+    Returns None when the stand-ins cannot follow the regrouping."""
+    out = []
+    i = j = 0
+    ni, nj = len(real_in), len(real_out)
+    while i < ni or j < nj:
+        gi, gj = [], []
+        pi = pj = 1
+        # smallest groups of source / target dims with equal products
+        while True:
+            if (pi == pj and gi and gj) or (i >= ni and j >= nj):
+                break
+            take_in = (pi < pj) or (pi == pj and not gi)
+            if (take_in and i < ni) or j >= nj:
+                pi *= real_in[i]
+                gi.append(i)
+                i += 1
+            else:
+                pj *= real_out[j]
+                gj.append(j)
+                j += 1
+        if pi != pj:
+            return None
+        prod_in = math.prod(stand_in[k] for k in gi)
+        if len(gj) == 1:
+            out.append(prod_in)
+            continue
+        if not gj:
+            if prod_in != 1:
+                return None
+            continue
+        vals = []
+        for k in gj:
+            if real_out[k] == 1:
+                vals.append(1)
+            elif stand_out_hint[k] is None:
+                return None
+            else:
+                vals.append(stand_out_hint[k])
+        if math.prod(vals) != prod_in:
+            return None
+        out.extend(vals)
+    return out
+
+
 def _same_scalar(x, y) -> bool:
     """Two score factors (numbers, graph nodes, ("recip", f)) that are the same value by
     construction: identical, or the same pure computation on the same inputs."""
@@ -496,6 +545,28 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
             hints[s] = 8
     sizes = _stand_in_sizes(hints)
 
+    # Static dims normally keep their values (a head dim of 128 marked static).  A graph
+    # traced with static shapes at real sizes would need id tensors of the real size: then
+    # the static dims of the inputs get stand-ins too (one per distinct value, chosen
+    # together with the symbols' so that small ratios such as Hq = g * Hkv survive), and the
+    # literal shapes in view / expand nodes are re-derived from the nodes' real shapes.
+    CAP = 1 << 22
+    real = lambda d: _hint(d) if isinstance(d, torch.SymInt) else int(d)
+    fmap: dict = {}
+
+    def _numel_as_is(val) -> int:
+        return math.prod(int(d.node.expr.subs(sizes)) if isinstance(d, torch.SymInt) else int(d) for d in val.shape)
+
+    if any(isinstance(p.meta.get("val"), torch.Tensor) and _numel_as_is(p.meta["val"]) > CAP for p in placeholders):
+        statics = sorted({int(d) for p in placeholders if isinstance(p.meta.get("val"), torch.Tensor)
+                          for d in p.meta["val"].shape if not isinstance(d, torch.SymInt) and int(d) > 4})
+        joint = dict(hints)
+        joint.update({("static", v): v for v in statics})
+        both = _stand_in_sizes(joint)
+        sizes = {k: v for k, v in both.items() if not isinstance(k, tuple)}
+        fmap = {k[1]: v for k, v in both.items() if isinstance(k, tuple)}
+    shrink_static = bool(fmap)
+
     # Equalities the trace relies on without having solved them for one symbol (two page
     # pools with pages_k * page_k == pages_v * page_v tokens): where the stand-ins break a
     # matmul's contraction or batch dims, the symbols involved keep their traced values,
@@ -523,7 +594,30 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
     def concrete(d) -> int:
         if isinstance(d, torch.SymInt):
             return int(d.node.expr.subs(sizes))
-        return int(d)
+        d = int(d)
+        if d in fmap:
+            return fmap[d]
+        if shrink_static and d > 4:
+            # a literal product of two input dims (batch * heads, tokens * width)
+            for a_, fa in fmap.items():
+                if d % a_ == 0 and (d // a_) in fmap:
+                    return fa * fmap[d // a_]
+        return d
+
+    def stand_in_view_shape(node, in_shape):
+        """Target shape of a view / reshape / expand node for an input of stand-in shape
+        ``in_shape``, derived from the node's real shapes instead of its literal arguments."""
+        src = node.args[0]
+        rin = [real(d) for d in src.meta["val"].shape]
+        rout = [real(d) for d in node.meta["val"].shape]
+        hint = [concrete(d) for d in node.meta["val"].shape]
+        if node.target is aten.expand.default:
+            pad = len(rout) - len(rin)
+            return [in_shape[j - pad] if j >= pad and rin[j - pad] == rout[j] else hint[j] for j in range(len(rout))]
+        got = _regroup(rin, rout, list(in_shape), hint)
+        if got is None:
+            raise _Skip("view not reproducible on stand-in sizes")
+        return got
 
     def fresh_ids(node: torch.fx.Node, val) -> Any:
         """A tensor-valued node that simply runs: ids over its own (stand-in) shape."""
@@ -531,7 +625,7 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
             return Scalar(node, 1.0)       # e.g. a Python float that dynamo passes as a 0-dim tensor
         shape = tuple(concrete(d) for d in val.shape)
         n = math.prod(shape)
-        if n > (1 << 22):
+        if n > CAP:
             raise NoMatch("stand-in tensor too large")
         return Ids(Source("node", node, shape=shape), torch.arange(n, dtype=torch.int64).reshape(shape))
 
@@ -632,6 +726,9 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
         # -- views of tensors
         if isinstance(first, Ids):
             if tgt in _VIEW_OPS:
+                if shrink_static and tgt in (aten.view.default, aten._unsafe_view.default, aten.reshape.default,
+                                             aten.expand.default):
+                    a = (a[0], stand_in_view_shape(node, first.t.shape)) + tuple(a[2:])
                 try:
                     out = Ids(first.src, tgt(first.t, *a[1:], **kw))
                 except Exception as e:  # invalid for the stand-in sizes
@@ -667,6 +764,9 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
             st = first
             if tgt in _SHAPE_ONLY_VIEW_OPS:
                 kw2 = {k: v for k, v in kw.items() if k != "memory_format"}
+                if shrink_static and tgt in (aten.view.default, aten._unsafe_view.default, aten.reshape.default,
+                                             aten.expand.default):
+                    a = (a[0], stand_in_view_shape(node, st.shape)) + tuple(a[2:])
                 try:
                     new_shape = meta_view(tgt, st.shape, a[1:], kw2)
                 except Exception as e:

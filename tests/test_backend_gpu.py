@@ -364,6 +364,42 @@ def test_paged_pools_with_different_page_sizes():
     assert (got - want).abs().max() <= TOL
 
 
+def test_static_shapes_at_baseline_sizes():
+    """torch.compile WITHOUT dynamic=True (static shapes) on configs 2 and 5 at full size."""
+    from loopfuse_amd import workloads
+
+    def prefill(Q, K, V):
+        QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        return torch.softmax(torch.ops.loopfuse.causal_mask(QK), dim=-1) @ V
+
+    def decode(Q, Kc, kt, Vc, vt):
+        B, pages = kt.shape
+        P, H, D = Kc.shape[1:]
+        K = torch.ops.loopfuse.paged_load(Kc, kt).reshape(B, pages * P, H, D).transpose(1, 2)
+        V = torch.ops.loopfuse.paged_load(Vc, vt).reshape(B, pages * P, H, D).transpose(1, 2)
+        g = Q.shape[1] // H
+        K = K.repeat_interleave(g, dim=1)
+        V = V.repeat_interleave(g, dim=1)
+        return torch.softmax(Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5), dim=-1) @ V
+
+    for fn, w in ((prefill, workloads.make("c2", seed=1)), (decode, workloads.make("c5", seed=1))):
+        ins = (w.q, w.k, w.v) if w.k_table is None else (w.q, w.k, w.k_table, w.v, w.v_table)
+        torch._dynamo.reset()
+        before = dict(interface.stats)
+        got = torch.compile(fn, backend=loopfuse_backend)(*[t.to(DEV) for t in ins]).float().cpu()
+        torch.cuda.synchronize()
+        assert interface.stats["fused"] == before["fused"] + 1, "the static graph was not fused"
+        b, h = 3, 17                                   # one (batch, head) against the oracle
+        hk = h // (w.q.shape[1] // (w.k.shape[-2] if w.k_table is not None else w.k.shape[1]))
+        if w.k_table is None:
+            want = O.attention_reference(w.q[b:b + 1, h:h + 1], w.k[b:b + 1, hk:hk + 1], w.v[b:b + 1, hk:hk + 1], mask="causal")
+        else:
+            kk = O.gather_paged(w.k, w.k_table[b:b + 1])[:, hk:hk + 1]
+            vv = O.gather_paged(w.v, w.v_table[b:b + 1])[:, hk:hk + 1]
+            want = O.attention_reference(w.q[b:b + 1, h:h + 1], kk, vv)
+        assert (got[b:b + 1, h:h + 1] - want).abs().max() <= TOL
+
+
 def test_decode_contiguous():
     def fn(Q, K, V):
         QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)

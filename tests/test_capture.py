@@ -382,3 +382,55 @@ def test_codegen_only_returns_kernel_objects_without_a_gpu(shim_built, monkeypat
     torch._dynamo.reset()
     prg = torch.compile(two, backend=loopfuse_amd.loopfuse_backend, dynamic=True)(q, k, v, k, v)
     assert len(prg) == 2 and "-DLF_MASK=0" in prg[0].code and "-DLF_MASK=2" in prg[1].code
+
+
+@pytest.mark.parametrize("which", ["causal", "gqa_window_softcap", "paged_decode", "block"])
+def test_static_shapes_at_real_sizes_are_matched(which, monkeypatch):
+    """torch.compile without dynamic=True traces static shapes: the literal sizes in the
+    graph are then the real ones, too large for id tensors, and the front end has to shrink
+    static dims and re-derive the literal view shapes.  The fused call is the oracle here."""
+    monkeypatch.setattr(capture.AttentionMatch, "run", _oracle_run)
+    r = lambda *shape, seed=0: torch.randn(*shape, generator=torch.Generator().manual_seed(seed)).to(torch.bfloat16)
+    if which == "causal":
+        def fn(Q, K, V):
+            QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+            return torch.softmax(torch.ops.loopfuse.causal_mask(QK), dim=-1) @ V
+        ins = (r(4, 8, 1024, 128), r(4, 8, 1024, 128, seed=1), r(4, 8, 1024, 128, seed=2))
+    elif which == "gqa_window_softcap":
+        def fn(Q, K, V):
+            g = Q.shape[1] // K.shape[1]
+            K = K.repeat_interleave(g, dim=1)
+            V = V.repeat_interleave(g, dim=1)
+            QK = torch.tanh(Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5) / 30) * 30
+            return torch.softmax(torch.ops.loopfuse.sliding_mask(QK, 100), dim=-1) @ V
+        ins = (r(2, 16, 1024, 128), r(2, 4, 1024, 128, seed=1), r(2, 4, 1024, 128, seed=2))
+    elif which == "paged_decode":
+        def fn(Q, Kc, kt, Vc, vt):
+            B, pages = kt.shape
+            P, H, D = Kc.shape[1:]
+            K = torch.ops.loopfuse.paged_load(Kc, kt).reshape(B, pages * P, H, D).transpose(1, 2)
+            V = torch.ops.loopfuse.paged_load(Vc, vt).reshape(B, pages * P, H, D).transpose(1, 2)
+            g = Q.shape[1] // H
+            K = K.repeat_interleave(g, dim=1)
+            V = V.repeat_interleave(g, dim=1)
+            return torch.softmax(Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5), dim=-1) @ V
+        n = 16 * 64
+        gen = torch.Generator().manual_seed(3)
+        ins = (r(16, 32, 1, 128), r(n, 16, 8, 128, seed=1), torch.randperm(n, generator=gen).view(16, 64).int(),
+               r(n, 16, 8, 128, seed=2), torch.randperm(n, generator=gen).view(16, 64).int())
+    else:
+        def fn(x, wq, wk, wv, wo):
+            B, S, E = x.shape
+            H = 8
+            q = (x @ wq).view(B, S, H, E // H).transpose(1, 2)
+            k = (x @ wk).view(B, S, H, E // H).transpose(1, 2)
+            v = (x @ wv).view(B, S, H, E // H).transpose(1, 2)
+            a = torch.softmax(torch.ops.loopfuse.causal_mask(q @ k.transpose(-2, -1) * 0.125), dim=-1) @ v
+            return a.transpose(1, 2).reshape(B, S, E) @ wo + x
+        ins = (r(8, 1024, 1024),) + tuple((r(1024, 1024, seed=s).float() * 0.03).to(torch.bfloat16) for s in (1, 2, 3, 4))
+    torch._dynamo.reset()
+    before = dict(interface.stats)
+    got = torch.compile(fn, backend=loopfuse_amd.loopfuse_backend)(*ins)        # static shapes
+    assert interface.stats["fused"] == before["fused"] + 1, "static graph at real size was not matched"
+    want = fn(*ins)
+    assert (got.float() - want.float()).abs().max().item() <= 6e-2
