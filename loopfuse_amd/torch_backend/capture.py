@@ -96,6 +96,11 @@ class Stage:
     sm: str = ""                       # "" | "minus_run" (x - running max) | "exp_run" | "num" (b^(x - max))
     base2: bool = False                # the exponentials are exp2
     denom_add: tuple = ()              # probabilities = num / (sum num + these terms)
+    # scores / probabilities that currently sit in a permuted or regrouped layout (einsum lowers
+    # to view -> permute -> view chains): ids of the canonical [batch..., Sq, Sk] elements in the
+    # current shape; None while the value is a plain reshape of the canonical layout
+    lay: Any = None
+    mat: tuple = ()                    # (Sq, Sk) stand-ins
 
 
 @dataclasses.dataclass
@@ -240,6 +245,8 @@ class AttentionMatch:
         t = vals[op.index]
         if op.paged:
             return t, vals[op.table_index]
+        if t.dim() == 3:
+            t = t.unsqueeze(0)         # [B*H, S, D] given without a batch dim
         t = t.permute(op.perm)
         # the kernels read rows of D contiguous elements with 16-byte loads: a view that
         # walks D with a stride (K given as [B, H, D, S], reference tests/test_attention.py:265-282)
@@ -356,6 +363,8 @@ def _fit_operand(x: torch.Tensor, src: Source, rows_are_d: bool) -> tuple[tuple[
         # [B, pages, P, Hkv, D]: tokens = (page, slot) merged
         merged = shape[2]
         shape = [shape[0], shape[1] * shape[2], shape[3], shape[4]]
+    if len(shape) == 3 and src.kind == "node":
+        shape = [1] + shape            # [B*H, S, D] inputs: one batch of B*H heads
     if len(shape) != 4:
         raise NoMatch(f"attention operand has rank {len(shape)} (need [B, H, S, D])")
     strides = [0] * 4
@@ -756,12 +765,31 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
                 if qi.t.shape[:-2] != ki.t.shape[:-2] or qi.t.shape[-1] != ki.t.shape[-2]:
                     raise _Skip("QK^T shapes disagree")
                 shape = tuple(qi.t.shape[:-1]) + (ki.t.shape[-1],)
-                return Stage("scores", shape, qi, ki)
+                return Stage("scores", shape, qi, ki, mat=(shape[-2], shape[-1]))
             raise _Skip(f"op on a tensor view: {tgt}")
 
         # -- the attention pipeline
         if isinstance(first, Stage):
             st = first
+            if tgt in _VIEW_OPS and st.kind in ("scores", "probs"):
+                # executed on ids of the canonical layout, like the views of operands
+                kw2 = {k: v for k, v in kw.items() if k != "memory_format"}
+                if shrink_static and tgt in (aten.view.default, aten._unsafe_view.default, aten.reshape.default,
+                                             aten.expand.default):
+                    a = (a[0], stand_in_view_shape(node, st.shape)) + tuple(a[2:])
+                n = math.prod(st.shape)
+                lay = st.lay if st.lay is not None else torch.arange(n, dtype=torch.int64).reshape(st.shape)
+                try:
+                    new = tgt(lay, *a[1:], **kw2)
+                except Exception as e:
+                    raise _Skip(f"view of the scores not reproducible: {e}")
+                if new.numel() != n:
+                    raise _Skip("view changes the number of scores")
+                plain = tuple(new.shape[-2:]) == tuple(st.mat) and torch.equal(new.reshape(-1), torch.arange(n))
+                return dataclasses.replace(st, shape=tuple(new.shape), lay=None if plain else new)
+            if st.lay is not None and not (tgt in _CAST_OPS or tgt is aten.tanh.default or (
+                    tgt in (aten.mul.Tensor, aten.div.Tensor) and not isinstance(a[1], (Stage, Ids, Aux)))):
+                raise _Skip("scores are used in a permuted layout")
             if tgt in _SHAPE_ONLY_VIEW_OPS:
                 kw2 = {k: v for k, v in kw.items() if k != "memory_format"}
                 if shrink_static and tgt in (aten.view.default, aten._unsafe_view.default, aten.reshape.default,
@@ -947,7 +975,8 @@ def _build_match(out_node: torch.fx.Node, st: Stage) -> AttentionMatch:
         q2_op = operand(st.q2, q2perm, q2g)
         k2_op = operand(st.kt2, k2perm, k2g)
 
-    qshape = tuple(st.q.src.shape[i] for i in qperm)       # stand-in [B, Hq, Sq, D]
+    q_src_shape = tuple(st.q.src.shape) if len(st.q.src.shape) == 4 else (1,) + tuple(st.q.src.shape)
+    qshape = tuple(q_src_shape[i] for i in qperm)          # stand-in [B, Hq, Sq, D]
     if len(st.shape) == 4:
         if tuple(st.shape) != qshape:
             raise NoMatch("output is not shaped [B, Hq, Sq, D]")

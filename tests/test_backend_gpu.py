@@ -243,6 +243,32 @@ def test_query_reshaped_from_merged_batch_and_heads():
     assert (got - O.attention_reference(Q.view(B, H, S, D), K, V, mask="causal")).abs().max() <= TOL
 
 
+@pytest.mark.parametrize("which", ["einsum", "rank3", "bshd"])
+@pytest.mark.parametrize("dynamic", [True, None])
+def test_other_spellings_of_attention(which, dynamic):
+    """einsum-written products, [B*H, S, D] inputs, [B, S, H, D] storage; dynamic and static tracing."""
+    def fn(Q, K, V):
+        if which == "einsum":
+            sc = torch.einsum("bhqd,bhkd->bhqk", Q, K) * (Q.shape[-1] ** -0.5)
+            return torch.einsum("bhqk,bhkd->bhqd", torch.softmax(torch.ops.loopfuse.causal_mask(sc), dim=-1), V)
+        if which == "bshd":
+            Q, K, V = (t.transpose(1, 2) for t in (Q, K, V))
+        o = torch.softmax(torch.ops.loopfuse.causal_mask(Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)), dim=-1) @ V
+        return o.transpose(1, 2) if which == "bshd" else o
+
+    B, H, S, D = 4, 8, 1100, 128
+    shape = {"einsum": (B, H, S, D), "rank3": (B * H, S, D), "bshd": (B, S, H, D)}[which]
+    Q, K, V = (rand(shape, seed=s) for s in (1, 2, 3))
+    torch._dynamo.reset()
+    before = dict(interface.stats)
+    got = torch.compile(fn, backend=loopfuse_backend, dynamic=dynamic)(*[t.to(DEV) for t in (Q, K, V)]).float().cpu()
+    torch.cuda.synchronize()
+    assert interface.stats["fused"] == before["fused"] + 1, "the fused HIP path was not taken"
+    to4 = {"einsum": lambda t: t, "rank3": lambda t: t.view(B, H, S, D), "bshd": lambda t: t.transpose(1, 2)}[which]
+    want = O.attention_reference(to4(Q), to4(K), to4(V), mask="causal")
+    assert (to4(got) - want).abs().max() <= TOL
+
+
 def test_operands_computed_in_the_graph():
     # reference tests/test_attention.py:465-481: elementwise functions of Q, K, V feed the attention
     def fn(Q, K, V):

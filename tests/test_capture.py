@@ -240,7 +240,7 @@ def test_capture_explicit_softmax_with_shifted_denominator():
 
 
 @pytest.mark.parametrize("which", ["two_outputs", "prefix", "inside_block", "modified", "softmax1", "softmax_e",
-                                   "mla", "mla_shared_rope", "double_k"])
+                                   "mla", "mla_shared_rope", "double_k", "einsum", "rank3", "bshd"])
 def test_rewritten_graphs_compute_the_same(which, monkeypatch):
     """Sub-graph fusion: the attention(s) inside a larger graph are replaced by fused
     calls and the rest keeps running.  Here the fused call is the oracle (no GPU), so
@@ -287,6 +287,19 @@ def test_rewritten_graphs_compute_the_same(which, monkeypatch):
         ins = (f32(2, 3, 40, 64), f32(2, 3, 40, 16, seed=1), f32(2, 3, 40, 64, seed=2),
                f32(2, 1 if shared else 3, 40, 16, seed=3), f32(2, 3, 40, 64, seed=4))
         n_attn = 1
+    elif which in ("einsum", "rank3", "bshd"):
+        # other spellings of the same attention: einsum (lowers to view -> permute -> view
+        # chains around both products), inputs without a batch dim, [B, S, H, D] storage
+        def fn(Q, K, V):
+            if which == "einsum":
+                sc = torch.einsum("bhqd,bhkd->bhqk", Q, K) * (Q.shape[-1] ** -0.5)
+                return torch.einsum("bhqk,bhkd->bhqd", torch.softmax(torch.ops.loopfuse.causal_mask(sc), dim=-1), V)
+            if which == "bshd":
+                Q, K, V = (t.transpose(1, 2) for t in (Q, K, V))
+            o = torch.softmax(torch.ops.loopfuse.causal_mask(Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)), dim=-1) @ V
+            return o.transpose(1, 2) if which == "bshd" else o
+        shape = {"einsum": (2, 3, 40, 64), "rank3": (6, 40, 64), "bshd": (2, 40, 3, 64)}[which]
+        ins, n_attn = (f32(*shape), f32(*shape, seed=1), f32(*shape, seed=2)), 1
     elif which == "double_k":
         # reference tests/test_attention.py:441-462 with its commented-out tail restored
         def fn(Q, K, K2, V):
