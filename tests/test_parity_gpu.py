@@ -503,6 +503,28 @@ def test_full_size_causal_prefix_is_bit_equal():
         assert torch.equal(part, whole[:, :, :n]), n
 
 
+@pytest.mark.parametrize("variant", ["swp", "w32"])
+def test_long_sequence_rows(variant, monkeypatch):
+    """S = 32768 (byte offsets up to 2^23 rows x 256 B): sampled rows of the causal result
+    against the oracle, row i being plain attention over keys 0..i."""
+    monkeypatch.setenv("LOOPFUSE_PREFILL", variant)
+    S, D = 32768, 128
+    q, k, v = (rand((1, 2, S, D), torch.bfloat16, s) for s in (1, 2, 3))
+    got = lowering.attention(q.to(dev()), k.to(dev()), v.to(dev()), lowering.AttnPlan(mask="causal", scale=D ** -0.5))
+    torch.cuda.synchronize()
+    got = got.float().cpu()
+    for i in (0, 1, 127, 128, 12345, 20000, S - 1):
+        want = O.attention_reference(q[:, :, i:i + 1], k[:, :, :i + 1], v[:, :, :i + 1])
+        assert (got[:, :, i:i + 1] - want).abs().max().item() <= TOL[torch.bfloat16], i
+    # window variant at the same length: only the last 300 keys of each row count
+    got = lowering.attention(q.to(dev()), k.to(dev()), v.to(dev()),
+                             lowering.AttnPlan(mask="sliding", window=300, scale=D ** -0.5)).float().cpu()
+    for i in (5, 299, 300, 25000, S - 1):
+        lo = max(0, i - 299)
+        want = O.attention_reference(q[:, :, i:i + 1], k[:, :, lo:i + 1], v[:, :, lo:i + 1])
+        assert (got[:, :, i:i + 1] - want).abs().max().item() <= TOL[torch.bfloat16], i
+
+
 def test_c1_on_gpu_vs_cpu_eager():
     # config 1 (fp32, CPU-runnable): same tensors through the CPU eager graph and,
     # cast to bf16, through the GPU kernel
