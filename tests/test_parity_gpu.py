@@ -419,6 +419,21 @@ def test_decode_paged_one_token_pages_int64():
     check(q, kp, vp, k_table=kt, v_table=vt)
 
 
+@pytest.mark.parametrize("paged", [False, True])
+def test_decode_long_context(paged):
+    """K_len = 65536 with few (batch, head) units: the KV range is split 16 ways."""
+    B, Hq, Hkv, S, D, P = 2, 8, 2, 65536, 128, 16
+    q = rand((B, Hq, 1, D), torch.bfloat16, 1)
+    if paged:
+        n = B * S // P
+        kp, vp = rand((n, P, Hkv, D), torch.bfloat16, 2), rand((n, P, Hkv, D), torch.bfloat16, 3)
+        table = torch.randperm(n, generator=torch.Generator().manual_seed(4)).view(B, S // P).to(torch.int32)
+        check(q, kp, vp, k_table=table, v_table=table)
+    else:
+        check(q, rand((B, Hkv, S, D), torch.bfloat16, 2), rand((B, Hkv, S, D), torch.bfloat16, 3))
+    assert lowering.attention.last_launch["grid"][1] == 16
+
+
 def test_decode_equals_last_prefill_row():
     q = rand((2, 4, 256, 128), torch.bfloat16, 1)
     k = rand((2, 4, 256, 128), torch.bfloat16, 2)
