@@ -243,13 +243,16 @@ def decode_split(units: int, Sk: int, cus: int = 256, per_cu: int = 2) -> int:
     """Number of KV splits across workgroups.  One workgroup per unit is enough once
     there are ``per_cu`` workgroups per CU (8 resident waves, each with 32 KB of loads
     in flight: two workgroups of 4 waves, or one of 8); below that the KV range is
-    split, down to 512 tokens per split and 16 splits, and a second kernel merges the
-    partial results."""
+    split, down to 512 tokens per split and up to 64 splits, and a second kernel merges
+    the partial results."""
     env = os.environ.get("LOOPFUSE_DECODE_SPLITS")
     if env:
         return max(1, int(env))
     want = max(1, (per_cu * cus + units - 1) // units)
-    most = max(1, min(16, Sk // 512))      # measured: >= 512 tokens per split, at most 16 splits
+    if want > 4:
+        # few units (small batch, long context): one workgroup per CU measured best
+        want = max(4, (cus + units - 1) // units)
+    most = max(1, min(64, Sk // 512))      # measured: >= 512 tokens per split, at most 64 splits
     return max(1, min(want, most))
 
 

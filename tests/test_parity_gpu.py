@@ -421,7 +421,7 @@ def test_decode_paged_one_token_pages_int64():
 
 @pytest.mark.parametrize("paged", [False, True])
 def test_decode_long_context(paged):
-    """K_len = 65536 with few (batch, head) units: the KV range is split 16 ways."""
+    """K_len = 65536 with few (batch, head) units: the KV range is split 64 ways."""
     B, Hq, Hkv, S, D, P = 2, 8, 2, 65536, 128, 16
     q = rand((B, Hq, 1, D), torch.bfloat16, 1)
     if paged:
@@ -431,7 +431,7 @@ def test_decode_long_context(paged):
         check(q, kp, vp, k_table=table, v_table=table)
     else:
         check(q, rand((B, Hkv, S, D), torch.bfloat16, 2), rand((B, Hkv, S, D), torch.bfloat16, 3))
-    assert lowering.attention.last_launch["grid"][1] == 16
+    assert lowering.attention.last_launch["grid"][1] == 64
 
 
 def test_decode_equals_last_prefill_row():
