@@ -216,10 +216,12 @@ def _check_tensor(name: str, t: torch.Tensor, dtype: torch.dtype) -> None:
         raise RuntimeError(f"loopfuse_amd: {name} is not on the GPU; the HIP path has no CPU fallback")
     if t.dtype != dtype:
         raise UnsupportedPlan(f"{name} has dtype {t.dtype}, expected {dtype}")
-    if t.stride(-1) != 1:
-        raise UnsupportedPlan(f"{name} must have unit stride in its last dimension")
     if t.data_ptr() % 16:
         raise UnsupportedPlan(f"{name} is not 16-byte aligned")
+    if t.is_contiguous() and t.shape[-1] % 8 == 0:
+        return
+    if t.stride(-1) != 1:
+        raise UnsupportedPlan(f"{name} must have unit stride in its last dimension")
     for n, s in zip(t.shape[:-1], t.stride()[:-1]):
         if n > 1 and s % 8:
             raise UnsupportedPlan(f"{name} strides must be multiples of 8 elements (16-byte loads)")
@@ -231,7 +233,7 @@ _scratch: dict[tuple[int, int], torch.Tensor] = {}
 def _get_scratch(device: torch.device, nfloats: int) -> torch.Tensor:
     """Split-K scratch, one buffer per (device, stream): launches on one stream are
     ordered, so they can share it; launches on different streams must not."""
-    key = (device.index or 0, torch.cuda.current_stream(device).cuda_stream)
+    key = (device.index or 0, runtime.current_stream_handle())
     t = _scratch.get(key)
     if t is None or t.numel() < nfloats:
         t = torch.empty(max(nfloats, 1 << 20), dtype=torch.float32, device=device)

@@ -131,6 +131,15 @@ def compile_source(src: str, name: str, opts: Sequence[str], arch: str | None = 
     return data, bool(hit.value), log.value.decode("utf-8", "replace")
 
 
+def current_stream_handle() -> int:
+    """hipStream_t of torch's current stream on the current device, as an integer
+    (the raw accessor: the launch path is called once per kernel)."""
+    try:
+        return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device())
+    except AttributeError:            # older / newer torch without the raw accessor
+        return torch.cuda.current_stream().cuda_stream
+
+
 class Kernel:
     """A kernel of a loaded module; ``launch`` passes ONE by-value struct argument."""
 
@@ -140,15 +149,17 @@ class Kernel:
         fn = ctypes.c_void_p()
         _check(f"lf_get_function[{symbol}]", lib().lf_get_function(module.handle, symbol.encode(), ctypes.byref(fn)))
         self.handle = fn
+        self._launch = lib().lf_launch
 
     def launch(self, grid: tuple[int, int, int], block: tuple[int, int, int], params: ctypes.Structure,
                stream: int | None = None, lds_bytes: int = 0) -> None:
         if stream is None:
-            stream = torch.cuda.current_stream().cuda_stream
+            stream = current_stream_handle()
         args = (ctypes.c_void_p * 1)(ctypes.addressof(params))
-        rc = lib().lf_launch(self.handle, grid[0], grid[1], grid[2], block[0], block[1], block[2],
-                             lds_bytes, ctypes.c_void_p(stream), args)
-        _check(f"lf_launch[{self.symbol}]", rc)
+        rc = self._launch(self.handle, grid[0], grid[1], grid[2], block[0], block[1], block[2],
+                          lds_bytes, ctypes.c_void_p(stream), args)
+        if rc:
+            _check(f"lf_launch[{self.symbol}]", rc)
 
 
 class Module:
