@@ -101,6 +101,7 @@ class Stage:
     # current shape; None while the value is a plain reshape of the canonical layout
     lay: Any = None
     mat: tuple = ()                    # (Sq, Sk) stand-ins
+    late_factors: list = dataclasses.field(default_factory=list)   # run-time factors applied after the mask: must be > 0
 
 
 @dataclasses.dataclass
@@ -197,6 +198,7 @@ class AttentionMatch:
     base2: bool = False            # explicit softmax written with exp2: scores are in log2 units
     q2: Optional[Operand] = None   # second score product: scores = Q K^T + Q2 K2^T
     k2: Optional[Operand] = None
+    late_factors: tuple = ()       # factors (also listed above) that the graph applies after the mask
 
     def describe(self) -> str:
         nm = lambda i: self.inputs[i].name
@@ -226,6 +228,10 @@ class AttentionMatch:
         return r
 
     def plan_for(self, vals) -> lowering.AttnPlan:
+        for f in self.late_factors:
+            # x * f commutes with the mask only for f > 0 (-inf must stay -inf)
+            if not self._number(f, vals) > 0.0:
+                raise lowering.UnsupportedPlan("a non-positive factor is applied to masked scores")
         pre = self._product(self.factors, vals)
         if self.has_tanh:
             cap = self._product(self.post_factors, vals)
@@ -827,14 +833,23 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
                 if st.sm != "":
                     raise _Skip(f"op inside an explicit softmax: {tgt}")
                 # a positive constant factor commutes with the mask (-inf stays -inf)
-                if tgt in (aten.mul.Tensor, aten.div.Tensor) and st.mask is not None and st.bias is None \
-                        and is_number(a[1]) and a[1] > 0 and not isinstance(node.args[1], torch.fx.Node) and st.uid == 0:
-                    f = float(a[1]) if tgt is aten.mul.Tensor else 1.0 / float(a[1])
+                if tgt in (aten.mul.Tensor, aten.div.Tensor) and st.mask is not None and st.bias is None and st.uid == 0 \
+                        and (isinstance(a[1], Scalar) or (is_number(a[1]) and (a[1] > 0 or isinstance(node.args[1], torch.fx.Node)))):
+                    raw = node.args[1]
+                    if isinstance(a[1], Scalar):
+                        f = a[1].node
+                    else:
+                        f = raw if isinstance(raw, torch.fx.Node) else float(a[1])
+                    if tgt is aten.div.Tensor:
+                        f = ("recip", f)
                     new = dataclasses.replace(st)
                     if st.has_tanh:
                         new.post_factors = st.post_factors + [f]
                     else:
                         new.factors = st.factors + [f]
+                    if not is_number(f):
+                        # a factor only known per call (D ** -0.5 of a dynamic D): its sign is checked then
+                        new.late_factors = st.late_factors + [f]
                     return new
             if st.kind == "scores" and tgt is aten.add.Tensor and isinstance(a[1], Stage):
                 # Q K^T + Q2 K2^T: two bare products (or two products with the same factors)
@@ -1007,4 +1022,4 @@ def _build_match(out_node: torch.fx.Node, st: Stage) -> AttentionMatch:
     return AttentionMatch(out_node, inputs, q_op, k_op, v_op, [scalar(f) for f in st.factors],
                           [scalar(f) for f in st.post_factors], st.has_tanh, st.mask, window, out_rank,
                           bias_op, obias_op, denom_add=tuple(scalar(t) for t in st.denom_add), base2=st.base2,
-                          q2=q2_op, k2=k2_op)
+                          q2=q2_op, k2=k2_op, late_factors=tuple(scalar(f) for f in st.late_factors))

@@ -447,3 +447,25 @@ def test_static_shapes_at_real_sizes_are_matched(which, monkeypatch):
     assert interface.stats["fused"] == before["fused"] + 1, "static graph at real size was not matched"
     want = fn(*ins)
     assert (got.float() - want.float()).abs().max().item() <= 6e-2
+
+
+def test_factor_after_the_mask(monkeypatch):
+    """x * f commutes with the mask only for f > 0.  A literal positive factor is folded at
+    trace time; one that is only known per call is checked per call, and a non-positive
+    value sends that call down the unfused graph."""
+    monkeypatch.setattr(capture.AttentionMatch, "run", _oracle_run)
+
+    def fn(Q, K, V, alpha):
+        s = torch.ops.loopfuse.causal_mask(Q @ K.transpose(-2, -1)) * alpha
+        return torch.softmax(s, dim=-1) @ V
+
+    q, k, v = (torch.randn(2, 3, 24, 64, generator=torch.Generator().manual_seed(s)) for s in (0, 1, 2))
+    torch._dynamo.reset()
+    cf = torch.compile(fn, backend=loopfuse_amd.loopfuse_backend, dynamic=True)
+    before = dict(interface.stats)
+    pos = cf(q, k, v, torch.tensor(0.125))
+    assert interface.stats["fused"] == before["fused"] + 1
+    torch.testing.assert_close(pos, O.attention_reference(q, k, v, mask="causal", scale=0.125), rtol=2e-4, atol=2e-4)
+    neg = cf(q, k, v, torch.tensor(-0.125))      # -inf * negative = +inf: not a masked softmax any more
+    assert interface.stats["eager_runtime"] == before["eager_runtime"] + 1
+    torch.testing.assert_close(neg, fn(q, k, v, torch.tensor(-0.125)), equal_nan=True)
