@@ -69,7 +69,7 @@ def cpu_baseline(seconds: float = 12.0) -> dict:
                 O.eager_reference_graph(q, k, v)
             ts = []
             t_end = time.perf_counter() + budget
-            while time.perf_counter() < t_end and len(ts) < 200:
+            while time.perf_counter() < t_end and len(ts) < 2000:
                 t0 = time.perf_counter()
                 O.eager_reference_graph(q, k, v)
                 ts.append(time.perf_counter() - t0)
