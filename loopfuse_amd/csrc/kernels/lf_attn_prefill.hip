@@ -220,9 +220,15 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
   const lf_elem* k2_uni = p.k2 + (long long)b * p.k2_sb + (long long)(h / p.k2_group) * p.k2_sh;
 #endif
 
-#if LF_SOFTCAP
+#if LF_SOFTCAP && !(LF_BIAS & 1)
+  // capped score c*tanh(x) = c - 2c*r with r = 1 / (e^(2x) + 1), x = s*scale/c.  The
+  // constant c is the same for every key of a row, so the softmax does not see it: the
+  // kernel works on -r and folds the factor 2c into the exponent multiplier
+  const float sc_exp = p.scale / p.softcap * (2.0f * LF_LOG2E);   // 2^(s * sc_exp) = e^(2x)
+  const float cexp = 2.0f * p.softcap * LF_LOG2E;
+#elif LF_SOFTCAP
   const float sc_in = p.scale / p.softcap;   // tanh argument multiplier
-  const float cexp = LF_LOG2E;               // scores are final before exp
+  const float cexp = LF_LOG2E;               // scores are final before exp (a bias is added to them)
 #elif LF_BIAS & 1
   const float cexp = LF_LOG2E;               // scores are scaled explicitly, then biased
 #else
@@ -469,7 +475,12 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
       LF_T(1)
       // ---- score modifications and mask; element i of block kb is kv index
       // j = k0 + 32*kb + 8*(i/4) + 4*g + i%4, query my_q.
-#if LF_SOFTCAP
+#if LF_SOFTCAP && !(LF_BIAS & 1)
+#pragma unroll
+      for (int kb = 0; kb < LF_NKB; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[kb][i] = __builtin_amdgcn_rcpf(-1.0f - lf_exp2(s[kb][i] * sc_exp));   // -r
+#elif LF_SOFTCAP
 #pragma unroll
       for (int kb = 0; kb < LF_NKB; ++kb)
 #pragma unroll

@@ -155,8 +155,12 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
   };
 
 #if LF_SOFTCAP
-  const float sc_in = p.scale / p.softcap;
-  const float cexp = LF_LOG2E;
+  // capped score c*tanh(x) = c - 2c*r with r = 1 / (e^(2x) + 1), x = s*scale/c.  The
+  // constant c is the same for every key of a row, so the softmax does not see it: the
+  // kernel works on -r and folds the factor 2c into the exponent multiplier, which saves
+  // the three VALU operations per score that would turn r into the capped score
+  const float sc_exp = p.scale / p.softcap * (2.0f * LF_LOG2E);   // 2^(s * sc_exp) = e^(2x)
+  const float cexp = 2.0f * p.softcap * LF_LOG2E;
 #else
   const float cexp = p.scale * LF_LOG2E;
 #endif
@@ -339,7 +343,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
 #pragma unroll
         for (int kb = 0; kb < LF_NKB; ++kb)
 #pragma unroll
-          for (int i = 0; i < 16; ++i) s[kb][i] = p.softcap * lf_tanh(s[kb][i] * sc_in);
+          for (int i = 0; i < 16; ++i) s[kb][i] = __builtin_amdgcn_rcpf(-1.0f - lf_exp2(s[kb][i] * sc_exp));   // -r
 #endif
         if (!full) {
 #pragma unroll
