@@ -46,7 +46,20 @@
 #define LF_NW 4     /* waves per workgroup: 4 (two workgroups per CU) or 8 (one) */
 #endif
 #define LF_NT (LF_NW * 64)
+#ifndef LF_GQAPACK
+#define LF_GQAPACK 0     /* 1 (grouped-query attention, Hq / Hkv a multiple of LF_NW): the waves of a workgroup
+                            take the same 32 query rows of LF_NW consecutive query heads that share one kv head,
+                            instead of LF_NW blocks of 32 rows of one head: a q tile is then 32 rows tall, every
+                            wave needs exactly the same KV tiles (no wave idles on a tile of the diagonal or of
+                            the window's edge), and one K/V tile in LDS serves LF_NW heads */
+#endif
+#if LF_GQAPACK
+#define LF_BM 32
+#define LF_HEADS_PER_WG LF_NW
+#else
 #define LF_BM (32 * LF_NW)
+#define LF_HEADS_PER_WG 1
+#endif
 #define LF_BN 64
 #define LF_KSLOTS 3
 #define LF_VSLOTS 2
@@ -73,7 +86,7 @@ __device__ __forceinline__ int lf_v_phys(int row, int ch) {
 #define LF_BARRIER_VM0() asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory")
 
 // slots per XCD class: (batch, head) pairs of the class, padded to groups of 4, times q-tile pairs
-#define LF_NSLOTS(p, npair) ((((p.B * p.Hq + 7) / 8 + 3) / 4 * 4) * (npair))
+#define LF_NSLOTS(p, npair) ((((p.B * (p.Hq / LF_HEADS_PER_WG) + 7) / 8 + 3) / 4 * 4) * (npair))
 
 extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_swp(const LfAttnParams p) {
   __shared__ __attribute__((aligned(16))) lf_elem lds_k[LF_KSLOTS][LF_BN * LF_D];
@@ -93,7 +106,8 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
   // ---- workgroup -> (batch*head, pair of q tiles), as in lf_attn_prefill.hip
   const int nqt = (p.Sq + LF_BM - 1) / LF_BM;
   const int npair = (nqt + 1) / 2;
-  const int nbh = p.B * p.Hq;
+  const int nhv = p.Hq / LF_HEADS_PER_WG;     // head units per batch element (heads, or packs of heads)
+  const int nbh = p.B * nhv;
   const int xcd = blockIdx.x & 7;
   // a workgroup takes slots blockIdx.x/8, + gridDim.x/8, ... of its XCD class (the host
   // may launch fewer workgroups than slots: the resident set, which then stays)
@@ -103,9 +117,13 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
   const int bh = (grp * 4 + (in_grp & 3)) * 8 + xcd;
   if (bh >= nbh) continue;
   const int pair = in_grp >> 2;
-  const int b = bh / p.Hq;
-  const int h = bh % p.Hq;
-  const int hkv = h / (p.Hq / p.Hkv);
+  const int b = bh / nhv;
+#if LF_GQAPACK
+  const int h = (bh % nhv) * LF_NW + wave;    // this wave's query head
+#else
+  const int h = bh % nhv;
+#endif
+  const int hkv = h / (p.Hq / p.Hkv);         // the same for all waves: the pack lies inside one group
   const int nkt = (p.Sk + LF_BN - 1) / LF_BN;
 
   // ---- direct-to-LDS staging: a wave-level load writes 64 lanes x 16 B at
@@ -227,7 +245,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
         p.visits[((long long)bh * nqt + qt) * nkt + kt] = 1;
     }
 
-    const int wq0 = q0 + 32 * wave;
+    const int wq0 = LF_GQAPACK ? q0 : q0 + 32 * wave;
     const int wqlast = min(wq0 + 31, p.Sq - 1);
     const bool wave_has_rows = wq0 < p.Sq;
     const int my_q = wq0 + l32;
