@@ -571,7 +571,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
             extra += ("-DLF_DMA=1",)     # frees the staging registers the bias values / Q2 fragments need
         # grouped-query attention: the 4 waves of a workgroup take 4 query heads of one group
         # (same 32 rows) and share every K/V tile in LDS
-        pack = family == "prefill_swp" and group % 4 == 0 and \
+        pack = family == "prefill_swp" and group % 4 == 0 and not any(e.startswith("-DLF_NW=") for e in extra) and \
             choice.get("pack", os.environ.get("LOOPFUSE_GQAPACK", "1") == "1")
         spec = KernelSpec(family, _DTYPE_CODE[dtype], D, mask, plan.softcap is not None, paged,
                           page_size, table_i64, v_tr=v_tr if family == "prefill" else True, bias=bias_bits,
