@@ -44,6 +44,7 @@ typedef struct LfAttnParamsHost {
   int64_t ob_sb, ob_sh, ob_sq;
   int64_t q2_sb, q2_sh, q2_ss;
   int64_t k2_sb, k2_sh, k2_ss;
+  int64_t k_span, v_span;     /* paged: elements from the pool's base pointer to the end of the pool */
   int32_t B, Hq, Hkv, Sq, Sk;
   int32_t window;             /* sliding-window width (LF_MASK == 2) */
   int32_t kt_stride, vt_stride;
@@ -55,10 +56,10 @@ typedef struct LfAttnParamsHost {
 } LfAttnParamsHost;
 
 #ifdef __cplusplus
-static_assert(sizeof(LfAttnParamsHost) == 360, "LfAttnParamsHost must match the device struct");
+static_assert(sizeof(LfAttnParamsHost) == 376, "LfAttnParamsHost must match the device struct");
 }
 #else
-_Static_assert(sizeof(LfAttnParamsHost) == 360, "LfAttnParamsHost must match the device struct");
+_Static_assert(sizeof(LfAttnParamsHost) == 376, "LfAttnParamsHost must match the device struct");
 #endif
 
 #endif /* LF_ATTN_PARAMS_H */

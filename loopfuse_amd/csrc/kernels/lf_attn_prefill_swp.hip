@@ -134,11 +134,29 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
   constexpr int kRowsPerWave = 64 / LF_CPR;
   const int srow = tid / LF_CPR;
   const int sch = tid % LF_CPR;
-  const lf_elem* k_uni = p.k + (long long)b * p.k_sb + (long long)hkv * p.k_sh;
-  const lf_elem* v_uni = p.v + (long long)b * p.v_sb + (long long)hkv * p.v_sh;
-  const unsigned k_bytes = (unsigned)(((long long)(p.Sk - 1) * p.k_ss + LF_D) * 2);
-  const unsigned v_bytes = (unsigned)(((long long)(p.Sk - 1) * p.v_ss + LF_D) * 2);
+  // Dense K/V: one buffer resource per (batch, kv head), rows 0..Sk-1.  Paged K/V
+  // (LF_PAGED, pages of a multiple of 64/LF_CPR tokens, pool < 4 GiB): the resource
+  // covers the whole pool, and the uniform part of a load's offset comes from the page
+  // table: page id * page stride + head + row inside the page.  The 64/LF_CPR rows of
+  // one wave-level load never straddle a page.  Rows past Sk get an offset beyond the
+  // resource, so they arrive as zeros in both cases.
+  constexpr bool kPagedK = (LF_PAGED & 1) != 0, kPagedV = (LF_PAGED & 2) != 0;
+  const lf_elem* k_uni = kPagedK ? p.k : p.k + (long long)b * p.k_sb + (long long)hkv * p.k_sh;
+  const lf_elem* v_uni = kPagedV ? p.v : p.v + (long long)b * p.v_sb + (long long)hkv * p.v_sh;
+  const unsigned k_bytes = kPagedK ? (unsigned)(p.k_span * 2) : (unsigned)(((long long)(p.Sk - 1) * p.k_ss + LF_D) * 2);
+  const unsigned v_bytes = kPagedV ? (unsigned)(p.v_span * 2) : (unsigned)(((long long)(p.Sk - 1) * p.v_ss + LF_D) * 2);
   const unsigned k_rowb = (unsigned)p.k_ss * 2u, v_rowb = (unsigned)p.v_ss * 2u;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  // page id (as a byte offset of the page + this kv head) for the rows of this wave in
+  // pass ps of tile kt; tiles / rows past Sk re-use the last page (their rows are zeroed)
+  auto page_off = [&](int which, int kt, int ps) -> unsigned {
+    const int tok = min(kt * LF_BN + (LF_NT / LF_CPR) * ps + (64 / LF_CPR) * wave_u, p.Sk - 1);
+    const lf_table_t* tab = reinterpret_cast<const lf_table_t*>(which ? p.v_table : p.k_table);
+    const int psz = which ? LF_PAGE_SIZE_V : LF_PAGE_SIZE;
+    const unsigned id = (unsigned)tab[(long long)b * (which ? p.vt_stride : p.kt_stride) + tok / psz];
+    return which ? id * (unsigned)(p.v_sb * 2) + (unsigned)hkv * (unsigned)(p.v_sh * 2)
+                 : id * (unsigned)(p.k_sb * 2) + (unsigned)hkv * (unsigned)(p.k_sh * 2);
+  };
   lf_u32x4 k_rsq, v_rsq;
   {
     const unsigned long long ka = (unsigned long long)k_uni, va = (unsigned long long)v_uni;
@@ -151,8 +169,9 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
     v_rsq[2] = __builtin_amdgcn_readfirstlane(v_bytes);
     v_rsq[3] = 0x00020000u;
   }
-  const unsigned k_doff = (unsigned)srow * k_rowb + 16u * (unsigned)lf_k_phys(srow, sch);
-  const unsigned v_doff = (unsigned)srow * v_rowb + 16u * (unsigned)lf_v_phys(srow, sch);
+  // per-lane part of the offset: dense = row inside the pass, paged = row inside the wave's load
+  const unsigned k_doff = (unsigned)(kPagedK ? srow % (64 / LF_CPR) : srow) * k_rowb + 16u * (unsigned)lf_k_phys(srow, sch);
+  const unsigned v_doff = (unsigned)(kPagedV ? srow % (64 / LF_CPR) : srow) * v_rowb + 16u * (unsigned)lf_v_phys(srow, sch);
   bool dma_on = true;
   auto dma = [&](const lf_u32x4& rs, unsigned voff, const lf_elem* lds_row0) {
     const unsigned m0v = __builtin_amdgcn_readfirstlane(
@@ -163,13 +182,28 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                  :: "s"(m0v), "v"(voff), "s"(rs) : "memory");
   };
-  auto dma_k_pass = [&](int kt, int sl, int ps) {
-    dma(k_rsq, k_doff + (unsigned)(kt * LF_BN + kRowsPerPass * ps) * k_rowb,
-        &lds_k[sl][(kRowsPerPass * ps + kRowsPerWave * wave) * LF_D]);
+  // pg: page_off() of the pass (paged operands only; fetched a tile ahead by the caller)
+  auto dma_k_pass = [&](int kt, int sl, int ps, unsigned pg) {
+    unsigned off;
+    if (kPagedK) {
+      const int tokw = kt * LF_BN + kRowsPerPass * ps + kRowsPerWave * wave_u;     // first row of this wave's load
+      off = pg + (unsigned)(tokw % LF_PAGE_SIZE) * k_rowb + k_doff;
+      if (tokw + (int)(srow % kRowsPerWave) >= p.Sk) off = 0xffffffffu;
+    } else {
+      off = k_doff + (unsigned)(kt * LF_BN + kRowsPerPass * ps) * k_rowb;
+    }
+    dma(k_rsq, off, &lds_k[sl][(kRowsPerPass * ps + kRowsPerWave * wave) * LF_D]);
   };
-  auto dma_v_pass = [&](int kt, int sl, int ps) {
-    dma(v_rsq, v_doff + (unsigned)(kt * LF_BN + kRowsPerPass * ps) * v_rowb,
-        &lds_v[sl][(kRowsPerPass * ps + kRowsPerWave * wave) * LF_D]);
+  auto dma_v_pass = [&](int kt, int sl, int ps, unsigned pg) {
+    unsigned off;
+    if (kPagedV) {
+      const int tokw = kt * LF_BN + kRowsPerPass * ps + kRowsPerWave * wave_u;
+      off = pg + (unsigned)(tokw % LF_PAGE_SIZE_V) * v_rowb + v_doff;
+      if (tokw + (int)(srow % kRowsPerWave) >= p.Sk) off = 0xffffffffu;
+    } else {
+      off = v_doff + (unsigned)(kt * LF_BN + kRowsPerPass * ps) * v_rowb;
+    }
+    dma(v_rsq, off, &lds_v[sl][(kRowsPerPass * ps + kRowsPerWave * wave) * LF_D]);
   };
 
 #if LF_SOFTCAP
@@ -279,15 +313,29 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
     float l_run = 0.0f;          // this lane's share of the running sum
 
     // ---- prologue: K(begin), K(begin+1), V(begin) resident; first K fragments in flight
+    // paged operands: page offsets of the passes issued during the coming tile (K two
+    // tiles ahead, V one tile ahead), fetched a tile before they are needed
+    unsigned kpg[LF_NPASS], vpg[LF_NPASS];
+    {
+      unsigned k0pg[LF_NPASS], k1pg[LF_NPASS], v0pg[LF_NPASS];
 #pragma unroll
-    for (int ps = 0; ps < LF_NPASS; ++ps) {
-      dma_k_pass(kt_begin, 0, ps);
-      if (kt_begin + 1 < kt_end) dma_k_pass(kt_begin + 1, 1, ps);
-      dma_v_pass(kt_begin, 0, ps);
+      for (int ps = 0; ps < LF_NPASS; ++ps) {
+        k0pg[ps] = kPagedK ? page_off(0, kt_begin, ps) : 0u;
+        k1pg[ps] = kPagedK ? page_off(0, kt_begin + 1, ps) : 0u;
+        v0pg[ps] = kPagedV ? page_off(1, kt_begin, ps) : 0u;
+        kpg[ps] = kPagedK ? page_off(0, kt_begin + 2, ps) : 0u;
+        vpg[ps] = kPagedV ? page_off(1, kt_begin + 1, ps) : 0u;
+      }
+#pragma unroll
+      for (int ps = 0; ps < LF_NPASS; ++ps) {
+        dma_k_pass(kt_begin, 0, ps, k0pg[ps]);
+        if (kt_begin + 1 < kt_end) dma_k_pass(kt_begin + 1, 1, ps, k1pg[ps]);
+        dma_v_pass(kt_begin, 0, ps, v0pg[ps]);
 #if LF_ABLATE & 2
-      dma_k_pass(kt_begin, 2, ps);
-      dma_v_pass(kt_begin, 1, ps);
+        dma_k_pass(kt_begin, 2, ps, k0pg[ps]);
+        dma_v_pass(kt_begin, 1, ps, v0pg[ps]);
 #endif
+      }
     }
 #if LF_ABLATE & 2
     dma_on = false;
@@ -310,11 +358,18 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
       // (tiles past the last one are not fetched: wave-uniform tests)
       auto dma_step = [&](int d) {
         if (d < LF_NPASS) {
-          if (kt + 2 < kt_end) dma_k_pass(kt + 2, ks_ld, d);
+          if (kt + 2 < kt_end) dma_k_pass(kt + 2, ks_ld, d, kpg[d]);
         } else if (kt + 1 < kt_end) {
-          dma_v_pass(kt + 1, vs_ld, d - LF_NPASS);
+          dma_v_pass(kt + 1, vs_ld, d - LF_NPASS, vpg[d - LF_NPASS]);
         }
       };
+      // page offsets for the next tile's loads (table reads: in flight during this tile)
+      unsigned kpg_n[LF_NPASS], vpg_n[LF_NPASS];
+#pragma unroll
+      for (int ps = 0; ps < LF_NPASS; ++ps) {
+        kpg_n[ps] = kPagedK ? page_off(0, kt + 3, ps) : 0u;
+        vpg_n[ps] = kPagedV ? page_off(1, kt + 2, ps) : 0u;
+      }
 
       const int k0 = kt * LF_BN;
       bool need = wave_has_rows;
@@ -439,6 +494,11 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
       }
       LF_BARRIER_VM0();
       ks_cur = ks_nxt;
+#pragma unroll
+      for (int ps = 0; ps < LF_NPASS; ++ps) {
+        kpg[ps] = kpg_n[ps];
+        vpg[ps] = vpg_n[ps];
+      }
     }
 
     // ---- epilogue: O[q][d] = O^T[d][q] / l.  Element i of block db is

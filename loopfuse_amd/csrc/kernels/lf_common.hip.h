@@ -104,6 +104,8 @@ struct LfAttnParams {
   long long ob_sb, ob_sh, ob_sq;         // element strides of obias (0 = broadcast)
   long long q2_sb, q2_sh, q2_ss;         // Q2 [B, Hq, Sq, LF_D2] (d stride 1)
   long long k2_sb, k2_sh, k2_ss;         // K2 [B, Hq / k2_group, Sk, LF_D2] (d stride 1)
+  long long k_span, v_span;              // paged: elements from the pool's base to its end (the range the
+                                         // direct-to-LDS loads are checked against)
   int B, Hq, Hkv, Sq, Sk;
   int window;                // sliding-window width (LF_MASK == 2)
   int kt_stride, vt_stride;  // row strides (elements) of k_table / v_table

@@ -46,7 +46,7 @@ class AttnParams(ctypes.Structure):
         + [(n, ctypes.c_longlong) for n in (
             "q_sb", "q_sh", "q_ss", "k_sb", "k_sh", "k_ss", "v_sb", "v_sh", "v_ss", "o_sb", "o_sh", "o_ss",
             "bias_sb", "bias_sh", "bias_sq", "ob_sb", "ob_sh", "ob_sq",
-            "q2_sb", "q2_sh", "q2_ss", "k2_sb", "k2_sh", "k2_ss")]
+            "q2_sb", "q2_sh", "q2_ss", "k2_sb", "k2_sh", "k2_ss", "k_span", "v_span")]
         + [(n, ctypes.c_int) for n in (
             "B", "Hq", "Hkv", "Sq", "Sk", "window", "kt_stride", "vt_stride", "nsplit", "rows", "split_len", "k2_group")]
         + [("scale", ctypes.c_float), ("softcap", ctypes.c_float), ("denom_add", ctypes.c_float)]
@@ -550,15 +550,25 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     if family == "prefill" and not bias_bits and plan.denom_add == 0.0 and not d2:
         family = {"swp": "prefill_swp", "w32": "prefill"}.get(choice.get("prefill"), None) or prefill_variant(Sq, v_tr)
     if family == "prefill_swp":
-        # direct-to-LDS staging: dense K/V only, 32-bit byte offsets per (batch, kv head)
-        # span; the kernel also addresses up to three tiles past Sk (those reads are
-        # range-checked to zeros, but their offsets must not wrap)
-        reach = max(abs(P.k_ss), abs(P.v_ss)) * 2 * (Sk + 3 * 64) + 2 * D
-        if paged or reach >= (1 << 32) or P.k_ss < 0 or P.v_ss < 0:
+        # direct-to-LDS staging addresses memory with 32-bit byte offsets.  Dense operands:
+        # offsets inside one (batch, kv head) span; the kernel also addresses up to three
+        # tiles past Sk (those reads are range-checked to zeros, but their offsets must
+        # not wrap).  Paged operands: offsets inside the whole pool (< 4 GiB), pages of a
+        # multiple of 8 tokens (the rows of one wave-level load stay inside a page).
+        def swp_ok(t, is_paged, ps_, ss):
+            if is_paged:
+                span_b = 2 * (sum((n - 1) * abs(st) for n, st in zip(t.shape, t.stride())) + 1)
+                return ps_ % 8 == 0 and span_b < (1 << 32) - 64 and all(st >= 0 for st in t.stride())
+            reach = abs(ss) * 2 * (Sk + 3 * 64) + 2 * D
+            return ss >= 0 and reach < (1 << 32) and (Sk - 1) * abs(ss) * 2 + 2 * D < (1 << 31)
+        if not (swp_ok(k, plan.k_paged, page_size, P.k_ss)
+                and swp_ok(v, plan.v_paged, page_size_v or page_size, P.v_ss)) \
+                or (paged and os.environ.get("LOOPFUSE_PAGED_SWP", "1") != "1"):
             family = "prefill"
-        span = max((Sk - 1) * abs(P.k_ss), (Sk - 1) * abs(P.v_ss)) * 2 + 2 * D
-        if span >= (1 << 31):
-            family = "prefill"
+        if plan.k_paged:
+            P.k_span = sum((n - 1) * st for n, st in zip(k.shape, k.stride())) + 1
+        if plan.v_paged:
+            P.v_span = sum((n - 1) * st for n, st in zip(v.shape, v.stride())) + 1
     if family in ("prefill", "prefill_swp"):
         P.q_sb, P.q_sh, P.q_ss = q.stride(0), q.stride(1), q.stride(2)
         P.o_sb, P.o_sh, P.o_ss = out.stride(0), out.stride(1), out.stride(2)

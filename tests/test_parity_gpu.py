@@ -205,6 +205,43 @@ def test_shifted_denominator_single_row_and_gqa_paged():
     check(rand((B, Hq, S, D), torch.bfloat16, 3), kp, vp, mask="causal", k_table=table, v_table=table, denom_add=1.0)
 
 
+# ---------------------------------------------------------------- paged prefill, direct-to-LDS loads
+@pytest.mark.parametrize("D,P,S,i64,which", [(128, 16, 336, False, 3), (128, 32, 352, True, 3), (64, 16, 336, False, 3),
+                                             (64, 8, 200, True, 3), (128, 16, 1040, False, 1), (128, 64, 448, False, 2)])
+@pytest.mark.parametrize("mask,window", [("causal", 0), ("sliding", 90), (None, 0)])
+def test_paged_prefill_direct_loads(D, P, S, i64, which, mask, window):
+    """lf_attn_prefill_swp on page pools: page sizes 8..64, lengths that end inside a KV tile,
+    int32 / int64 tables, K only / V only / both paged, GQA (packed heads) and not."""
+    B, Hq, Hkv = 2, 8, 2
+    n = B * S // P
+    gen = torch.Generator().manual_seed(S + P)
+    q = rand((B, Hq, S, D), torch.bfloat16, 1)
+    table = torch.randperm(n, generator=gen).view(B, S // P).to(torch.int64 if i64 else torch.int32)
+    pool = lambda seed: rand((n, P, Hkv, D), torch.bfloat16, seed)
+    dense = lambda seed: O.gather_paged(pool(seed), table).contiguous()
+    k, kt = (pool(2), table) if which & 1 else (dense(2), None)
+    v, vt = (pool(3), table) if which & 2 else (dense(3), None)
+    check(q, k, v, mask=mask, window=window, k_table=kt, v_table=vt)
+    assert lowering.attention.last_launch["kernels"] == ["lf_attn_prefill_swp"]
+
+
+def test_paged_prefill_falls_back_where_direct_loads_cannot_serve(monkeypatch):
+    B, Hq, Hkv, S, D = 2, 4, 4, 256, 128
+    q = rand((B, Hq, S, D), torch.bfloat16, 1)
+    for P in (1, 4):                       # pages smaller than the rows of one wave-level load
+        n = B * S // P
+        table = torch.randperm(n, generator=torch.Generator().manual_seed(P)).view(B, S // P).to(torch.int32)
+        shape = (n, P, Hkv, D) if P > 1 else (n, Hkv, D)
+        check(q, rand(shape, torch.bfloat16, 2), rand(shape, torch.bfloat16, 3), mask="causal", k_table=table, v_table=table)
+        assert lowering.attention.last_launch["kernels"] == ["lf_attn_prefill"]
+    monkeypatch.setenv("LOOPFUSE_PAGED_SWP", "0")
+    n = B * S // 16
+    table = torch.randperm(n, generator=torch.Generator().manual_seed(3)).view(B, S // 16).to(torch.int32)
+    check(q, rand((n, 16, Hkv, D), torch.bfloat16, 2), rand((n, 16, Hkv, D), torch.bfloat16, 3), mask="causal",
+          k_table=table, v_table=table)
+    assert lowering.attention.last_launch["kernels"] == ["lf_attn_prefill"]
+
+
 # ---------------------------------------------------------------- empty inputs
 def test_empty_inputs():
     dt, d = torch.bfloat16, dev()

@@ -67,14 +67,15 @@ def test_launch_geometry_checks(shim_built):
 def test_params_struct_layout():
     from loopfuse_amd.lowering import AttnParams
 
-    # 13 pointers, 24 int64 strides, 12 ints, 3 floats (+4 bytes tail padding to the 8-byte alignment)
+    # 13 pointers, 26 int64 strides / spans, 12 ints, 3 floats (+4 bytes tail padding to the 8-byte alignment)
     assert AttnParams.q.offset == 0 and AttnParams.q2.offset == 88 and AttnParams.q_sb.offset == 104
     assert AttnParams.q2_sb.offset == 104 + 144
-    assert AttnParams.B.offset == 104 + 192
-    assert AttnParams.k2_group.offset == 104 + 192 + 44
-    assert AttnParams.scale.offset == 104 + 192 + 48
-    assert AttnParams.denom_add.offset == 104 + 192 + 48 + 8
-    assert ctypes.sizeof(AttnParams) == 360
+    assert AttnParams.k_span.offset == 104 + 192
+    assert AttnParams.B.offset == 104 + 208
+    assert AttnParams.k2_group.offset == 104 + 208 + 44
+    assert AttnParams.scale.offset == 104 + 208 + 48
+    assert AttnParams.denom_add.offset == 104 + 208 + 48 + 8
+    assert ctypes.sizeof(AttnParams) == 376
 
 
 def test_c_header_matches_the_ctypes_mirror_and_the_device_struct(tmp_path):
