@@ -369,8 +369,10 @@ def test_paged_decode_page16_config5_shape():
     assert (got - want).abs().max() <= TOL
 
 
-def test_paged_pools_with_different_page_sizes():
-    # K pool in pages of 16 tokens, V pool in pages of 4, each with its own table
+@pytest.mark.parametrize("pv,kernel", [(4, "lf_attn_prefill"), (64, "lf_attn_prefill_swp")])
+def test_paged_pools_with_different_page_sizes(pv, kernel):
+    # K pool in pages of 16 tokens, V pool in pages of 4 (register-staged kernel) or 64
+    # (direct-to-LDS kernel), each with its own table
     def fn(Q, Kc, kt, Vc, vt):
         B = kt.shape[0]
         H, D = Kc.shape[2:]
@@ -381,13 +383,15 @@ def test_paged_pools_with_different_page_sizes():
 
     B, H, S, D = 2, 4, 512, 128
     g = torch.Generator().manual_seed(5)
-    Kc, Vc = rand((B * S // 16, 16, H, D), seed=1), rand((B * S // 4, 4, H, D), seed=2)
+    Kc, Vc = rand((B * S // 16, 16, H, D), seed=1), rand((B * S // pv, pv, H, D), seed=2)
     kt = torch.randperm(B * S // 16, generator=g).view(B, -1).to(torch.int32)
-    vt = torch.randperm(B * S // 4, generator=g).view(B, -1).to(torch.int32)
+    vt = torch.randperm(B * S // pv, generator=g).view(B, -1).to(torch.int32)
     Q = rand((B, H, S, D), seed=3)
     got = run_fused(fn, (Q, Kc, kt, Vc, vt))
     want = O.attention_reference(Q, Kc, Vc, mask="causal", k_table=kt, v_table=vt)
     assert (got - want).abs().max() <= TOL
+    from loopfuse_amd import lowering
+    assert lowering.attention.last_launch["kernels"] == [kernel]
 
 
 def test_static_shapes_at_baseline_sizes():
