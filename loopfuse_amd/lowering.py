@@ -398,7 +398,10 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     output is then not written): for timing the streaming kernel alone.
     ``choice`` overrides the launch heuristics (what ``tuned_attention`` searches over):
     ``{"prefill": "swp" | "w32"}``, ``{"head_per_wave": bool, "splits": n}``.
-    Returns O [B, Hq, Sq, D] (and the visited-tile record if asked).
+    Returns O [B, Hq, Sq, D] and, with ``record_visits``, the uint8 record of the KV tiles
+    each workgroup walked, ``[B * heads * q_tiles, kv_tiles]`` with ``heads = Hq`` and
+    128-row q tiles, or ``heads = Hq / 4`` and 32-row q tiles when query heads are packed
+    (``last_launch["heads_per_workgroup"] == 4``).
     """
     choice = choice or {}
     dtype = q.dtype
