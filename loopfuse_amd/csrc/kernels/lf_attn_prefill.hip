@@ -31,37 +31,25 @@
 #ifndef LF_VPF
 #define LF_VPF 4         /* V fragments (two transposed reads each) in flight */
 #endif
-#ifndef LF_SCHED
-#define LF_SCHED 0       /* 1: pin read/MFMA interleaving with sched_group_barrier (measured slower) */
-#endif
 #ifndef LF_KVBUF
 #define LF_KVBUF 1       /* dense K/V staged with range-checked buffer loads (needs < 2 GiB per (batch, head) span) */
 #endif
 #ifndef LF_DMA
-#define LF_DMA 0   /* 1 (needs LF_KVBUF, no LF_PAD): dense K/V tiles go global -> LDS directly
-                      (buffer_load ... lds through inline asm); parity-clean, no faster than the
-                      register path on the measured shapes, so off by default.
-                      2: the same, with the loads of the next tile issued one pass at a time
-                      between the MFMAs of the current tile instead of in a burst at the top */
+#define LF_DMA 0   /* 1 (needs LF_KVBUF): dense K/V tiles go global -> LDS directly (buffer_load ... lds
+                      through inline asm), which frees the staging registers; used where the kernel
+                      needs them for bias values or the second score product */
 #endif
-#define LF_DMA_SPREAD (LF_DMA == 2 && !LF_PAGED)
+#if LF_DMA > 1
+#error "LF_DMA is 0 or 1"
+#endif
 #define LF_DMA_K (LF_DMA && !(LF_PAGED & 1))
 #define LF_DMA_V (LF_DMA && !(LF_PAGED & 2))
-#ifndef LF_TIMING
-#define LF_TIMING 0      /* profiling aid: per-phase s_memtime totals of one wave into part_acc */
-#endif
-#ifndef LF_ABLATE
-#define LF_ABLATE 0      /* profiling aid: 1 = no softmax math, 2 = no staging/barrier, 4 = no PV, 8 = no QK^T (results are wrong) */
-#endif
 #ifndef LF_LAZY_LOG2
 #define LF_LAZY_LOG2 8   /* slack of the softmax exponent offset, log2 units */
 #endif
 
 #ifndef LF_D2
 #define LF_D2 0     /* depth of a second score product: S = Q K^T + Q2 K2^T (16, 32 or 64; 0 = none) */
-#endif
-#if LF_D2 && LF_DMA == 2
-#error "the second score product is staged through registers: LF_DMA 0 or 1"
 #endif
 
 #ifndef LF_BN
@@ -87,31 +75,15 @@
 #define LF_NKS2 (LF_D2 / 16)                 /* k-steps of the Q2 K2^T product */
 #define LF_RPS2 (LF_D2 ? 256 / (LF_D2 * 2) : 1)
 #define LF_NP2 ((LF_BN * LF_CPR2 + LF_NT - 1) / LF_NT)   /* staging passes of a K2 tile */
-// LDS row strides (elements).  LF_PAD: rows are padded instead of XOR-swizzled, so
-// every fragment address is one per-lane base plus a compile-time offset (no
-// per-fragment address arithmetic): +16 bytes per K row spreads 16 consecutive
-// rows over all 64 banks for ds_read_b128, +64 bytes per V row does the same for
-// the 4 rows x 64 bytes a transposed read touches.
-#ifndef LF_PAD
-#define LF_PAD 0
-#endif
-#if LF_PAD
-#define LF_KS (LF_D + 8)
-#define LF_VS (LF_D + 32)
-#else
+// LDS row strides (elements): rows are not padded, the tiles are XOR-swizzled
 #define LF_KS LF_D
 #define LF_VS LF_D
-#endif
 
 // Physical 16-byte chunk of logical chunk `ch` in row `row` of the K tile: rows
 // that a ds_read_b128 touches together (16 consecutive rows, same logical chunk)
 // land in 16 different chunks, i.e. on all 64 banks.
 __device__ __forceinline__ int lf_k_phys(int row, int ch) {
-#if LF_PAD
-  return ch;
-#else
   return ch ^ ((row / LF_RPS) & (LF_CPR - 1));
-#endif
 }
 #if LF_D2
 // The K2 tile (rows of LF_D2 elements, several rows per 256-byte bank span): the same
@@ -123,11 +95,7 @@ __device__ __forceinline__ int lf_k2_phys(int row, int ch) {
 // Same for the V tile, where a transposed read touches 4 consecutive rows x 64
 // contiguous bytes per 32 lanes: permute the 64-byte groups by the row.
 __device__ __forceinline__ int lf_v_phys(int row, int ch) {
-#if LF_PAD
-  return ch;
-#else
   return ch ^ (4 * ((row / LF_RPS) & (LF_CPR / 4 - 1)));
-#endif
 }
 
 extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(const LfAttnParams p) {
@@ -295,16 +263,6 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                  :: "s"(m0v), "v"(voff), "s"(rs) : "memory");
   };
-  // one staging pass (LF_BN / LF_NPASS rows) of tile kt into buffer buf; rows past
-  // Sk arrive as zeros, so a tile index past the last tile is harmless
-  auto dma_k_pass = [&](int kt, int buf, int ps) {
-    dma(k_rsq, k_doff + (unsigned)(kt * LF_BN + kRowsPerPass * ps) * k_rowb,
-        &lds_k[buf][(kRowsPerPass * ps + kRowsPerWave * wave) * LF_KS]);
-  };
-  auto dma_v_pass = [&](int kt, int buf, int ps) {
-    dma(v_rsq, v_doff + (unsigned)(kt * LF_BN + kRowsPerPass * ps) * v_rowb,
-        &lds_v[buf][(kRowsPerPass * ps + kRowsPerWave * wave) * LF_VS]);
-  };
 #endif
   auto load_tile = [&](int kt, int buf) {
 #pragma unroll
@@ -380,19 +338,10 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
   store_tile(0);
   __syncthreads();
 
-#if LF_TIMING
-  unsigned long long tacc[6] = {0, 0, 0, 0, 0, 0};
-#define LF_T(i) { unsigned long long now_ = __builtin_amdgcn_s_memtime(); tacc[i] += now_ - tprev; tprev = now_; }
-  unsigned long long tprev = __builtin_amdgcn_s_memtime();
-#else
-#define LF_T(i)
-#endif
   for (int kt = kt_begin; kt < kt_end; ++kt) {
     const int cur = (kt - kt_begin) & 1;
     const bool have_next = kt + 1 < kt_end;
-#if !(LF_ABLATE & 2) && !LF_DMA_SPREAD
     if (have_next) load_tile(kt + 1, cur ^ 1);
-#endif
 
     const int k0 = kt * LF_BN;
     bool need = wave_has_rows;
@@ -406,7 +355,6 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
     full = full && (wq0 + 31 - k0 < p.window);
 #endif
 
-    LF_T(0)
     if (need) {
       const lf_elem* kbuf = lds_k[cur];
       const lf_elem* vbuf = lds_v[cur];
@@ -424,7 +372,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
       {
         // K fragments are fetched LF_KPF MFMAs ahead of their use: the LDS round
         // trip (well over 100 cycles) spans several 32-cycle MFMAs
-        constexpr int kNF = ((LF_ABLATE & 8) ? 0 : LF_NKS * LF_NKB);
+        constexpr int kNF = (LF_NKS * LF_NKB);
         lf_u32x4 kf[kNF > 0 ? kNF : 1];
         auto k_frag = [&](int f) {
           const int ks = f / LF_NKB, kb = f % LF_NKB;
@@ -432,14 +380,11 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
           return *reinterpret_cast<const lf_u32x4*>(&kbuf[row * LF_KS + 8 * lf_k_phys(row, 2 * ks + g)]);
         };
 #pragma unroll
-        for (int f = 0; f < LF_KPF && f < kNF; ++f) kf[f] = (LF_ABLATE & 16) ? __builtin_bit_cast(lf_u32x4, qf[f % LF_NKS]) : k_frag(f);
+        for (int f = 0; f < LF_KPF && f < kNF; ++f) kf[f] = k_frag(f);
 #pragma unroll
         for (int f = 0; f < kNF; ++f) {
-          if (f + LF_KPF < kNF) kf[f + LF_KPF] = (LF_ABLATE & 16) ? __builtin_bit_cast(lf_u32x4, qf[f % LF_NKS]) : k_frag(f + LF_KPF);
+          if (f + LF_KPF < kNF) kf[f + LF_KPF] = k_frag(f + LF_KPF);
           s[f % LF_NKB] = lf_mfma32(__builtin_bit_cast(lf_elem8, kf[f]), qf[f / LF_NKB], s[f % LF_NKB]);
-#if LF_DMA_SPREAD
-          if (f % (kNF / LF_NPASS) == 1) dma_k_pass(kt + 1, cur ^ 1, f / (kNF / LF_NPASS));
-#endif
         }
 #if LF_D2
         // + Q2 K2^T into the same accumulators
@@ -454,25 +399,11 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
           }
         }
 #endif
-#if LF_SCHED
-        // pin the order: LF_KPF reads, then (MFMA, read) pairs, then the last MFMAs
-        __builtin_amdgcn_sched_group_barrier(0x100, LF_KPF, 0);
-#pragma unroll
-        for (int f = 0; f < kNF - LF_KPF; ++f) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, LF_KPF, 0);
-#endif
       }
 #if LF_SETPRIO
       __builtin_amdgcn_s_setprio(0);
 #endif
 
-#if LF_TIMING
-      asm volatile("" :: "v"(s[0][0]), "v"(s[LF_NKB - 1][15]));   // results needed here
-#endif
-      LF_T(1)
       // ---- score modifications and mask; element i of block kb is kv index
       // j = k0 + 32*kb + 8*(i/4) + 4*g + i%4, query my_q.
 #if LF_SOFTCAP && !(LF_BIAS & 1)
@@ -541,13 +472,11 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
       // slack -- a wave-uniform branch that is rarely taken after the first tiles.
       // O / l is independent of the offset, so the result is unchanged.
       float mx = LF_NEG_INF;
-#if !(LF_ABLATE & 1)
 #pragma unroll
       for (int kb = 0; kb < LF_NKB; ++kb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kb][i]);
       mx = fmaxf(mx, lf_swap32(mx));
-#endif
       const float mxc = mx * cexp;
 #if LF_DENOM
       mc_true = fmaxf(mc_true, mxc);
@@ -573,24 +502,19 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
       for (int kb = 0; kb < LF_NKB; ++kb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-#if LF_ABLATE & 1
-          float e = s[kb][i];
-#else
           float e = lf_exp2(s[kb][i] * cexp - mc_sub);
-#endif
           rs += e;
           pf[2 * kb + i / 8][i % 8] = lf_from_float(e);
         }
       l_run += rs;
 
-      LF_T(2)
 #if LF_SETPRIO
       __builtin_amdgcn_s_setprio(2);
 #endif
       // ---- O^T += V^T P^T.  k-slot s of step kk is kv row
       // 16*kk + 8*(s/4) + 4*g + s%4 (the order P is held in); A row = d.
       {
-        constexpr int kNF = ((LF_ABLATE & 4) ? 0 : LF_NKK * LF_NDB);
+        constexpr int kNF = (LF_NKK * LF_NDB);
         lf_elem8 vf[kNF > 0 ? kNF : 1];
         auto v_frag = [&](int f) {
           const int kk = f / LF_NDB, db = f % LF_NDB;
@@ -625,56 +549,21 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
           return a;
         };
 #pragma unroll
-        for (int f = 0; f < LF_VPF && f < kNF; ++f) vf[f] = (LF_ABLATE & 32) ? qf[f % LF_NKS] : v_frag(f);
+        for (int f = 0; f < LF_VPF && f < kNF; ++f) vf[f] = v_frag(f);
 #pragma unroll
         for (int f = 0; f < kNF; ++f) {
-          if (f + LF_VPF < kNF) vf[f + LF_VPF] = (LF_ABLATE & 32) ? qf[f % LF_NKS] : v_frag(f + LF_VPF);
+          if (f + LF_VPF < kNF) vf[f + LF_VPF] = v_frag(f + LF_VPF);
           o[f % LF_NDB] = lf_mfma32(vf[f], pf[f / LF_NDB], o[f % LF_NDB]);
-#if LF_DMA_SPREAD
-          if (f % (kNF / LF_NPASS) == 1) dma_v_pass(kt + 1, cur ^ 1, f / (kNF / LF_NPASS));
-#endif
         }
-#if LF_SCHED && LF_V_TR
-        __builtin_amdgcn_sched_group_barrier(0x100, 2 * LF_VPF, 0);
-#pragma unroll
-        for (int f = 0; f < kNF - LF_VPF; ++f) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, LF_VPF, 0);
-#endif
       }
 #if LF_SETPRIO
       __builtin_amdgcn_s_setprio(0);
 #endif
     }
-#if LF_DMA_SPREAD
-    else {
-#pragma unroll
-      for (int ps = 0; ps < LF_NPASS; ++ps) {
-        dma_k_pass(kt + 1, cur ^ 1, ps);
-        dma_v_pass(kt + 1, cur ^ 1, ps);
-      }
-    }
-#endif
 
-#if LF_TIMING
-    asm volatile("" :: "v"(o[0][0]), "v"(o[LF_NDB - 1][15]));
-#endif
-    LF_T(3)
-#if !(LF_ABLATE & 2)
-    if (have_next || LF_DMA_SPREAD) store_tile(cur ^ 1);
-    LF_T(4)
+    if (have_next) store_tile(cur ^ 1);
     __syncthreads();
-    LF_T(5)
-#endif
   }
-#if LF_TIMING
-  if (blockIdx.x == 8 * 5 && tid == 0 && p.part_acc != nullptr) {
-    for (int i = 0; i < 6; ++i) p.part_acc[i] += (float)tacc[i];
-    p.part_acc[6] += (float)(kt_end - kt_begin);
-  }
-#endif
 
   // ---- epilogue: O[q][d] = O^T[d][q] / l.  Element i of block db is
   // d = 32*db + 8*(i/4) + 4*g + i%4.

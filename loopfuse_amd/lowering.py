@@ -589,9 +589,6 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         spec = KernelSpec(family, _DTYPE_CODE[dtype], D, mask, plan.softcap is not None, paged,
                           page_size, table_i64, v_tr=v_tr if family == "prefill" else True, bias=bias_bits,
                           denom=plan.denom_add != 0.0, d2=d2, page_size_v=page_size_v, pack=bool(pack), extra=extra)
-        if os.environ.get("LOOPFUSE_TIMING"):       # profiling aid, see LF_TIMING in the kernel
-            attention.timing = torch.zeros(16, dtype=torch.float32, device=q.device)
-            P.part_acc = attention.timing.data_ptr()
         bm, bn = TILE_SHAPES[family]
         nw = 4
         for e in spec.extra:                    # tuning: -DLF_NW=8 doubles the q tile
