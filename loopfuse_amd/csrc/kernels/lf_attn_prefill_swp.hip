@@ -32,10 +32,7 @@
 #define LF_VPF 4         /* V fragments (two transposed reads each) in flight */
 #endif
 #ifndef LF_SETPRIO
-#define LF_SETPRIO 1     /* 1: raise the wave priority while it issues MFMAs; 2: static, by workgroup:
-                            the workgroup whose LDS allocation starts at 0 runs at low priority, the
-                            one above it at high priority, which keeps the two workgroups of a CU out
-                            of phase (one in its MFMAs while the other is in its softmax) */
+#define LF_SETPRIO 1     /* raise the wave priority while it issues MFMAs */
 #endif
 #ifndef LF_ABLATE
 #define LF_ABLATE 0      /* profiling aid (wrong results): 1 no exp, 2 no direct loads, 4 no O store, 8 no Q load, 16 no K reads,
@@ -97,11 +94,6 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
   const int wave = tid >> 6;
   const int l32 = lane & 31;
   const int g = lane >> 5;
-#if LF_SETPRIO == 2
-  // hardware register LDS_ALLOC (id 6), field LDS_BASE (low 12 bits read here)
-  if ((__builtin_amdgcn_s_getreg((11 << 11) | 6) & 0xfff) != 0) __builtin_amdgcn_s_setprio(3);
-  else __builtin_amdgcn_s_setprio(0);
-#endif
 
   // ---- workgroup -> (batch*head, pair of q tiles), as in lf_attn_prefill.hip
   const int nqt = (p.Sq + LF_BM - 1) / LF_BM;
@@ -394,7 +386,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
         lf_elem8 vf[LF_NFV];
 #pragma unroll
         for (int f = 0; f < LF_KPF; ++f) kf[f] = kpre[f];
-#if LF_SETPRIO == 1
+#if LF_SETPRIO
         __builtin_amdgcn_s_setprio(2);
 #endif
         __builtin_amdgcn_sched_barrier(0);
@@ -406,7 +398,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
           s[f % LF_NKB] = lf_mfma32(__builtin_bit_cast(lf_elem8, kf[f]), qf[f / LF_NKB], s[f % LF_NKB]);
           __builtin_amdgcn_sched_barrier(0);
         }
-#if LF_SETPRIO == 1
+#if LF_SETPRIO
         __builtin_amdgcn_s_setprio(0);
 #endif
 
@@ -471,7 +463,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
         l_run += rs;
 
         // ---- O^T += V^T P^T; the last steps also read the first fragments of K(kt+1)
-#if LF_SETPRIO == 1
+#if LF_SETPRIO
         __builtin_amdgcn_s_setprio(2);
 #endif
         __builtin_amdgcn_sched_barrier(0);
@@ -482,7 +474,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
           o[f % LF_NDB] = lf_mfma32(vf[f], pf[f / LF_NDB], o[f % LF_NDB]);
           __builtin_amdgcn_sched_barrier(0);
         }
-#if LF_SETPRIO == 1
+#if LF_SETPRIO
         __builtin_amdgcn_s_setprio(0);
 #endif
       } else {
