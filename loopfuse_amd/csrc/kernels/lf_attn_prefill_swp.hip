@@ -44,15 +44,16 @@
 #endif
 #define LF_NT (LF_NW * 64)
 #ifndef LF_GQAPACK
-#define LF_GQAPACK 0     /* 1 (grouped-query attention, Hq / Hkv a multiple of LF_NW): the waves of a workgroup
-                            take the same 32 query rows of LF_NW consecutive query heads that share one kv head,
-                            instead of LF_NW blocks of 32 rows of one head: a q tile is then 32 rows tall, every
-                            wave needs exactly the same KV tiles (no wave idles on a tile of the diagonal or of
-                            the window's edge), and one K/V tile in LDS serves LF_NW heads */
+#define LF_GQAPACK 0     /* g = 2 or 4 (grouped-query attention, Hq / Hkv a multiple of g): the waves of a
+                            workgroup take the same query rows of g consecutive query heads that share one kv
+                            head -- wave w: head w % g, row block w / g -- instead of LF_NW row blocks of one
+                            head.  A q tile is then 32 * LF_NW / g rows tall; with g = LF_NW every wave needs
+                            exactly the same KV tiles (no wave idles on a tile of the diagonal or of the
+                            window's edge), and one K/V tile in LDS serves g heads */
 #endif
 #if LF_GQAPACK
-#define LF_BM 32
-#define LF_HEADS_PER_WG LF_NW
+#define LF_BM (32 * LF_NW / LF_GQAPACK)
+#define LF_HEADS_PER_WG LF_GQAPACK
 #else
 #define LF_BM (32 * LF_NW)
 #define LF_HEADS_PER_WG 1
@@ -111,7 +112,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
   const int pair = in_grp >> 2;
   const int b = bh / nhv;
 #if LF_GQAPACK
-  const int h = (bh % nhv) * LF_NW + wave;    // this wave's query head
+  const int h = (bh % nhv) * LF_GQAPACK + wave % LF_GQAPACK;    // this wave's query head
 #else
   const int h = bh % nhv;
 #endif
@@ -271,7 +272,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
         p.visits[((long long)bh * nqt + qt) * nkt + kt] = 1;
     }
 
-    const int wq0 = LF_GQAPACK ? q0 : q0 + 32 * wave;
+    const int wq0 = q0 + 32 * (LF_GQAPACK ? wave / LF_GQAPACK : wave);
     const int wqlast = min(wq0 + 31, p.Sq - 1);
     const bool wave_has_rows = wq0 < p.Sq;
     const int my_q = wq0 + l32;

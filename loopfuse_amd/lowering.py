@@ -71,7 +71,7 @@ class KernelSpec:
     headwave: bool = False  # decode: one kv head per wave (8 waves) instead of 4 waves sharing a head
     denom: bool = False    # prefill: softmax denominator sum + c (c a run-time parameter)
     bias: int = 0          # prefill: bit 0 additive score bias tensor, bit 1 additive output bias tensor, bit 2 unaligned rows
-    pack: bool = False     # prefill_swp, grouped-query attention: a workgroup's waves take 4 heads of one group
+    pack: int = 0          # prefill_swp, grouped-query attention: a workgroup's waves take 2 or 4 heads of one group
     page_size_v: int = 0   # tokens per page of the V pool when it differs from K's (0 = same)
     d2: int = 0            # prefill: depth of a second score product Q2 K2^T (0, 16, 32, 64)
     extra: tuple = ()      # further -D options (tuning experiments)
@@ -95,7 +95,7 @@ class KernelSpec:
             if self.d2:
                 o += [f"-DLF_D2={self.d2}"]
         elif self.family == "prefill_swp" and self.pack:
-            o += ["-DLF_GQAPACK=1"]
+            o += [f"-DLF_GQAPACK={int(self.pack)}"]
         return o + list(self.extra)
 
     def files(self) -> tuple[str, ...]:
@@ -109,7 +109,7 @@ class KernelSpec:
     def name(self) -> str:
         return (f"lf_{self.family}_t{self.dtype}_d{self.head_dim}_m{self.mask}_c{int(self.softcap)}"
                 f"_p{self.paged}x{self.page_size}i{int(self.table_i64)}_r{self.rows}w{self.waves}v{int(self.v_tr)}h{int(self.headwave)}b{self.bias}n{int(self.denom)}"
-                + (f"_q{self.d2}" if self.d2 else "") + ("_gp" if self.pack else "") + (f"_pv{self.page_size_v}" if self.page_size_v else "")
+                + (f"_q{self.d2}" if self.d2 else "") + (f"_gp{int(self.pack)}" if self.pack else "") + (f"_pv{self.page_size_v}" if self.page_size_v else "")
                 + "".join("_" + e.replace("-D", "").replace("=", "") for e in self.extra))
 
     def source(self) -> str:
@@ -341,7 +341,7 @@ def tuned_attention(q, k, v, plan: AttnPlan, k_table=None, v_table=None, **kw):
                      for sp in (None, 1, 2, 4, 8)]
         elif not (plan.k_paged or plan.v_paged):
             cands = [{"prefill": "swp"}, {"prefill": "w32"}]
-            if group % 4 == 0:
+            if group % 2 == 0:
                 cands.insert(1, {"prefill": "swp", "pack": False})
         else:
             cands = [{}]
@@ -400,8 +400,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     ``{"prefill": "swp" | "w32"}``, ``{"head_per_wave": bool, "splits": n}``.
     Returns O [B, Hq, Sq, D] and, with ``record_visits``, the uint8 record of the KV tiles
     each workgroup walked, ``[B * heads * q_tiles, kv_tiles]`` with ``heads = Hq`` and
-    128-row q tiles, or ``heads = Hq / 4`` and 32-row q tiles when query heads are packed
-    (``last_launch["heads_per_workgroup"] == 4``).
+    128-row q tiles, or ``heads = Hq / g`` and ``128 / g``-row q tiles when g = 2 or 4 query heads
+    are packed (``last_launch["heads_per_workgroup"] == g``).
     """
     choice = choice or {}
     dtype = q.dtype
@@ -582,13 +582,15 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
             extra += ("-DLF_KVBUF=0",)
         elif family == "prefill" and (bias_bits or d2) and not paged:
             extra += ("-DLF_DMA=1",)     # frees the staging registers the bias values / Q2 fragments need
-        # grouped-query attention: the 4 waves of a workgroup take 4 query heads of one group
-        # (same 32 rows) and share every K/V tile in LDS
-        pack = family == "prefill_swp" and group % 4 == 0 and not any(e.startswith("-DLF_NW=") for e in extra) and \
-            choice.get("pack", os.environ.get("LOOPFUSE_GQAPACK", "1") == "1")
+        # grouped-query attention: the 4 waves of a workgroup take 4 (or 2) query heads of one
+        # group over the same query rows and share every K/V tile in LDS
+        pack = 0
+        if family == "prefill_swp" and group % 2 == 0 and not any(e.startswith("-DLF_NW=") for e in extra) and \
+                choice.get("pack", os.environ.get("LOOPFUSE_GQAPACK", "1") == "1"):
+            pack = 4 if group % 4 == 0 else 2
         spec = KernelSpec(family, _DTYPE_CODE[dtype], D, mask, plan.softcap is not None, paged,
                           page_size, table_i64, v_tr=v_tr if family == "prefill" else True, bias=bias_bits,
-                          denom=plan.denom_add != 0.0, d2=d2, page_size_v=page_size_v, pack=bool(pack), extra=extra)
+                          denom=plan.denom_add != 0.0, d2=d2, page_size_v=page_size_v, pack=pack, extra=extra)
         bm, bn = TILE_SHAPES[family]
         nw = 4
         for e in spec.extra:                    # tuning: -DLF_NW=8 doubles the q tile
@@ -597,7 +599,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
                 bm = 32 * nw
         heads = Hq
         if spec.pack:
-            bm, heads = 32, Hq // 4          # q tiles of 32 rows x 4 heads
+            bm, heads = 128 // spec.pack, Hq // spec.pack      # q tiles of 32 rows x 4 heads, or 64 rows x 2 heads
         nqt = (Sq + bm - 1) // bm
         nkt = (Sk + bn - 1) // bn
         visits = None
@@ -614,7 +616,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
             grid = min(grid, 8 * int(persist))
         get_kernel(spec, spec.entry()).launch((grid, 1, 1), (64 * nw, 1, 1), P)
         attention.last_launch = {"kernels": [spec.entry()], "grid": grid, "block": 64 * nw, "q_tile_rows": bm,
-                                 "heads_per_workgroup": 4 if spec.pack else 1}
+                                 "heads_per_workgroup": spec.pack or 1}
         return (out, visits) if record_visits else out
 
     if family != "decode":

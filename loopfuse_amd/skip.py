@@ -17,7 +17,8 @@ from __future__ import annotations
 # (query rows per workgroup, KV rows per LDS tile) of each prefill kernel
 TILE_SHAPES = {
     "prefill": (128, 64),        # lf_attn_prefill: 4 waves x 32 rows, two waves per SIMD
-    "prefill_swp_pack": (32, 64),   # lf_attn_prefill_swp -DLF_GQAPACK=1: 32 rows x 4 query heads of one group
+    "prefill_swp_pack": (32, 64),   # lf_attn_prefill_swp -DLF_GQAPACK=4: 32 rows x 4 query heads of one group
+    "prefill_swp_pack2": (64, 64),  # lf_attn_prefill_swp -DLF_GQAPACK=2: 64 rows x 2 query heads of one group
     "prefill_swp": (128, 64),    # lf_attn_prefill_swp: 4 waves x 32 rows, direct-to-LDS staging, reads issued ahead
 }
 PREFILL_BM, PREFILL_BN = TILE_SHAPES["prefill"]

@@ -349,10 +349,12 @@ class AttentionMatch:
             raise lowering.UnsupportedPlan("depth of the second score product not served by the HIP kernels")
         family = "prefill" if (paged or bias or d2) else lowering.prefill_variant(q.shape[-2])
         extra = ("-DLF_DMA=1",) if ((bias or d2) and not paged) else ()
-        pack = False
+        pack = 0
         if family == "prefill_swp":
             kd, _ = self._operand(self.k, vals)
-            pack = (q.shape[1] // max(kd.shape[1], 1)) % 4 == 0 and q.shape[1] % max(kd.shape[1], 1) == 0
+            grp = q.shape[1] // max(kd.shape[1], 1)
+            if q.shape[1] % max(kd.shape[1], 1) == 0 and grp % 2 == 0:
+                pack = 4 if grp % 4 == 0 else 2
         return [lowering.KernelSpec(family, dt, D, mask, plan.softcap is not None, paged, ps, i64, bias=bias, d2=d2,
                                     page_size_v=psv, pack=pack, extra=extra)]
 

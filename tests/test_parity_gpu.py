@@ -338,21 +338,22 @@ def test_visited_tiles_bit_exact(mask, window, S, variant, monkeypatch):
     assert torch.equal(host, dense)
 
 
+@pytest.mark.parametrize("g", [4, 2])
 @pytest.mark.parametrize("mask,window,S", [("causal", 0, 593), ("sliding", 256, 2048), ("sliding", 100, 700), (None, 0, 300)])
-def test_visited_tiles_bit_exact_with_packed_query_heads(mask, window, S):
-    """Grouped-query attention: a workgroup takes 32 rows of 4 query heads of one group; its
-    walked KV tiles == tiles with any unmasked score for those 32 rows."""
-    bm, bn = skip.TILE_SHAPES["prefill_swp_pack"]
+def test_visited_tiles_bit_exact_with_packed_query_heads(mask, window, S, g):
+    """Grouped-query attention: a workgroup takes 32 rows of 4 query heads (or 64 rows of 2) of
+    one group; its walked KV tiles == tiles with any unmasked score for those rows."""
+    bm, bn = skip.TILE_SHAPES["prefill_swp_pack" if g == 4 else "prefill_swp_pack2"]
     q = rand((2, 8, S, 128), torch.bfloat16, 1).to(dev())
-    k, v = (rand((2, 2, S, 128), torch.bfloat16, s).to(dev()) for s in (2, 3))
+    k, v = (rand((2, 8 // g, S, 128), torch.bfloat16, s).to(dev()) for s in (2, 3))
     plan = lowering.AttnPlan(mask=mask, window=window, scale=128 ** -0.5)
     out, visits = lowering.attention(q, k, v, plan, record_visits=True)
     torch.cuda.synchronize()
-    assert lowering.attention.last_launch["heads_per_workgroup"] == 4 and lowering.attention.last_launch["q_tile_rows"] == 32
+    assert lowering.attention.last_launch["heads_per_workgroup"] == g and lowering.attention.last_launch["q_tile_rows"] == bm
     nqt = skip.cdiv(S, bm)
-    visits = visits.cpu().view(2 * 2, nqt, -1).bool()          # (batch x packs of 4 heads, q tile, kv tile)
+    visits = visits.cpu().view(2 * (8 // g), nqt, -1).bool()   # (batch x packs of g heads, q tile, kv tile)
     dense = O.visited_tiles_dense(mask, S, S, window, bm, bn)
-    for u in range(4):
+    for u in range(2 * (8 // g)):
         assert torch.equal(visits[u], dense)
     want = O.attention_reference(q.cpu(), k.cpu(), v.cpu(), mask=mask, window=window)
     assert (out.float().cpu() - want).abs().max().item() <= TOL[torch.bfloat16]
