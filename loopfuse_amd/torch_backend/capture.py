@@ -73,6 +73,9 @@ class Ids:
 class Scalar:
     node: torch.fx.Node            # re-evaluated at call time
     value: float                   # value for the stand-in sizes (unused beyond sanity)
+    # how to compute it in plain Python at call time, if every step is understood:
+    # ("lit", x) | ("arg", fx node holding a number) | ("op", name, operand, ...); None = run the node
+    expr: Any = None
 
 
 @dataclasses.dataclass
@@ -217,6 +220,8 @@ class AttentionMatch:
     def _number(x, vals) -> float:
         if isinstance(x, tuple) and x[0] == "recip":
             return 1.0 / AttentionMatch._number(x[1], vals)
+        if isinstance(x, tuple) and x[0] == "expr":
+            return _eval_scalar(x[1], lambda i: AttentionMatch._number(("arg", i), vals))
         if isinstance(x, tuple) and x[0] == "arg":
             x = vals[x[1]]
         return float(x.item() if isinstance(x, torch.Tensor) else x)
@@ -495,11 +500,79 @@ def _regroup(real_in, real_out, stand_in, stand_out_hint):
     return out
 
 
+_SCALAR_BINARY = {aten.mul.Tensor: "mul", aten.div.Tensor: "div", aten.add.Tensor: "add", aten.sub.Tensor: "sub",
+                  aten.pow.Tensor_Tensor: "pow", aten.pow.Tensor_Scalar: "pow"}
+_SCALAR_UNARY = {aten.reciprocal.default: "recip", aten.sqrt.default: "sqrt", aten.rsqrt.default: "rsqrt",
+                 aten.neg.default: "neg"}
+
+
+def _scalar_expr(node: torch.fx.Node, tgt, a, kw):
+    """Python-evaluable form of a 0-dim computation on shape-derived values, or None."""
+    def operand(i):
+        x = a[i]
+        if isinstance(x, Scalar):
+            return x.expr
+        raw = node.args[i]
+        if isinstance(raw, torch.fx.Node):
+            return ("arg", raw)
+        return ("lit", float(x)) if isinstance(x, (int, float)) and not isinstance(x, bool) else None
+
+    if tgt in _CAST_OPS or tgt in (aten.clone.default, aten.alias.default, aten.detach.default):
+        return operand(0)
+    if tgt in _SCALAR_BINARY and len(a) >= 2 and kw.get("alpha", 1) == 1:
+        x, y = operand(0), operand(1)
+        return None if x is None or y is None else ("op", _SCALAR_BINARY[tgt], x, y)
+    if tgt in _SCALAR_UNARY:
+        x = operand(0)
+        return None if x is None else ("op", _SCALAR_UNARY[tgt], x)
+    return None
+
+
+def _eval_scalar(e, leaf) -> float:
+    kind = e[0]
+    if kind == "lit":
+        return float(e[1])
+    if kind == "arg":
+        return float(leaf(e[1]))
+    name, xs = e[1], [_eval_scalar(x, leaf) for x in e[2:]]
+    if name == "mul":
+        return xs[0] * xs[1]
+    if name == "div":
+        return xs[0] / xs[1]
+    if name == "add":
+        return xs[0] + xs[1]
+    if name == "sub":
+        return xs[0] - xs[1]
+    if name == "pow":
+        return xs[0] ** xs[1]
+    if name == "recip":
+        return 1.0 / xs[0]
+    if name == "sqrt":
+        return math.sqrt(xs[0])
+    if name == "rsqrt":
+        return 1.0 / math.sqrt(xs[0])
+    if name == "neg":
+        return -xs[0]
+    raise ValueError(name)
+
+
+def _same_expr(x, y) -> bool:
+    if x is None or y is None or x[0] != y[0]:
+        return False
+    if x[0] == "lit":
+        return x[1] == y[1]
+    if x[0] == "arg":
+        return x[1] is y[1]
+    return x[1] == y[1] and len(x) == len(y) and all(_same_expr(p, q) for p, q in zip(x[2:], y[2:]))
+
+
 def _same_scalar(x, y) -> bool:
     """Two score factors (numbers, graph nodes, ("recip", f)) that are the same value by
     construction: identical, or the same pure computation on the same inputs."""
     if x is y:
         return True
+    if isinstance(x, Scalar) and isinstance(y, Scalar):
+        return _same_expr(x.expr, y.expr) or _same_scalar(x.node, y.node)
     if isinstance(x, tuple) and isinstance(y, tuple):
         return len(x) == len(y) and all(_same_scalar(a, b) for a, b in zip(x, y))
     if isinstance(x, torch.fx.Node) and isinstance(y, torch.fx.Node):
@@ -643,7 +716,7 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
     def fresh_ids(node: torch.fx.Node, val) -> Any:
         """A tensor-valued node that simply runs: ids over its own (stand-in) shape."""
         if val.dim() == 0:
-            return Scalar(node, 1.0)       # e.g. a Python float that dynamo passes as a 0-dim tensor
+            return Scalar(node, 1.0, ("arg", node))    # e.g. a Python float that dynamo passes as a 0-dim tensor
         shape = tuple(concrete(d) for d in val.shape)
         n = math.prod(shape)
         if n > CAP:
@@ -658,7 +731,7 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
         elif isinstance(val, (torch.SymInt, int)):
             env[p] = concrete(val)
         elif isinstance(val, (torch.SymFloat, float)):
-            env[p] = Scalar(p, float(val) if isinstance(val, float) else 1.0)
+            env[p] = Scalar(p, float(val) if isinstance(val, float) else 1.0, ("arg", p))
         else:
             raise NoMatch(f"unsupported placeholder {p.name}")
 
@@ -710,12 +783,13 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
 
         # -- scalars derived from sizes
         if tgt is aten.scalar_tensor.default and is_number(a[0]):
-            return Scalar(node, float(a[0]))
+            raw0 = node.args[0]
+            return Scalar(node, float(a[0]), ("arg", raw0) if isinstance(raw0, torch.fx.Node) else ("lit", float(a[0])))
         val = node.meta.get("val")
         if isinstance(first, Scalar) and isinstance(val, torch.Tensor) and val.dim() == 0 and all(
                 isinstance(x, (Scalar, int, float, bool, str, torch.dtype, type(None)))
                 for x in list(a) + list(kw.values())):
-            return Scalar(node, 1.0)       # any arithmetic among shape-derived 0-dim values
+            return Scalar(node, 1.0, _scalar_expr(node, tgt, a, kw))   # any arithmetic among shape-derived 0-dim values
 
         # -- explicit softmax by-products (running / final max, their gap, the denominator)
         if tgt is operator.getitem and isinstance(first, list) and isinstance(a[1], int):
@@ -730,7 +804,7 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
             if tgt is aten.add.Tensor and x.kind == "den" and kw.get("alpha", 1) == 1 and (
                     (is_number(a[1]) and a[1] >= 0) or isinstance(a[1], Scalar)):
                 raw = node.args[1]
-                term = a[1].node if isinstance(a[1], Scalar) else (raw if isinstance(raw, torch.fx.Node) else float(a[1]))
+                term = a[1] if isinstance(a[1], Scalar) else (raw if isinstance(raw, torch.fx.Node) else float(a[1]))
                 return Aux("den", x.uid, c=x.c + (term,))
             if tgt is aten.mul.Tensor and x.kind == "expgap" and isinstance(a[1], Stage):
                 a = (a[1], a[0])            # handled below with the stage first
@@ -843,7 +917,7 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
                         and (isinstance(a[1], Scalar) or (is_number(a[1]) and (a[1] > 0 or isinstance(node.args[1], torch.fx.Node)))):
                     raw = node.args[1]
                     if isinstance(a[1], Scalar):
-                        f = a[1].node
+                        f = a[1]
                     else:
                         f = raw if isinstance(raw, torch.fx.Node) else float(a[1])
                     if tgt is aten.div.Tensor:
@@ -881,7 +955,7 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
                     other = a[1]
                     raw = node.args[1]
                     if isinstance(other, Scalar):
-                        f = other.node
+                        f = other
                     elif is_number(other):
                         f = raw if isinstance(raw, torch.fx.Node) else float(other)
                     else:
@@ -947,7 +1021,7 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
         elif isinstance(val, (torch.SymInt, int)) and not isinstance(val, bool):
             env[node] = concrete(val)
         elif isinstance(val, (torch.SymFloat, float)):
-            env[node] = Scalar(node, 1.0)
+            env[node] = Scalar(node, 1.0, ("arg", node))
         else:
             env[node] = None
 
@@ -1012,6 +1086,15 @@ def _build_match(out_node: torch.fx.Node, st: Stage) -> AttentionMatch:
     def scalar(f):
         if isinstance(f, tuple) and f[0] == "recip":
             return ("recip", scalar(f[1]))
+        if isinstance(f, Scalar):
+            if f.expr is None:
+                return ("arg", slot(f.node))        # not understood: the graph computes it, the call reads it
+
+            def conv(e):
+                if e[0] == "arg":
+                    return ("arg", slot(e[1]))
+                return e if e[0] == "lit" else e[:2] + tuple(conv(x) for x in e[2:])
+            return ("expr", conv(f.expr))
         if isinstance(f, torch.fx.Node):
             return ("arg", slot(f))
         return f
