@@ -151,16 +151,19 @@ def compile_spec(spec: KernelSpec, arch: str = runtime.DEFAULT_ARCH) -> Compiled
     """hipRTC-compile (or fetch from the on-disk cache) one specialisation.  Needs no GPU."""
     with _lock:
         ck = _compiled.get(spec)
-        override = os.environ.get("LOOPFUSE_HSACO_" + spec.family.upper())   # tuning aid: prebuilt code object
-        if ck is None and override:
-            with open(override, "rb") as fh:
-                ck = CompiledKernel(spec, fh.read(), False, "override " + override)
-            _compiled[spec] = ck
-        if ck is None:
-            code, hit, log = runtime.compile_source(spec.source(), spec.name(), spec.options(), arch)
-            ck = CompiledKernel(spec, code, hit, log)
-            _compiled[spec] = ck
+    if ck is not None:
         return ck
+    override = os.environ.get("LOOPFUSE_HSACO_" + spec.family.upper())   # tuning aid: prebuilt code object
+    if override:
+        with open(override, "rb") as fh:
+            ck = CompiledKernel(spec, fh.read(), False, "override " + override)
+    else:
+        # outside the lock: different specialisations compile concurrently (the shim is re-entrant;
+        # two threads asking for the same one both compile, the results are identical)
+        code, hit, log = runtime.compile_source(spec.source(), spec.name(), spec.options(), arch)
+        ck = CompiledKernel(spec, code, hit, log)
+    with _lock:
+        return _compiled.setdefault(spec, ck)
 
 
 def load_spec(spec: KernelSpec) -> runtime.Module:
