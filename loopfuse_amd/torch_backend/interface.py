@@ -32,7 +32,7 @@ from functools import partial
 from typing import Any, Callable
 
 import torch
-from torch._functorch.aot_autograd import aot_module_simplified
+from torch._functorch.aot_autograd import aot_module_simplified, make_boxed_func
 
 from .. import lowering
 from . import capture
@@ -46,7 +46,8 @@ USE_HARDCODE_KERNEL = os.environ.get("USE_HARDCODE_KERNEL", "0") == "1"
 # route taken by compiled callables since import: "fused" = HIP kernel launched,
 # "eager_graph" = graph not recognised, "eager_runtime" = recognised but the call's
 # tensors could not be served (CPU tensors, dtype, alignment ...)
-stats = {"fused": 0, "eager_graph": 0, "eager_runtime": 0, "compiled_graphs": 0, "matched_graphs": 0}
+# "eager_training" = graph traced with gradients enabled (forward or backward half)
+stats = {"fused": 0, "eager_graph": 0, "eager_runtime": 0, "eager_training": 0, "compiled_graphs": 0, "matched_graphs": 0}
 
 
 def _strict() -> bool:
@@ -67,8 +68,35 @@ def loopfuse_backend(gm: torch.fx.GraphModule, sample_inputs, mode="max-autotune
     """
     if mode:
         kwargs["mode"] = mode
+    if torch.is_grad_enabled() and (any(isinstance(t, torch.Tensor) and t.requires_grad for t in sample_inputs)
+                                    or any(t.requires_grad for t in gm.parameters())):
+        # AOTAutograd is about to trace a forward + backward pair: the forward graph must
+        # hand the probabilities to the backward graph, which a fused forward never forms
+        global _warned_training
+        if _strict():
+            raise NotImplementedError("loopfuse_amd: the attention kernels are forward-only and this graph is "
+                                      "traced with gradients enabled")
+        if not _warned_training:
+            _warned_training = True
+            log.warning("loopfuse_amd: graph traced with gradients enabled (an input requires grad); the attention "
+                        "kernels are forward-only, so this graph runs unfused.  Wrap inference in torch.no_grad().")
+        return aot_module_simplified(gm, sample_inputs, fw_compiler=_unfused_compiler)
     compiler = partial(loopfuse_compiler, input_names=get_input_names(gm), **kwargs)
     return aot_module_simplified(gm, sample_inputs, fw_compiler=compiler)
+
+
+_warned_training = False
+
+
+def _unfused_compiler(gm: torch.fx.GraphModule, sample_inputs) -> Callable:
+    """fw_compiler / bw_compiler of graphs traced for training: they run as captured."""
+    stats["compiled_graphs"] += 1
+
+    def eager_fn(*args):
+        stats["eager_training"] += 1
+        return gm(*args)
+
+    return make_boxed_func(eager_fn)
 
 
 # attention sub-graphs of the graphs compiled so far; the rewritten graphs call

@@ -330,6 +330,45 @@ def test_attention_inside_a_transformer_block():
     assert (got - want).abs().max() <= 4 * TOL and (got - want).abs().mean() <= 4e-3
 
 
+def test_module_with_parameters_outside_and_inside_no_grad():
+    """A module's parameters require grad: called outside torch.no_grad() the graph is
+    traced for training and runs unfused (and can be differentiated); inside it the
+    attention takes the HIP kernels."""
+    class Attn(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            torch.manual_seed(0)
+            self.qkv = torch.nn.Linear(512, 3 * 512, bias=False)
+            self.out = torch.nn.Linear(512, 512, bias=False)
+
+        def forward(self, x):
+            B, S, E = x.shape
+            q, k, v = (t.view(B, S, 8, 64).transpose(1, 2) for t in self.qkv(x).chunk(3, dim=-1))
+            a = torch.softmax(torch.ops.loopfuse.causal_mask(q @ k.transpose(-2, -1) * 0.125), dim=-1) @ v
+            return self.out(a.transpose(1, 2).reshape(B, S, E))
+
+    m = Attn().to(DEV).to(torch.bfloat16)
+    x = rand((2, 200, 512), seed=3).to(DEV)
+    torch._dynamo.reset()
+    before = dict(interface.stats)
+    cm = torch.compile(m, backend=loopfuse_backend, dynamic=True, mode=None)
+    y = cm(x)
+    y.float().square().mean().backward()
+    g_compiled = m.qkv.weight.grad.float().clone()
+    m.zero_grad()
+    y_eager = m(x)
+    y_eager.float().square().mean().backward()
+    assert interface.stats["fused"] == before["fused"] and interface.stats["eager_training"] >= before["eager_training"] + 2
+    assert (y.float() - y_eager.float()).abs().max() <= 1e-2
+    assert (g_compiled - m.qkv.weight.grad.float()).abs().max() <= 1e-3 * m.qkv.weight.grad.float().abs().max() + 1e-6
+    torch._dynamo.reset()
+    with torch.no_grad():
+        y2 = torch.compile(m, backend=loopfuse_backend, dynamic=True, mode=None)(x)
+    torch.cuda.synchronize()
+    assert interface.stats["fused"] == before["fused"] + 1
+    assert (y2.float() - y_eager.float()).abs().max() <= 4 * TOL
+
+
 def test_paged_decode_gqa_reference_format():
     # tests/benchmark.py:400-443: one-token pages, Q viewed [B, Hkv, group, D]
     def fn(Q, Kc, kt, Vc, vt):

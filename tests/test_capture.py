@@ -25,6 +25,69 @@ def test_custom_op_semantics():
     assert torch.equal(torch.ops.loopfuse.paged_load(buf, tab), buf[tab.long()])
 
 
+def test_custom_op_gradients():
+    """The operators' autograd formulas against the same functions spelled with
+    differentiable torch ops (double precision), and against finite differences."""
+    g = torch.Generator().manual_seed(1)
+    a = torch.randn(2, 5, 5, generator=g, dtype=torch.float64, requires_grad=True)
+    w = torch.randn(2, 5, 5, generator=g, dtype=torch.float64)
+    for op, keep in ((torch.ops.loopfuse.causal_mask, O.dense_mask("causal", 5, 5)),
+                     (lambda x: torch.ops.loopfuse.sliding_mask(x, 2), O.dense_mask("sliding", 5, 5, 2))):
+        (got,) = torch.autograd.grad((torch.softmax(op(a), -1) * w).sum(), a)
+        (want,) = torch.autograd.grad((torch.softmax(a.masked_fill(~keep, float("-inf")), -1) * w).sum(), a)
+        assert torch.allclose(got, want, atol=1e-12) and got[:, ~keep].abs().max() == 0
+    run, fin = torch.ops.loopfuse.scan_max(a)
+    (got,) = torch.autograd.grad((run * w).sum() + (fin * w[..., :1]).sum(), a)
+    cm = torch.cummax(a, -1).values
+    (want,) = torch.autograd.grad((cm * w).sum() + (cm[..., -1:] * w[..., :1]).sum(), a)
+    assert torch.allclose(got, want, atol=1e-12)
+    buf = torch.randn(7, 2, 3, generator=g, dtype=torch.float64, requires_grad=True)
+    tab = torch.tensor([[1, 4, 1], [6, 1, 0]], dtype=torch.int32)          # page 1 is gathered three times
+    wl = torch.randn(2, 3, 2, 3, generator=g, dtype=torch.float64)
+    (got,) = torch.autograd.grad((torch.ops.loopfuse.paged_load(buf, tab) * wl).sum(), buf)
+    (want,) = torch.autograd.grad((buf[tab.long()] * wl).sum(), buf)
+    assert torch.allclose(got, want, atol=1e-12) and got[[2, 3, 5]].abs().max() == 0
+    assert torch.autograd.gradcheck(lambda x: torch.ops.loopfuse.paged_load(x, tab), (buf,))
+    assert torch.autograd.gradcheck(lambda x: torch.softmax(torch.ops.loopfuse.sliding_mask(x, 3), -1), (a,))
+
+
+def test_graph_traced_for_training_runs_unfused_and_differentiates():
+    """Inputs that require grad (a module's parameters outside torch.no_grad()): the
+    reference fails while tracing (its operators have no autograd formula); here the
+    graph runs as captured and gradients equal those of the uncompiled function."""
+    def fn(q, k, v):
+        s = q @ k.transpose(-2, -1) * q.shape[-1] ** -0.5
+        return torch.softmax(torch.ops.loopfuse.causal_mask(s), dim=-1) @ v
+
+    g = torch.Generator().manual_seed(2)
+    ins = [torch.randn(1, 2, 24, 16, generator=g, requires_grad=True) for _ in range(3)]
+    ref = [t.detach().clone().requires_grad_() for t in ins]
+    torch._dynamo.reset()
+    before = dict(interface.stats)
+    out = torch.compile(fn, backend=loopfuse_amd.loopfuse_backend, dynamic=True)(*ins)
+    out.square().sum().backward()
+    fn(*ref).square().sum().backward()
+    for a, b in zip(ins, ref):
+        assert torch.allclose(a.grad, b.grad, atol=1e-5, rtol=1e-5)
+    assert interface.stats["eager_training"] - before["eager_training"] == 2      # forward and backward graph
+    assert interface.stats["fused"] == before["fused"] and interface.stats["matched_graphs"] == before["matched_graphs"]
+    # the same function under no_grad takes the matching route
+    torch._dynamo.reset()
+    with torch.no_grad():
+        torch.compile(fn, backend=loopfuse_amd.loopfuse_backend, dynamic=True)(*ins)
+    assert interface.stats["matched_graphs"] == before["matched_graphs"] + 1
+
+
+def test_strict_mode_refuses_training_graphs(monkeypatch):
+    monkeypatch.setenv("LOOPFUSE_STRICT", "1")
+    torch._dynamo.reset()
+    x = torch.randn(1, 1, 8, 16, requires_grad=True)
+    fn = lambda q: torch.softmax(torch.ops.loopfuse.causal_mask(q @ q.transpose(-2, -1)), -1) @ q
+    with pytest.raises(Exception, match="forward-only"):
+        torch.compile(fn, backend=loopfuse_amd.loopfuse_backend, dynamic=True)(x)
+    torch._dynamo.reset()
+
+
 def capture_graph(fn, inputs, marks=()):
     """Trace fn with dynamic shapes and return the AttentionMatch (or the NoMatch)."""
     box = {}
