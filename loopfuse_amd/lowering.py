@@ -441,6 +441,12 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
             raise RuntimeError(f"loopfuse_amd: {which} page table is not on the GPU")
         if table.stride(1) != 1:
             table = table.contiguous()
+        if os.environ.get("LOOPFUSE_CHECK_TABLES", "0") == "1" and table.numel():
+            # debugging aid (waits for the stream): the kernels trust page ids, an id outside
+            # the pool is a read outside the allocation
+            lo, hi = int(table.min()), int(table.max())
+            if lo < 0 or hi >= t.shape[0]:
+                raise ValueError(f"loopfuse_amd: {which} page table holds ids in [{lo}, {hi}] for a pool of {t.shape[0]} pages")
         if t.dim() == 3:       # [N, Hkv, D], one token per page (the reference's format)
             ps, hk, sp, st, sh = 1, t.shape[1], t.stride(0), 0, t.stride(1)
         elif t.dim() == 4:     # [N, P, Hkv, D]

@@ -731,3 +731,19 @@ def test_launches_can_be_captured_in_a_hip_graph(name):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, want), f"replay {rep} differs from the eager launch"
+
+
+def test_page_ids_outside_the_pool_are_reported_when_asked(monkeypatch):
+    """LOOPFUSE_CHECK_TABLES=1 validates page ids on the host before anything is launched."""
+    monkeypatch.setenv("LOOPFUSE_CHECK_TABLES", "1")
+    w = workloads.make("c5", seed=0, B=2, S=256).to(dev())
+    plan = lowering.AttnPlan(scale=w.scale, k_paged=True, v_paged=True)
+    good = lowering.attention(w.q, w.k, w.v, plan, w.k_table, w.v_table)
+    bad = w.k_table.clone()
+    bad[1, 3] = w.k.shape[0]
+    with pytest.raises(ValueError, match="page table holds ids"):
+        lowering.attention(w.q, w.k, w.v, plan, bad, w.v_table)
+    bad[1, 3] = -1
+    with pytest.raises(ValueError, match="page table holds ids"):
+        lowering.attention(w.q, w.k, w.v, plan, w.k_table, bad)
+    assert torch.equal(good, lowering.attention(w.q, w.k, w.v, plan, w.k_table, w.v_table))
