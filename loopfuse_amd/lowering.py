@@ -17,6 +17,7 @@ from __future__ import annotations
 
 import ctypes
 import dataclasses
+import functools
 import math
 import os
 import threading
@@ -378,6 +379,19 @@ def tuned_attention(q, k, v, plan: AttnPlan, k_table=None, v_table=None, **kw):
     return attention(q, k, v, plan, k_table, v_table, **{**kw, "choice": _tuned[key]})
 
 
+def _on_device_of_first_argument(fn):
+    """Kernel modules, the stream and the split-K scratch are looked up for the current
+    device: make the device of Q current for the duration of the call when it is not."""
+    @functools.wraps(fn)
+    def guarded(q, *args, **kw):
+        if isinstance(q, torch.Tensor) and q.is_cuda and q.device.index != torch.cuda.current_device():
+            with torch.cuda.device(q.device):
+                return fn(q, *args, **kw)
+        return fn(q, *args, **kw)
+    return guarded
+
+
+@_on_device_of_first_argument
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
               k_table: Optional[torch.Tensor] = None, v_table: Optional[torch.Tensor] = None,
               *, out: Optional[torch.Tensor] = None, record_visits: bool = False,
@@ -420,6 +434,10 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     _check_tensor("Q", q, dtype)
     _check_tensor("K", k, dtype)
     _check_tensor("V", v, dtype)
+    for name, t in (("K", k), ("V", v), ("K page table", k_table), ("V page table", v_table), ("score bias", score_bias),
+                    ("output bias", out_bias), ("Q2", q2), ("K2", k2), ("O", out)):
+        if t is not None and t.device != q.device:
+            raise RuntimeError(f"loopfuse_amd: {name} is on {t.device}, Q on {q.device}")
 
     P = AttnParams()
     paged = 0

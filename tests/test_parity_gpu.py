@@ -747,3 +747,16 @@ def test_page_ids_outside_the_pool_are_reported_when_asked(monkeypatch):
     with pytest.raises(ValueError, match="page table holds ids"):
         lowering.attention(w.q, w.k, w.v, plan, w.k_table, bad)
     assert torch.equal(good, lowering.attention(w.q, w.k, w.v, plan, w.k_table, w.v_table))
+
+
+def test_operands_on_another_device_are_refused():
+    """Every operand must live where Q lives; nothing is launched otherwise."""
+    w = workloads.make("c5", seed=0, B=2, S=256).to(dev())
+    plan = lowering.AttnPlan(scale=w.scale, k_paged=True, v_paged=True)
+    with pytest.raises(RuntimeError, match="K page table is on cpu"):
+        lowering.attention(w.q, w.k, w.v, plan, w.k_table.cpu(), w.v_table)
+    q, k, v = (rand((1, 2, 64, 64), torch.bfloat16, s).to(dev()) for s in (1, 2, 3))
+    with pytest.raises(RuntimeError, match="score bias is on cpu"):
+        lowering.attention(q, k, v, lowering.AttnPlan(scale=0.125), score_bias=rand((1, 2, 64, 64), torch.bfloat16, 4))
+    with pytest.raises(RuntimeError, match="not on the GPU"):
+        lowering.attention(q, k.cpu(), v, lowering.AttnPlan(scale=0.125))
