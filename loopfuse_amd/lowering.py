@@ -18,6 +18,7 @@ from __future__ import annotations
 import ctypes
 import dataclasses
 import functools
+import json
 import math
 import os
 import threading
@@ -163,8 +164,26 @@ def compile_spec(spec: KernelSpec, arch: str = runtime.DEFAULT_ARCH) -> Compiled
         # two threads asking for the same one both compile, the results are identical)
         code, hit, log = runtime.compile_source(spec.source(), spec.name(), spec.options(), arch)
         ck = CompiledKernel(spec, code, hit, log)
+    record = os.environ.get("LOOPFUSE_RECORD_SPECS")
     with _lock:
+        if record and spec not in _compiled:
+            # one JSON line per specialisation a workload asked for: specs_from_file() reads
+            # them back, so a deployment can fill the code-object cache ahead of time
+            with open(record, "a") as fh:
+                fh.write(json.dumps(dataclasses.asdict(spec), sort_keys=True) + "\n")
         return _compiled.setdefault(spec, ck)
+
+
+def specs_from_file(path: str) -> list[KernelSpec]:
+    """Specialisations recorded with ``LOOPFUSE_RECORD_SPECS=<path>`` (duplicates dropped)."""
+    seen: dict[KernelSpec, None] = {}
+    with open(path) as fh:
+        for line in fh:
+            if line.strip():
+                d = json.loads(line)
+                d["extra"] = tuple(d.get("extra", ()))
+                seen.setdefault(KernelSpec(**d))
+    return list(seen)
 
 
 def load_spec(spec: KernelSpec) -> runtime.Module:
