@@ -423,6 +423,23 @@ def test_unfused_graph_still_correct():
     assert torch.equal(out, torch.relu(a) + b)
 
 
+def test_requested_specialisations_are_recorded_and_read_back(shim_built, monkeypatch, tmp_path):
+    """LOOPFUSE_RECORD_SPECS: one line per specialisation asked for, first request only;
+    specs_from_file gives the same KernelSpec objects back (extra options included)."""
+    path = tmp_path / "specs.jsonl"
+    monkeypatch.setenv("LOOPFUSE_RECORD_SPECS", str(path))
+    monkeypatch.setattr(lowering, "_compiled", {})
+    a = lowering.KernelSpec("decode", 0, 128, paged=3, page_size=16, rows=16, waves=8, headwave=True)
+    b = lowering.KernelSpec("prefill", 1, 64, lowering.MASK_SLIDING, True, bias=5, extra=("-DLF_DMA=1",))
+    for spec in (a, b, a):
+        lowering.compile_spec(spec)
+    assert len(path.read_text().splitlines()) == 2
+    assert lowering.specs_from_file(str(path)) == [a, b]
+    import __graft_entry__
+    listed = __graft_entry__.standard_specs()
+    assert len(listed) == len(set(listed)) and a in listed
+
+
 def test_kernel_specs_compile_without_gpu(shim_built):
     spec = lowering.KernelSpec("prefill", 0, 128, lowering.MASK_CAUSAL)
     ck = lowering.compile_spec(spec)
