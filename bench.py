@@ -97,6 +97,36 @@ def cpu_baseline(seconds: float = 12.0) -> dict:
     }
 
 
+def torch_sdpa(args, dev) -> dict:
+    """PyTorch's own fused attention on the same GPU and inputs: a same-hardware point of
+    comparison (not the reference, which has no AMD path).  Softcap and the sliding window
+    have no SDPA spelling, so only the causal config is timed for prefill; the decode config
+    gets contiguous K/V (the page gather is done before the timed region)."""
+    import torch
+    import torch.nn.functional as F
+
+    from loopfuse_amd import workloads
+
+    res: dict = {}
+    if args.workload == "c2" and args.only in (None, "prefill"):
+        w = workloads.make("c2", seed=0).to(dev)
+        t, _ = time_gpu(lambda i: F.scaled_dot_product_attention(w.q, w.k, w.v, is_causal=True), args.steps, args.warmup)
+        res["prefill"] = {"workload": "c2", "us_per_launch": t * 1e6, "tflops": w.flops() / t / 1e12}
+        del w
+    if args.only in (None, "decode"):
+        w = workloads.make(args.decode_workload, seed=0).to(dev)
+        k, v = w.k, w.v
+        if w.k_table is not None:
+            B, hkv, d = w.q.shape[0], w.k.shape[-2], w.k.shape[-1]
+            k = w.k[w.k_table.long()].reshape(B, -1, hkv, d).transpose(1, 2).contiguous()
+            v = w.v[w.v_table.long()].reshape(B, -1, hkv, d).transpose(1, 2).contiguous()
+        gqa = w.q.shape[1] != k.shape[1]
+        t, _ = time_gpu(lambda i: F.scaled_dot_product_attention(w.q, k, v, enable_gqa=gqa), args.steps, min(args.warmup, 20))
+        res["decode"] = {"workload": args.decode_workload + (" (contiguous K/V)" if w.k_table is not None else ""),
+                         "us_per_launch": t * 1e6, "gbs": w.kv_bytes() / t / 1e9}
+    return res
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -107,6 +137,9 @@ def main() -> int:
                     help="time only one of the two kernels (profiling aid)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 512 MiB device copy (reference point for FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--torch-sdpa", action="store_true",
+                    help="also time torch.nn.functional.scaled_dot_product_attention on the same GPU and inputs "
+                         "(config 2 as is; the decode config with its pages gathered into contiguous K/V beforehand)")
     ap.add_argument("--workload", default="c2", help="prefill workload: c2 | c2_softcap | c3")
     ap.add_argument("--decode-workload", default="c5", help="decode workload: c5 | c4")
     args = ap.parse_args()
@@ -196,6 +229,8 @@ def main() -> int:
                    "decode_workload": "config 5: paged GQA decode bf16 B64 Hq32/Hkv8 K_len2048 D128 page16"
                    if args.decode_workload == "c5" else args.decode_workload},
     })
+    if args.torch_sdpa:
+        out["torch_sdpa"] = torch_sdpa(args, dev)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
