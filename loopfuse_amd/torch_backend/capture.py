@@ -74,7 +74,8 @@ class Scalar:
     node: torch.fx.Node            # re-evaluated at call time
     value: float                   # value for the stand-in sizes (unused beyond sanity)
     # how to compute it in plain Python at call time, if every step is understood:
-    # ("lit", x) | ("arg", fx node holding a number) | ("op", name, operand, ...); None = run the node
+    # ("lit", x) | ("arg", fx node holding a number) | ("dim", fx node holding a tensor, axis) |
+    # ("op", name, operand, ...); None = run the node
     expr: Any = None
 
 
@@ -126,6 +127,10 @@ _VIEW_OPS = {
 _SHAPE_ONLY_VIEW_OPS = {aten.view.default, aten._unsafe_view.default, aten.reshape.default,
                         aten.expand.default, aten.clone.default, aten.alias.default,
                         aten.detach.default, aten.contiguous.default}
+# F.scaled_dot_product_attention in an ATen graph (which one depends on the device and dtype)
+_SDPA_OPS = {getattr(aten, name).default for name in (
+    "_scaled_dot_product_flash_attention", "_scaled_dot_product_efficient_attention",
+    "_scaled_dot_product_flash_attention_for_cpu") if hasattr(aten, name)}
 _CAST_OPS = {prims.convert_element_type.default, aten._to_copy.default}
 
 
@@ -202,6 +207,18 @@ class AttentionMatch:
     q2: Optional[Operand] = None   # second score product: scores = Q K^T + Q2 K2^T
     k2: Optional[Operand] = None
     late_factors: tuple = ()       # factors (also listed above) that the graph applies after the mask
+    # memory order of the traced output when it is not row-major (torch's fused attention ops
+    # return [B, H, S, D] views of [B, S, H, D] storage, and the graph after them may rely on
+    # it): dims from outermost to innermost; () = row-major
+    out_order: tuple = ()
+
+    def empty_out(self, vals, dtype, device) -> torch.Tensor:
+        """Uninitialised output in the traced shape and memory order."""
+        shape = self.out_shape(vals)
+        if not self.out_order:
+            return torch.empty(shape, dtype=dtype, device=device)
+        inverse = [self.out_order.index(i) for i in range(len(shape))]
+        return torch.empty([shape[i] for i in self.out_order], dtype=dtype, device=device).permute(inverse)
 
     def describe(self) -> str:
         nm = lambda i: self.inputs[i].name
@@ -221,7 +238,7 @@ class AttentionMatch:
         if isinstance(x, tuple) and x[0] == "recip":
             return 1.0 / AttentionMatch._number(x[1], vals)
         if isinstance(x, tuple) and x[0] == "expr":
-            return _eval_scalar(x[1], lambda i: AttentionMatch._number(("arg", i), vals))
+            return _eval_scalar(x[1], lambda i: vals[i])
         if isinstance(x, tuple) and x[0] == "arg":
             x = vals[x[1]]
         return float(x.item() if isinstance(x, torch.Tensor) else x)
@@ -316,7 +333,8 @@ class AttentionMatch:
         v, vt = self._operand(self.v, vals)
         B, Hq, Sq, Sk, D = self._shapes(vals)
         run = lowering.tuned_attention if self.tune else lowering.attention
-        out = run(q, k, v, self.plan_for(vals), kt, vt,
+        given = {"out": self.empty_out(vals, q.dtype, q.device)} if self.out_order else {}
+        out = run(q, k, v, self.plan_for(vals), kt, vt, **given,
                                  score_bias=self._bias_view(self.bias, vals, (B, Hq, Sq, Sk)),
                                  out_bias=self._bias_view(self.out_bias, vals, (B, Hq, Sq, D)),
                                  **self._second_product(vals))
@@ -533,7 +551,10 @@ def _eval_scalar(e, leaf) -> float:
     if kind == "lit":
         return float(e[1])
     if kind == "arg":
-        return float(leaf(e[1]))
+        x = leaf(e[1])
+        return float(x.item() if isinstance(x, torch.Tensor) else x)
+    if kind == "dim":
+        return float(leaf(e[1]).shape[e[2]])
     name, xs = e[1], [_eval_scalar(x, leaf) for x in e[2:]]
     if name == "mul":
         return xs[0] * xs[1]
@@ -563,6 +584,8 @@ def _same_expr(x, y) -> bool:
         return x[1] == y[1]
     if x[0] == "arg":
         return x[1] is y[1]
+    if x[0] == "dim":
+        return x[1] is y[1] and x[2] == y[2]
     return x[1] == y[1] and len(x) == len(y) and all(_same_expr(p, q) for p, q in zip(x[2:], y[2:]))
 
 
@@ -766,6 +789,44 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
             if isinstance(x, torch.fx.Node) and isinstance(env.get(x), Stage) and env[x].kind == "out":
                 finalise(x)
 
+    def sdpa_stage(node, tgt, a, kw) -> Stage:
+        """torch's fused attention ops (what F.scaled_dot_product_attention becomes in an
+        ATen graph) as a finished attention: softmax(causal?(Q K^T * scale)) V."""
+        names = [arg_.name for arg_ in tgt._schema.arguments]
+        given = dict(zip(names, a))
+        given.update(kw)
+        qi, ki, vi = given["query"], given["key"], given["value"]
+        if not all(isinstance(x, Ids) and x.t.dim() == 4 for x in (qi, ki, vi)):
+            raise _Skip("fused attention op on operands that are not rank-4 tensors")
+        if given.get("attn_mask") is not None or given.get("attn_bias") is not None:
+            raise _Skip("fused attention op with a mask tensor")
+        if given.get("dropout_p", 0.0) != 0.0:
+            raise _Skip("fused attention op with dropout")
+        if qi.t.shape[0] != ki.t.shape[0] or qi.t.shape[-1] != ki.t.shape[-1] or vi.t.shape[:3] != ki.t.shape[:3] \
+                or ki.t.shape[1] < 1 or qi.t.shape[1] % ki.t.shape[1]:
+            raise _Skip("fused attention op: Q, K, V shapes disagree")
+        if qi.t.shape[1] != ki.t.shape[1]:
+            # enable_gqa: query head h reads kv head h // group, as repeat_interleave would give
+            group = qi.t.shape[1] // ki.t.shape[1]
+            ki = Ids(ki.src, ki.t.repeat_interleave(group, dim=1))
+            vi = Ids(vi.src, vi.t.repeat_interleave(group, dim=1))
+        scale = given.get("scale")
+        if scale is None:
+            d = node.args[0].meta["val"].shape[-1]
+            if isinstance(d, int):
+                scale = float(d) ** -0.5
+            else:
+                # fully dynamic graph: the head dim is read off the query tensor at call time
+                scale = Scalar(node, float(qi.t.shape[-1]) ** -0.5, ("op", "rsqrt", ("dim", node.args[0], -1)))
+        elif isinstance(scale, (int, float)):
+            raw = node.kwargs.get("scale")
+            scale = raw if isinstance(raw, torch.fx.Node) else float(scale)
+        elif not isinstance(scale, Scalar):
+            raise _Skip("fused attention op: scale not understood")
+        sq, sk = qi.t.shape[-2], ki.t.shape[-2]
+        return Stage("out", tuple(qi.t.shape[:-1]) + (vi.t.shape[-1],), qi, Ids(ki.src, ki.t.transpose(-1, -2)), vi,
+                     factors=[scale], mask="causal" if given.get("is_causal", False) else None, mat=(sq, sk))
+
     def pattern_step(node, tgt, a, kw, first):
         """The abstract value of ``node`` if it continues a pattern; raises _Skip otherwise."""
         # -- integer / float arithmetic on sizes
@@ -844,6 +905,8 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
                 shape = tuple(table.src.shape) + tuple(pool.src.shape[1:])
                 src = Source("paged", pool.src.node, table.src.node, shape, len(table.src.shape))
                 return Ids(src, torch.arange(math.prod(shape), dtype=torch.int64).reshape(shape))
+            if tgt in _SDPA_OPS:
+                return [sdpa_stage(node, tgt, a, kw)] + [None] * 8      # (output, log-sum-exp, ...)
             if tgt in (aten.bmm.default, aten.mm.default, aten.matmul.default) and isinstance(a[1], Ids):
                 qi, ki = a[0], a[1]
                 if qi.t.dim() < 3 or ki.t.dim() != qi.t.dim():
@@ -1009,7 +1072,7 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
             env[node] = pattern_step(node, node.target, a, kw, first)
             continue
         except _Skip as e:
-            if any(isinstance(x, Stage) for x in list(a) + list(kw.values())):
+            if node.target in _SDPA_OPS or any(isinstance(x, Stage) for x in list(a) + list(kw.values())):
                 reasons.append(str(e))
         # an ordinary op: it keeps running as it is; finished attentions it reads are fused
         consume(node.all_input_nodes)
@@ -1093,6 +1156,8 @@ def _build_match(out_node: torch.fx.Node, st: Stage) -> AttentionMatch:
             def conv(e):
                 if e[0] == "arg":
                     return ("arg", slot(e[1]))
+                if e[0] == "dim":
+                    return ("dim", slot(e[1]), e[2])
                 return e if e[0] == "lit" else e[:2] + tuple(conv(x) for x in e[2:])
             return ("expr", conv(f.expr))
         if isinstance(f, torch.fx.Node):
@@ -1108,7 +1173,17 @@ def _build_match(out_node: torch.fx.Node, st: Stage) -> AttentionMatch:
         n, dims = _fit_bias(st.out_bias, qshape)
         obias_op = BiasOperand(slot(n), dims)
     window = scalar(st.window) if st.mask == "sliding" else 0
+    out_order = ()
+    val = out_node.meta.get("val")
+    if out_rank == 4 and isinstance(val, torch.Tensor) and val.dim() == 4:
+        strides = [s_ if isinstance(s_, int) else _hint(s_) for s_ in val.stride()]
+        order = tuple(sorted(range(4), key=lambda i: (-strides[i], i)))
+        if order[3] != 3:
+            raise NoMatch("traced output does not keep the head dim innermost")
+        if order != (0, 1, 2, 3):
+            out_order = order
     return AttentionMatch(out_node, inputs, q_op, k_op, v_op, [scalar(f) for f in st.factors],
                           [scalar(f) for f in st.post_factors], st.has_tanh, st.mask, window, out_rank,
                           bias_op, obias_op, denom_add=tuple(scalar(t) for t in st.denom_add), base2=st.base2,
-                          q2=q2_op, k2=k2_op, late_factors=tuple(scalar(f) for f in st.late_factors))
+                          q2=q2_op, k2=k2_op, late_factors=tuple(scalar(f) for f in st.late_factors),
+                          out_order=out_order)

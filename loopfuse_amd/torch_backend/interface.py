@@ -111,7 +111,7 @@ def _fused_call(match_id: int, *vals):
     if _codegen_sink is not None:
         _codegen_sink.extend(lowering.compile_spec(s) for s in match.kernel_specs_for(vals))
         q = vals[match.q.index]
-        return torch.empty(match.out_shape(vals), dtype=q.dtype, device=q.device)
+        return match.empty_out(vals, q.dtype, q.device)
     return match.run(vals)
 
 

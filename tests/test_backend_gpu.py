@@ -330,6 +330,46 @@ def test_attention_inside_a_transformer_block():
     assert (got - want).abs().max() <= 4 * TOL and (got - want).abs().mean() <= 4e-3
 
 
+@pytest.mark.parametrize("which", ["causal", "gqa_decode", "scale_rect", "module"])
+@pytest.mark.parametrize("dynamic", [True, False])
+def test_torch_fused_attention_calls_are_taken_over(which, dynamic):
+    """F.scaled_dot_product_attention arrives as one aten._scaled_dot_product_* node;
+    without a mask tensor or dropout it is the same attention and runs on the HIP kernels
+    (the output keeps the memory order the traced op gives, which later views rely on)."""
+    import torch.nn.functional as F
+    if which == "causal":
+        fn = lambda q, k, v: F.scaled_dot_product_attention(q, k, v, is_causal=True)
+        ins = (rand((2, 8, 333, 128), seed=1), rand((2, 8, 333, 128), seed=2), rand((2, 8, 333, 128), seed=3))
+        want = O.attention_reference(*ins, mask="causal")
+    elif which == "gqa_decode":
+        fn = lambda q, k, v: F.scaled_dot_product_attention(q, k, v, enable_gqa=True)
+        ins = (rand((4, 32, 1, 128), seed=1), rand((4, 8, 1000, 128), seed=2), rand((4, 8, 1000, 128), seed=3))
+        want = O.attention_reference(*ins)
+    elif which == "scale_rect":
+        fn = lambda q, k, v: F.scaled_dot_product_attention(q, k, v, scale=0.05) * 2
+        ins = (rand((2, 4, 100, 64), seed=1), rand((2, 4, 260, 64), seed=2), rand((2, 4, 260, 64), seed=3))
+        want = O.attention_reference(*ins, scale=0.05) * 2
+    else:
+        def fn(x, wqkv, wo):
+            B, S, E = x.shape
+            q, k, v = ((x @ w).view(B, S, 8, E // 8).transpose(1, 2) for w in wqkv.unbind(0))
+            a = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+            return a.transpose(1, 2).reshape(B, S, E) @ wo
+        ins = (rand((2, 200, 512), seed=1), rand((3, 512, 512), seed=2) * 0.04, rand((512, 512), seed=3) * 0.04)
+        want = None
+    torch._dynamo.reset()
+    before = dict(interface.stats)
+    dev_ins = [t.to(DEV) for t in ins]
+    with torch.no_grad():
+        got = torch.compile(fn, backend=loopfuse_backend, dynamic=dynamic, mode=None)(*dev_ins)
+        if want is None:
+            want = fn(*dev_ins).float().cpu()
+    torch.cuda.synchronize()
+    assert interface.stats["fused"] == before["fused"] + 1, "the fused HIP path was not taken"
+    err = (got.float().cpu() - want).abs().max().item()
+    assert err <= (4 * TOL if which == "module" else 2 * TOL if which == "scale_rect" else TOL), err
+
+
 def test_module_with_parameters_outside_and_inside_no_grad():
     """A module's parameters require grad: called outside torch.no_grad() the graph is
     traced for training and runs unfused (and can be differentiated); inside it the

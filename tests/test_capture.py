@@ -275,7 +275,7 @@ def _oracle_run(self, vals):
                                 score_bias=self._bias_view(self.bias, vals, (B, Hq, Sq, Sk)),
                                 out_bias=self._bias_view(self.out_bias, vals, (B, Hq, Sq, D)),
                                 **self._second_product(vals)).to(q.dtype)
-    return out.reshape(self.out_shape(vals))
+    return self.empty_out(vals, out.dtype, out.device).copy_(out.reshape(self.out_shape(vals)))
 
 
 def _explicit_softmax(X, base2=True, c=1.0):
@@ -303,7 +303,8 @@ def test_capture_explicit_softmax_with_shifted_denominator():
 
 
 @pytest.mark.parametrize("which", ["two_outputs", "prefix", "inside_block", "modified", "softmax1", "softmax_e",
-                                   "mla", "mla_shared_rope", "double_k", "einsum", "rank3", "bshd"])
+                                   "mla", "mla_shared_rope", "double_k", "einsum", "rank3", "bshd",
+                                   "sdpa_causal_gqa", "sdpa_scale_expand", "sdpa_bshd_block"])
 def test_rewritten_graphs_compute_the_same(which, monkeypatch):
     """Sub-graph fusion: the attention(s) inside a larger graph are replaced by fused
     calls and the rest keeps running.  Here the fused call is the oracle (no GPU), so
@@ -363,6 +364,24 @@ def test_rewritten_graphs_compute_the_same(which, monkeypatch):
             return o.transpose(1, 2) if which == "bshd" else o
         shape = {"einsum": (2, 3, 40, 64), "rank3": (6, 40, 64), "bshd": (2, 40, 3, 64)}[which]
         ins, n_attn = (f32(*shape), f32(*shape, seed=1), f32(*shape, seed=2)), 1
+    elif which.startswith("sdpa"):
+        # torch's own fused attention call: one aten._scaled_dot_product_* node in the graph
+        import torch.nn.functional as F
+        if which == "sdpa_causal_gqa":          # default scale, kv heads grouped by the op itself
+            fn = lambda Q, K, V: F.scaled_dot_product_attention(Q, K, V, is_causal=True, enable_gqa=True)
+            ins = (f32(2, 8, 40, 64), f32(2, 2, 40, 64, seed=1), f32(2, 2, 40, 64, seed=2))
+        elif which == "sdpa_scale_expand":      # explicit scale, one kv head expanded, rectangular, something after it
+            fn = lambda Q, K, V: F.scaled_dot_product_attention(Q, K.expand(-1, 4, -1, -1), V.expand(-1, 4, -1, -1),
+                                                                scale=0.3) + 1
+            ins = (f32(2, 4, 24, 64), f32(2, 1, 56, 64, seed=1), f32(2, 1, 56, 64, seed=2))
+        else:                                   # the usual module spelling: [B, S, H*D] -> heads -> attention -> back
+            def fn(x, wqkv, wo):
+                B, S, E = x.shape
+                q, k, v = ((x @ w).view(B, S, 4, E // 4).transpose(1, 2) for w in wqkv.unbind(0))
+                a = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+                return a.transpose(1, 2).reshape(B, S, E) @ wo
+            ins = (f32(2, 24, 256), f32(3, 256, 256, seed=1) * 0.06, f32(256, 256, seed=2) * 0.06)
+        n_attn = 1
     elif which == "double_k":
         # reference tests/test_attention.py:441-462 with its commented-out tail restored
         def fn(Q, K, K2, V):
@@ -549,3 +568,22 @@ def test_factor_after_the_mask(monkeypatch):
     neg = cf(q, k, v, torch.tensor(-0.125))      # -inf * negative = +inf: not a masked softmax any more
     assert interface.stats["eager_runtime"] == before["eager_runtime"] + 1
     torch.testing.assert_close(neg, fn(q, k, v, torch.tensor(-0.125)), equal_nan=True)
+
+
+def test_fused_attention_op_with_a_mask_tensor_is_left_alone():
+    """A mask tensor given to F.scaled_dot_product_attention is not taken over: the graph
+    runs as captured, and the reason is reported."""
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(1, 2, 16, 32, generator=g) for _ in range(3))
+    m = torch.rand(1, 1, 16, 16, generator=g) > 0.3
+    m[..., 0] = True
+    fn = lambda q, k, v, m: F.scaled_dot_product_attention(q, k, v, attn_mask=m)
+    box = capture_graph(fn, (q, k, v, m))
+    assert "match" not in box and "mask tensor" in str(box["nomatch"])
+    torch._dynamo.reset()
+    before = dict(interface.stats)
+    with torch.no_grad():
+        got = torch.compile(fn, backend=loopfuse_amd.loopfuse_backend, dynamic=True)(q, k, v, m)
+    assert interface.stats["eager_graph"] == before["eager_graph"] + 1
+    torch.testing.assert_close(got, fn(q, k, v, m))
