@@ -798,8 +798,11 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
         qi, ki, vi = given["query"], given["key"], given["value"]
         if not all(isinstance(x, Ids) and x.t.dim() == 4 for x in (qi, ki, vi)):
             raise _Skip("fused attention op on operands that are not rank-4 tensors")
-        if given.get("attn_mask") is not None or given.get("attn_bias") is not None:
-            raise _Skip("fused attention op with a mask tensor")
+        bias = given.get("attn_mask") if given.get("attn_mask") is not None else given.get("attn_bias")
+        if bias is not None and not isinstance(bias, Ids):
+            raise _Skip("fused attention op with a mask that is not a tensor")
+        if bias is not None and given.get("is_causal", False):
+            raise _Skip("fused attention op with a mask tensor and is_causal")
         if given.get("dropout_p", 0.0) != 0.0:
             raise _Skip("fused attention op with dropout")
         if qi.t.shape[0] != ki.t.shape[0] or qi.t.shape[-1] != ki.t.shape[-1] or vi.t.shape[:3] != ki.t.shape[:3] \
@@ -824,8 +827,11 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
         elif not isinstance(scale, Scalar):
             raise _Skip("fused attention op: scale not understood")
         sq, sk = qi.t.shape[-2], ki.t.shape[-2]
+        # a mask tensor reaches the op as an additive term in the query's dtype (torch turns
+        # boolean masks into 0 / -inf before it dispatches): the kernels' score bias
         return Stage("out", tuple(qi.t.shape[:-1]) + (vi.t.shape[-1],), qi, Ids(ki.src, ki.t.transpose(-1, -2)), vi,
-                     factors=[scale], mask="causal" if given.get("is_causal", False) else None, mat=(sq, sk))
+                     factors=[scale], mask="causal" if given.get("is_causal", False) else None, mat=(sq, sk),
+                     bias=None if bias is None else (bias, tuple(qi.t.shape[:-1]) + (sk,)))
 
     def pattern_step(node, tgt, a, kw, first):
         """The abstract value of ``node`` if it continues a pattern; raises _Skip otherwise."""

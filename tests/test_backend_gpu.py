@@ -330,7 +330,7 @@ def test_attention_inside_a_transformer_block():
     assert (got - want).abs().max() <= 4 * TOL and (got - want).abs().mean() <= 4e-3
 
 
-@pytest.mark.parametrize("which", ["causal", "gqa_decode", "scale_rect", "module"])
+@pytest.mark.parametrize("which", ["causal", "gqa_decode", "scale_rect", "module", "bool_mask", "float_mask"])
 @pytest.mark.parametrize("dynamic", [True, False])
 def test_torch_fused_attention_calls_are_taken_over(which, dynamic):
     """F.scaled_dot_product_attention arrives as one aten._scaled_dot_product_* node;
@@ -349,6 +349,17 @@ def test_torch_fused_attention_calls_are_taken_over(which, dynamic):
         fn = lambda q, k, v: F.scaled_dot_product_attention(q, k, v, scale=0.05) * 2
         ins = (rand((2, 4, 100, 64), seed=1), rand((2, 4, 260, 64), seed=2), rand((2, 4, 260, 64), seed=3))
         want = O.attention_reference(*ins, scale=0.05) * 2
+    elif which in ("bool_mask", "float_mask"):
+        fn = lambda q, k, v, m: F.scaled_dot_product_attention(q, k, v, attn_mask=m)
+        if which == "bool_mask":
+            m = torch.rand(2, 1, 200, 264, generator=torch.Generator().manual_seed(5)) > 0.3
+            m[..., 0] = True
+            bias = torch.zeros(m.shape).masked_fill(~m, float("-inf"))
+        else:
+            m = rand((1, 4, 200, 264), seed=5)
+            bias = m.float()
+        ins = (rand((2, 4, 200, 64), seed=1), rand((2, 4, 264, 64), seed=2), rand((2, 4, 264, 64), seed=3), m)
+        want = O.attention_reference(*ins[:3], score_bias=bias)
     else:
         def fn(x, wqkv, wo):
             B, S, E = x.shape
