@@ -887,6 +887,14 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
 
         # -- views of tensors
         if isinstance(first, Ids):
+            if tgt is aten.slice.Tensor:
+                # x[:, :, None] style indexing leaves one whole-range slice per dim in a dynamic graph
+                rest = list(a[1:]) + [None] * 4
+                start, end, step = rest[1], rest[2], rest[3]
+                if start in (0, None) and step in (1, None) and (end is None or (is_number(end) and end >= 1 << 62)) \
+                        and not kw:
+                    return first
+                raise _Skip("a slice that is not the whole range")
             if tgt in _VIEW_OPS:
                 if shrink_static and tgt in (aten.view.default, aten._unsafe_view.default, aten.reshape.default,
                                              aten.expand.default):

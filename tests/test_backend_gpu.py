@@ -381,6 +381,29 @@ def test_torch_fused_attention_calls_are_taken_over(which, dynamic):
     assert err <= (4 * TOL if which == "module" else 2 * TOL if which == "scale_rect" else TOL), err
 
 
+@pytest.mark.parametrize("S,P,use_mask", [(300, 0, False), (1, 700, False), (64, 700, True)])
+def test_decoder_layer_with_cache_and_repeated_kv_heads(S, P, use_mask):
+    """The decoder-layer attention block of tests/test_capture.py (rotary embedding, cache
+    concatenation, kv heads repeated by expand + reshape, F.scaled_dot_product_attention)
+    in bf16 with D = 128: prefill, one-token decode and a masked chunk all run on the HIP
+    kernels with the un-repeated cache as K and V."""
+    from test_capture import DecoderLayerAttention, decoder_layer_inputs
+    torch.manual_seed(0)
+    m = DecoderLayerAttention(E=1024, H=8, Hkv=2).eval().to(DEV).to(torch.bfloat16)
+    ins = [None if t is None else t.to(DEV) for t in decoder_layer_inputs(1024, 8, 2, S, P, use_mask, torch.bfloat16)]
+    torch._dynamo.reset()
+    before = dict(interface.stats)
+    with torch.no_grad():
+        got = torch.compile(m, backend=loopfuse_backend, dynamic=True, mode=None)(*ins)
+        want = m(*ins)
+    torch.cuda.synchronize()
+    assert interface.stats["fused"] == before["fused"] + 1, "the fused HIP path was not taken"
+    match = interface._MATCHES[-1]
+    assert match.k.group == 4 and match.inputs[match.k.index].name.startswith("cat")
+    assert (got[0].float() - want[0].float()).abs().max().item() <= 4 * TOL
+    assert torch.equal(got[1], want[1]) and torch.equal(got[2], want[2])
+
+
 def test_module_with_parameters_outside_and_inside_no_grad():
     """A module's parameters require grad: called outside torch.no_grad() the graph is
     traced for training and runs unfused (and can be differentiated); inside it the

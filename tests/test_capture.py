@@ -588,3 +588,76 @@ def test_fused_attention_op_with_dropout_is_left_alone():
     q, k, v = (torch.randn(1, 2, 16, 32, generator=g) for _ in range(3))
     box = capture_graph(lambda q, k, v: F.scaled_dot_product_attention(q, k, v, dropout_p=0.5), (q, k, v))
     assert "match" not in box and "nomatch" in box
+
+
+def _rotate_half(x):
+    x1, x2 = x[..., : x.shape[-1] // 2], x[..., x.shape[-1] // 2:]
+    return torch.cat((-x2, x1), dim=-1)
+
+
+def _repeat_kv(h, n):
+    b, hk, s, d = h.shape
+    return h[:, :, None, :, :].expand(b, hk, n, s, d).reshape(b, hk * n, s, d)
+
+
+class DecoderLayerAttention(torch.nn.Module):
+    """Attention block as decoder models commonly write it: projections, rotary embedding,
+    key/value cache appended by concatenation, kv heads repeated with expand + reshape,
+    F.scaled_dot_product_attention, output projection, residual."""
+
+    def __init__(self, E=256, H=8, Hkv=2):
+        super().__init__()
+        self.H, self.Hkv, self.D = H, Hkv, E // H
+        self.q = torch.nn.Linear(E, H * self.D, bias=False)
+        self.k = torch.nn.Linear(E, Hkv * self.D, bias=False)
+        self.v = torch.nn.Linear(E, Hkv * self.D, bias=False)
+        self.o = torch.nn.Linear(E, E, bias=False)
+        self.norm = torch.nn.LayerNorm(E)
+
+    def forward(self, x, cos, sin, past_k, past_v, mask=None):
+        import torch.nn.functional as F
+        B, S, E = x.shape
+        h = self.norm(x)
+        q = self.q(h).view(B, S, self.H, self.D).transpose(1, 2)
+        k = self.k(h).view(B, S, self.Hkv, self.D).transpose(1, 2)
+        v = self.v(h).view(B, S, self.Hkv, self.D).transpose(1, 2)
+        q = q * cos + _rotate_half(q) * sin
+        k = k * cos + _rotate_half(k) * sin
+        k = torch.cat([past_k, k], dim=2)
+        v = torch.cat([past_v, v], dim=2)
+        g = self.H // self.Hkv
+        a = F.scaled_dot_product_attention(q, _repeat_kv(k, g), _repeat_kv(v, g), attn_mask=mask,
+                                           is_causal=mask is None and S > 1 and past_k.shape[2] == 0)
+        return x + self.o(a.transpose(1, 2).contiguous().view(B, S, E)), k, v
+
+
+def decoder_layer_inputs(E, H, Hkv, S, P, use_mask, dtype=torch.float32):
+    g = torch.Generator().manual_seed(S + P)
+    D = E // H
+    r = lambda *shape: torch.randn(*shape, generator=g).to(dtype)
+    mask = None
+    if use_mask:      # causal mask of a chunk of S rows appended to P cached positions
+        mask = torch.zeros(2, 1, S, P + S).masked_fill(torch.ones(S, P + S).triu(P + 1).bool(), float("-inf")).to(dtype)
+    return r(2, S, E), r(1, 1, S, D), r(1, 1, S, D), r(2, Hkv, P, D), r(2, Hkv, P, D), mask
+
+
+@pytest.mark.parametrize("S,P,use_mask", [(24, 0, False), (1, 40, False), (8, 40, True)])
+@pytest.mark.parametrize("dynamic", [True, False])
+def test_decoder_layer_with_cache_and_repeated_kv_heads(S, P, use_mask, dynamic, monkeypatch):
+    """Prefill, one-token decode and a masked chunk of a decoder layer: the attention is
+    taken over, K and V are the un-repeated cache tensors (grouped heads are not copied)."""
+    monkeypatch.setattr(capture.AttentionMatch, "run", _oracle_run)
+    torch.manual_seed(0)
+    m = DecoderLayerAttention().eval()
+    ins = decoder_layer_inputs(256, 8, 2, S, P, use_mask)
+    torch._dynamo.reset()
+    before = dict(interface.stats)
+    with torch.no_grad():
+        got = torch.compile(m, backend=loopfuse_amd.loopfuse_backend, dynamic=dynamic)(*ins)
+        want = m(*ins)
+    assert interface.stats["fused"] == before["fused"] + 1
+    match = interface._MATCHES[-1]
+    assert match.k.group == 4 and match.v.group == 4
+    assert match.inputs[match.k.index].name.startswith("cat") and (match.bias is not None) == use_mask
+    for a, b in zip(got, want):
+        torch.testing.assert_close(a, b, rtol=2e-4, atol=2e-4)
