@@ -192,15 +192,27 @@ def loopfuse_compiler(gm: torch.fx.GraphModule, sample_inputs, input_names: list
 
         return codegen_fn
 
+    refused = [0]       # consecutive calls of this graph that the kernels could not serve
+
     def optimized_fn(*args):
+        if refused[0] >= 2:
+            # what the kernels refuse (dtype, head dim, layout) is a property of the traced
+            # graph, which dynamo re-traces when it changes: stop trying, each attempt runs
+            # the graph up to the fused call for nothing
+            stats["eager_runtime"] += 1
+            return gm(*args)
         try:
             out = fused_gm(*args)
         except lowering.UnsupportedPlan as e:
             if _strict():
                 raise
-            log.info("fused path not applicable to this call (%s); running the graph unfused", e)
+            refused[0] += 1
+            (log.warning if refused[0] == 2 else log.info)(
+                "fused path not applicable to this call (%s); running the graph unfused%s", e,
+                " from now on" if refused[0] == 2 else "")
             stats["eager_runtime"] += 1
             return gm(*args)
+        refused[0] = 0
         stats["fused"] += 1
         return out
 

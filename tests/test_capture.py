@@ -442,6 +442,27 @@ def test_backend_on_cpu_tensors_runs_graph_unfused():
     assert interface.stats["fused"] == before["fused"]
 
 
+def test_repeated_refusals_stop_the_attempts(monkeypatch):
+    """After two consecutive calls the kernels cannot serve, a compiled graph goes straight
+    to its captured form: the part of the rewritten graph before the fused call is not run
+    for nothing any more."""
+    attempts = []
+
+    def refuse(self, vals):
+        attempts.append(1)
+        raise lowering.UnsupportedPlan("not served")
+
+    monkeypatch.setattr(capture.AttentionMatch, "run", refuse)
+    fn = lambda q, k, v: torch.softmax(q @ k.transpose(-2, -1), dim=-1) @ v
+    q, k, v = (torch.randn(1, 2, 16, 64, generator=torch.Generator().manual_seed(s)) for s in (0, 1, 2))
+    torch._dynamo.reset()
+    before = dict(interface.stats)
+    compiled = torch.compile(fn, backend=loopfuse_amd.loopfuse_backend, dynamic=True)
+    for _ in range(5):
+        assert torch.allclose(compiled(q, k, v), fn(q, k, v), atol=1e-6)
+    assert len(attempts) == 2 and interface.stats["eager_runtime"] == before["eager_runtime"] + 5
+
+
 def test_unfused_graph_still_correct():
     def fn(a, b):
         return torch.relu(a) + b
