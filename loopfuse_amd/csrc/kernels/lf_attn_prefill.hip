@@ -98,9 +98,30 @@ __device__ __forceinline__ int lf_v_phys(int row, int ch) {
   return ch ^ (4 * ((row / LF_RPS) & (LF_CPR / 4 - 1)));
 }
 
+// Mask tensors reach the kernel as score biases of 0 / -inf.  Before the loop over a q
+// tile's KV tiles the workgroup looks for tiles whose bias is -inf for all of its rows and
+// keys: they add nothing (every probability is 0) and the loop leaves them out, loads
+// included.  Needs 8-byte aligned bias rows; not combined with the second score product
+// (no LDS left for the list at two workgroups per CU).
+#ifndef LF_BIAS_EARLY
+/* request a tile's bias values before its S^T products (not where the registers are short:
+   second score product, element-wise loads of unaligned rows) */
+#define LF_BIAS_EARLY (!LF_D2 && !(LF_BIAS & 4))
+#endif
+#ifndef LF_LIVE_LIST
+#define LF_LIVE_LIST 1        /* 0: walk every tile (for comparisons) */
+#endif
+#define LF_USE_LIVE_LIST (LF_LIVE_LIST && (LF_BIAS & 1) && !(LF_BIAS & 4) && !LF_D2)
+#define LF_LIVE_WORDS 64      /* 64-bit words of the list: q tiles with up to 4096 KV tiles use it */
+
 extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(const LfAttnParams p) {
   __shared__ __attribute__((aligned(16))) lf_elem lds_k[2][LF_BN * LF_KS];
   __shared__ __attribute__((aligned(16))) lf_elem lds_v[2][LF_BN * LF_VS];
+#if LF_USE_LIVE_LIST
+  __shared__ unsigned long long lds_dead[LF_LIVE_WORDS];     // bit r of word w: KV tile kt_begin + 64 w + r is dead
+  static_assert(sizeof(lf_elem) * LF_BN * LF_VS >= 5 * LF_LIVE_WORDS * sizeof(unsigned long long),
+                "the second V buffer holds the scratch of the dead-tile search");
+#endif
 #if LF_D2
   __shared__ __attribute__((aligned(16))) lf_elem lds_k2[2][LF_BN * LF_D2];
 #endif
@@ -332,6 +353,107 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
 #endif
   };
 
+#if LF_USE_LIVE_LIST
+  // ---- dead KV tiles of this q tile.  Scratch: the second V buffer, which nothing uses
+  // before the loop's first iteration (and the previous q tile's loop ended on a barrier).
+  const int nrel = kt_end - kt_begin;
+  const bool use_list = nrel <= 64 * LF_LIVE_WORDS;
+  if (use_list) {
+    constexpr unsigned short kNegInf = LF_DTYPE == 0 ? 0xff80u : 0xfc00u;
+    constexpr unsigned kNegInf2 = (unsigned)kNegInf * 0x10001u;
+    unsigned long long* cand = reinterpret_cast<unsigned long long*>(&lds_v[1][0]);      // [LF_LIVE_WORDS]
+    unsigned long long* part = cand + LF_LIVE_WORDS;                                      // [LF_NW][LF_LIVE_WORDS]
+    const int nwords = (nrel + 63) / 64;
+    const lf_elem* bbase = p.bias + (long long)b * p.bias_sb + (long long)h * p.bias_sh;
+    // (1) candidates: whole tiles (not the one that crosses Sk) with -inf at the bottom-left
+    // and the top-right corner (a dense bias stops here: two loads per tile)
+    for (int wi = wave; wi < nwords; wi += LF_NW) {
+      const int rel = 64 * wi + lane;
+      const int kc = min(kt_begin + rel, kt_end - 1) * LF_BN;        // first key of the tile, < Sk
+      const unsigned short bl = __builtin_bit_cast(unsigned short, bbase[(long long)qlast * p.bias_sq + kc]);
+      const unsigned short tr = __builtin_bit_cast(unsigned short, bbase[(long long)q0 * p.bias_sq + min(kc + LF_BN, p.Sk) - 1]);
+      const unsigned long long word = __builtin_amdgcn_ballot_w64(rel < nrel && kc + LF_BN <= p.Sk &&
+                                                                  bl == kNegInf && tr == kNegInf);
+      if (lane == 0) cand[wi] = word;
+    }
+    __syncthreads();
+    // (2) every wave checks its own 32 rows of each candidate, four candidates at a time
+    // (their loads are in flight together): lane (l32, g) reads row wq0 + l32 (clamped),
+    // keys 32 g .. 32 g + 31 of the tile
+    {
+      const lf_elem* brow_w = bbase + (long long)min(wq0 + l32, p.Sq - 1) * p.bias_sq + 32 * g;
+      for (int wi = 0; wi < nwords; ++wi) {
+        const unsigned long long cw = cand[wi];
+        const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)cw);
+        const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(cw >> 32));
+        unsigned long long mine = ((unsigned long long)hi << 32) | lo;
+        unsigned long long todo = mine;
+        while (todo != 0ull) {
+          int bits[4];
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            bits[c] = todo != 0ull ? __builtin_ctzll(todo) : bits[0];     // a repeat of the first is harmless
+            todo &= todo - 1ull;                                           // 0 stays 0
+          }
+          lf_u32x2 raw[4][8];
+#pragma unroll
+          for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+              raw[c][i] = *reinterpret_cast<const lf_u32x2*>(brow_w + (kt_begin + 64 * wi + bits[c]) * LF_BN + 4 * i);
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            bool dead = true;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) dead = dead && raw[c][i][0] == kNegInf2 && raw[c][i][1] == kNegInf2;
+            if (__builtin_amdgcn_ballot_w64(dead) != ~0ull) mine &= ~(1ull << bits[c]);
+          }
+        }
+        if (lane == 0) part[wave * LF_LIVE_WORDS + wi] = mine;
+      }
+    }
+    __syncthreads();
+    // (3) dead for the workgroup = dead for each of its waves
+    if (tid < nwords) {
+      unsigned long long d = part[tid];
+#pragma unroll
+      for (int w = 1; w < LF_NW; ++w) d &= part[w * LF_LIVE_WORDS + tid];
+      lds_dead[tid] = d;
+    }
+    __syncthreads();
+  }
+  // first live KV tile at or after kt (kt_end if there is none); wave-uniform
+  auto next_live = [&](int kt) -> int {
+    if (!use_list) return kt;
+    int rel = kt - kt_begin;
+    while (rel < nrel) {
+      const unsigned long long dw = lds_dead[rel >> 6];
+      const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)dw);
+      const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(dw >> 32));
+      const unsigned long long live = ~(((unsigned long long)hi << 32) | lo) >> (rel & 63);
+      if (live != 0ull) {
+        rel += __builtin_ctzll(live);
+        break;
+      }
+      rel = (rel | 63) + 1;
+    }
+    return min(kt_begin + rel, kt_end);
+  };
+
+  // the loop walks the live tiles only (all of them can be dead)
+  const int kt_first = next_live(kt_begin);
+  if (kt_first < kt_end) {
+    load_tile(kt_first, 0);
+    store_tile(0);
+  }
+  __syncthreads();
+
+  int cur = 0;
+  for (int kt = kt_first, kt_next; kt < kt_end; kt = kt_next, cur ^= 1) {
+    kt_next = next_live(kt + 1);
+    const bool have_next = kt_next < kt_end;
+    if (have_next) load_tile(kt_next, cur ^ 1);
+#else
   // every valid q tile has at least one KV tile (kt_end >= 1 > kt_begin is not
   // guaranteed only for Sk == 0, which the host rejects)
   load_tile(kt_begin, 0);
@@ -342,6 +464,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
     const int cur = (kt - kt_begin) & 1;
     const bool have_next = kt + 1 < kt_end;
     if (have_next) load_tile(kt + 1, cur ^ 1);
+#endif
 
     const int k0 = kt * LF_BN;
     bool need = wave_has_rows;
@@ -358,6 +481,26 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
     if (need) {
       const lf_elem* kbuf = lds_k[cur];
       const lf_elem* vbuf = lds_v[cur];
+#if (LF_BIAS & 1) && LF_BIAS_EARLY
+      // the tile's bias values are requested before the S^T products, which hide the latency
+      lf_elem4 bias_v[LF_NKB][4];
+      {
+        const lf_elem* brow = p.bias + (long long)b * p.bias_sb + (long long)h * p.bias_sh +
+                              (long long)min(my_q, p.Sq - 1) * p.bias_sq;
+#pragma unroll
+        for (int kb = 0; kb < LF_NKB; ++kb)
+#pragma unroll
+          for (int i4 = 0; i4 < 4; ++i4) {
+            const int j0 = k0 + 32 * kb + 8 * i4 + 4 * g;
+            if (!(LF_BIAS & 4) && j0 + 3 < p.Sk) {
+              bias_v[kb][i4] = *reinterpret_cast<const lf_elem4*>(brow + j0);
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) bias_v[kb][i4][e] = brow[min(j0 + e, p.Sk - 1)];
+            }
+          }
+      }
+#endif
 
       // ---- S^T = K Q^T (the LF_NKB accumulator chains are interleaved so that
       // consecutive MFMAs are independent)
@@ -430,12 +573,18 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
           for (int i4 = 0; i4 < 4; ++i4) {
             const int j0 = k0 + 32 * kb + 8 * i4 + 4 * g;
             lf_elem4 bv;
+#if LF_BIAS_EARLY
+            (void)j0;
+            (void)brow;
+            bv = bias_v[kb][i4];
+#else
             if (!(LF_BIAS & 4) && j0 + 3 < p.Sk) {
               bv = *reinterpret_cast<const lf_elem4*>(brow + j0);
             } else {
 #pragma unroll
               for (int e = 0; e < 4; ++e) bv[e] = brow[min(j0 + e, p.Sk - 1)];
             }
+#endif
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
 #if LF_SOFTCAP

@@ -760,3 +760,63 @@ def test_operands_on_another_device_are_refused():
         lowering.attention(q, k, v, lowering.AttnPlan(scale=0.125), score_bias=rand((1, 2, 64, 64), torch.bfloat16, 4))
     with pytest.raises(RuntimeError, match="not on the GPU"):
         lowering.attention(q, k.cpu(), v, lowering.AttnPlan(scale=0.125))
+
+
+def _mask_bias(kind, Sq, Sk, dtype, seed=0):
+    """Additive masks as a caller would pass them: 0 where a key is visible, -inf elsewhere."""
+    i = torch.arange(Sq)[:, None]
+    j = torch.arange(Sk)[None, :]
+    if kind == "causal":
+        keep = j <= i
+    elif kind == "window":
+        keep = (j <= i) & (i - j < 100)
+    elif kind == "documents":            # block-diagonal: three documents packed into one sequence
+        edges = torch.tensor([0, Sk // 3, Sk // 2, Sk])
+        doc = lambda t: torch.bucketize(t, edges[1:-1], right=True)
+        keep = (doc(i) == doc(j)) & (j <= i)
+    elif kind == "padding":              # the last keys are padding; a finite bias elsewhere
+        keep = (j < Sk - 200).expand(Sq, Sk)
+    else:
+        raise ValueError(kind)
+    m = torch.zeros(Sq, Sk).masked_fill(~keep, float("-inf"))
+    if kind == "padding":
+        m = m + torch.randn(Sq, Sk, generator=torch.Generator().manual_seed(seed)) * keep
+    return m.to(dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("kind", ["causal", "window", "documents", "padding"])
+@pytest.mark.parametrize("S,D", [(593, 64), (1300, 128)])
+def test_mask_tensors_skip_dead_tiles_without_changing_the_result(dtype, kind, S, D, monkeypatch):
+    """Mask tensors are biases of 0 / -inf; KV tiles that are -inf for a whole q tile are left
+    out of the loop.  The result must equal the oracle's and, bit for bit, the result of the
+    same kernel walking every tile."""
+    q, k, v = (rand((2, 3, S, D), dtype, s) for s in (1, 2, 3))
+    bias = _mask_bias(kind, S, S, dtype)[None, None].expand(2, 1, S, S).contiguous()
+    plan = lowering.AttnPlan(scale=D ** -0.5)
+    on = [t.to(dev()) for t in (q, k, v, bias)]
+    got = lowering.attention(*on[:3], plan, score_bias=on[3])
+    want = O.attention_reference(q, k, v, score_bias=bias.float())
+    assert (got.float().cpu() - want).abs().max().item() <= TOL[dtype]
+    monkeypatch.setenv("LOOPFUSE_KOPTS", "-DLF_LIVE_LIST=0")
+    every_tile = lowering.attention(*on[:3], plan, score_bias=on[3])
+    assert torch.equal(got, every_tile)
+
+
+def test_mask_tensor_with_rows_that_see_nothing():
+    """Rows whose keys are all masked come out as NaN, as softmax of all -inf does; the
+    other rows are unaffected (a q tile may have no live KV tile at all)."""
+    S, D = 400, 64
+    q, k, v = (rand((1, 2, S, D), torch.bfloat16, s) for s in (1, 2, 3))
+    bias = _mask_bias("causal", S, S, torch.bfloat16).clone()
+    bias[128:256] = float("-inf")          # one whole q tile
+    bias[300] = float("-inf")              # one row of another
+    bias = bias[None, None]
+    got = lowering.attention(*[t.to(dev()) for t in (q, k, v)], lowering.AttnPlan(scale=D ** -0.5),
+                             score_bias=bias.to(dev())).float().cpu()
+    want = O.attention_reference(q, k, v, score_bias=bias.float())
+    blind = torch.zeros(S, dtype=torch.bool)
+    blind[128:256] = True
+    blind[300] = True
+    assert torch.isnan(want[:, :, blind]).all() and torch.isnan(got[:, :, blind]).all()
+    assert (got[:, :, ~blind] - want[:, :, ~blind]).abs().max().item() <= TOL[torch.bfloat16]
