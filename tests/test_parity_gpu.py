@@ -820,3 +820,20 @@ def test_mask_tensor_with_rows_that_see_nothing():
     blind[300] = True
     assert torch.isnan(want[:, :, blind]).all() and torch.isnan(got[:, :, blind]).all()
     assert (got[:, :, ~blind] - want[:, :, ~blind]).abs().max().item() <= TOL[torch.bfloat16]
+
+
+@pytest.mark.parametrize("Sk", [200_000, 270_000])
+def test_mask_tensor_over_a_long_key_range(Sk):
+    """Dead-tile list over many 64-bit words (3125 KV tiles) and, past 4096 tiles, the
+    walk over every tile: live keys are scattered islands, the rest is masked."""
+    Sq, D = 128, 64
+    q, k, v = rand((1, 2, Sq, D), torch.bfloat16, 1), rand((1, 1, Sk, D), torch.bfloat16, 2), rand((1, 1, Sk, D), torch.bfloat16, 3)
+    bias = torch.full((Sq, Sk), float("-inf"))
+    for start in (0, 4096 + 17, 64 * 1000, 64 * 2047 + 5, Sk - 300):      # islands, some across tile and word borders
+        bias[:, start:start + 150] = 0.0
+    bias[5, 64 * 3000:64 * 3000 + 3] = 0.5                                # one row keeps a far tile alive
+    bias = bias.to(torch.bfloat16)[None, None]
+    got = lowering.attention(*[t.to(dev()) for t in (q, k, v)], lowering.AttnPlan(scale=D ** -0.5),
+                             score_bias=bias.to(dev())).float().cpu()
+    want = O.attention_reference(q, k, v, score_bias=bias.float())
+    assert (got - want).abs().max().item() <= TOL[torch.bfloat16]
