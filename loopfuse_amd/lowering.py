@@ -549,6 +549,13 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
             raise UnsupportedPlan(f"{what} must be a {dtype} GPU tensor")
         if t.dim() > 4:
             raise UnsupportedPlan(f"{what} has more than 4 dims")
+        if os.environ.get("LOOPFUSE_BIAS_COPY", "1") == "1" and \
+                t.dim() >= 2 and t.shape[-1] == last and t.stride(-1) == 1 and t.numel() <= (1 << 25) and \
+                (t.data_ptr() % 8 or any(st % 4 for n, st in zip(t.shape[:-1], t.stride()[:-1]) if n > 1)):
+            # rows that do not start on 8-byte borders (a mask over an odd number of keys) would
+            # be read element by element: a copy with padded rows is cheaper for tensors this small
+            padded = torch.empty((*t.shape[:-1], (last + 3) // 4 * 4), dtype=t.dtype, device=t.device)
+            t = padded[..., :last].copy_(t)
         try:
             t = t.expand(B, Hq, Sq, last)
         except RuntimeError:

@@ -170,8 +170,11 @@ def test_biased_attention_paged_kv():
     check(q, kp, vp, mask="causal", k_table=table, v_table=table, score_bias=sb)
 
 
-def test_unaligned_bias_rows():
-    # contiguous [.., 333, 333] bias: rows start at odd element offsets -> element loads
+@pytest.mark.parametrize("copy", ["1", "0"])
+def test_unaligned_bias_rows(copy, monkeypatch):
+    # contiguous [.., 333, 333] bias: rows start at odd element offsets -> a copy with padded
+    # rows (small tensors, the default) or element loads in the kernel
+    monkeypatch.setenv("LOOPFUSE_BIAS_COPY", copy)
     B, H, S, D = 1, 2, 333, 64
     q, k, v = (rand((B, H, S, D), torch.bfloat16, s) for s in (1, 2, 3))
     sb = rand((B, H, S, S), torch.bfloat16, 4)
@@ -837,3 +840,17 @@ def test_mask_tensor_over_a_long_key_range(Sk):
                              score_bias=bias.to(dev())).float().cpu()
     want = O.attention_reference(q, k, v, score_bias=bias.float())
     assert (got - want).abs().max().item() <= TOL[torch.bfloat16]
+
+
+def test_mask_tensor_over_an_odd_number_of_keys():
+    """Rows of a [.., 593, 593] mask do not start on 8-byte borders: the launcher pads them
+    in a copy, and the dead-tile list applies as for aligned masks."""
+    S, D = 593, 128
+    q, k, v = (rand((2, 2, S, D), torch.bfloat16, s) for s in (1, 2, 3))
+    bias = _mask_bias("window", S, S, torch.bfloat16)[None, None]
+    on = [t.to(dev()) for t in (q, k, v, bias)]
+    got = lowering.attention(*on[:3], lowering.AttnPlan(scale=D ** -0.5), score_bias=on[3])
+    want = O.attention_reference(q, k, v, score_bias=bias.float())
+    assert (got.float().cpu() - want).abs().max().item() <= TOL[torch.bfloat16]
+    flagged = lowering.attention(*on[:3], lowering.AttnPlan(mask="sliding", window=100, scale=D ** -0.5))
+    assert (got.float() - flagged.float()).abs().max().item() <= 2 ** -6
