@@ -53,9 +53,17 @@
 #define LF_QROWS 16          /* query rows one unit can hold (MFMA N) */
 #define LF_OSTRIDE (LF_D + 4) /* floats per row of the merge buffer */
 
+#ifndef LF_BIAS
+#define LF_BIAS 0            /* 1: additive score bias [B, kv head, row, key] (8-byte aligned rows), e.g. a mask
+                                tensor of 0 / -inf; travels with the K/V registers of its step */
+#endif
+
 struct LfDecStage {
   lf_u32x4 k[LF_NJ];
   lf_u32x4 v[LF_NJ];
+#if LF_BIAS
+  lf_elem4 bias;             // lane (q = c, g): keys 4g .. 4g + 3 of the step, query row q
+#endif
 };
 struct LfDecIds {            // page ids of one step
   long long k, v;
@@ -145,6 +153,11 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 8 / LF_DW) lf_attn_decode(co
     }
     return id;
   };
+#if LF_BIAS
+  // bias row of query column c (columns past nrows repeat the last row; their results are dropped)
+  const lf_elem* bias_row = p.bias + (long long)b * p.bias_sb + (long long)hkv * p.bias_sh +
+                            (long long)(row0 + min(c, nrows - 1)) * p.bias_sq;
+#endif
   auto issue = [&](LfDecStage& sg, int st, const LfDecIds& id) {
     const int tok = min(step_tok0(st) + c, p.Sk - 1);      // clamp: masked later, never out of bounds
     const lf_elem *kp, *vp;
@@ -160,6 +173,18 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 8 / LF_DW) lf_attn_decode(co
     for (int j = 0; j < LF_NJ; ++j) sg.k[j] = *reinterpret_cast<const lf_u32x4*>(kp + 32 * j);
 #pragma unroll
     for (int j = 0; j < LF_NJ; ++j) sg.v[j] = *reinterpret_cast<const lf_u32x4*>(vp + 32 * j);
+#if LF_BIAS
+    {
+      // keys past Sk read clamped positions: their scores are masked in consume()
+      const int t4 = step_tok0(st) + 4 * g;
+      if (t4 + 3 < p.Sk) {
+        sg.bias = *reinterpret_cast<const lf_elem4*>(bias_row + t4);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sg.bias[e] = bias_row[min(t4 + e, p.Sk - 1)];
+      }
+    }
+#endif
   };
 
   lf_elem* my_v = reinterpret_cast<lf_elem*>(smem) + wave * 2 * 16 * LF_D;
@@ -196,7 +221,12 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 8 / LF_DW) lf_attn_decode(co
       s = p.softcap * lf_tanh(s * sc_in);
 #endif
       const int tok = t0 + (i < 4 ? i : 12 + i);
+#if LF_BIAS
+      // (scaled or capped score + bias) in log2 units
+      x[i] = (tok < tok_end) ? s * cexp + lf_to_float(i < 4 ? sa.bias[i] : sb.bias[i - 4]) * LF_LOG2E : LF_NEG_INF;
+#else
       x[i] = (tok < tok_end) ? s * cexp : LF_NEG_INF;
+#endif
       mx = fmaxf(mx, x[i]);
     }
     if (__builtin_amdgcn_ballot_w64(mx > mc + (float)LF_LAZY_LOG2) != 0ull) {

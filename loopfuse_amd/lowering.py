@@ -92,6 +92,8 @@ class KernelSpec:
             o += [f"-DLF_PAGE_SIZE_V={self.page_size_v}"]
         if self.family == "decode":
             o += [f"-DLF_DW={self.waves}", f"-DLF_HEADWAVE={int(self.headwave)}"]
+            if self.bias:
+                o += ["-DLF_BIAS=1"]
         elif self.family == "prefill":
             o += [f"-DLF_V_TR={int(self.v_tr)}", f"-DLF_BIAS={self.bias}", f"-DLF_DENOM={int(self.denom)}"]
             if self.d2:
@@ -593,8 +595,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         P.q2_sb, P.q2_sh, P.q2_ss = q2.stride(0), q2.stride(1), q2.stride(2)
         P.k2_sb, P.k2_sh, P.k2_ss = k2.stride(0), k2.stride(1), k2.stride(2)
         P.k2_group = Hq // k2.shape[1]
-    if bias_bits & 3 or plan.denom_add != 0.0 or d2:
-        force_family = "prefill"
+    if bias_bits not in (0, 1) or plan.denom_add != 0.0 or d2:
+        force_family = "prefill"       # the decode kernel takes an aligned score bias and nothing else of these
 
     # ---- family: decode when there is no mask and few query rows share a KV head
     family = force_family
@@ -681,6 +683,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         rows = group
         P.q_sb, P.q_sh, P.q_ss = q.stride(0), group * q.stride(1), q.stride(1)
         P.o_sb, P.o_sh, P.o_ss = out.stride(0), group * out.stride(1), out.stride(1)
+        if bias_bits:
+            P.bias_sh, P.bias_sq = group * score_bias.stride(1), score_bias.stride(1)
     elif group == 1:
         rows = Sq
         P.q_sb, P.q_sh, P.q_ss = q.stride(0), q.stride(1), q.stride(2)
@@ -705,7 +709,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     P.rows, P.nsplit, P.split_len = rows, nsplit, split_len
     spec = KernelSpec("decode", _DTYPE_CODE[dtype], D, MASK_NONE, plan.softcap is not None, paged,
                       page_size, table_i64, rows=DECODE_QROWS, waves=waves, headwave=headwave, page_size_v=page_size_v,
-                      extra=tuple(os.environ.get("LOOPFUSE_KOPTS", "").split()))
+                      bias=bias_bits, extra=tuple(os.environ.get("LOOPFUSE_KOPTS", "").split()))
     if nsplit > 1:
         nrow = B * Hkv * rows * nsplit
         scratch = _get_scratch(q.device, nrow * (D + 2))

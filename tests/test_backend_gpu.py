@@ -404,6 +404,26 @@ def test_decoder_layer_with_cache_and_repeated_kv_heads(S, P, use_mask):
     assert torch.equal(got[1], want[1]) and torch.equal(got[2], want[2])
 
 
+def test_batched_decode_with_a_padding_mask_stays_on_the_decode_kernel():
+    """One-token decode of a left-padded batch: F.scaled_dot_product_attention with a boolean
+    [B, 1, 1, Sk] mask and grouped kv heads runs on the streaming decode kernel."""
+    import torch.nn.functional as F
+    from loopfuse_amd import lowering
+    B, Hq, Hkv, Sk, D = 4, 32, 8, 1500, 128
+    q, k, v = rand((B, Hq, 1, D), seed=1), rand((B, Hkv, Sk, D), seed=2), rand((B, Hkv, Sk, D), seed=3)
+    pad = torch.tensor([0, 1200, 64, 333])
+    keep = (torch.arange(Sk)[None, :] >= pad[:, None])[:, None, None, :]
+    def repeat_kv(h, n):
+        b, hk, s, d = h.shape
+        return h[:, :, None, :, :].expand(b, hk, n, s, d).reshape(b, hk * n, s, d)
+
+    fn = lambda q, k, v, m: F.scaled_dot_product_attention(q, repeat_kv(k, Hq // Hkv), repeat_kv(v, Hq // Hkv), attn_mask=m)
+    got = run_fused(fn, (q, k, v, keep))
+    assert lowering.attention.last_launch["kernels"][0] == "lf_attn_decode"
+    want = O.attention_reference(q, k, v, score_bias=torch.zeros(keep.shape).masked_fill(~keep, float("-inf")))
+    assert (got - want).abs().max().item() <= TOL
+
+
 def test_module_with_parameters_outside_and_inside_no_grad():
     """A module's parameters require grad: called outside torch.no_grad() the graph is
     traced for training and runs unfused (and can be differentiated); inside it the

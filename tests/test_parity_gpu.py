@@ -854,3 +854,64 @@ def test_mask_tensor_over_an_odd_number_of_keys():
     assert (got.float().cpu() - want).abs().max().item() <= TOL[torch.bfloat16]
     flagged = lowering.attention(*on[:3], lowering.AttnPlan(mask="sliding", window=100, scale=D ** -0.5))
     assert (got.float() - flagged.float()).abs().max().item() <= 2 ** -6
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", ["gqa_left_padding", "per_head_bias_softcap", "rows_view", "paged_page16", "paged_one_token",
+                                  "paged_head_per_wave"])
+def test_decode_with_score_bias(dtype, case):
+    """Decode shapes with an additive score bias (mask tensors of batched generation: left
+    padding; per-head biases) stay on the streaming decode kernel."""
+    g = torch.Generator().manual_seed(11)
+    B, Hkv, group, D, Sk, Sq = 3, 2, 4, 128, 1000, 1
+    softcap = None
+    kw = {}
+    if case == "rows_view":
+        group, Sq, Sk, D = 1, 5, 333, 64
+    if case == "paged_head_per_wave":
+        Hkv, B = 8, 2
+        kw["choice"] = {"head_per_wave": True, "splits": 2}
+    Hq = Hkv * group
+    q = rand((B, Hq, Sq, D), dtype, 1)
+    k, v = rand((B, Hkv, Sk, D), dtype, 2), rand((B, Hkv, Sk, D), dtype, 3)
+    if case == "gqa_left_padding":
+        pad = torch.tensor([0, 700, 37])            # batch 1 has its first splits fully masked
+        bias = torch.zeros(B, 1, 1, Sk).masked_fill(torch.arange(Sk)[None, None, None, :] < pad[:, None, None, None], float("-inf"))
+        kw["num_splits"] = 4
+    elif case == "per_head_bias_softcap":
+        bias, softcap = torch.randn(1, Hq, 1, Sk, generator=g), 20.0
+    elif case == "rows_view":
+        bias = torch.randn(B, Hq, Sq, Sk + 3, generator=g)[..., :Sk]       # row stride Sk + 3 = 336: aligned rows
+    else:
+        bias = torch.randn(B, 1, 1, Sk, generator=g).masked_fill(torch.rand(B, 1, 1, Sk, generator=g) < 0.2, float("-inf"))
+    bias = bias.to(dtype)
+    k_in, v_in, kt, vt = k, v, None, None
+    if case.startswith("paged"):
+        P = 1 if case == "paged_one_token" else 16
+        Skp = (Sk + P - 1) // P * P
+        n = B * Skp // P
+        perm = torch.randperm(n, generator=g)
+        table = perm.view(B, Skp // P).to(torch.int32)
+        pool_k = torch.zeros(n, P, Hkv, D, dtype=dtype)
+        pool_v = torch.zeros(n, P, Hkv, D, dtype=dtype)
+        kp = torch.nn.functional.pad(k, (0, 0, 0, Skp - Sk)).transpose(1, 2).reshape(B, Skp // P, P, Hkv, D)
+        vp = torch.nn.functional.pad(v, (0, 0, 0, Skp - Sk)).transpose(1, 2).reshape(B, Skp // P, P, Hkv, D)
+        pool_k[table.long()] = kp
+        pool_v[table.long()] = vp
+        if P == 1:
+            pool_k, pool_v = pool_k[:, 0], pool_v[:, 0]
+        k_in, v_in, kt, vt = pool_k, pool_v, table, table.clone()
+        if Skp != Sk:      # the padded keys exist in the pool: mask them
+            bias = torch.nn.functional.pad(bias, (0, Skp - Sk), value=float("-inf"))
+            k = torch.nn.functional.pad(k, (0, 0, 0, Skp - Sk))
+            v = torch.nn.functional.pad(v, (0, 0, 0, Skp - Sk))
+    plan = lowering.AttnPlan(scale=D ** -0.5, softcap=softcap, k_paged=kt is not None, v_paged=vt is not None)
+    on = lambda t: None if t is None else t.to(dev())
+    got = lowering.attention(on(q), on(k_in), on(v_in), plan, on(kt), on(vt), score_bias=on(bias), **kw)
+    assert lowering.attention.last_launch["kernels"][0] == "lf_attn_decode"
+    assert lowering.attention.last_launch["head_per_wave"] == (case == "paged_head_per_wave")
+    want = O.attention_reference(q, k, v, softcap=softcap, score_bias=bias.float())
+    assert (got.float().cpu() - want).abs().max().item() <= TOL[dtype]
+    if case == "gqa_left_padding":
+        one = lowering.attention(on(q), on(k_in), on(v_in), plan, score_bias=on(bias), num_splits=1)
+        assert (got.float() - one.float()).abs().max().item() <= 2 ** -7
