@@ -32,7 +32,7 @@ typedef struct LfAttnParamsHost {
   float* part_acc;      /* decode split-K scratch: [units, nsplit, rows, D] floats */
   float* part_ml;       /* decode split-K scratch: [units, nsplit, rows, 2] floats */
   unsigned char* visits;/* optional [B*Hq*q_tiles, kv_tiles] visited-tile record, else NULL */
-  const void* bias;     /* LF_BIAS & 1: additive score bias [B, Hq, Sq, Sk] */
+  const void* bias;     /* LF_BIAS & 1: additive score bias [B, Hq, Sq, Sk]; lf_attn_decode -DLF_BIAS=1: [B, Hkv, rows, Sk] */
   const void* obias;    /* LF_BIAS & 2: additive output bias [B, Hq, Sq, D] */
   const void* q2;       /* LF_D2: second score product Q2 [B, Hq, Sq, D2] ... */
   const void* k2;       /* ... K2 [B, Hq / k2_group, Sk, D2] */
