@@ -327,7 +327,7 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 8 / LF_DW) lf_attn_decode(co
     const int qr = row0 + c;
     if (p.nsplit == 1) {
       lf_elem* orow = p.o + (long long)b * p.o_sb + (long long)hkv * p.o_sh + (long long)qr * p.o_ss;
-      const float inv = 1.0f / l_wave;
+      const float inv = lf_inv_sum(l_wave);
 #pragma unroll
       for (int db = 0; db < LF_NDB; ++db) {
         lf_elem4 w4;
@@ -386,7 +386,7 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 8 / LF_DW) lf_attn_decode(co
     const int qr = row0 + qi;
     if (p.nsplit == 1) {
       lf_elem* orow = p.o + (long long)b * p.o_sb + (long long)hkv * p.o_sh + (long long)qr * p.o_ss;
-      const float inv = 1.0f / l_tot;
+      const float inv = lf_inv_sum(l_tot);
       lf_elem8 w8;
 #pragma unroll
       for (int e = 0; e < 8; ++e) w8[e] = lf_from_float(sum[e] * inv);
@@ -449,7 +449,7 @@ extern "C" __global__ void __launch_bounds__(256) lf_attn_decode_combine(const L
     m = mc;
   }
   lf_elem* orow = p.o + (long long)b * p.o_sb + (long long)hkv * p.o_sh + (long long)qr * p.o_ss;
-  const float inv = 1.0f / l;
+  const float inv = lf_inv_sum(l);
   lf_elem4 w;
 #pragma unroll
   for (int e = 0; e < 4; ++e) w[e] = lf_from_float(a[e] * inv);

@@ -722,7 +722,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
     // sum and extra term in the same units: l is relative to the lagging offset
     l_tot += p.denom_add * lf_exp2(mc_true - mc_ref);
 #endif
-    const float inv = 1.0f / l_tot;
+    const float inv = lf_inv_sum(l_tot);
     lf_elem* orow = p.o + (long long)b * p.o_sb + (long long)h * p.o_sh + (long long)my_q * p.o_ss;
 #pragma unroll
     for (int db = 0; db < LF_NDB; ++db)

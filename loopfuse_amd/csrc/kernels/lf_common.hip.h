@@ -78,6 +78,20 @@ typedef int lf_table_t;
 #define LF_NEG_INF (-__builtin_inff())
 #define LF_LOG2E 1.4426950408889634f
 
+// 1 / l for the final normalisation.  -DLF_SAFE=1: a query row that saw no key at all
+// (l == 0: every score was -inf) comes out as zeros, which is what torch's fused attention
+// ops return for it; the default is 0 * inf = NaN, what softmax of a row of -inf gives.
+#ifndef LF_SAFE
+#define LF_SAFE 0
+#endif
+__device__ __forceinline__ float lf_inv_sum(float l) {
+#if LF_SAFE
+  return l > 0.0f ? 1.0f / l : 0.0f;
+#else
+  return 1.0f / l;
+#endif
+}
+
 // Kernel parameter block.  Mirrors loopfuse_amd/lowering.py::AttnParams field
 // for field (pointers, then 64-bit element strides, then 32-bit scalars).
 struct LfAttnParams {

@@ -76,6 +76,7 @@ class KernelSpec:
     pack: int = 0          # prefill_swp, grouped-query attention: a workgroup's waves take 2 or 4 heads of one group
     page_size_v: int = 0   # tokens per page of the V pool when it differs from K's (0 = same)
     d2: int = 0            # prefill: depth of a second score product Q2 K2^T (0, 16, 32, 64)
+    safe: bool = False     # rows that saw no key come out as zeros instead of NaN
     extra: tuple = ()      # further -D options (tuning experiments)
 
     def options(self) -> list[str]:
@@ -100,6 +101,8 @@ class KernelSpec:
                 o += [f"-DLF_D2={self.d2}"]
         elif self.family == "prefill_swp" and self.pack:
             o += [f"-DLF_GQAPACK={int(self.pack)}"]
+        if self.safe:
+            o += ["-DLF_SAFE=1"]
         return o + list(self.extra)
 
     def files(self) -> tuple[str, ...]:
@@ -114,6 +117,7 @@ class KernelSpec:
         return (f"lf_{self.family}_t{self.dtype}_d{self.head_dim}_m{self.mask}_c{int(self.softcap)}"
                 f"_p{self.paged}x{self.page_size}i{int(self.table_i64)}_r{self.rows}w{self.waves}v{int(self.v_tr)}h{int(self.headwave)}b{self.bias}n{int(self.denom)}"
                 + (f"_q{self.d2}" if self.d2 else "") + (f"_gp{int(self.pack)}" if self.pack else "") + (f"_pv{self.page_size_v}" if self.page_size_v else "")
+                + ("_z" if self.safe else "")
                 + "".join("_" + e.replace("-D", "").replace("=", "") for e in self.extra))
 
     def source(self) -> str:
@@ -233,6 +237,8 @@ class AttnPlan:
     k_paged: bool = False
     v_paged: bool = False
     denom_add: float = 0.0             # probabilities are e^(x-max) / (sum e^(x-max) + denom_add)
+    zero_blind_rows: bool = False      # a row whose keys are all masked by the score bias gives zeros (as torch's
+                                       # fused attention ops do) instead of the NaN of a softmax over -inf
 
 
 class UnsupportedPlan(ValueError):
@@ -645,7 +651,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
             pack = 4 if group % 4 == 0 else 2
         spec = KernelSpec(family, _DTYPE_CODE[dtype], D, mask, plan.softcap is not None, paged,
                           page_size, table_i64, v_tr=v_tr if family == "prefill" else True, bias=bias_bits,
-                          denom=plan.denom_add != 0.0, d2=d2, page_size_v=page_size_v, pack=pack, extra=extra)
+                          denom=plan.denom_add != 0.0, d2=d2, page_size_v=page_size_v, pack=pack, extra=extra,
+                          safe=plan.zero_blind_rows and bool(bias_bits & 1) and family == "prefill")
         bm, bn = TILE_SHAPES[family]
         nw = 4
         for e in spec.extra:                    # tuning: -DLF_NW=8 doubles the q tile
@@ -709,7 +716,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     P.rows, P.nsplit, P.split_len = rows, nsplit, split_len
     spec = KernelSpec("decode", _DTYPE_CODE[dtype], D, MASK_NONE, plan.softcap is not None, paged,
                       page_size, table_i64, rows=DECODE_QROWS, waves=waves, headwave=headwave, page_size_v=page_size_v,
-                      bias=bias_bits, extra=tuple(os.environ.get("LOOPFUSE_KOPTS", "").split()))
+                      bias=bias_bits, safe=plan.zero_blind_rows and bool(bias_bits),
+                      extra=tuple(os.environ.get("LOOPFUSE_KOPTS", "").split()))
     if nsplit > 1:
         nrow = B * Hkv * rows * nsplit
         scratch = _get_scratch(q.device, nrow * (D + 2))

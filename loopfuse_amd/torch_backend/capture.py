@@ -106,6 +106,7 @@ class Stage:
     lay: Any = None
     mat: tuple = ()                    # (Sq, Sk) stand-ins
     late_factors: list = dataclasses.field(default_factory=list)   # run-time factors applied after the mask: must be > 0
+    zero_blind_rows: bool = False      # torch's fused attention ops: a row with every key masked gives zeros
 
 
 @dataclasses.dataclass
@@ -211,6 +212,7 @@ class AttentionMatch:
     # return [B, H, S, D] views of [B, S, H, D] storage, and the graph after them may rely on
     # it): dims from outermost to innermost; () = row-major
     out_order: tuple = ()
+    zero_blind_rows: bool = False  # rows whose keys are all masked give zeros (torch's fused attention ops), not NaN
 
     def empty_out(self, vals, dtype, device) -> torch.Tensor:
         """Uninitialised output in the traced shape and memory order."""
@@ -267,7 +269,8 @@ class AttentionMatch:
             scale *= math.log(2.0)
         return lowering.AttnPlan(mask=self.mask, window=int(window), scale=scale, softcap=softcap,
                                  k_paged=self.k.paged, v_paged=self.v.paged,
-                                 denom_add=sum(self._number(t, vals) for t in self.denom_add))
+                                 denom_add=sum(self._number(t, vals) for t in self.denom_add),
+                                 zero_blind_rows=self.zero_blind_rows)
 
     def _operand(self, op: Operand, vals):
         t = vals[op.index]
@@ -831,7 +834,7 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
         # boolean masks into 0 / -inf before it dispatches): the kernels' score bias
         return Stage("out", tuple(qi.t.shape[:-1]) + (vi.t.shape[-1],), qi, Ids(ki.src, ki.t.transpose(-1, -2)), vi,
                      factors=[scale], mask="causal" if given.get("is_causal", False) else None, mat=(sq, sk),
-                     bias=None if bias is None else (bias, tuple(qi.t.shape[:-1]) + (sk,)))
+                     bias=None if bias is None else (bias, tuple(qi.t.shape[:-1]) + (sk,)), zero_blind_rows=True)
 
     def pattern_step(node, tgt, a, kw, first):
         """The abstract value of ``node`` if it continues a pattern; raises _Skip otherwise."""
@@ -1200,4 +1203,4 @@ def _build_match(out_node: torch.fx.Node, st: Stage) -> AttentionMatch:
                           [scalar(f) for f in st.post_factors], st.has_tanh, st.mask, window, out_rank,
                           bias_op, obias_op, denom_add=tuple(scalar(t) for t in st.denom_add), base2=st.base2,
                           q2=q2_op, k2=k2_op, late_factors=tuple(scalar(f) for f in st.late_factors),
-                          out_order=out_order)
+                          out_order=out_order, zero_blind_rows=st.zero_blind_rows)

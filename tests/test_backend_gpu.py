@@ -424,6 +424,22 @@ def test_batched_decode_with_a_padding_mask_stays_on_the_decode_kernel():
     assert (got - want).abs().max().item() <= TOL
 
 
+def test_rows_without_a_visible_key_give_zeros_like_the_stock_op():
+    """Left-padded prefill: the padded query rows see no key.  torch's fused attention returns
+    zeros for them (NaN there would leak into later layers through K and V); so does the take-over."""
+    import torch.nn.functional as F
+    B, H, S, D = 2, 4, 300, 64
+    q, k, v = (rand((B, H, S, D), seed=s) for s in (1, 2, 3))
+    pad = torch.tensor([0, 130])
+    i, j = torch.arange(S)[:, None], torch.arange(S)[None, :]
+    keep = ((j <= i)[None] & (j[None] >= pad[:, None, None]))[:, None]            # causal and not padding
+    fn = lambda q, k, v, m: F.scaled_dot_product_attention(q, k, v, attn_mask=m)
+    got = run_fused(fn, (q, k, v, keep))
+    stock = fn(*[t.to(DEV) for t in (q, k, v, keep)]).float().cpu()
+    assert (got[1, :, :130] == 0).all() and (stock[1, :, :130] == 0).all()
+    assert (got - stock).abs().max().item() <= TOL
+
+
 def test_module_with_parameters_outside_and_inside_no_grad():
     """A module's parameters require grad: called outside torch.no_grad() the graph is
     traced for training and runs unfused (and can be differentiated); inside it the

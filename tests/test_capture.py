@@ -275,6 +275,8 @@ def _oracle_run(self, vals):
                                 score_bias=self._bias_view(self.bias, vals, (B, Hq, Sq, Sk)),
                                 out_bias=self._bias_view(self.out_bias, vals, (B, Hq, Sq, D)),
                                 **self._second_product(vals)).to(q.dtype)
+    if plan.zero_blind_rows:
+        out = out.nan_to_num(nan=0.0)
     return self.empty_out(vals, out.dtype, out.device).copy_(out.reshape(self.out_shape(vals)))
 
 

@@ -915,3 +915,36 @@ def test_decode_with_score_bias(dtype, case):
     if case == "gqa_left_padding":
         one = lowering.attention(on(q), on(k_in), on(v_in), plan, score_bias=on(bias), num_splits=1)
         assert (got.float() - one.float()).abs().max().item() <= 2 ** -7
+
+
+@pytest.mark.parametrize("shape", ["prefill", "decode", "decode_split"])
+def test_rows_that_see_nothing_give_zeros_when_asked(shape):
+    """AttnPlan.zero_blind_rows (what torch's fused attention ops do, and what the front end
+    sets for them): zeros instead of NaN for rows whose keys are all masked; other rows unchanged."""
+    D = 64
+    if shape == "prefill":
+        B, H, Sq, Sk = 1, 2, 400, 400
+        bias = _mask_bias("causal", Sq, Sk, torch.bfloat16).clone()
+        bias[128:256] = float("-inf")
+        bias[300] = float("-inf")
+        bias = bias[None, None]
+        blind = torch.isinf(bias[0, 0]).all(-1)[None, None].expand(B, H, Sq)
+        kw = {}
+    else:
+        B, H, Sq, Sk = 3, 4, 1, 1200
+        bias = torch.zeros(B, 1, 1, Sk)
+        bias[1] = float("-inf")                     # one sequence of the batch sees nothing
+        bias[2, ..., :900] = float("-inf")
+        bias = bias.to(torch.bfloat16)
+        blind = torch.zeros(B, H, Sq, dtype=torch.bool)
+        blind[1] = True
+        kw = {"num_splits": 4 if shape == "decode_split" else 1}
+    q, k, v = rand((B, H, Sq, D), torch.bfloat16, 1), rand((B, H, Sk, D), torch.bfloat16, 2), rand((B, H, Sk, D), torch.bfloat16, 3)
+    on = [t.to(dev()) for t in (q, k, v, bias)]
+    want = O.attention_reference(q, k, v, score_bias=bias.float())
+    assert torch.isnan(want[blind]).all()
+    for zero in (False, True):
+        got = lowering.attention(*on[:3], lowering.AttnPlan(scale=D ** -0.5, zero_blind_rows=zero), score_bias=on[3], **kw).float().cpu()
+        assert lowering.attention.last_launch["kernels"][0] == ("lf_attn_prefill" if shape == "prefill" else "lf_attn_decode")
+        assert (got[blind] == 0).all() if zero else torch.isnan(got[blind]).all()
+        assert (got[~blind] - want[~blind]).abs().max().item() <= TOL[torch.bfloat16]
