@@ -948,3 +948,49 @@ def test_rows_that_see_nothing_give_zeros_when_asked(shape):
         assert lowering.attention.last_launch["kernels"][0] == ("lf_attn_prefill" if shape == "prefill" else "lf_attn_decode")
         assert (got[blind] == 0).all() if zero else torch.isnan(got[blind]).all()
         assert (got[~blind] - want[~blind]).abs().max().item() <= TOL[torch.bfloat16]
+
+
+def _mask_sweep_case(i):
+    """Case i of a seeded sweep over score biases that hold -inf regions (mask tensors)."""
+    g = torch.Generator().manual_seed(5000 + i)
+    ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    pick = lambda xs: xs[ri(0, len(xs) - 1)]
+    kind = pick(["prefill", "prefill", "rect", "decode", "decode"])
+    c = dict(dtype=pick([torch.bfloat16, torch.float16]), D=pick([64, 128]), B=ri(1, 3), Hkv=pick([1, 2, 8]),
+             group=pick([1, 2, 4]), kind=kind, softcap=pick([None, None, 30.0]),
+             bcast=pick(["none", "batch", "head", "both", "row"]), noise=pick([False, True]),
+             blocks=ri(1, 6), flag=pick([None, None, "causal"]) if kind == "prefill" else None, seed=6000 + i)
+    if kind == "prefill":
+        c["Sq"] = c["Sk"] = ri(1, 900)
+    elif kind == "rect":
+        c["Sq"], c["Sk"] = ri(1, 300), ri(1, 1500)
+    else:
+        c["Sq"], c["Sk"] = 1, ri(16, 4000)
+        c["splits"] = pick([None, None, 1, 3])
+    return c
+
+
+@pytest.mark.parametrize("i", range(24))
+def test_seeded_mask_sweep(i):
+    c = _mask_sweep_case(i)
+    dt, D, B, Hkv, Sq, Sk = c["dtype"], c["D"], c["B"], c["Hkv"], c["Sq"], c["Sk"]
+    Hq = Hkv * c["group"]
+    g = torch.Generator().manual_seed(c["seed"])
+    bshape = [B, Hq, Sq, Sk]
+    if c["bcast"] in ("batch", "both"):
+        bshape[0] = 1
+    if c["bcast"] in ("head", "both"):
+        bshape[1] = 1
+    if c["bcast"] == "row":
+        bshape[2] = 1
+    bias = torch.randn(bshape, generator=g) if c["noise"] else torch.zeros(bshape)
+    for _ in range(c["blocks"]):              # rectangles of -inf, some larger than a 128 x 64 tile
+        r0, c0 = int(torch.randint(0, bshape[2], (1,), generator=g)), int(torch.randint(0, Sk, (1,), generator=g))
+        h, w = int(torch.randint(1, 400, (1,), generator=g)), int(torch.randint(1, 900, (1,), generator=g))
+        bias[..., r0:r0 + h, c0:c0 + w] = float("-inf")
+    bias[..., 0] = 0.0                        # every row keeps a visible key
+    bias = bias.to(dt)
+    q, k, v = rand((B, Hq, Sq, D), dt, c["seed"] + 1), rand((B, Hkv, Sk, D), dt, c["seed"] + 2), rand((B, Hkv, Sk, D), dt, c["seed"] + 3)
+    print("mask sweep case", i, {**c, "bias_shape": bshape}, flush=True)
+    kw = {"num_splits": c["splits"]} if c.get("splits") else {}
+    check(q, k, v, mask=c["flag"], softcap=c["softcap"], score_bias=bias, **kw)
