@@ -373,6 +373,17 @@ class AttentionMatch:
         d2 = self._operand(self.q2, vals)[0].shape[-1] if self.q2 is not None else 0
         if d2 not in (0, 16, 32, 64):
             raise lowering.UnsupportedPlan("depth of the second score product not served by the HIP kernels")
+        kd, _ = self._operand(self.k, vals)
+        B, Hq, Sq, Sk, _ = self._shapes(vals)
+        hkv = kd.shape[-2] if self.k.paged else kd.shape[1]
+        grp = Hq // max(hkv, 1)
+        if plan.mask is None and bias in (0, 1) and not d2 and plan.denom_add == 0.0 and Sk >= 16 and \
+                ((Sq == 1 and grp <= 64) or (grp == 1 and Sq <= 16)):
+            # decode shapes stream K/V once (which of the two work splits serves them depends on the
+            # device; the four-wave one is reported)
+            return [lowering.KernelSpec("decode", dt, D, lowering.MASK_NONE, plan.softcap is not None, paged, ps, i64,
+                                        rows=lowering.DECODE_QROWS, waves=4, page_size_v=psv, bias=bias,
+                                        safe=plan.zero_blind_rows and bool(bias))]
         family = "prefill" if (paged or bias or d2) else lowering.prefill_variant(q.shape[-2])
         extra = ("-DLF_DMA=1",) if ((bias or d2) and not paged) else ()
         pack = 0
@@ -382,7 +393,8 @@ class AttentionMatch:
             if q.shape[1] % max(kd.shape[1], 1) == 0 and grp % 2 == 0:
                 pack = 4 if grp % 4 == 0 else 2
         return [lowering.KernelSpec(family, dt, D, mask, plan.softcap is not None, paged, ps, i64, bias=bias, d2=d2,
-                                    page_size_v=psv, pack=pack, extra=extra)]
+                                    page_size_v=psv, pack=pack, extra=extra,
+                                    safe=plan.zero_blind_rows and bool(bias & 1) and family == "prefill")]
 
 
 # ----------------------------------------------------------------------------

@@ -528,6 +528,15 @@ def test_codegen_only_returns_kernel_objects_without_a_gpu(shim_built, monkeypat
     prg = torch.compile(two, backend=loopfuse_amd.loopfuse_backend, dynamic=True)(q, k, v, k, v)
     assert len(prg) == 2 and "-DLF_MASK=0" in prg[0].code and "-DLF_MASK=2" in prg[1].code
 
+    def decode(Q, K, V, M):          # one query row per head, grouped kv heads, a padding mask: the streaming kernel
+        S = (Q @ K.repeat_interleave(4, dim=1).transpose(-2, -1)) * 0.125 + M
+        return torch.softmax(S, dim=-1) @ V.repeat_interleave(4, dim=1)
+
+    torch._dynamo.reset()
+    prg = torch.compile(decode, backend=loopfuse_amd.loopfuse_backend, dynamic=True)(
+        bf(2, 8, 1, 64), bf(2, 2, 320, 64, seed=1), bf(2, 2, 320, 64, seed=2), bf(2, 1, 1, 320, seed=3))
+    assert len(prg) == 1 and "lf_attn_decode" in prg.code and "-DLF_BIAS=1" in prg.code
+
 
 @pytest.mark.parametrize("which", ["causal", "gqa_window_softcap", "paged_decode", "block"])
 def test_static_shapes_at_real_sizes_are_matched(which, monkeypatch):
