@@ -106,8 +106,46 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 8 / LF_DW) lf_attn_decode(co
   const int row0 = rc * LF_QROWS;
   const int nrows = min(p.rows - row0, LF_QROWS);          // query rows of this unit
 
-  const int tok_begin = z * p.split_len;
-  const int tok_end = min(tok_begin + p.split_len, p.Sk);
+  int tok_begin = z * p.split_len;
+  int tok_end = min(tok_begin + p.split_len, p.Sk);
+#if LF_BIAS
+  // Keys whose bias is -inf for every query row of the unit add nothing.  The split is narrowed
+  // to the span from its first to its last live key (the left padding of a batch, the unused
+  // tail of a fixed-size cache are then never read); a split without a live key does no work.
+  // Every wave scans the same values (4 keys per lane, 256 per step) and finds the same span.
+  {
+    constexpr unsigned short kNegInf = LF_DTYPE == 0 ? 0xff80u : 0xfc00u;
+    constexpr unsigned kNegInf2 = (unsigned)kNegInf * 0x10001u;
+    const lf_elem* bb = p.bias + (long long)b * p.bias_sb + (long long)hkv * p.bias_sh + (long long)row0 * p.bias_sq;
+    const int nscan = p.bias_sq == 0 ? 1 : nrows;       // rows that share one bias row are scanned once
+    int first = 0x7fffffff, last = -1;                  // relative to tok_begin
+    for (int base = tok_begin; base < tok_end; base += 256) {
+      const int t4 = base + 4 * lane;
+      bool lv = false;
+      for (int r = 0; r < nscan; ++r) {
+        const lf_elem* br = bb + (long long)r * p.bias_sq;
+        if (t4 + 3 < tok_end) {
+          const lf_u32x2 raw = *reinterpret_cast<const lf_u32x2*>(br + t4);
+          lv = lv || raw[0] != kNegInf2 || raw[1] != kNegInf2;
+        } else {
+          for (int e = 0; e < 4; ++e)
+            if (t4 + e < tok_end) lv = lv || __builtin_bit_cast(unsigned short, br[t4 + e]) != kNegInf;
+        }
+      }
+      const unsigned long long live = __builtin_amdgcn_ballot_w64(lv);
+      if (live != 0ull) {
+        first = min(first, base - tok_begin + 4 * (int)__builtin_ctzll(live));
+        last = max(last, base - tok_begin + 4 * (63 - (int)__builtin_clzll(live)) + 3);
+      }
+    }
+    if (last < 0) {
+      tok_end = tok_begin;
+    } else {
+      tok_end = min(tok_end, tok_begin + last + 1);
+      tok_begin += first & ~31;                         // whole pairs of 16-key steps
+    }
+  }
+#endif
   const int npairs = (max(tok_end - tok_begin, 0) + 31) / 32;
 
   // ---- B operand of S^T = K Q^T: lane (q = c, g) holds Q[row0 + q][32*j + 8*g .. +7];

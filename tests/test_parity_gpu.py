@@ -988,9 +988,41 @@ def test_seeded_mask_sweep(i):
         r0, c0 = int(torch.randint(0, bshape[2], (1,), generator=g)), int(torch.randint(0, Sk, (1,), generator=g))
         h, w = int(torch.randint(1, 400, (1,), generator=g)), int(torch.randint(1, 900, (1,), generator=g))
         bias[..., r0:r0 + h, c0:c0 + w] = float("-inf")
-    bias[..., 0] = 0.0                        # every row keeps a visible key
+    # every row keeps a visible key: the first one, or any one for decode shapes (spans that
+    # start and end anywhere)
+    bias[..., int(torch.randint(0, Sk, (1,), generator=g)) if c["kind"] == "decode" else 0] = 0.0
     bias = bias.to(dt)
     q, k, v = rand((B, Hq, Sq, D), dt, c["seed"] + 1), rand((B, Hkv, Sk, D), dt, c["seed"] + 2), rand((B, Hkv, Sk, D), dt, c["seed"] + 3)
     print("mask sweep case", i, {**c, "bias_shape": bshape}, flush=True)
     kw = {"num_splits": c["splits"]} if c.get("splits") else {}
     check(q, k, v, mask=c["flag"], softcap=c["softcap"], score_bias=bias, **kw)
+
+
+@pytest.mark.parametrize("paged", [False, True])
+def test_decode_reads_only_the_live_span_of_a_fixed_size_cache(paged):
+    """A cache allocated for 4096 keys with 37..700 of them filled, left padding in front: the
+    mask leaves a short live span per sequence; results equal attention over exactly those keys."""
+    B, Hkv, group, D, Sk = 4, 8, 4, 128, 4096
+    Hq = Hkv * group
+    lo = torch.tensor([0, 100, 33, 512])
+    hi = torch.tensor([37, 700, 34, 4096])           # one sequence with a single live key, one filled to the end
+    j = torch.arange(Sk)[None, :]
+    keep = (j >= lo[:, None]) & (j < hi[:, None])
+    bias = torch.zeros(B, 1, 1, Sk).masked_fill(~keep[:, None, None, :], float("-inf")).to(torch.bfloat16)
+    q, k, v = rand((B, Hq, 1, D), torch.bfloat16, 1), rand((B, Hkv, Sk, D), torch.bfloat16, 2), rand((B, Hkv, Sk, D), torch.bfloat16, 3)
+    want = torch.stack([O.attention_reference(q[b:b + 1], k[b:b + 1, :, lo[b]:hi[b]], v[b:b + 1, :, lo[b]:hi[b]])[0] for b in range(B)])
+    k_in, v_in, kt, vt = k, v, None, None
+    if paged:
+        P = 16
+        n = B * Sk // P
+        table = torch.randperm(n, generator=torch.Generator().manual_seed(4)).view(B, Sk // P).to(torch.int32)
+        pool_k = torch.empty(n, P, Hkv, D, dtype=torch.bfloat16)
+        pool_v = torch.empty(n, P, Hkv, D, dtype=torch.bfloat16)
+        pool_k[table.long()] = k.transpose(1, 2).reshape(B, Sk // P, P, Hkv, D)
+        pool_v[table.long()] = v.transpose(1, 2).reshape(B, Sk // P, P, Hkv, D)
+        k_in, v_in, kt, vt = pool_k, pool_v, table, table.clone()
+    on = lambda t: None if t is None else t.to(dev())
+    plan = lowering.AttnPlan(scale=D ** -0.5, k_paged=paged, v_paged=paged)
+    got = lowering.attention(on(q), on(k_in), on(v_in), plan, on(kt), on(vt), score_bias=on(bias)).float().cpu()
+    assert lowering.attention.last_launch["kernels"][0] == "lf_attn_decode"
+    assert (got - want).abs().max().item() <= TOL[torch.bfloat16]
