@@ -114,8 +114,6 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 8 / LF_DW) lf_attn_decode(co
   // tail of a fixed-size cache are then never read); a split without a live key does no work.
   // Every wave scans the same values (4 keys per lane, 256 per step) and finds the same span.
   {
-    constexpr unsigned short kNegInf = LF_DTYPE == 0 ? 0xff80u : 0xfc00u;
-    constexpr unsigned kNegInf2 = (unsigned)kNegInf * 0x10001u;
     const lf_elem* bb = p.bias + (long long)b * p.bias_sb + (long long)hkv * p.bias_sh + (long long)row0 * p.bias_sq;
     const int nscan = p.bias_sq == 0 ? 1 : nrows;       // rows that share one bias row are scanned once
     int first = 0x7fffffff, last = -1;                  // relative to tok_begin
@@ -126,10 +124,10 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 8 / LF_DW) lf_attn_decode(co
         const lf_elem* br = bb + (long long)r * p.bias_sq;
         if (t4 + 3 < tok_end) {
           const lf_u32x2 raw = *reinterpret_cast<const lf_u32x2*>(br + t4);
-          lv = lv || raw[0] != kNegInf2 || raw[1] != kNegInf2;
+          lv = lv || !lf_bias_masked2(raw[0]) || !lf_bias_masked2(raw[1]);
         } else {
           for (int e = 0; e < 4; ++e)
-            if (t4 + e < tok_end) lv = lv || __builtin_bit_cast(unsigned short, br[t4 + e]) != kNegInf;
+            if (t4 + e < tok_end) lv = lv || !lf_bias_masked(__builtin_bit_cast(unsigned short, br[t4 + e]));
         }
       }
       const unsigned long long live = __builtin_amdgcn_ballot_w64(lv);

@@ -359,8 +359,6 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
   const int nrel = kt_end - kt_begin;
   const bool use_list = nrel <= 64 * LF_LIVE_WORDS;
   if (use_list) {
-    constexpr unsigned short kNegInf = LF_DTYPE == 0 ? 0xff80u : 0xfc00u;
-    constexpr unsigned kNegInf2 = (unsigned)kNegInf * 0x10001u;
     unsigned long long* cand = reinterpret_cast<unsigned long long*>(&lds_v[1][0]);      // [LF_LIVE_WORDS]
     unsigned long long* part = cand + LF_LIVE_WORDS;                                      // [LF_NW][LF_LIVE_WORDS]
     const int nwords = (nrel + 63) / 64;
@@ -373,7 +371,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
       const unsigned short bl = __builtin_bit_cast(unsigned short, bbase[(long long)qlast * p.bias_sq + kc]);
       const unsigned short tr = __builtin_bit_cast(unsigned short, bbase[(long long)q0 * p.bias_sq + min(kc + LF_BN, p.Sk) - 1]);
       const unsigned long long word = __builtin_amdgcn_ballot_w64(rel < nrel && kc + LF_BN <= p.Sk &&
-                                                                  bl == kNegInf && tr == kNegInf);
+                                                                  lf_bias_masked(bl) && lf_bias_masked(tr));
       if (lane == 0) cand[wi] = word;
     }
     __syncthreads();
@@ -405,7 +403,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
           for (int c = 0; c < 4; ++c) {
             bool dead = true;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) dead = dead && raw[c][i][0] == kNegInf2 && raw[c][i][1] == kNegInf2;
+            for (int i = 0; i < 8; ++i) dead = dead && lf_bias_masked2(raw[c][i][0]) && lf_bias_masked2(raw[c][i][1]);
             if (__builtin_amdgcn_ballot_w64(dead) != ~0ull) mine &= ~(1ull << bits[c]);
           }
         }

@@ -84,6 +84,26 @@ typedef int lf_table_t;
 #ifndef LF_SAFE
 #define LF_SAFE 0
 #endif
+// Score-bias values that mark a key as masked, for the searches that leave keys out which
+// no query row can see (16-bit patterns; the second form takes two packed values).  -inf
+// always.  With LF_SAFE also the finite values masks are commonly filled with, the most
+// negative finite number of the storage type and its binade (<= -1.7e38 for bf16,
+// <= -57344 for fp16): next to any visible key their probabilities underflow to exactly 0,
+// so leaving them out changes nothing for a row that sees a key; a row that sees none
+// gives zeros under LF_SAFE either way.  NaN never counts.
+__device__ __forceinline__ bool lf_bias_masked(unsigned bits) {
+  constexpr unsigned kNegInf = LF_DTYPE == 0 ? 0xff80u : 0xfc00u;
+#if LF_SAFE
+  constexpr unsigned kFloor = LF_DTYPE == 0 ? 0xff00u : 0xfb00u;
+  return bits >= kFloor && bits <= kNegInf;
+#else
+  return bits == kNegInf;
+#endif
+}
+__device__ __forceinline__ bool lf_bias_masked2(unsigned raw) {
+  return lf_bias_masked(raw & 0xffffu) && lf_bias_masked(raw >> 16);
+}
+
 __device__ __forceinline__ float lf_inv_sum(float l) {
 #if LF_SAFE
   return l > 0.0f ? 1.0f / l : 0.0f;

@@ -1026,3 +1026,32 @@ def test_decode_reads_only_the_live_span_of_a_fixed_size_cache(paged):
     got = lowering.attention(on(q), on(k_in), on(v_in), plan, on(kt), on(vt), score_bias=on(bias)).float().cpu()
     assert lowering.attention.last_launch["kernels"][0] == "lf_attn_decode"
     assert (got - want).abs().max().item() <= TOL[torch.bfloat16]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", ["prefill", "decode"])
+def test_masks_filled_with_the_most_negative_finite_value(dtype, shape):
+    """Masks are often filled with torch.finfo(dtype).min instead of -inf.  With
+    zero_blind_rows (attentions taken over from torch's fused op) such keys are left out like
+    -inf ones: bit-equal to the -inf mask, equal to the oracle on rows that see a key, finite
+    on rows that see none."""
+    D = 64
+    if shape == "prefill":
+        B, H, Sq, Sk = 2, 2, 700, 700
+        keep = (torch.arange(Sk)[None, :] <= torch.arange(Sq)[:, None]) & (torch.arange(Sk)[None, :] >= 200)
+        keep = keep[None, None].expand(B, 1, Sq, Sk)
+    else:
+        B, H, Sq, Sk = 3, 4, 1, 3000
+        keep = ((torch.arange(Sk)[None, :] >= torch.tensor([0, 2100, 64])[:, None]) &
+                (torch.arange(Sk)[None, :] < torch.tensor([500, 2600, 65])[:, None]))[:, None, None, :]
+    lowest = torch.zeros(keep.shape).masked_fill(~keep, torch.finfo(dtype).min).to(dtype)
+    ninf = torch.zeros(keep.shape).masked_fill(~keep, float("-inf")).to(dtype)
+    q, k, v = rand((B, H, Sq, D), dtype, 1), rand((B, H, Sk, D), dtype, 2), rand((B, H, Sk, D), dtype, 3)
+    on = [t.to(dev()) for t in (q, k, v)]
+    plan = lowering.AttnPlan(scale=D ** -0.5, zero_blind_rows=True)
+    a = lowering.attention(*on, plan, score_bias=lowest.to(dev()))
+    b = lowering.attention(*on, plan, score_bias=ninf.to(dev()))
+    sees = keep.any(-1).expand(B, H, Sq)
+    assert torch.isfinite(a).all() and torch.equal(a[sees.to(dev())], b[sees.to(dev())])
+    want = O.attention_reference(q, k, v, score_bias=ninf.float())
+    assert (a.float().cpu()[sees] - want[sees]).abs().max().item() <= TOL[dtype]
