@@ -15,6 +15,7 @@ timed region.  One JSON line on stdout.
 from __future__ import annotations
 
 import argparse
+import dataclasses
 import json
 import os
 import statistics
@@ -140,8 +141,8 @@ def main() -> int:
     ap.add_argument("--torch-sdpa", action="store_true",
                     help="also time torch.nn.functional.scaled_dot_product_attention on the same GPU and inputs "
                          "(config 2 as is; the decode config with its pages gathered into contiguous K/V beforehand)")
-    ap.add_argument("--workload", default="c2", help="prefill workload: c2 | c2_softcap | c3")
-    ap.add_argument("--decode-workload", default="c5", help="decode workload: c5 | c4")
+    ap.add_argument("--workload", default="c2", help="prefill workload: c2 | c2_softcap | c3 | c2_mask (the causal mask given as a tensor)")
+    ap.add_argument("--decode-workload", default="c5", help="decode workload: c5 | c4 | c5_padded | cache4096 (mask tensors: left padding / partly filled cache)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus 1); "
@@ -184,8 +185,7 @@ def main() -> int:
         nrot = max(2, int(1.5e9 // base.kv_bytes()) + 1)
         ws = [base.to(dev)]
         for _ in range(nrot - 1):
-            ws.append(workloads.Workload(base.name, ws[0].q, ws[0].k.clone(), ws[0].v.clone(), base.mask,
-                                         base.window, base.softcap, ws[0].k_table, ws[0].v_table))
+            ws.append(dataclasses.replace(ws[0], k=ws[0].k.clone(), v=ws[0].v.clone()))
         o = workloads.run(ws[0])
         torch.cuda.synchronize()
         t, wall = time_gpu(lambda i: workloads.run(ws[i % nrot], out=o), args.steps, args.warmup)
