@@ -1055,3 +1055,25 @@ def test_masks_filled_with_the_most_negative_finite_value(dtype, shape):
     assert torch.isfinite(a).all() and torch.equal(a[sees.to(dev())], b[sees.to(dev())])
     want = O.attention_reference(q, k, v, score_bias=ninf.float())
     assert (a.float().cpu()[sees] - want[sees]).abs().max().item() <= TOL[dtype]
+
+
+@pytest.mark.parametrize("name,B,S", [("c2_mask", 2, 512), ("c5_padded", 4, 1024), ("cache4096", 4, 1024)])
+def test_mask_tensor_workloads_of_the_bench(name, B, S):
+    """The bench's workloads whose mask is a tensor of 0 / -inf (causal mask as [1,1,S,S], left
+    padding, partly filled cache), at sizes the oracle finishes in seconds: same result as the
+    oracle given the same tensor, and as the kernel's own flag path where one exists."""
+    w = workloads.make(name, seed=7, B=B, S=S)
+    got = workloads.run(w.to(dev())).float().cpu()
+    want = O.attention_reference(w.q, w.k, w.v, mask=w.mask, k_table=w.k_table, v_table=w.v_table,
+                                 score_bias=w.score_bias)
+    assert (got - want).abs().max().item() <= TOL[w.q.dtype]
+    if name == "c2_mask":
+        flag = workloads.make("c2", seed=7, B=B, S=S)
+        assert torch.equal(flag.q, w.q) and w.flops() == flag.flops()
+        by_flag = workloads.run(flag.to(dev())).float().cpu()
+        assert (got - by_flag).abs().max().item() <= TOL[w.q.dtype]
+    else:
+        # only the keys a sequence can see count as traffic
+        seen = int(torch.isfinite(w.score_bias.float()).sum())
+        assert w.visible_keys == seen
+        assert w.kv_bytes() == 2 * 2 * w.kv_heads() * seen * w.q.shape[-1]

@@ -1,4 +1,6 @@
 """Block-skip set: closed-form tile ranges == brute force over the dense mask, bit-exact."""
+import dataclasses
+
 import pytest
 import torch
 
@@ -48,3 +50,21 @@ def test_tuning_key_buckets_sizes():
     c = lowering._tune_key(mk(2, 4, 1025), mk(2, 4, 1025), plan, None, 0)
     assert a == b != c
     assert lowering._tune_key(mk(2, 8, 1000), mk(2, 4, 1000), plan, None, 0) != a       # GQA group differs
+
+
+def test_mask_tensor_workloads_are_consistent():
+    """Host side of the bench's mask-tensor workloads: the bias is 0 / -inf, every sequence keeps
+    a visible key, and the byte count covers exactly the visible keys."""
+    from loopfuse_amd import workloads
+    w = workloads.make("c2_mask", seed=1, B=1, S=128)
+    i = torch.arange(128)
+    assert torch.equal(torch.isfinite(w.score_bias.float())[0, 0], i[None, :] <= i[:, None])
+    assert w.mask is None and w.flops() == workloads.make("c2", seed=1, B=1, S=128).flops()
+    for name in ("c5_padded", "cache4096"):
+        w = workloads.make(name, seed=1, B=3, S=256)
+        live = torch.isfinite(w.score_bias.float())
+        assert w.score_bias.shape == (3, 1, 1, 256) and set(w.score_bias.float().unique().tolist()) <= {0.0, float("-inf")}
+        assert live.any(dim=-1).all()
+        assert w.visible_keys == int(live.sum())
+        assert w.kv_bytes() == 2 * w.k.element_size() * w.kv_heads() * w.visible_keys * w.q.shape[-1]
+        assert w.kv_bytes() < dataclasses.replace(w, visible_keys=None).kv_bytes()
