@@ -11,6 +11,14 @@ memory-bound half of the metric, config 5 (paged GQA decode, B64 K_len 2048, pag
 16), reported under "decode" in GB/s with the reference's byte convention
 (K and V only, tests/benchmark.py:452).  Inputs are resident in HBM before the
 timed region.  One JSON line on stdout.
+
+Order of the legs.  The GPU's power management makes the launches that follow an idle
+period unrepresentative (the first few run at boost clocks, the next few dozen slower than
+the steady state), so each kernel is first brought to its steady state the way the
+reference's harness does it (``triton.testing.do_bench``, reference tests/benchmark.py:19-22:
+about 25 ms of untimed launches, then about 100 ms of timed ones) -- that measurement is
+reported as ``settled`` -- and the ``--warmup W`` untimed + ``--steps K`` timed launches that
+``value`` is computed from follow immediately.
 """
 from __future__ import annotations
 
@@ -50,6 +58,106 @@ def time_gpu(fn, steps: int, warmup: int):
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     return start.elapsed_time(stop) * 1e-3 / steps, wall / steps
+
+
+def time_settled(fn, warm_ms: float = 25.0, timed_ms: float = 100.0) -> dict:
+    """Time-based conditioning like the reference's ``do_bench`` (tests/benchmark.py:19-22):
+    an estimate from 5 launches sizes ~``warm_ms`` of untimed and ~``timed_ms`` of timed launches."""
+    import torch
+
+    fn(0)
+    torch.cuda.synchronize()
+    est, _ = time_gpu(fn, 5, 0)
+    n_warm = max(1, int(warm_ms * 1e-3 / est))
+    n_rep = max(1, int(timed_ms * 1e-3 / est))
+    t, _ = time_gpu(fn, n_rep, n_warm)
+    return {"us_per_launch": t * 1e6, "warmup_launches": n_warm + 6, "timed_launches": n_rep}
+
+
+def mfma_ceiling(dev) -> dict:
+    """What a loop of nothing but MFMAs sustains on this GPU for zeros and for N(0,1) bf16
+    operands (csrc/kernels/lf_mfma_probe.hip): the chip lowers its clock with the switching
+    activity of the operands, so the second figure, not the published peak, bounds any
+    kernel on the benchmark's inputs."""
+    import ctypes
+
+    import torch
+
+    from loopfuse_amd import lowering, runtime
+
+    class Probe(ctypes.Structure):
+        _fields_ = [("out", ctypes.c_void_p), ("data", ctypes.c_void_p), ("clk", ctypes.c_void_p), ("iters", ctypes.c_int)]
+
+    nwg, iters = 512, 3000
+    out = torch.zeros(nwg * 256, dtype=torch.float32, device=dev)
+    clk = torch.zeros(2 * nwg, dtype=torch.int64, device=dev)
+    res = {}
+    for kind, shape in ((0, "32x32x16"), (1, "16x16x32")):
+        code, _, _ = runtime.compile_source(runtime.read_kernel_source("lf_mfma_probe.hip"), f"lf_mfma_probe_k{kind}",
+                                            list(lowering.COMMON_OPTS) + [f"-DLF_PROBE_KIND={kind}"])
+        kern = runtime.Module(code).kernel("lf_mfma_probe")
+        for name, data in (("zeros", torch.zeros(65536 * 8, dtype=torch.bfloat16, device=dev)),
+                           ("normal", torch.randn(65536 * 8, device=dev).to(torch.bfloat16))):
+            prm = Probe(out.data_ptr(), data.data_ptr(), clk.data_ptr(), iters)
+            t, _ = time_gpu(lambda i: kern.launch((nwg, 1, 1), (256, 1, 1), prm), 6, 3)
+            c = clk.cpu().view(-1, 2).double()
+            res[f"{shape}_{name}"] = {"tflops": iters * 32 * 32768.0 * 4 * nwg / t / 1e12,
+                                      "shader_mhz": float((c[:, 0] / c[:, 1]).median() * 100)}
+    return res
+
+
+def via_backend(dev, steps: int, warmup: int) -> dict:
+    """The two headline workloads through the drop-in path: the reference's own graph
+    spellings (tests/benchmark.py:78-84 causal prefill, 400-406 paged GQA decode with the
+    pool's pages folded into the sequence) under ``torch.compile(backend=loopfuse_backend,
+    dynamic=True)``; device and host time per call."""
+    import torch
+
+    from loopfuse_amd import loopfuse_backend, workloads
+    from loopfuse_amd.torch_backend import interface
+
+    def prefill(q, k, v):
+        qk = q @ k.transpose(-2, -1) * (q.shape[-1] ** -0.5)
+        return torch.softmax(torch.ops.loopfuse.causal_mask(qk), dim=-1) @ v
+
+    def decode(Q, Kc, kt, Vc, vt):
+        B, pages = kt.shape
+        P, H, D = Kc.shape[1:]
+        K = torch.ops.loopfuse.paged_load(Kc, kt).reshape(B, pages * P, H, D).transpose(-3, -2)
+        V = torch.ops.loopfuse.paged_load(Vc, vt).reshape(B, pages * P, H, D).transpose(-3, -2)
+        QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+        return torch.softmax(QK, dim=-1) @ V
+
+    res = {}
+    with torch.inference_mode():
+        w = workloads.make("c2", seed=0).to(dev)
+        fn = torch.compile(prefill, backend=loopfuse_backend, dynamic=True)
+        before = interface.stats["fused"]
+        fn(w.q, w.k, w.v)
+        torch.cuda.synchronize()
+        st = time_settled(lambda i: fn(w.q, w.k, w.v))
+        t, wall = time_gpu(lambda i: fn(w.q, w.k, w.v), steps, warmup)
+        res["prefill_c2"] = {"us_per_call": t * 1e6, "host_us_per_call": wall * 1e6, "settled_us_per_call": st["us_per_launch"],
+                             "tflops": w.flops() / t / 1e12, "fused_calls": interface.stats["fused"] - before}
+        del w
+        base = workloads.make("c5", seed=0)
+        nrot = max(2, int(1.5e9 // base.kv_bytes()) + 1)
+        ws = [base.to(dev)]
+        for _ in range(nrot - 1):
+            ws.append(dataclasses.replace(ws[0], k=ws[0].k.clone(), v=ws[0].v.clone()))
+        B, Hq, _, D = base.q.shape
+        Hkv = base.k.shape[2]
+        qv = [x.q.view(B, Hkv, Hq // Hkv, D) for x in ws]      # the reference's [B, Hkv, group, D] view of Q
+        fn = torch.compile(decode, backend=loopfuse_backend, dynamic=True)
+        before = interface.stats["fused"]
+        call = lambda i: fn(qv[i % nrot], ws[i % nrot].k, ws[i % nrot].k_table, ws[i % nrot].v, ws[i % nrot].v_table)
+        call(0)
+        torch.cuda.synchronize()
+        st = time_settled(call)
+        t, wall = time_gpu(call, steps, warmup)
+        res["decode_c5"] = {"us_per_call": t * 1e6, "host_us_per_call": wall * 1e6, "settled_us_per_call": st["us_per_launch"],
+                            "gbs": base.kv_bytes() / t / 1e9, "fused_calls": interface.stats["fused"] - before}
+    return res
 
 
 def cpu_baseline(seconds: float = 12.0) -> dict:
@@ -131,8 +239,8 @@ def torch_sdpa(args, dev) -> dict:
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="time only one of the two kernels (profiling aid)")
@@ -141,6 +249,10 @@ def main() -> int:
     ap.add_argument("--torch-sdpa", action="store_true",
                     help="also time torch.nn.functional.scaled_dot_product_attention on the same GPU and inputs "
                          "(config 2 as is; the decode config with its pages gathered into contiguous K/V beforehand)")
+    ap.add_argument("--no-via-backend", action="store_true",
+                    help="skip the legs that time the two headline workloads through torch.compile(backend=loopfuse_backend)")
+    ap.add_argument("--mfma-ceiling", action="store_true",
+                    help="also run the MFMA-only probe on zeros and on N(0,1) operands (the data-dependent clock ceiling)")
     ap.add_argument("--workload", default="c2", help="prefill workload: c2 | c2_softcap | c3 | c2_mask (the causal mask given as a tensor)")
     ap.add_argument("--decode-workload", default="c5", help="decode workload: c5 | c4 | c5_padded | cache4096 (mask tensors: left padding / partly filled cache)")
     args = ap.parse_args()
@@ -173,9 +285,11 @@ def main() -> int:
         w = workloads.make(args.workload, seed=0).to(dev)
         o = workloads.run(w)     # first call compiles / loads the code object
         torch.cuda.synchronize()
+        settled = time_settled(lambda i: workloads.run(w, out=o))
         t, wall = time_gpu(lambda i: workloads.run(w, out=o), args.steps, args.warmup)
-        pre = {"workload": args.workload, "sec": t, "wall_sec": wall, "flops": w.flops(),
+        pre = {"workload": args.workload, "sec": t, "wall_sec": wall, "flops": w.flops(), "settled": settled,
                "kernels": lowering.attention.last_launch["kernels"]}
+        del w, o
 
     dec = None
     if args.only in (None, "decode"):
@@ -188,14 +302,15 @@ def main() -> int:
             ws.append(dataclasses.replace(ws[0], k=ws[0].k.clone(), v=ws[0].v.clone()))
         o = workloads.run(ws[0])
         torch.cuda.synchronize()
+        dsettled = time_settled(lambda i: workloads.run(ws[i % nrot], out=o))
         t, wall = time_gpu(lambda i: workloads.run(ws[i % nrot], out=o), args.steps, args.warmup)
         dec = {"workload": args.decode_workload, "sec": t, "wall_sec": wall, "bytes": base.kv_bytes(), "rotation": nrot,
-               "kernels": lowering.attention.last_launch["kernels"]}
-        # the streaming kernel alone (its partial results left unmerged): the launch the HBM
-        # roofline is about; `value` keeps the whole step with the combine launch
+               "settled": dsettled, "kernels": lowering.attention.last_launch["kernels"]}
+        # extra field: the streaming kernel alone (its partial results left unmerged, O not written)
         tk, _ = time_gpu(lambda i: workloads.run(ws[i % nrot], out=o, merge_splits=False), args.steps, 20)
         dec["kernel_sec"] = tk
         dec["stream_kernels"] = lowering.attention.last_launch["kernels"]
+        del ws, o
 
     primary = pre if pre is not None else dec
     if pre is not None:
@@ -207,15 +322,24 @@ def main() -> int:
         out["roofline"] = {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                            "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": TRAFFIC_BYTES.get(args.workload),
                            "kernel": "+".join(pre["kernels"]), "us_per_launch": pre["sec"] * 1e6}
+        st = pre["settled"]
+        out["settled"] = {"value": pre["flops"] / st["us_per_launch"] / 1e6, "unit": "TFLOP/s",
+                          "frac": pre["flops"] / st["us_per_launch"] / 1e6 / MFMA_BF16_PEAK_TFLOPS, **st,
+                          "protocol": "about 25 ms of untimed launches, then about 100 ms of timed ones (the reference's do_bench)"}
     if dec is not None:
         gbs = dec["bytes"] / dec["sec"] / 1e9
         kgbs = dec["bytes"] / dec["kernel_sec"] / 1e9
         d = {"workload": dec["workload"], "value": gbs, "unit": "GB/s", "us_per_launch": dec["sec"] * 1e6,
              "frac_of_hbm_peak": gbs / HBM_PEAK_GBS, "kernels": "+".join(dec["kernels"]),
              "host_us_per_launch": dec["wall_sec"] * 1e6, "kv_pool_rotation": dec["rotation"],
-             "roofline": {"bound": "hbm", "achieved": kgbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                          "frac": kgbs / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES.get(args.decode_workload),
-                          "kernel": "+".join(dec["stream_kernels"]), "us_per_launch": dec["kernel_sec"] * 1e6}}
+             # the roofline is read on the whole step (every launch that it takes to write O)
+             "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": gbs / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES.get(args.decode_workload),
+                          "kernel": "+".join(dec["kernels"]), "us_per_launch": dec["sec"] * 1e6},
+             "settled": {"value": dec["bytes"] / dec["settled"]["us_per_launch"] / 1e3, "unit": "GB/s",
+                         "frac": dec["bytes"] / dec["settled"]["us_per_launch"] / 1e3 / HBM_PEAK_GBS, **dec["settled"]},
+             "stream_kernel_alone": {"kernel": "+".join(dec["stream_kernels"]), "us_per_launch": dec["kernel_sec"] * 1e6,
+                                     "gbs": kgbs, "note": "partials left unmerged, O not written"}}
         if pre is None:
             out.update({"metric": "prefill TFLOP/s + decode HBM GB/s on 1 MI355X (% of roofline)",
                         "value": gbs, "unit": "GB/s", "roofline": d["roofline"]})
@@ -229,6 +353,10 @@ def main() -> int:
                    "decode_workload": "config 5: paged GQA decode bf16 B64 Hq32/Hkv8 K_len2048 D128 page16"
                    if args.decode_workload == "c5" else args.decode_workload},
     })
+    if not args.no_via_backend and args.only is None and args.workload == "c2" and args.decode_workload == "c5":
+        out["via_backend"] = via_backend(dev, args.steps, args.warmup)
+    if args.mfma_ceiling:
+        out["mfma_ceiling"] = mfma_ceiling(dev)
     if args.torch_sdpa:
         out["torch_sdpa"] = torch_sdpa(args, dev)
     if not args.no_cpu_baseline:

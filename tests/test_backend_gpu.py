@@ -611,30 +611,48 @@ def test_recompile_free_new_sequence_length():
     assert outs[1] == 0
 
 
+def _softmax64(x):
+    e = (x - x.amax(dim=-1, keepdim=True)).exp()
+    return e / e.sum(dim=-1, keepdim=True)
+
+
 @pytest.mark.parametrize("which", ["add", "add_2dim", "matmul_add", "matmul_add_3dim", "modified_attn", "softmax_matmul",
                                    "paged_add", "simplified_attn"])
 def test_unlowered_graphs_still_correct(which):
-    """Reference tests/test_accuracy.py:29-82, 172-211: not attention-shaped for this
-    backend; they run unfused and must still be numerically right."""
+    """Reference tests/test_accuracy.py:29-82, 172-211, 233-250, 314-333: graphs that are not
+    attention-shaped for this backend (no kernel is lowered for them: they run as captured),
+    plus the modified-attention graph.  Each result is checked against an independent float64
+    computation on the CPU, spelled differently from the compiled function (einsum / explicit
+    exponentials / index loops), not against the same graph run eagerly."""
+    f64 = lambda ts: [t.double() if t.is_floating_point() else t for t in ts]
     if which == "add":
         fn = lambda a, b: a + b
         ins = (rand((4, 1024, 128), torch.float32, 1), rand((4, 1024, 128), torch.float32, 2))
+        ref = lambda a, b: torch.stack([a, b]).sum(dim=0)
     elif which == "add_2dim":          # reference tests/test_accuracy.py:40-50
         fn = lambda a, b: a + b
         ins = (rand((512, 1024), torch.float32, 1), rand((512, 1024), torch.float32, 2))
+        ref = lambda a, b: torch.stack([a, b]).sum(dim=0)
     elif which == "matmul_add_3dim":   # reference tests/test_accuracy.py:66-82
         fn = lambda a, b, c: a @ b + c
         ins = (rand((4, 256, 64), torch.float32, 1) * 0.1, rand((4, 64, 128), torch.float32, 2) * 0.1,
                rand((4, 256, 128), torch.float32, 3))
+        ref = lambda a, b, c: torch.einsum("bik,bkj->bij", a, b) + c
     elif which == "simplified_attn":   # reference tests/test_accuracy.py:314-332: no exponential, not a softmax
         def fn(Q, K, V):
             QK = Q @ K.transpose(-2, -1)
             m = torch.max(QK, dim=-1, keepdim=True)[0] + torch.sum(QK, dim=-1, keepdim=True)
             return (QK / (m + 1e-3)) @ V
         ins = tuple(rand((2, 4, 256, 64), torch.float32, s) * 0.2 for s in (1, 2, 3))
+
+        def ref(Q, K, V):
+            s = torch.einsum("bhid,bhjd->bhij", Q, K)
+            den = s.amax(dim=-1) + torch.einsum("bhij->bhi", s) + 1e-3
+            return torch.einsum("bhij,bhjd->bhid", s, V) / den[..., None]
     elif which == "matmul_add":
         fn = lambda a, b, c: a @ b + c
         ins = (rand((256, 128), torch.float32, 1), rand((128, 128), torch.float32, 2), rand((256, 128), torch.float32, 3))
+        ref = lambda a, b, c: torch.einsum("ik,kj->ij", a, b) + c
     elif which == "modified_attn":
         def fn(Q, K, V, qb, sb, ob):
             QK = (Q + qb) @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
@@ -642,16 +660,26 @@ def test_unlowered_graphs_still_correct(which):
             return torch.softmax(torch.ops.loopfuse.causal_mask(QK), dim=-1) @ V + ob
         ins = tuple(rand((2, 2, 128, 64), torch.float32, s) for s in (1, 2, 3, 4)) + \
             (rand((2, 2, 128, 128), torch.float32, 5), rand((2, 2, 128, 64), torch.float32, 6))
+
+        def ref(Q, K, V, qb, sb, ob):
+            s = torch.einsum("bhid,bhjd->bhij", Q + qb, K) * (3.5 / 8.0) + sb
+            i = torch.arange(s.shape[-2])[:, None]
+            j = torch.arange(s.shape[-1])[None, :]
+            s = torch.where(j <= i, s, torch.full_like(s, float("-inf")))
+            return torch.einsum("bhij,bhjd->bhid", _softmax64(s), V) + ob
     elif which == "paged_add":       # reference tests/test_accuracy.py:233-250
         fn = lambda buf, tab: torch.ops.loopfuse.paged_load(buf, tab) + 1
         ins = (rand((64, 4, 32), torch.float32, 1),
                torch.randint(0, 64, (3, 20), generator=torch.Generator().manual_seed(2), dtype=torch.int32))
+        ref = lambda buf, tab: torch.stack([torch.stack([buf[int(tab[b, s])] for s in range(tab.shape[1])])
+                                            for b in range(tab.shape[0])]) + 1
     else:
         fn = lambda x, y: torch.softmax(x, dim=-1) @ y
         ins = (rand((2, 4, 128, 64), torch.float32, 1), rand((2, 4, 64, 128), torch.float32, 2))
+        ref = lambda x, y: torch.einsum("bhij,bhjd->bhid", _softmax64(x), y)
     torch._dynamo.reset()
     dev_ins = [t.to(DEV) for t in ins]
-    want = fn(*dev_ins)
+    want = ref(*f64(ins))
     got = torch.compile(fn, backend=loopfuse_backend, dynamic=True)(*dev_ins)
     tol = 1e-2 if which == "simplified_attn" else 1e-4      # the reference checks that case at rtol 1e-2 too
-    torch.testing.assert_close(got, want, rtol=tol, atol=tol)
+    torch.testing.assert_close(got.double().cpu(), want, rtol=tol, atol=tol)

@@ -693,3 +693,17 @@ def test_decoder_layer_with_cache_and_repeated_kv_heads(S, P, use_mask, dynamic,
     assert match.inputs[match.k.index].name.startswith("cat") and (match.bias is not None) == use_mask
     for a, b in zip(got, want):
         torch.testing.assert_close(a, b, rtol=2e-4, atol=2e-4)
+
+
+def test_reference_import_path_is_a_drop_in():
+    # reference loopfuse/__init__.py:1-3 and its tests import `from loopfuse import loopfuse_backend`
+    import loopfuse
+    from loopfuse import loopfuse_backend as ref_path_backend
+    from loopfuse_amd import loopfuse_backend as own_backend
+
+    assert ref_path_backend is own_backend and loopfuse.__all__ == ["loopfuse_backend"]
+    for op in ("causal_mask", "sliding_mask", "scan_max", "paged_load"):
+        assert hasattr(torch.ops.loopfuse, op)
+    x = torch.randn(2, 3, 5, 5)
+    fn = torch.compile(lambda a: torch.ops.loopfuse.causal_mask(a) + 1, backend=ref_path_backend, dynamic=True)
+    assert torch.equal(fn(x), torch.ops.loopfuse.causal_mask(x) + 1)
