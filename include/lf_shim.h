@@ -14,7 +14,9 @@
  *     hip/hiprtc error code (or a negative LF_E* code); a human-readable
  *     message for the calling thread is available from lf_last_error().
  *   - the shim never allocates device memory; every device buffer (inputs,
- *     outputs, split-K scratch) belongs to the caller.
+ *     outputs, split-K scratch) belongs to the caller.  lf_launch_decode_static
+ *     is the one exception to the last item: its split-K scratch is a static
+ *     device array inside the library.
  *   - all entry points are re-entrant; the only shared state is an
  *     internally locked table of loaded modules.
  */
@@ -30,6 +32,11 @@ extern "C" {
 #define LF_EINVAL (-1)   /* bad argument */
 #define LF_EIO    (-2)   /* cache file could not be read/written */
 #define LF_ENOSYM (-3)   /* kernel symbol not found in module */
+#define LF_ENOSPC (-4)   /* request larger than the library's static scratch */
+
+/* Size of the static device array behind lf_launch_decode_static (one copy per GPU the
+ * library runs on, held until the process ends). */
+#define LF_STATIC_SCRATCH_BYTES (8u << 20)
 
 /* ABI version of this header; bumped on any signature change. */
 int lf_abi_version(void);
@@ -82,6 +89,31 @@ int lf_module_unload(void* mod);
 int lf_launch(void* fn, unsigned gx, unsigned gy, unsigned gz,
               unsigned bx, unsigned by, unsigned bz,
               unsigned lds_bytes, void* stream, void** args);
+
+/*
+ * No counterpart in the reference.  For callers that cannot allocate device memory
+ * (a stream under HIP graph capture, a tight serving loop, a harness that forbids
+ * hipMalloc): one split decode step -- `fn_decode` (lf_attn_decode) on a (gx, gy)
+ * grid of bx threads, then `fn_combine` (lf_attn_decode_combine) on combine_gx
+ * blocks of combine_bx threads, both from one code object and both taking
+ * `params` (an LfAttnParamsHost, include/lf_attn_params.h) by value -- with the
+ * split-K partials in a static device array of LF_STATIC_SCRATCH_BYTES instead of a
+ * caller-owned buffer: the part_acc / part_ml fields of `params` are ignored and
+ * replaced.  part_acc_bytes / part_ml_bytes say how much the step needs
+ * (units * nsplit * rows * D * 4 and units * nsplit * rows * 2 * 4); more than the
+ * array holds is refused with LF_ENOSPC.  Allocates nothing and frees nothing.
+ * Every call on a GPU shares that GPU's array: calls on one stream are ordered,
+ * calls that overlap on one GPU (different streams) race.  The array keeps the last
+ * call's partials; nothing in it has to start at zero.
+ */
+int lf_launch_decode_static(void* fn_decode, void* fn_combine,
+                            const void* params, size_t params_bytes,
+                            size_t part_acc_bytes, size_t part_ml_bytes,
+                            unsigned gx, unsigned gy, unsigned bx,
+                            unsigned combine_gx, unsigned combine_bx, void* stream);
+
+/* LF_STATIC_SCRATCH_BYTES as the built library has it. */
+size_t lf_static_scratch_bytes(void);
 
 /* Architecture name, compute-unit count and LDS bytes per workgroup of a
  * device.  Fails (non-zero) when there is no usable GPU. */

@@ -6,6 +6,7 @@
 // that already holds PyTorch-ROCm, the dynamic linker resolves both by soname to
 // the copies torch loaded, so streams and device pointers are shared with torch.
 #include "lf_shim.h"
+#include "lf_shim_internal.h"
 
 #include <hip/hip_runtime_api.h>
 #include <hip/hiprtc.h>
@@ -90,9 +91,11 @@ int resolve_arch(const char* arch, std::string* out) {
 
 }  // namespace
 
+int lf_internal_fail(int code, const std::string& msg) { return fail(code, msg); }
+
 extern "C" {
 
-int lf_abi_version(void) { return 1; }
+int lf_abi_version(void) { return 2; }
 
 const char* lf_last_error(void) { return g_err.c_str(); }
 

@@ -425,7 +425,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
               force_family: str | None = None, num_splits: int | None = None, v_tr: bool = True,
               score_bias: Optional[torch.Tensor] = None, out_bias: Optional[torch.Tensor] = None,
               choice: Optional[dict] = None, merge_splits: bool = True,
-              q2: Optional[torch.Tensor] = None, k2: Optional[torch.Tensor] = None):
+              q2: Optional[torch.Tensor] = None, k2: Optional[torch.Tensor] = None,
+              static_scratch: bool = False):
     """Run fused attention on the GPU.
 
     q : [B, Hq, Sq, D];  k, v : [B, Hkv, Sk, D], or page pools [N, P, Hkv, D]
@@ -440,6 +441,10 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     ``lf_attn_prefill`` with dense K2.
     ``merge_splits=False`` leaves the partial results of a split decode unmerged (the
     output is then not written): for timing the streaming kernel alone.
+    ``static_scratch=True`` (split decode only, ``out`` given): the step goes through the C ABI's
+    ``lf_launch_decode_static``, whose split-K partials live in a static device array of the
+    library -- no device memory is allocated anywhere in the call; a step whose partials exceed
+    that array raises ``runtime.ShimError``.
     ``choice`` overrides the launch heuristics (what ``tuned_attention`` searches over):
     ``{"prefill": "swp" | "w32"}``, ``{"head_per_wave": bool, "splits": n}``.
     Returns O [B, Hq, Sq, D] and, with ``record_visits``, the uint8 record of the KV tiles
@@ -718,6 +723,17 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
                       page_size, table_i64, rows=DECODE_QROWS, waves=waves, headwave=headwave, page_size_v=page_size_v,
                       bias=bias_bits, safe=plan.zero_blind_rows and bool(bias_bits),
                       extra=tuple(os.environ.get("LOOPFUSE_KOPTS", "").split()))
+    rows_per_block = 1024 // D       # combine kernel: 256 threads, 4 consecutive d each
+    combine_grid = (B * Hkv * rows + rows_per_block - 1) // rows_per_block
+    if static_scratch:
+        if nsplit <= 1 or not merge_splits:
+            raise UnsupportedPlan("static_scratch serves split decode steps (this call does not split the keys)")
+        nrow = B * Hkv * rows * nsplit
+        runtime.launch_decode_static(get_kernel(spec, "lf_attn_decode"), get_kernel(spec, "lf_attn_decode_combine"), P,
+                                     4 * nrow * D, 4 * nrow * 2, (units, nsplit), 64 * spec.waves, combine_grid, 256)
+        attention.last_launch = {"kernels": ["lf_attn_decode", "lf_attn_decode_combine"], "grid": (units, nsplit),
+                                 "block": 64 * spec.waves, "head_per_wave": headwave, "static_scratch": True}
+        return out
     if nsplit > 1:
         nrow = B * Hkv * rows * nsplit
         scratch = _get_scratch(q.device, nrow * (D + 2))
@@ -725,9 +741,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         P.part_ml = scratch.data_ptr() + 4 * nrow * D
     get_kernel(spec, "lf_attn_decode").launch((units, nsplit, 1), (64 * spec.waves, 1, 1), P)
     if nsplit > 1 and merge_splits:
-        rows_per_block = 1024 // D       # 256 threads, 4 consecutive d each
-        get_kernel(spec, "lf_attn_decode_combine").launch(
-            ((B * Hkv * rows + rows_per_block - 1) // rows_per_block, 1, 1), (256, 1, 1), P)
+        get_kernel(spec, "lf_attn_decode_combine").launch((combine_grid, 1, 1), (256, 1, 1), P)
     attention.last_launch = {"kernels": ["lf_attn_decode"] + (["lf_attn_decode_combine"] if nsplit > 1 and merge_splits else []),
                              "grid": (units, nsplit), "block": 64 * spec.waves, "head_per_wave": headwave}
     return out

@@ -35,6 +35,8 @@ ABI_SYMBOLS = (
     "lf_get_function",
     "lf_module_unload",
     "lf_launch",
+    "lf_launch_decode_static",
+    "lf_static_scratch_bytes",
     "lf_device_info",
     "lf_device_count",
 )
@@ -92,6 +94,10 @@ def lib() -> ctypes.CDLL:
         L.lf_module_unload.argtypes = [ctypes.c_void_p]
         L.lf_launch.restype = ctypes.c_int
         L.lf_launch.argtypes = [ctypes.c_void_p] + [ctypes.c_uint] * 7 + [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p)]
+        L.lf_launch_decode_static.restype = ctypes.c_int
+        L.lf_launch_decode_static.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+                                              ctypes.c_size_t, ctypes.c_size_t] + [ctypes.c_uint] * 5 + [ctypes.c_void_p]
+        L.lf_static_scratch_bytes.restype = ctypes.c_size_t
         L.lf_device_info.restype = ctypes.c_int
         L.lf_device_info.argtypes = [
             ctypes.c_int, ctypes.c_char_p, ctypes.c_size_t,
@@ -160,6 +166,24 @@ class Kernel:
                           lds_bytes, ctypes.c_void_p(stream), args)
         if rc:
             _check(f"lf_launch[{self.symbol}]", rc)
+
+
+def launch_decode_static(decode: Kernel, combine: Kernel, params: ctypes.Structure, part_acc_bytes: int,
+                         part_ml_bytes: int, grid: tuple[int, int], block: int, combine_grid: int,
+                         combine_block: int, stream: int | None = None) -> None:
+    """One split decode step through ``lf_launch_decode_static``: both kernels, with the
+    split-K partials in the library's static device array (nothing is allocated)."""
+    if stream is None:
+        stream = current_stream_handle()
+    rc = lib().lf_launch_decode_static(decode.handle, combine.handle, ctypes.addressof(params), ctypes.sizeof(params),
+                                       part_acc_bytes, part_ml_bytes, grid[0], grid[1], block,
+                                       combine_grid, combine_block, ctypes.c_void_p(stream))
+    if rc:
+        _check("lf_launch_decode_static", rc)
+
+
+def static_scratch_bytes() -> int:
+    return int(lib().lf_static_scratch_bytes())
 
 
 class Module:

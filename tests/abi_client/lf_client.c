@@ -234,7 +234,7 @@ static int run_decode(const char* dir) {
 
 int main(int argc, char** argv) {
   if (argc < 2) { fprintf(stderr, "usage: %s <kernel source dir> [prefill|decode]\n", argv[0]); return 64; }
-  if (lf_abi_version() != 1) { fprintf(stderr, "unexpected ABI version %d\n", lf_abi_version()); return 5; }
+  if (lf_abi_version() != 2) { fprintf(stderr, "unexpected ABI version %d\n", lf_abi_version()); return 5; }
   char arch[64];
   int cus = 0, lds = 0;
   CHECK_LF(lf_device_info(0, arch, sizeof arch, &cus, &lds));

@@ -19,11 +19,11 @@ def header_symbols():
 
 def test_exports_every_declared_symbol(shim_built):
     syms = header_symbols()
-    assert len(syms) >= 11
+    assert len(syms) >= 13
     for s in syms:
         assert hasattr(shim_built, s), f"{s} declared in lf_shim.h but not exported"
     assert sorted(runtime.ABI_SYMBOLS) == syms
-    assert shim_built.lf_abi_version() == 1
+    assert shim_built.lf_abi_version() == 2
 
 
 def test_compile_without_gpu_and_cache(shim_built, tmp_path):
