@@ -259,7 +259,7 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 8 / LF_DW) lf_attn_decode(co
       const int tok = t0 + (i < 4 ? i : 12 + i);
 #if LF_BIAS
       // (scaled or capped score + bias) in log2 units
-      x[i] = (tok < tok_end) ? s * cexp + lf_to_float(i < 4 ? sa.bias[i] : sb.bias[i - 4]) * LF_LOG2E : LF_NEG_INF;
+      x[i] = (tok < tok_end) ? s * cexp + lf_bias_value(i < 4 ? sa.bias[i] : sb.bias[i - 4]) * LF_LOG2E : LF_NEG_INF;
 #else
       x[i] = (tok < tok_end) ? s * cexp : LF_NEG_INF;
 #endif

@@ -52,9 +52,6 @@
 #define LF_D2 0     /* depth of a second score product: S = Q K^T + Q2 K2^T (16, 32 or 64; 0 = none) */
 #endif
 
-#ifndef LF_BN
-#define LF_BN 64
-#endif
 #ifndef LF_OCC
 #define LF_OCC 2    /* waves per SIMD the register budget is set for */
 #endif
@@ -63,14 +60,7 @@
 #endif
 #define LF_NT (LF_NW * 64)
 #define LF_BM (32 * LF_NW)
-#define LF_D LF_HEAD_DIM
-#define LF_CPR (LF_D / 8)                    /* 16-byte chunks per K/V row    */
-#define LF_RPS (256 / (LF_D * 2))            /* rows per 256-byte bank span   */
 #define LF_NPASS (LF_BN * LF_CPR / LF_NT)    /* staging passes per tile       */
-#define LF_NKB (LF_BN / 32)                  /* 32-row blocks of S^T per tile */
-#define LF_NKS (LF_D / 16)                   /* k-steps of the QK^T product   */
-#define LF_NDB (LF_D / 32)                   /* 32-row blocks of O^T          */
-#define LF_NKK (LF_BN / 16)                  /* k-steps of the PV product     */
 #define LF_CPR2 (LF_D2 / 8)                  /* 16-byte chunks per K2 row      */
 #define LF_NKS2 (LF_D2 / 16)                 /* k-steps of the Q2 K2^T product */
 #define LF_RPS2 (LF_D2 ? 256 / (LF_D2 * 2) : 1)
@@ -79,24 +69,14 @@
 #define LF_KS LF_D
 #define LF_VS LF_D
 
-// Physical 16-byte chunk of logical chunk `ch` in row `row` of the K tile: rows
-// that a ds_read_b128 touches together (16 consecutive rows, same logical chunk)
-// land in 16 different chunks, i.e. on all 64 banks.
-__device__ __forceinline__ int lf_k_phys(int row, int ch) {
-  return ch ^ ((row / LF_RPS) & (LF_CPR - 1));
-}
 #if LF_D2
-// The K2 tile (rows of LF_D2 elements, several rows per 256-byte bank span): the same
-// permutation with its own row length.
+// The K2 tile (rows of LF_D2 elements, several rows per 256-byte bank span): the K tile's
+// permutation (lf_k_phys) with its own row length.
 __device__ __forceinline__ int lf_k2_phys(int row, int ch) {
   return ch ^ ((row / LF_RPS2) & (LF_CPR2 - 1));
 }
 #endif
-// Same for the V tile, where a transposed read touches 4 consecutive rows x 64
-// contiguous bytes per 32 lanes: permute the 64-byte groups by the row.
-__device__ __forceinline__ int lf_v_phys(int row, int ch) {
-  return ch ^ (4 * ((row / LF_RPS) & (LF_CPR / 4 - 1)));
-}
+
 
 // Mask tensors reach the kernel as score biases of 0 / -inf.  Before the loop over a q
 // tile's KV tiles the workgroup looks for tiles whose bias is -inf for all of its rows and
@@ -263,27 +243,11 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
   // (unpadded, row-major) tile; the XOR swizzle is applied on the global side: the
   // lane that lands on physical chunk `sch` fetches logical chunk sch ^ swizzle(row).
   // No staging registers, no ds_write, and rows past Sk arrive as zeros.
-  lf_u32x4 k_rsq, v_rsq;
-  {
-    const unsigned long long ka = (unsigned long long)k_uni, va = (unsigned long long)v_uni;
-    k_rsq[0] = __builtin_amdgcn_readfirstlane((unsigned)ka);
-    k_rsq[1] = __builtin_amdgcn_readfirstlane((unsigned)(ka >> 32) & 0xffffu);
-    k_rsq[2] = __builtin_amdgcn_readfirstlane(k_bytes);
-    k_rsq[3] = 0x00020000u;
-    v_rsq[0] = __builtin_amdgcn_readfirstlane((unsigned)va);
-    v_rsq[1] = __builtin_amdgcn_readfirstlane((unsigned)(va >> 32) & 0xffffu);
-    v_rsq[2] = __builtin_amdgcn_readfirstlane(v_bytes);
-    v_rsq[3] = 0x00020000u;
-  }
+  const lf_u32x4 k_rsq = lf_make_buffer(k_uni, k_bytes), v_rsq = lf_make_buffer(v_uni, v_bytes);
   const unsigned k_doff = (unsigned)srow * k_rowb + 16u * (unsigned)lf_k_phys(srow, sch);
   const unsigned v_doff = (unsigned)srow * v_rowb + 16u * (unsigned)lf_v_phys(srow, sch);
   constexpr int kRowsPerWave = 64 / LF_CPR;
-  auto dma = [&](const lf_u32x4& rs, unsigned voff, const lf_elem* lds_row0) {
-    const unsigned m0v = __builtin_amdgcn_readfirstlane(
-        (unsigned)(size_t)(__attribute__((address_space(3))) const void*)lds_row0);
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-                 :: "s"(m0v), "v"(voff), "s"(rs) : "memory");
-  };
+  auto dma = [&](const lf_u32x4& rs, unsigned voff, const lf_elem* lds_row0) { lf_dma_to_lds(rs, voff, lds_row0); };
 #endif
   auto load_tile = [&](int kt, int buf) {
 #pragma unroll
@@ -515,11 +479,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
         // trip (well over 100 cycles) spans several 32-cycle MFMAs
         constexpr int kNF = (LF_NKS * LF_NKB);
         lf_u32x4 kf[kNF > 0 ? kNF : 1];
-        auto k_frag = [&](int f) {
-          const int ks = f / LF_NKB, kb = f % LF_NKB;
-          const int row = 32 * kb + l32;
-          return *reinterpret_cast<const lf_u32x4*>(&kbuf[row * LF_KS + 8 * lf_k_phys(row, 2 * ks + g)]);
-        };
+        auto k_frag = [&](int f) { return lf_read_k_frag(kbuf, l32, g, f); };
 #pragma unroll
         for (int f = 0; f < LF_KPF && f < kNF; ++f) kf[f] = k_frag(f);
 #pragma unroll
@@ -586,9 +546,9 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
 #if LF_SOFTCAP
-              s[kb][4 * i4 + e] += lf_to_float(bv[e]);
+              s[kb][4 * i4 + e] += lf_bias_value(bv[e]);
 #else
-              s[kb][4 * i4 + e] = s[kb][4 * i4 + e] * p.scale + lf_to_float(bv[e]);
+              s[kb][4 * i4 + e] = s[kb][4 * i4 + e] * p.scale + lf_bias_value(bv[e]);
 #endif
             }
           }
@@ -667,24 +627,9 @@ extern "C" __global__ void __launch_bounds__(LF_NT, LF_OCC) lf_attn_prefill(cons
           const int kk = f / LF_NDB, db = f % LF_NDB;
           lf_elem8 a;
 #if LF_V_TR
-          // 16-lane group (2g + dh) asks for rows r0..r0+3, columns 32db+16dh..+15:
-          // lane j of the group supplies the 8-byte piece (row r0 + j/4, cols +4*(j%4))
-          // and receives column j of the 4 rows.
-          const int j16 = lane & 15;
-          const int dh = (lane >> 4) & 1;
-          const int col = 32 * db + 16 * dh + 4 * (j16 & 3);
-#pragma unroll
-          for (int half = 0; half < 2; ++half) {
-            const int row = 16 * kk + 8 * half + 4 * g + (j16 >> 2);
-            const lf_elem* src = &vbuf[row * LF_VS + 8 * lf_v_phys(row, col / 8) + (col % 8)];
-            lf_s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (__attribute__((address_space(3))) lf_s16x4*)(src));
-            lf_elem4 te = __builtin_bit_cast(lf_elem4, t);
-            a[4 * half + 0] = te[0];
-            a[4 * half + 1] = te[1];
-            a[4 * half + 2] = te[2];
-            a[4 * half + 3] = te[3];
-          }
+          (void)kk;
+          (void)db;
+          a = lf_read_v_frag_tr(vbuf, lane, g, f);
 #else
           const int col = 32 * db + l32;
 #pragma unroll

@@ -34,11 +34,6 @@
 #ifndef LF_SETPRIO
 #define LF_SETPRIO 1     /* raise the wave priority while it issues MFMAs */
 #endif
-#ifndef LF_ABLATE
-#define LF_ABLATE 0      /* profiling aid (wrong results): 1 no exp, 2 no direct loads, 4 no O store, 8 no Q load, 16 no K reads,
-                            32 V fragments by one plain 16-byte read, 64 no V reads */
-#endif
-
 #ifndef LF_NW
 #define LF_NW 4     /* waves per workgroup: 4 (two workgroups per CU) or 8 (one) */
 #endif
@@ -58,26 +53,11 @@
 #define LF_BM (32 * LF_NW)
 #define LF_HEADS_PER_WG 1
 #endif
-#define LF_BN 64
 #define LF_KSLOTS 3
 #define LF_VSLOTS 2
-#define LF_D LF_HEAD_DIM
-#define LF_CPR (LF_D / 8)
-#define LF_RPS (256 / (LF_D * 2))
 #define LF_NPASS (LF_BN * LF_CPR / LF_NT)
-#define LF_NKB (LF_BN / 32)
-#define LF_NKS (LF_D / 16)
-#define LF_NDB (LF_D / 32)
-#define LF_NKK (LF_BN / 16)
 #define LF_NFK (LF_NKS * LF_NKB)      /* MFMAs (= K fragments) of S^T per tile */
 #define LF_NFV (LF_NKK * LF_NDB)      /* MFMAs (= V fragments) of O^T per tile */
-
-__device__ __forceinline__ int lf_k_phys(int row, int ch) {
-  return ch ^ ((row / LF_RPS) & (LF_CPR - 1));
-}
-__device__ __forceinline__ int lf_v_phys(int row, int ch) {
-  return ch ^ (4 * ((row / LF_RPS) & (LF_CPR / 4 - 1)));
-}
 
 // workgroup barrier that waits for this wave's direct-to-LDS loads but leaves LDS
 // reads in flight (the compiler's own barrier would wait for those too)
@@ -150,31 +130,11 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
     return which ? id * (unsigned)(p.v_sb * 2) + (unsigned)hkv * (unsigned)(p.v_sh * 2)
                  : id * (unsigned)(p.k_sb * 2) + (unsigned)hkv * (unsigned)(p.k_sh * 2);
   };
-  lf_u32x4 k_rsq, v_rsq;
-  {
-    const unsigned long long ka = (unsigned long long)k_uni, va = (unsigned long long)v_uni;
-    k_rsq[0] = __builtin_amdgcn_readfirstlane((unsigned)ka);
-    k_rsq[1] = __builtin_amdgcn_readfirstlane((unsigned)(ka >> 32) & 0xffffu);
-    k_rsq[2] = __builtin_amdgcn_readfirstlane(k_bytes);
-    k_rsq[3] = 0x00020000u;
-    v_rsq[0] = __builtin_amdgcn_readfirstlane((unsigned)va);
-    v_rsq[1] = __builtin_amdgcn_readfirstlane((unsigned)(va >> 32) & 0xffffu);
-    v_rsq[2] = __builtin_amdgcn_readfirstlane(v_bytes);
-    v_rsq[3] = 0x00020000u;
-  }
+  const lf_u32x4 k_rsq = lf_make_buffer(k_uni, k_bytes), v_rsq = lf_make_buffer(v_uni, v_bytes);
   // per-lane part of the offset: dense = row inside the pass, paged = row inside the wave's load
   const unsigned k_doff = (unsigned)(kPagedK ? srow % (64 / LF_CPR) : srow) * k_rowb + 16u * (unsigned)lf_k_phys(srow, sch);
   const unsigned v_doff = (unsigned)(kPagedV ? srow % (64 / LF_CPR) : srow) * v_rowb + 16u * (unsigned)lf_v_phys(srow, sch);
-  bool dma_on = true;
-  auto dma = [&](const lf_u32x4& rs, unsigned voff, const lf_elem* lds_row0) {
-    const unsigned m0v = __builtin_amdgcn_readfirstlane(
-        (unsigned)(size_t)(__attribute__((address_space(3))) const void*)lds_row0);
-#if LF_ABLATE & 2
-    if (dma_on)
-#endif
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-                 :: "s"(m0v), "v"(voff), "s"(rs) : "memory");
-  };
+  auto dma = [&](const lf_u32x4& rs, unsigned voff, const lf_elem* lds_row0) { lf_dma_to_lds(rs, voff, lds_row0); };
   // pg: page_off() of the pass (paged operands only; fetched a tile ahead by the caller)
   auto dma_k_pass = [&](int kt, int sl, int ps, unsigned pg) {
     unsigned off;
@@ -210,48 +170,8 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
   const float cexp = p.scale * LF_LOG2E;
 #endif
 
-  // per-lane fragment offsets (elements) inside a tile
-  auto k_off = [&](int f) {
-    const int ks = f / LF_NKB, kb = f % LF_NKB;
-    const int row = 32 * kb + l32;
-    return row * LF_D + 8 * lf_k_phys(row, 2 * ks + g);
-  };
-  auto k_frag = [&](const lf_elem* kbuf, int f) {
-#if LF_ABLATE & 16
-    lf_u32x4 z = {(unsigned)f, 1u, 2u, 3u};
-    return z;
-#else
-    return *reinterpret_cast<const lf_u32x4*>(&kbuf[k_off(f)]);
-#endif
-  };
-  // 16-lane group (2g + dh) asks for rows r0..r0+3, columns 32db+16dh..+15: lane j
-  // of the group supplies the 8-byte piece (row r0 + j/4, cols +4*(j%4)) and
-  // receives column j of the 4 rows.
-  auto v_frag = [&](const lf_elem* vbuf, int f) {
-    const int kk = f / LF_NDB, db = f % LF_NDB;
-    lf_elem8 a;
-#if LF_ABLATE & 64
-    for (int e = 0; e < 8; ++e) a[e] = (lf_elem)(float)(f + e);
-    return a;
-#elif LF_ABLATE & 32
-    return __builtin_bit_cast(lf_elem8, *reinterpret_cast<const lf_u32x4*>(&vbuf[k_off(f)]));
-#endif
-    const int j16 = lane & 15;
-    const int dh = (lane >> 4) & 1;
-    const int col = 32 * db + 16 * dh + 4 * (j16 & 3);
-#pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      const int row = 16 * kk + 8 * half + 4 * g + (j16 >> 2);
-      const lf_elem* src = &vbuf[row * LF_D + 8 * lf_v_phys(row, col / 8) + (col % 8)];
-      lf_s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_s16x4*)(src));
-      lf_elem4 te = __builtin_bit_cast(lf_elem4, t);
-      a[4 * half + 0] = te[0];
-      a[4 * half + 1] = te[1];
-      a[4 * half + 2] = te[2];
-      a[4 * half + 3] = te[3];
-    }
-    return a;
-  };
+  auto k_frag = [&](const lf_elem* kbuf, int f) { return lf_read_k_frag(kbuf, l32, g, f); };
+  auto v_frag = [&](const lf_elem* vbuf, int f) { return lf_read_v_frag_tr(vbuf, lane, g, f); };
 
   auto run_q_tile = [&](const int qt) {
     const int q0 = qt * LF_BM;
@@ -284,11 +204,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
                             (long long)min(my_q, p.Sq - 1) * p.q_ss;
 #pragma unroll
       for (int ks = 0; ks < LF_NKS; ++ks)
-#if LF_ABLATE & 8
-        qf[ks] = __builtin_bit_cast(lf_elem8, lf_u32x4{0x3e803f00u + lane * 65537u * ks, 0xbe803e00u, 0x3f000000u + lane, 0xbf003d80u});
-#else
         qf[ks] = __builtin_bit_cast(lf_elem8, *reinterpret_cast<const lf_u32x4*>(qrow + 16 * ks + 8 * g));
-#endif
     }
     // the compiler waits for the Q loads here (a use it can see) and all older vector
     // memory operations are drained, so its bookkeeping is clear before the direct
@@ -324,15 +240,8 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
         dma_k_pass(kt_begin, 0, ps, k0pg[ps]);
         if (kt_begin + 1 < kt_end) dma_k_pass(kt_begin + 1, 1, ps, k1pg[ps]);
         dma_v_pass(kt_begin, 0, ps, v0pg[ps]);
-#if LF_ABLATE & 2
-        dma_k_pass(kt_begin, 2, ps, k0pg[ps]);
-        dma_v_pass(kt_begin, 1, ps, v0pg[ps]);
-#endif
       }
     }
-#if LF_ABLATE & 2
-    dma_on = false;
-#endif
     LF_BARRIER_VM0();
     lf_u32x4 kpre[LF_KPF];
 #pragma unroll
@@ -417,13 +326,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
               const int j = k0 + 32 * kb + 8 * (i / 4) + 4 * g + (i % 4);
-              bool ok = j < p.Sk;
-#if LF_MASK >= 1
-              ok = ok && (j <= my_q);
-#endif
-#if LF_MASK == 2
-              ok = ok && (my_q - j < p.window);
-#endif
+              const bool ok = lf_mask_keep(my_q, j, p.Sk, p.window);
               s[kb][i] = ok ? s[kb][i] : LF_NEG_INF;
             }
         }
@@ -453,11 +356,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
         for (int kb = 0; kb < LF_NKB; ++kb)
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
-#if LF_ABLATE & 1
-            const float e = s[kb][i] * cexp - mc_sub;
-#else
             const float e = lf_exp2(s[kb][i] * cexp - mc_sub);
-#endif
             rs += e;
             pf[2 * kb + i / 8][i % 8] = lf_from_float(e);
           }
@@ -496,9 +395,6 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
 
     // ---- epilogue: O[q][d] = O^T[d][q] / l.  Element i of block db is
     // d = 32*db + 8*(i/4) + 4*g + i%4.
-#if LF_ABLATE & 2
-    dma_on = true;
-#endif
     const float l_tot = l_run + lf_swap32(l_run);
     {
       // Lane (q, g) holds, per block db, four 4-value chunks d = 32*db + 8*i4 + 4*g + 0..3.
@@ -525,9 +421,6 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
           auto r0 = __builtin_amdgcn_permlane32_swap(ch[2 * j][0], ch[2 * j + 1][0], false, false);
           auto r1 = __builtin_amdgcn_permlane32_swap(ch[2 * j][1], ch[2 * j + 1][1], false, false);
           const lf_u32x4 out = {r0[0], r1[0], r0[1], r1[1]};
-#if LF_ABLATE & 4
-          if (out[0] == 0x12345678u)
-#endif
           if (my_q < p.Sq) *reinterpret_cast<lf_u32x4*>(orow + 32 * db + 16 * j + 8 * g) = out;
         }
       }

@@ -104,6 +104,17 @@ __device__ __forceinline__ bool lf_bias_masked2(unsigned raw) {
   return lf_bias_masked(raw & 0xffffu) && lf_bias_masked(raw >> 16);
 }
 
+// Value a score-bias element adds to a score.  With LF_SAFE the values that count as masked
+// (see above) add -inf, so a key gets probability exactly 0 whether its tile / span was walked
+// or left out: a row that sees no key then gives zeros in every case.
+__device__ __forceinline__ float lf_bias_value(lf_elem b) {
+#if LF_SAFE
+  return lf_bias_masked(__builtin_bit_cast(unsigned short, b)) ? LF_NEG_INF : (float)b;
+#else
+  return (float)b;
+#endif
+}
+
 __device__ __forceinline__ float lf_inv_sum(float l) {
 #if LF_SAFE
   return l > 0.0f ? 1.0f / l : 0.0f;

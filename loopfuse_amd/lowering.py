@@ -106,8 +106,12 @@ class KernelSpec:
         return o + list(self.extra)
 
     def files(self) -> tuple[str, ...]:
-        return ("lf_common.hip.h", {"prefill": "lf_attn_prefill.hip",
-                                    "prefill_swp": "lf_attn_prefill_swp.hip", "decode": "lf_attn_decode.hip"}[self.family])
+        kernel = {"prefill": "lf_attn_prefill.hip", "prefill_swp": "lf_attn_prefill_swp.hip",
+                  "decode": "lf_attn_decode.hip"}[self.family]
+        if self.family == "decode":
+            return ("lf_common.hip.h", kernel)
+        # the two prefill kernels: their own tuning macros come first (the shared blocks use LF_BN)
+        return ("lf_common.hip.h", "lf_prefill_blocks.hip.h", kernel)
 
     def entry(self) -> str:
         return {"prefill": "lf_attn_prefill",
@@ -161,15 +165,10 @@ def compile_spec(spec: KernelSpec, arch: str = runtime.DEFAULT_ARCH) -> Compiled
         ck = _compiled.get(spec)
     if ck is not None:
         return ck
-    override = os.environ.get("LOOPFUSE_HSACO_" + spec.family.upper())   # tuning aid: prebuilt code object
-    if override:
-        with open(override, "rb") as fh:
-            ck = CompiledKernel(spec, fh.read(), False, "override " + override)
-    else:
-        # outside the lock: different specialisations compile concurrently (the shim is re-entrant;
-        # two threads asking for the same one both compile, the results are identical)
-        code, hit, log = runtime.compile_source(spec.source(), spec.name(), spec.options(), arch)
-        ck = CompiledKernel(spec, code, hit, log)
+    # outside the lock: different specialisations compile concurrently (the shim is re-entrant;
+    # two threads asking for the same one both compile, the results are identical)
+    code, hit, log = runtime.compile_source(spec.source(), spec.name(), spec.options(), arch)
+    ck = CompiledKernel(spec, code, hit, log)
     record = os.environ.get("LOOPFUSE_RECORD_SPECS")
     with _lock:
         if record and spec not in _compiled:
@@ -406,6 +405,32 @@ def tuned_attention(q, k, v, plan: AttnPlan, k_table=None, v_table=None, **kw):
     return attention(q, k, v, plan, k_table, v_table, **{**kw, "choice": _tuned[key]})
 
 
+class _LastLaunch:
+    """What the calling THREAD's last ``attention`` call launched (kernels, grid, block, tile
+    shape): ``attention.last_launch["kernels"]``.  Each thread sees its own record."""
+
+    def __init__(self):
+        self._tls = threading.local()
+
+    def set(self, record: dict) -> None:
+        self._tls.record = record
+
+    def _get(self) -> dict:
+        return getattr(self._tls, "record", {})
+
+    def __getitem__(self, key):
+        return self._get()[key]
+
+    def get(self, key, default=None):
+        return self._get().get(key, default)
+
+    def __repr__(self) -> str:
+        return repr(self._get())
+
+
+_last_launch = _LastLaunch()
+
+
 def _on_device_of_first_argument(fn):
     """Kernel modules, the stream and the split-K scratch are looked up for the current
     device: make the device of Q current for the duration of the call when it is not."""
@@ -415,6 +440,7 @@ def _on_device_of_first_argument(fn):
             with torch.cuda.device(q.device):
                 return fn(q, *args, **kw)
         return fn(q, *args, **kw)
+    guarded.last_launch = _last_launch
     return guarded
 
 
@@ -463,6 +489,13 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         raise UnsupportedPlan(f"head dim {D} not supported (64, 128)")
     if not (plan.scale > 0.0) or not math.isfinite(plan.scale):
         raise UnsupportedPlan("score scale must be positive and finite")
+    softcap = None
+    if plan.softcap is not None:
+        # cap * tanh(s / cap) is even in cap: a negative cap (pre- and post-factor both negative
+        # in the graph) is served as its magnitude; zero or a non-finite cap is not a softcap
+        softcap = abs(float(plan.softcap))
+        if not (softcap > 0.0) or not math.isfinite(softcap):
+            raise UnsupportedPlan("softcap must be finite and non-zero")
     _check_tensor("Q", q, dtype)
     _check_tensor("K", k, dtype)
     _check_tensor("V", v, dtype)
@@ -503,6 +536,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
             ps, hk, sp, st, sh = t.shape[1], t.shape[2], t.stride(0), t.stride(1), t.stride(2)
         else:
             raise UnsupportedPlan(f"{which} pool must be [N, Hkv, D] or [N, P, Hkv, D]")
+        if t.shape[-1] != D:
+            raise UnsupportedPlan(f"{which} pool has head dim {t.shape[-1]}, Q has {D}")
         if ps & (ps - 1):
             raise UnsupportedPlan("page size must be a power of two")
         i64 = table.dtype == torch.int64
@@ -538,7 +573,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
             raise UnsupportedPlan(f"O must be [{B}, {Hq}, {Sq}, {D}]")
     if B == 0 or Hq == 0 or Sq == 0:
         # no query rows: the (empty) output is the whole result, nothing to launch
-        attention.last_launch = {"kernels": [], "grid": 0, "block": 0}
+        _last_launch.set({"kernels": [], "grid": 0, "block": 0})
         return (out, torch.zeros((0, 0), dtype=torch.uint8, device=q.device)) if record_visits else out
 
     P.q, P.k, P.v, P.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
@@ -547,7 +582,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     P.B, P.Hq, P.Hkv, P.Sq, P.Sk = B, Hq, Hkv, Sq, Sk
     P.window = int(plan.window)
     P.scale = float(plan.scale)
-    P.softcap = float(plan.softcap) if plan.softcap else 0.0
+    P.softcap = softcap if softcap is not None else 0.0
     P.denom_add = float(plan.denom_add)
     if plan.denom_add < 0.0 or not math.isfinite(plan.denom_add):
         raise UnsupportedPlan("the denominator offset must be finite and >= 0")
@@ -682,8 +717,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         if family == "prefill_swp" and persist:
             grid = min(grid, 8 * int(persist))
         get_kernel(spec, spec.entry()).launch((grid, 1, 1), (64 * nw, 1, 1), P)
-        attention.last_launch = {"kernels": [spec.entry()], "grid": grid, "block": 64 * nw, "q_tile_rows": bm,
-                                 "heads_per_workgroup": spec.pack or 1}
+        _last_launch.set({"kernels": [spec.entry()], "grid": grid, "block": 64 * nw, "q_tile_rows": bm,
+                                 "heads_per_workgroup": spec.pack or 1})
         return (out, visits) if record_visits else out
 
     if family != "decode":
@@ -731,8 +766,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         nrow = B * Hkv * rows * nsplit
         runtime.launch_decode_static(get_kernel(spec, "lf_attn_decode"), get_kernel(spec, "lf_attn_decode_combine"), P,
                                      4 * nrow * D, 4 * nrow * 2, (units, nsplit), 64 * spec.waves, combine_grid, 256)
-        attention.last_launch = {"kernels": ["lf_attn_decode", "lf_attn_decode_combine"], "grid": (units, nsplit),
-                                 "block": 64 * spec.waves, "head_per_wave": headwave, "static_scratch": True}
+        _last_launch.set({"kernels": ["lf_attn_decode", "lf_attn_decode_combine"], "grid": (units, nsplit),
+                                 "block": 64 * spec.waves, "head_per_wave": headwave, "static_scratch": True})
         return out
     if nsplit > 1:
         nrow = B * Hkv * rows * nsplit
@@ -742,6 +777,6 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     get_kernel(spec, "lf_attn_decode").launch((units, nsplit, 1), (64 * spec.waves, 1, 1), P)
     if nsplit > 1 and merge_splits:
         get_kernel(spec, "lf_attn_decode_combine").launch((combine_grid, 1, 1), (256, 1, 1), P)
-    attention.last_launch = {"kernels": ["lf_attn_decode"] + (["lf_attn_decode_combine"] if nsplit > 1 and merge_splits else []),
-                             "grid": (units, nsplit), "block": 64 * spec.waves, "head_per_wave": headwave}
+    _last_launch.set({"kernels": ["lf_attn_decode"] + (["lf_attn_decode_combine"] if nsplit > 1 and merge_splits else []),
+                             "grid": (units, nsplit), "block": 64 * spec.waves, "head_per_wave": headwave})
     return out

@@ -47,7 +47,9 @@ USE_HARDCODE_KERNEL = os.environ.get("USE_HARDCODE_KERNEL", "0") == "1"
 # "eager_graph" = graph not recognised, "eager_runtime" = recognised but the call's
 # tensors could not be served (CPU tensors, dtype, alignment ...)
 # "eager_training" = graph traced with gradients enabled (forward or backward half)
-stats = {"fused": 0, "eager_graph": 0, "eager_runtime": 0, "eager_training": 0, "compiled_graphs": 0, "matched_graphs": 0}
+# "refused_signatures" = argument layouts latched as not servable (see optimized_fn)
+stats = {"fused": 0, "eager_graph": 0, "eager_runtime": 0, "eager_training": 0, "compiled_graphs": 0, "matched_graphs": 0,
+         "refused_signatures": 0}
 
 
 def _strict() -> bool:
@@ -99,15 +101,13 @@ def _unfused_compiler(gm: torch.fx.GraphModule, sample_inputs) -> Callable:
     return make_boxed_func(eager_fn)
 
 
-# attention sub-graphs of the graphs compiled so far; the rewritten graphs call
-# ``_fused_call(id, *inputs)`` where the unfused chain used to end
-_MATCHES: list = []
 _codegen_sink: list | None = None     # CODEGEN_ONLY: compiled specialisations are collected here
+last_matches: list = []               # attention sub-graphs of the most recently compiled graph (debugging, tests)
 
 
-def _fused_call(match_id: int, *vals):
-    """Stand-in for one attention sub-graph inside a rewritten graph."""
-    match = _MATCHES[match_id]
+def _fused_call(match, *vals):
+    """Stand-in for one attention sub-graph inside a rewritten graph; ``match`` is an attribute
+    of the rewritten graph module, so it lives exactly as long as that compiled graph does."""
     if _codegen_sink is not None:
         _codegen_sink.extend(lowering.compile_spec(s) for s in match.kernel_specs_for(vals))
         q = vals[match.q.index]
@@ -122,15 +122,26 @@ def rewrite_graph(gm: torch.fx.GraphModule, matches: list) -> torch.fx.GraphModu
     val_map: dict = {}
     out = new_graph.graph_copy(gm.graph, val_map)
     new_graph.output(out)
-    for m in matches:
-        _MATCHES.append(m)
+    last_matches[:] = matches
+    names = []
+    for i, m in enumerate(matches):
+        name = f"_lf_match_{i}"
+        setattr(gm, name, m)          # GraphModule() below copies the attributes its get_attr nodes name
+        names.append(name)
         old = val_map[m.out_node]
         with new_graph.inserting_after(old):
-            call = new_graph.call_function(_fused_call, (len(_MATCHES) - 1, *[val_map[n] for n in m.inputs]))
+            attr = new_graph.get_attr(name)
+        with new_graph.inserting_after(attr):
+            call = new_graph.call_function(_fused_call, (attr, *[val_map[n] for n in m.inputs]))
         old.replace_all_uses_with(call)
     new_graph.eliminate_dead_code()
-    new_graph.lint()
-    return torch.fx.GraphModule(gm, new_graph)
+    try:
+        fused = torch.fx.GraphModule(gm, new_graph)
+    finally:
+        for name in names:
+            delattr(gm, name)
+    fused.graph.lint()
+    return fused
 
 
 def loopfuse_compiler(gm: torch.fx.GraphModule, sample_inputs, input_names: list[str] | None = None,
@@ -192,13 +203,20 @@ def loopfuse_compiler(gm: torch.fx.GraphModule, sample_inputs, input_names: list
 
         return codegen_fn
 
-    refused = [0]       # consecutive calls of this graph that the kernels could not serve
+    # Calls the kernels could not serve, by what the refusal depends on: dtype, shape, strides,
+    # alignment and device of every tensor argument (and the integer arguments).  A call with a
+    # signature refused before goes straight to the unfused graph -- each failed attempt runs the
+    # graph up to the fused call for nothing -- while a call with another signature (another
+    # shape under dynamic=True, an aligned tensor after an unaligned one) is tried again.
+    refused: set = set()
+
+    def signature(args):
+        return tuple((a.dtype, tuple(a.shape), a.stride(), a.data_ptr() % 16, a.device) if isinstance(a, torch.Tensor) else a
+                     for a in args)
 
     def optimized_fn(*args):
-        if refused[0] >= 2:
-            # what the kernels refuse (dtype, head dim, layout) is a property of the traced
-            # graph, which dynamo re-traces when it changes: stop trying, each attempt runs
-            # the graph up to the fused call for nothing
+        sig = signature(args) if refused else None
+        if sig is not None and sig in refused:
             stats["eager_runtime"] += 1
             return gm(*args)
         try:
@@ -206,13 +224,14 @@ def loopfuse_compiler(gm: torch.fx.GraphModule, sample_inputs, input_names: list
         except lowering.UnsupportedPlan as e:
             if _strict():
                 raise
-            refused[0] += 1
-            (log.warning if refused[0] == 2 else log.info)(
-                "fused path not applicable to this call (%s); running the graph unfused%s", e,
-                " from now on" if refused[0] == 2 else "")
+            if len(refused) >= 64:      # bounded: forget old refusals rather than grow
+                refused.clear()
+            refused.add(signature(args))
+            stats["refused_signatures"] += 1
+            log.warning("fused path not applicable to this call (%s); calls with these argument layouts run "
+                        "the graph unfused", e)
             stats["eager_runtime"] += 1
             return gm(*args)
-        refused[0] = 0
         stats["fused"] += 1
         return out
 

@@ -2,9 +2,9 @@
  * lf_client.c — a C host that drives the attention kernels through the C ABI alone
  * (include/lf_shim.h + include/lf_attn_params.h): no Python, no torch.
  *
- *   lf_client <kernel source dir> [prefill|decode]
+ *   lf_client <kernel source dir> [prefill|prefill_swp|decode]
  *
- * It compiles lf_attn_prefill.hip (causal, bf16, D = 128) or lf_attn_decode.hip
+ * It compiles lf_attn_prefill.hip or lf_attn_prefill_swp.hip (causal, bf16, D = 128) or lf_attn_decode.hip
  * (paged GQA, bf16, D = 128, pages of 16 tokens) with lf_compile, loads and
  * launches it with lf_module_load / lf_get_function / lf_launch on device buffers
  * of its own, and checks the result against double-precision loops over the same
@@ -67,18 +67,24 @@ static char* read_file(const char* dir, const char* name, size_t* len) {
   return buf;
 }
 
-/* common header + kernel file = one translation unit */
+/* common header (+ the prefill building blocks) + kernel file = one translation unit */
 static char* kernel_source(const char* dir, const char* file) {
-  size_t a, b;
-  char* h = read_file(dir, "lf_common.hip.h", &a);
-  char* k = read_file(dir, file, &b);
-  if (!h || !k) return NULL;
-  char* s = (char*)malloc(a + b + 2);
-  memcpy(s, h, a);
-  s[a] = '\n';
-  memcpy(s + a + 1, k, b + 1);
-  free(h);
-  free(k);
+  const char* parts[3] = {"lf_common.hip.h", strstr(file, "prefill") ? "lf_prefill_blocks.hip.h" : NULL, file};
+  char* s = (char*)malloc(1);
+  size_t total = 0;
+  s[0] = 0;
+  for (int i = 0; i < 3; ++i) {
+    if (!parts[i]) continue;
+    size_t n;
+    char* t = read_file(dir, parts[i], &n);
+    if (!t) { free(s); return NULL; }
+    s = (char*)realloc(s, total + n + 2);
+    memcpy(s + total, t, n);
+    s[total + n] = '\n';
+    s[total + n + 1] = 0;
+    total += n + 1;
+    free(t);
+  }
   return s;
 }
 
@@ -104,7 +110,7 @@ static const char* kCommon[] = {"-O3", "-std=c++17", "-Xclang", "-target-feature
                                 "-DLF_DTYPE=0", "-DLF_HEAD_DIM=128", "-DLF_SOFTCAP=0", "-DLF_TABLE_I64=0"};
 #define NCOMMON ((int)(sizeof kCommon / sizeof kCommon[0]))
 
-static int run_prefill(const char* dir) {
+static int run_prefill(const char* dir, const char* file, const char* symbol) {
   enum { B = 2, H = 3, S = 200, D = 128 };
   const size_t n = (size_t)B * H * S * D;
   uint16_t *q = malloc(2 * n), *k = malloc(2 * n), *v = malloc(2 * n), *o = malloc(2 * n);
@@ -120,7 +126,7 @@ static int run_prefill(const char* dir) {
   memcpy(opts, kCommon, sizeof kCommon);
   opts[NCOMMON] = "-DLF_MASK=1"; opts[NCOMMON + 1] = "-DLF_PAGED=0"; opts[NCOMMON + 2] = "-DLF_PAGE_SIZE=1";
   void* fn = NULL;
-  int rc = load_kernel(dir, "lf_attn_prefill.hip", opts, NCOMMON + 3, "lf_attn_prefill", &fn);
+  int rc = load_kernel(dir, file, opts, NCOMMON + 3, symbol, &fn);
   if (rc) return rc;
 
   LfAttnParamsHost p;
@@ -160,7 +166,7 @@ static int run_prefill(const char* dir) {
       if (!(err <= worst)) worst = err;      /* NaN-proof */
     }
   }
-  printf("prefill causal bf16 B%d H%d S%d D%d through the C ABI: max abs err %.3g\n", B, H, S, D, worst);
+  printf("%s causal bf16 B%d H%d S%d D%d through the C ABI: max abs err %.3g\n", symbol, B, H, S, D, worst);
   return worst <= 2e-2 ? 0 : 1;
 }
 
@@ -233,14 +239,15 @@ static int run_decode(const char* dir) {
 }
 
 int main(int argc, char** argv) {
-  if (argc < 2) { fprintf(stderr, "usage: %s <kernel source dir> [prefill|decode]\n", argv[0]); return 64; }
+  if (argc < 2) { fprintf(stderr, "usage: %s <kernel source dir> [prefill|prefill_swp|decode]\n", argv[0]); return 64; }
   if (lf_abi_version() != 2) { fprintf(stderr, "unexpected ABI version %d\n", lf_abi_version()); return 5; }
   char arch[64];
   int cus = 0, lds = 0;
   CHECK_LF(lf_device_info(0, arch, sizeof arch, &cus, &lds));
   printf("device 0: %s, %d CUs, %d bytes of LDS per workgroup\n", arch, cus, lds);
   int rc = 0;
-  if (argc < 3 || !strcmp(argv[2], "prefill")) rc |= run_prefill(argv[1]);
+  if (argc < 3 || !strcmp(argv[2], "prefill")) rc |= run_prefill(argv[1], "lf_attn_prefill.hip", "lf_attn_prefill");
+  if (argc < 3 || !strcmp(argv[2], "prefill_swp")) rc |= run_prefill(argv[1], "lf_attn_prefill_swp.hip", "lf_attn_prefill_swp");
   if (argc < 3 || !strcmp(argv[2], "decode")) rc |= run_decode(argv[1]);
   if (rc == 0) printf("OK\n");
   return rc;

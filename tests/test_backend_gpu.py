@@ -187,9 +187,8 @@ def test_prefix_attention_two_fused_calls():
     B, H, Sq, Sp, D = 3, 4, 320, 512, 128
     Q, Ks, Vs = (rand((B, H, Sq, D), seed=s) for s in (1, 2, 3))
     Kp, Vp = (rand((B, H, Sp, D), seed=s) for s in (4, 5))
-    n0 = len(interface._MATCHES)
     got = run_fused(fn, (Q, Kp, Vp, Ks, Vs))
-    assert len(interface._MATCHES) == n0 + 2
+    assert len(interface.last_matches) == 2
     want = O.attention_reference(Q, Kp, Vp) + O.attention_reference(Q, Ks, Vs, mask="causal")
     assert (got - want).abs().max() <= 2 * TOL      # two bf16 results added in bf16
 
@@ -398,7 +397,7 @@ def test_decoder_layer_with_cache_and_repeated_kv_heads(S, P, use_mask):
         want = m(*ins)
     torch.cuda.synchronize()
     assert interface.stats["fused"] == before["fused"] + 1, "the fused HIP path was not taken"
-    match = interface._MATCHES[-1]
+    match = interface.last_matches[-1]
     assert match.k.group == 4 and match.inputs[match.k.index].name.startswith("cat")
     assert (got[0].float() - want[0].float()).abs().max().item() <= 4 * TOL
     assert torch.equal(got[1], want[1]) and torch.equal(got[2], want[2])

@@ -418,10 +418,9 @@ def test_rewritten_graphs_compute_the_same(which, monkeypatch):
         n_attn = 1
     torch._dynamo.reset()
     before = dict(interface.stats)
-    n_before = len(interface._MATCHES)
     got = torch.compile(fn, backend=loopfuse_amd.loopfuse_backend, dynamic=True)(*ins)
     assert interface.stats["fused"] == before["fused"] + 1
-    assert len(interface._MATCHES) == n_before + n_attn
+    assert len(interface.last_matches) == n_attn
     want = fn(*ins)
     for g, w in zip(got if isinstance(got, tuple) else (got,), want if isinstance(want, tuple) else (want,)):
         torch.testing.assert_close(g, w, rtol=2e-4, atol=2e-4)
@@ -445,9 +444,9 @@ def test_backend_on_cpu_tensors_runs_graph_unfused():
 
 
 def test_repeated_refusals_stop_the_attempts(monkeypatch):
-    """After two consecutive calls the kernels cannot serve, a compiled graph goes straight
-    to its captured form: the part of the rewritten graph before the fused call is not run
-    for nothing any more."""
+    """A call the kernels cannot serve latches its argument layout: later calls with the same
+    layout go straight to the captured graph (the part of the rewritten graph before the fused
+    call is not run for nothing), a call with another layout is tried again."""
     attempts = []
 
     def refuse(self, vals):
@@ -462,7 +461,15 @@ def test_repeated_refusals_stop_the_attempts(monkeypatch):
     compiled = torch.compile(fn, backend=loopfuse_amd.loopfuse_backend, dynamic=True)
     for _ in range(5):
         assert torch.allclose(compiled(q, k, v), fn(q, k, v), atol=1e-6)
-    assert len(attempts) == 2 and interface.stats["eager_runtime"] == before["eager_runtime"] + 5
+    assert len(attempts) == 1 and interface.stats["eager_runtime"] == before["eager_runtime"] + 5
+    assert interface.stats["refused_signatures"] == before["refused_signatures"] + 1
+    # another layout of the same graph (a strided view of K) is a new signature: tried once more
+    k2 = torch.randn(1, 2, 16, 128, generator=torch.Generator().manual_seed(3))[..., :64]
+    graphs = interface.stats["compiled_graphs"]
+    for _ in range(3):
+        assert torch.allclose(compiled(q, k2, v), fn(q, k2, v), atol=1e-6)
+    if interface.stats["compiled_graphs"] == graphs:      # same compiled graph served the new layout
+        assert len(attempts) == 2
 
 
 def test_unfused_graph_still_correct():
@@ -688,7 +695,7 @@ def test_decoder_layer_with_cache_and_repeated_kv_heads(S, P, use_mask, dynamic,
         got = torch.compile(m, backend=loopfuse_amd.loopfuse_backend, dynamic=dynamic)(*ins)
         want = m(*ins)
     assert interface.stats["fused"] == before["fused"] + 1
-    match = interface._MATCHES[-1]
+    match = interface.last_matches[-1]
     assert match.k.group == 4 and match.v.group == 4
     assert match.inputs[match.k.index].name.startswith("cat") and (match.bias is not None) == use_mask
     for a, b in zip(got, want):

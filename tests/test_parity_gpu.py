@@ -1046,9 +1046,9 @@ def test_masks_filled_with_the_most_negative_finite_value(dtype, shape):
         keep = (torch.arange(Sk)[None, :] <= torch.arange(Sq)[:, None]) & (torch.arange(Sk)[None, :] >= 200)
         keep = keep[None, None].expand(B, 1, Sq, Sk)
     else:
-        B, H, Sq, Sk = 3, 4, 1, 3000
-        keep = ((torch.arange(Sk)[None, :] >= torch.tensor([0, 2100, 64])[:, None]) &
-                (torch.arange(Sk)[None, :] < torch.tensor([500, 2600, 65])[:, None]))[:, None, None, :]
+        B, H, Sq, Sk = 4, 4, 1, 3000          # the last sequence sees no key at all
+        keep = ((torch.arange(Sk)[None, :] >= torch.tensor([0, 2100, 64, 7])[:, None]) &
+                (torch.arange(Sk)[None, :] < torch.tensor([500, 2600, 65, 7])[:, None]))[:, None, None, :]
     lowest = torch.zeros(keep.shape).masked_fill(~keep, torch.finfo(dtype).min).to(dtype)
     ninf = torch.zeros(keep.shape).masked_fill(~keep, float("-inf")).to(dtype)
     q, k, v = rand((B, H, Sq, D), dtype, 1), rand((B, H, Sk, D), dtype, 2), rand((B, H, Sk, D), dtype, 3)
@@ -1058,6 +1058,10 @@ def test_masks_filled_with_the_most_negative_finite_value(dtype, shape):
     b = lowering.attention(*on, plan, score_bias=ninf.to(dev()))
     sees = keep.any(-1).expand(B, H, Sq)
     assert torch.isfinite(a).all() and torch.equal(a[sees.to(dev())], b[sees.to(dev())])
+    # rows that see no key give zeros with either fill, also where they share a walked tile / span
+    # with rows that do see keys (fp16: the finite fill times log2(e) stays finite, so it has to be
+    # mapped to -inf where it is added, not only where tiles are left out)
+    assert (~sees).any() and (a[(~sees).to(dev())] == 0).all() and (b[(~sees).to(dev())] == 0).all()
     want = O.attention_reference(q, k, v, score_bias=ninf.float())
     assert (a.float().cpu()[sees] - want[sees]).abs().max().item() <= TOL[dtype]
 
