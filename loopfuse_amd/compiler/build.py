@@ -1,0 +1,297 @@
+"""ATen graph -> one loop nest per compute op (the counterpart of the reference's graph
+parser and op builders, ``loopfuse/torch_backend/interface.py:357-527`` and
+``loopfuse/torch_backend/ops.py:344-751``).
+
+View ops (transpose, expand, unsqueeze, view/reshape, clone, ``loopfuse::paged_load``) build
+nothing: they regroup the atoms of a ``View``.  Compute ops (bmm, scalar multiply / divide,
+tanh, the two mask ops, softmax) instantiate their operands with fresh atoms, unify the index
+ranges that must agree, and append one nest that writes a temporary buffer.
+"""
+from __future__ import annotations
+
+import dataclasses
+import math
+import operator
+from typing import Optional
+
+import torch
+
+from . import ir
+from .ir import Atom, Buffer
+
+aten = torch.ops.aten
+
+
+class Unsupported(Exception):
+    """The graph uses something these builders do not cover."""
+
+
+@dataclasses.dataclass
+class View:
+    """A tensor value: ``dims[k]`` = atoms of view dimension k; ``idx[d]`` = atoms that index
+    dimension d of ``buf``; ``gather`` = (d, table View): buffer dimension d is read at
+    ``table[...]`` (page gather)."""
+
+    buf: Buffer
+    idx: list[list[Atom]]
+    dims: list[list[Atom]]
+    gather: Optional[tuple] = None
+
+    def instantiate(self, memo: Optional[dict] = None) -> "View":
+        """The same structure over fresh atoms (every use of a value gets its own)."""
+        memo = {} if memo is None else memo
+
+        def cp(a: Atom) -> Atom:
+            a = a.rep()
+            if a.id not in memo:
+                n = Atom(a.size, a.hint, a.name.rstrip("'") + "'")
+                n.broadcast = a.broadcast
+                memo[a.id] = n
+                if a.children is not None:
+                    n.children = [cp(c) for c in a.children]
+            return memo[a.id]
+
+        g = None
+        if self.gather is not None:
+            g = (self.gather[0], self.gather[1].instantiate(memo))
+        return View(self.buf, [[cp(a) for a in d] for d in self.idx], [[cp(a) for a in d] for d in self.dims], g)
+
+    def read(self) -> ir.Read:
+        g = None if self.gather is None else (self.gather[0], self.gather[1].buf, self.gather[1].idx)
+        return ir.Read(self.buf, self.idx, g)
+
+
+def _hint(x) -> int:
+    if isinstance(x, int):
+        return x
+    return int(x.node.hint)
+
+
+def _sym(x) -> str:
+    return str(x)
+
+
+class Parser:
+    """Walks the graph once; ``nests`` and ``out`` (the View of the graph's single output) result."""
+
+    def __init__(self, gm: torch.fx.GraphModule):
+        self.gm = gm
+        self.env: dict = {}              # fx node -> View | ("scalar", fn, text) | ("size", fn, text, hint)
+        self.nests: list[ir.Nest] = []
+        self.inputs: list[Buffer] = []
+        self.sizes: dict[str, int] = {}  # size symbol -> placeholder index (SymInt inputs), for evaluation per call
+        self.ntemp = 0
+        self.out: Optional[View] = None
+
+    # ------------------------------------------------------------ helpers
+    def temp(self, name: str, dims: list[list[Atom]]) -> Buffer:
+        self.ntemp += 1
+        return Buffer(f"{name}{self.ntemp}", dims, "temp")
+
+    def size_of(self, a):
+        """(symbol text, hint) of a size argument: int, SymInt-valued node or python int."""
+        if isinstance(a, torch.fx.Node):
+            v = self.env[a]
+            if v[0] != "size":
+                raise Unsupported(f"{a} is not a size")
+            return v[2], v[3]
+        return str(int(a)), int(a)
+
+    def emit(self, name: str, out_dims: list[list[Atom]], red: list[Atom], value: ir.Expr, accum=None) -> View:
+        buf = self.temp(name, out_dims)
+        stmt = ir.Assign(buf, value) if accum is None else ir.Accum(buf, accum[0], value, accum[1])
+        self.nests.append(ir.Nest(buf.name, [a for d in out_dims for a in d], red, stmt))
+        return View(buf, [list(d) for d in out_dims], [list(d) for d in out_dims])
+
+    # ------------------------------------------------------------ the walk
+    def run(self) -> "Parser":
+        ph = 0
+        for n in self.gm.graph.nodes:
+            if n.op == "placeholder":
+                v = n.meta.get("val")
+                if isinstance(v, torch.Tensor) and v.dim() == 0:
+                    # a python float of the traced function that dynamo lifted into a 0-dim tensor input
+                    # (a softcap held in a variable): a run-time scalar
+                    self.env[n] = ("scalar", (lambda args, i=ph: float(args[i])), n.name)
+                elif isinstance(v, torch.Tensor):
+                    dims = [[Atom(_sym(s), _hint(s), f"{n.name}.{k}")] for k, s in enumerate(v.shape)]
+                    buf = Buffer(n.name, dims, "input", str(v.dtype).replace("torch.", ""), ph)
+                    self.inputs.append(buf)
+                    self.env[n] = View(buf, [list(d) for d in dims], [list(d) for d in dims])
+                elif isinstance(v, (torch.SymInt, int)):
+                    idx = ph
+                    self.sizes[_sym(v)] = idx
+                    self.env[n] = ("size", (lambda args, i=idx: int(args[i])), _sym(v), _hint(v))
+                elif isinstance(v, (torch.SymFloat, float)):
+                    # a python float of the traced function that dynamo made a graph input (a softcap
+                    # held in a variable): a run-time scalar
+                    self.env[n] = ("scalar", (lambda args, i=ph: float(args[i])), n.name)
+                else:
+                    raise Unsupported(f"placeholder {n.name} of type {type(v).__name__}")
+                ph += 1
+            elif n.op == "call_function":
+                self.env[n] = self.call(n)
+            elif n.op == "output":
+                outs = n.args[0]
+                outs = outs if isinstance(outs, (tuple, list)) else (outs,)
+                if len(outs) != 1 or not isinstance(self.env.get(outs[0]), View):
+                    raise Unsupported("graphs with one tensor output only")
+                self.out = self.env[outs[0]]
+            else:
+                raise Unsupported(f"node kind {n.op}")
+        return self
+
+    def call(self, n: torch.fx.Node):
+        t, a = n.target, n.args
+        val = lambda x: self.env[x] if isinstance(x, torch.fx.Node) else x
+        # ---- integer arithmetic on sizes
+        if t in (operator.mul, operator.floordiv, operator.add, operator.sub):
+            (sa, ha), (sb, hb) = self.size_of(a[0]), self.size_of(a[1])
+            fa = val(a[0])[1] if isinstance(a[0], torch.fx.Node) else (lambda args, c=int(a[0]): c)
+            fb = val(a[1])[1] if isinstance(a[1], torch.fx.Node) else (lambda args, c=int(a[1]): c)
+            sym = {operator.mul: "*", operator.floordiv: "//", operator.add: "+", operator.sub: "-"}[t]
+            return ("size", (lambda args, f=t, x=fa, y=fb: f(x(args), y(args))), f"({sa}{sym}{sb})", t(ha, hb))
+        # ---- 0-dim values computed from sizes (D ** -0.5 and the like)
+        if t is aten.scalar_tensor.default:
+            x = a[0]
+            if isinstance(x, torch.fx.Node):
+                s = self.env[x]
+                return ("scalar", (lambda args, f=s[1]: float(f(args))), s[2])
+            return ("scalar", (lambda args, c=float(x): c), f"{float(x):g}")
+        if t is torch.ops.prims.convert_element_type.default and isinstance(val(a[0]), tuple):
+            return val(a[0])
+        if t is aten.pow.Tensor_Tensor and isinstance(val(a[0]), tuple) and isinstance(val(a[1]), tuple):
+            x, y = val(a[0]), val(a[1])
+            return ("scalar", (lambda args, f=x[1], g=y[1]: f(args) ** g(args)), f"{x[2]}**{y[2]}")
+        # ---- views
+        if t is aten.transpose.int:
+            v = val(a[0])
+            d0, d1 = a[1] % len(v.dims), a[2] % len(v.dims)
+            dims = list(v.dims)
+            dims[d0], dims[d1] = dims[d1], dims[d0]
+            return dataclasses.replace(v, dims=dims)
+        if t is aten.permute.default:
+            v = val(a[0])
+            return dataclasses.replace(v, dims=[v.dims[p % len(v.dims)] for p in a[1]])
+        if t is aten.unsqueeze.default:
+            v = val(a[0])
+            dims = list(v.dims)
+            dims.insert(a[1] % (len(dims) + 1), [])
+            return dataclasses.replace(v, dims=dims)
+        if t in (aten.clone.default, aten.alias.default, aten.contiguous.default if hasattr(aten, "contiguous") else None):
+            return val(a[0])
+        if t is torch.ops.prims.convert_element_type.default or t is aten._to_copy.default:
+            return val(a[0])             # precision of intermediates is the kernels' business (fp32 throughout)
+        if t is aten.expand.default:
+            v = val(a[0])
+            dims = [list(d) for d in v.dims]
+            dims = [[] for _ in range(len(a[1]) - len(dims))] + dims
+            for k, s in enumerate(a[1]):
+                sym, h = self.size_of(s)
+                have = math.prod(x.hint for x in ir.leaves(dims[k])) if dims[k] else 1
+                if have == 1 and h != 1:
+                    b = Atom(sym, h, f"{n.name}.bc{k}")
+                    b.broadcast = True
+                    dims[k] = [b]
+                elif have != h:
+                    raise Unsupported(f"expand of dim {k}: {have} -> {h}")
+            return dataclasses.replace(v, dims=dims)
+        if t in (aten.view.default, aten._unsafe_view.default, aten.reshape.default):
+            return self.reshape(val(a[0]), a[1])
+        if t is torch.ops.loopfuse.paged_load.default:
+            pool, table = val(a[0]), val(a[1])
+            if pool.gather is not None or table.gather is not None or len(table.dims) != 2:
+                raise Unsupported("paged_load of a view")
+            # out[b, pg, *t] = pool[table[b, pg], *t]
+            return View(pool.buf, pool.idx, [list(d) for d in table.dims] + [list(d) for d in pool.dims[1:]], (0, table))
+        # ---- compute ops
+        if t is aten.bmm.default:
+            return self.bmm(val(a[0]).instantiate(), val(a[1]).instantiate())
+        if t in (aten.mul.Tensor, aten.div.Tensor):
+            x, y = val(a[0]), val(a[1])
+            if isinstance(x, View) and not isinstance(y, View):
+                if isinstance(y, tuple):
+                    factor: ir.Expr = ir.Scalar(y[1], y[2])
+                else:
+                    factor = ir.Const(float(y))
+                v = x.instantiate()
+                return self.emit("mul" if t is aten.mul.Tensor else "div", v.dims, [],
+                                 ir.Bin("mul" if t is aten.mul.Tensor else "div", v.read(), factor))
+            raise Unsupported("tensor-by-tensor products other than bmm")
+        if t is aten.tanh.default:
+            v = val(a[0]).instantiate()
+            return self.emit("tanh", v.dims, [], ir.Un("tanh", v.read()))
+        if t is torch.ops.loopfuse.causal_mask.default:
+            v = val(a[0]).instantiate()
+            row, col = v.dims[-2], v.dims[-1]
+            return self.emit("mask", v.dims, [], ir.Select([ir.Clause(-1, 1, 0, row, col)], v.read(), float("-inf")))
+        if t is torch.ops.loopfuse.sliding_mask.default:
+            v = val(a[0]).instantiate()
+            row, col = v.dims[-2], v.dims[-1]
+            # 0 <= i - j <= w - 1, top-left aligned (reference ops.py:733-741); the window may be a
+            # run-time integer of the graph
+            if isinstance(a[1], torch.fx.Node):
+                wv = self.env[a[1]]
+                w, wfn = wv[3], (lambda args, f=wv[1]: -(int(f(args)) - 1))
+            else:
+                w, wfn = int(a[1]), None
+            cl = [ir.Clause(-1, 1, 0, row, col), ir.Clause(1, -1, -(w - 1), row, col, wfn)]
+            return self.emit("mask", v.dims, [], ir.Select(cl, v.read(), float("-inf")))
+        if t is aten._softmax.default:
+            return self.softmax(val(a[0]), a[1])
+        raise Unsupported(f"op {t}")
+
+    def reshape(self, v: View, shape) -> View:
+        """Regroup the atoms of all dims, outer to inner, into the requested sizes; an atom
+        that straddles a boundary is split."""
+        flat = [x for d in v.dims for x in ir.leaves(d)]
+        out: list[list[Atom]] = []
+        for s in shape:
+            sym, want = self.size_of(s)
+            cur: list[Atom] = []
+            have = 1
+            while have < want or (flat and flat[0].hint == 1 and have == want and len(out) == len(shape) - 1):
+                if not flat:
+                    raise Unsupported("reshape sizes do not multiply out")
+                x = flat.pop(0)
+                if have * x.hint <= want and want % (have * x.hint) == 0:
+                    cur.append(x)
+                    have *= x.hint
+                else:
+                    need = want // have
+                    if x.hint % need:
+                        raise Unsupported("reshape splits a dimension unevenly")
+                    x.split(need, f"({sym})" if have == 1 else f"({sym})//{have}", f"({x.size})//({need})")
+                    cur.append(x.children[0])
+                    flat.insert(0, x.children[1])
+                    have = want
+            out.append(cur)
+        if any(x.hint != 1 for x in flat):
+            raise Unsupported("reshape sizes do not multiply out")
+        return dataclasses.replace(v, dims=out)
+
+    def bmm(self, x: View, y: View) -> View:
+        # x [bh, m, k] @ y [bh, k, n]
+        if len(x.dims) != 3 or len(y.dims) != 3:
+            raise Unsupported("bmm of non-3-d operands")
+        ir.unify(x.dims[0], y.dims[0])
+        ir.unify(x.dims[2], y.dims[1])
+        return self.emit("dot", [x.dims[0], x.dims[1], y.dims[2]], [], ir.Dot(x.read(), y.read(), list(x.dims[2])))
+
+    def softmax(self, v: View, dim: int) -> View:
+        """max, exp(x - max), sum, divide: four nests, as the reference decomposes it
+        (ops.py:416-452)."""
+        if dim % len(v.dims) != len(v.dims) - 1:
+            raise Unsupported("softmax over a dim other than the last")
+        x = v.instantiate()
+        outer, red = x.dims[:-1], x.dims[-1]
+        m = self.emit("max", outer, list(red), x.read(), ("max", float("-inf")))
+        # the next nests read x and the row statistics over the same atoms
+        e = self.emit("exp", x.dims, [], ir.Un("exp", ir.Bin("sub", x.read(), m.read())))
+        e_in = e
+        l = self.emit("sum", outer, list(red), e_in.read(), ("add", 0.0))
+        return self.emit("prob", x.dims, [], ir.Bin("div", e_in.read(), l.read()))
+
+
+def parse(gm: torch.fx.GraphModule) -> Parser:
+    return Parser(gm).run()

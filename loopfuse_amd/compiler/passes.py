@@ -1,0 +1,278 @@
+"""Passes over the loop nests (reference ``loopfuse/optimize.py:34-60``).
+
+  fuse             pointwise producer -> consumer inlining (reference compiler/passes/fuse.py
+                   + store/load forwarding of cleanup_passes.py:183-208, as one step: a
+                   temporary written by an ``Assign`` nest is substituted where it is read)
+  online_softmax   the three reductions over the key atoms -- row maximum, sum of exponentials,
+                   probabilities @ V -- become one pass with rescaled accumulators
+                   (reference compiler/passes/factor_acc.py:23-109)
+  block_skip       the mask clauses, evaluated over whole (q tile, kv tile) boxes, give the
+                   range of kv tiles a q tile has to visit
+                   (reference compiler/passes/skip_loop_iterations.py:26-81, 267-378)
+"""
+from __future__ import annotations
+
+import dataclasses
+import math
+from typing import Callable, Optional, Sequence
+
+from . import ir
+from .ir import Atom, Nest
+
+
+class PassError(Exception):
+    pass
+
+
+# ---------------------------------------------------------------- atom renaming
+def _refinement(prod: Sequence[Atom], cons: Sequence[Atom]) -> dict:
+    """Map each leaf of ``prod`` to the consumer leaves that index the same range (the consumer
+    may have split an atom the producer iterates whole)."""
+    ps = [a for a in ir.leaves(prod)]
+    cs = [a for a in ir.leaves(cons)]
+    out: dict = {}
+    ci = 0
+    for p in ps:
+        if p.hint == 1:
+            out[p.id] = []
+            continue
+        got, have = [], 1
+        while have < p.hint:
+            while ci < len(cs) and cs[ci].hint == 1:
+                ci += 1
+            if ci >= len(cs):
+                raise PassError("consumer indexes a smaller range than the producer writes")
+            got.append(cs[ci])
+            have *= cs[ci].hint
+            ci += 1
+        if have != p.hint:
+            raise PassError("consumer atoms do not refine the producer's")
+        out[p.id] = got
+    return out
+
+
+def _rename_atoms(atoms: Sequence[Atom], m: dict) -> list[Atom]:
+    out = []
+    for a in ir.leaves(atoms):
+        out.extend(m.get(a.id, [a]))
+    return out
+
+
+def rename(e: ir.Expr, m: dict) -> ir.Expr:
+    """``e`` with every atom replaced through ``m`` (atom id -> list of atoms)."""
+    def fn(x):
+        if isinstance(x, ir.Read):
+            g = None
+            if x.gather is not None:
+                g = (x.gather[0], x.gather[1], [_rename_atoms(t, m) for t in x.gather[2]])
+            return ir.Read(x.buf, [_rename_atoms(d, m) for d in x.idx], g)
+        if isinstance(x, ir.Select):
+            cl = [ir.Clause(c.ci, c.cj, c.c0, _rename_atoms(c.row, m), _rename_atoms(c.col, m), c.c0_fn) for c in x.clauses]
+            return ir.Select(cl, rename(x.a, m), x.other)
+        if isinstance(x, ir.Dot):
+            return ir.Dot(rename(x.a, m), rename(x.b, m), _rename_atoms(x.over, m))
+        return None
+    return ir.substitute(e, fn)
+
+
+# ---------------------------------------------------------------- fuse
+def fuse(nests: list[Nest], keep: ir.Buffer) -> list[Nest]:
+    """Inline every temporary written by a pointwise (``Assign``) nest into its readers and drop
+    its nest; reductions (``Accum``) and the result buffer stay.  Runs to a fixed point."""
+    nests = list(nests)
+    changed = True
+    while changed:
+        changed = False
+        for prod in nests:
+            if not isinstance(prod.stmt, ir.Assign) or prod.stmt.buf is keep or prod.red:
+                continue
+            buf = prod.stmt.buf
+            users = [n for n in nests if n is not prod and any(r.buf is buf for r in _stmt_reads(n.stmt))]
+            if not users:
+                continue
+
+            def inline(x, buf=buf, prod=prod):
+                if isinstance(x, ir.Read) and x.buf is buf:
+                    m: dict = {}
+                    for pd, cd in zip(buf.dims, x.idx):
+                        m.update(_refinement(pd, cd))
+                    return rename(prod.stmt.value, m)
+                return None
+
+            for u in users:
+                u.stmt.value = ir.substitute(u.stmt.value, inline)
+            nests.remove(prod)
+            changed = True
+            break
+    return nests
+
+
+def _stmt_reads(stmt) -> list[ir.Read]:
+    if isinstance(stmt, ir.Rescaled):
+        return ir.reads(stmt.score) + [stmt.weights]
+    return ir.reads(stmt.value)
+
+
+# ---------------------------------------------------------------- online softmax
+def _same_atoms(a: Sequence[Atom], b: Sequence[Atom]) -> bool:
+    la, lb = [x for x in ir.leaves(a) if x.hint != 1], [x for x in ir.leaves(b) if x.hint != 1]
+    return len(la) == len(lb) and all(x is y for x, y in zip(la, lb))
+
+
+def _struct_eq(a: ir.Expr, b: ir.Expr, m: dict) -> bool:
+    """Structural equality of two expressions up to the atom renaming ``m`` (ids of a's atoms ->
+    atoms of b), which is extended on the way."""
+    if type(a) is not type(b):
+        return False
+    def atoms_eq(x, y):
+        lx, ly = [t for t in ir.leaves(x) if t.hint != 1], [t for t in ir.leaves(y) if t.hint != 1]
+        if len(lx) != len(ly):
+            return False
+        for s, t in zip(lx, ly):
+            if m.setdefault(s.id, t) is not t:
+                return False
+        return True
+    if isinstance(a, ir.Const):
+        return a.value == b.value
+    if isinstance(a, ir.Scalar):
+        return a.text == b.text
+    if isinstance(a, ir.Read):
+        if a.buf is not b.buf or (a.gather is None) != (b.gather is None):
+            return False
+        if a.gather is not None and (a.gather[0] != b.gather[0] or a.gather[1] is not b.gather[1] or
+                                     not all(atoms_eq(x, y) for x, y in zip(a.gather[2], b.gather[2]))):
+            return False
+        return all(atoms_eq(x, y) for x, y in zip(a.idx, b.idx))
+    if isinstance(a, ir.Bin):
+        return a.op == b.op and _struct_eq(a.a, b.a, m) and _struct_eq(a.b, b.b, m)
+    if isinstance(a, ir.Un):
+        return a.op == b.op and _struct_eq(a.a, b.a, m)
+    if isinstance(a, ir.Dot):
+        return atoms_eq(a.over, b.over) and _struct_eq(a.a, b.a, m) and _struct_eq(a.b, b.b, m)
+    if isinstance(a, ir.Select):
+        return (a.other == b.other and len(a.clauses) == len(b.clauses) and
+                all((c.ci, c.cj, c.c0) == (d.ci, d.cj, d.c0) and atoms_eq(c.row, d.row) and atoms_eq(c.col, d.col)
+                    for c, d in zip(a.clauses, b.clauses)) and _struct_eq(a.a, b.a, m))
+    return False
+
+
+def online_softmax(nests: list[Nest], keep: ir.Buffer) -> list[Nest]:
+    """After ``fuse`` an attention graph is three nests over the same rows:
+
+        m[r]    = max_j  x[r, j]                                  (Accum max)
+        l[r]    = sum_j  exp(x[r, j] - m[r])                      (Accum add)
+        o[r, d] = dot_j( exp(x[r, j] - m[r]) / l[r],  v[j, d] )   (Assign of a Dot over j)
+
+    The divisor l[r] does not depend on j, so it moves out of the contraction; what remains of
+    the second and third nest are sums over j of terms that carry the same factor exp(-m[r]).
+    With a running maximum in place of m, growing it from m_old to m_new multiplies every term
+    already summed by exp(m_old - m_new) -- a factor free of j -- so one pass that rescales both
+    accumulators whenever the maximum grows computes the same values (the "online hoist" of the
+    reference, factor_acc.py:23-109).  The pass checks that the three nests have exactly this
+    form, with the same x, and replaces them by one ``Rescaled`` nest."""
+    out_nest = next((n for n in nests if n.writes() is keep), None)
+    if out_nest is None or not isinstance(out_nest.stmt, ir.Assign) or not isinstance(out_nest.stmt.value, ir.Dot):
+        raise PassError("the result is not a contraction")
+    dot = out_nest.stmt.value
+    p, v = dot.a, dot.b
+    # p = exp(x - m[r]) / l[r]
+    if not (isinstance(p, ir.Bin) and p.op == "div" and isinstance(p.b, ir.Read)):
+        raise PassError("left operand of the contraction is not a normalised value")
+    e, l_read = p.a, p.b
+    if not (isinstance(e, ir.Un) and e.op == "exp" and isinstance(e.a, ir.Bin) and e.a.op == "sub" and isinstance(e.a.b, ir.Read)):
+        raise PassError("numerator is not exp(x - m)")
+    x, m_read = e.a.a, e.a.b
+    if not isinstance(v, ir.Read):
+        raise PassError("right operand of the contraction is not a tensor read")
+    l_nest = next((n for n in nests if n.writes() is l_read.buf), None)
+    m_nest = next((n for n in nests if n.writes() is m_read.buf), None)
+    if l_nest is None or m_nest is None or not isinstance(l_nest.stmt, ir.Accum) or not isinstance(m_nest.stmt, ir.Accum):
+        raise PassError("row statistics are not reductions")
+    if l_nest.stmt.op != "add" or m_nest.stmt.op != "max":
+        raise PassError("row statistics are not a sum and a maximum")
+    # l's summand is the numerator, m's operand is x -- over the contraction's own atoms
+    ren: dict = {}
+    if not _struct_eq(l_nest.stmt.value, e, ren) or not _struct_eq(m_nest.stmt.value, x, ren):
+        raise PassError("sum / maximum are not taken of the contraction's own scores")
+    for a, b in ((l_nest.red, dot.over), (m_nest.red, dot.over)):
+        la = [ren.get(t.id, t) for t in ir.leaves(a) if t.hint != 1]
+        if not _same_atoms(la, dot.over):
+            raise PassError("reductions run over different key ranges")
+    # x may not depend on the statistics themselves
+    if any(r.buf in (l_read.buf, m_read.buf) for r in ir.reads(x)):
+        raise PassError("scores depend on their own statistics")
+    new = Nest(out_nest.name, out_nest.par, list(dot.over), ir.Rescaled(keep, x, v))
+    return [n for n in nests if n not in (out_nest, l_nest, m_nest)] + [new]
+
+
+# ---------------------------------------------------------------- block skip
+@dataclasses.dataclass
+class TileBounds:
+    """[start, end) of kv tiles for q tile ``qt``: callables over (qt, Sq, Sk) and their text."""
+
+    start: Callable
+    end: Callable
+    text: str
+
+    def range(self, qt: int, Sq: int, Sk: int, args=None) -> tuple[int, int]:
+        """``args``: the call's flat arguments, for clauses whose constant is a run-time integer of
+        the graph (a window passed as a variable); without them the traced value is used."""
+        b, e = self.start(qt, Sq, Sk, args), self.end(qt, Sq, Sk, args)
+        return b, max(b, e)
+
+
+def _floordiv(a: int, b: int) -> int:
+    return a // b
+
+
+def block_skip(nests: list[Nest], bm: int, bn: int) -> list[Nest]:
+    """Tighten the kv-tile loop of the ``Rescaled`` nest.  A kv tile whose every score is masked
+    leaves the running maximum, the sum and the accumulator unchanged (the masked value is
+    -inf: exp gives 0, max ignores it), so it can be left out (reference
+    skip_loop_iterations.py:318-341).  Whether a clause ci*i + cj*j + c0 <= 0 can hold anywhere
+    in the box i in [i_lo, i_hi], j in [j_lo, j_hi] follows from its minimum over the box
+    (interval arithmetic, reference :26-81); solved for the kv tile index this bounds the loop
+    from above (cj > 0) or from below (cj < 0) (reference :343-376).  Clauses over the same
+    difference i - j, which is all the two mask ops produce, make the conjunction exact."""
+    nest = next((n for n in nests if isinstance(n.stmt, ir.Rescaled)), None)
+    if nest is None:
+        raise PassError("no online-softmax nest to tile")
+    clauses: list[ir.Clause] = []
+    for x in ir.walk(nest.stmt.score):
+        if isinstance(x, ir.Select):
+            if x.other != float("-inf"):
+                raise PassError("masked value is not -inf: skipping would change the result")
+            clauses.extend(x.clauses)
+    uppers, lowers, texts = [], [], []
+    for c in clauses:
+        if c.cj == 0:
+            continue                                     # does not bound the key loop
+        # the row extreme that makes the clause easiest to satisfy
+        def i_ext(qt, Sq, c=c):
+            lo, hi = qt * bm, min(qt * bm + bm, Sq) - 1
+            return lo if c.ci > 0 else hi
+        if c.cj > 0:
+            # min over the box = ci*i_ext + cj*j_lo + c0 <= 0  <=>  kt*bn <= (-c0 - ci*i_ext) / cj
+            uppers.append(lambda qt, Sq, Sk, args, c=c, f=i_ext: _floordiv(_floordiv(-c.const(args) - c.ci * f(qt, Sq), c.cj), bn) + 1)
+            texts.append(f"kt*{bn} <= ({-c.c0} - {c.ci}*i_{'lo' if c.ci > 0 else 'hi'}) // {c.cj}")
+        else:
+            # min = ci*i_ext + cj*j_hi + c0 <= 0  <=>  j_hi >= ceil((ci*i_ext + c0) / -cj) =: L, j_hi = min(kt*bn + bn, Sk) - 1
+            def lower(qt, Sq, Sk, args, c=c, f=i_ext):
+                L = -_floordiv(-(c.ci * f(qt, Sq) + c.const(args)), -c.cj)
+                if L > Sk - 1:
+                    return 1 << 30                        # no key satisfies it: empty range
+                return max(0, _floordiv(L, bn)) if L > 0 else 0
+            lowers.append(lower)
+            texts.append(f"min(kt*{bn}+{bn}, Sk)-1 >= ceil(({c.ci}*i_{'lo' if c.ci > 0 else 'hi'} + {c.c0}) / {-c.cj})")
+
+    def start(qt, Sq, Sk, args=None):
+        return max([0] + [f(qt, Sq, Sk, args) for f in lowers])
+
+    def end(qt, Sq, Sk, args=None):
+        nkt = -(-Sk // bn)
+        if min(qt * bm + bm, Sq) - 1 < qt * bm:
+            return 0
+        return min([nkt] + [f(qt, Sq, Sk, args) for f in uppers])
+
+    nest.stmt.tile = (bm, bn, TileBounds(start, end, " and ".join(texts) or "all"))
+    return nests

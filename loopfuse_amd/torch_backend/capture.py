@@ -241,6 +241,8 @@ class AttentionMatch:
             return 1.0 / AttentionMatch._number(x[1], vals)
         if isinstance(x, tuple) and x[0] == "expr":
             return _eval_scalar(x[1], lambda i: vals[i])
+        if isinstance(x, tuple) and x[0] == "fn":        # a scalar the loop-nest front end derived: callable over the inputs
+            return float(x[1](vals))
         if isinstance(x, tuple) and x[0] == "arg":
             x = vals[x[1]]
         return float(x.item() if isinstance(x, torch.Tensor) else x)

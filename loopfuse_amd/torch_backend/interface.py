@@ -34,7 +34,7 @@ from typing import Any, Callable
 import torch
 from torch._functorch.aot_autograd import aot_module_simplified, make_boxed_func
 
-from .. import lowering
+from .. import compiler, lowering
 from . import capture
 
 log = logging.getLogger("loopfuse_amd")
@@ -49,7 +49,38 @@ USE_HARDCODE_KERNEL = os.environ.get("USE_HARDCODE_KERNEL", "0") == "1"
 # "eager_training" = graph traced with gradients enabled (forward or backward half)
 # "refused_signatures" = argument layouts latched as not servable (see optimized_fn)
 stats = {"fused": 0, "eager_graph": 0, "eager_runtime": 0, "eager_training": 0, "compiled_graphs": 0, "matched_graphs": 0,
-         "refused_signatures": 0}
+         "refused_signatures": 0, "derived_graphs": 0}
+
+
+def _frontend() -> str:
+    """Which front end turns the graph into fused calls: "match" (default) = the sub-graph
+    matcher of capture.py; "ir" = the loop-nest front end (loopfuse_amd/compiler: per-op nests,
+    fusion, online-softmax and block-skip passes, plan read off the fused nest), with the matcher
+    as fallback for graphs it does not cover; "check" = the matcher, cross-checked against the
+    loop-nest front end wherever that derives a plan."""
+    return os.environ.get("LOOPFUSE_FRONTEND", "match")
+
+
+def match_from_nests(gm: torch.fx.GraphModule, comp: "compiler.pipeline.Compiled") -> capture.AttentionMatch:
+    """The attention the loop-nest front end derived, in the form the fused call takes."""
+    att = comp.attention
+    placeholders = [n for n in gm.graph.nodes if n.op == "placeholder"]
+    out_node = next(n for n in gm.graph.nodes if n.op == "output").args[0]
+    out_node = out_node[0] if isinstance(out_node, (tuple, list)) else out_node
+
+    def operand(o) -> capture.Operand:
+        return capture.Operand(o.placeholder, tuple(o.perm), o.paged, o.table, o.group)
+
+    def factor(f):
+        kind, x = f
+        x = ("fn", x) if callable(x) else float(x)
+        return ("recip", x) if kind == "div" else x
+
+    return capture.AttentionMatch(out_node=out_node, inputs=placeholders, q=operand(att.q), k=operand(att.k),
+                                  v=operand(att.v), factors=[factor(f) for f in att.pre],
+                                  post_factors=[factor(f) for f in att.post], has_tanh=att.has_tanh,
+                                  mask=att.mask, window=("fn", att.window) if callable(att.window) else att.window,
+                                  out_rank=4)
 
 
 def _strict() -> bool:
@@ -152,13 +183,41 @@ def loopfuse_compiler(gm: torch.fx.GraphModule, sample_inputs, input_names: list
     if DEBUG:
         print("---- loopfuse_amd: ATen graph ----")
         print(gm.code)
-    try:
-        matches = capture.match_attention(gm)
-    except capture.NoMatch as e:
-        matches = []
-        reason = str(e)
+    frontend = _frontend()
+    derived = None
+    if frontend in ("ir", "check") or DEBUG:
+        try:
+            derived = compiler.compile_graph(gm)
+        except compiler.NotDerivable as e:
+            log.info("loop-nest front end: %s", e)
+            if DEBUG:
+                print(f"---- loopfuse_amd: loop-nest front end does not cover this graph ({e})")
+        else:
+            stats["derived_graphs"] += 1
+            if DEBUG:
+                print("---- loopfuse_amd: loop nests ----")
+                print(derived.before)
+                print("---- loopfuse_amd: after fuse / online-softmax / block-skip ----")
+                print(derived.after)
+                print("---- loopfuse_amd: derived:", derived.attention.describe())
+    if frontend == "ir" and derived is not None:
+        matches, reason = [match_from_nests(gm, derived)], ""
     else:
-        reason = ""
+        try:
+            matches = capture.match_attention(gm)
+        except capture.NoMatch as e:
+            matches = []
+            reason = str(e)
+        else:
+            reason = ""
+        if frontend == "check" and derived is not None:
+            a = derived.attention
+            same = (len(matches) == 1 and matches[0].mask == a.mask and matches[0].has_tanh == a.has_tanh
+                    and matches[0].k.paged == a.k.paged and matches[0].v.paged == a.v.paged
+                    and (a.mask != "sliding" or callable(a.window) or matches[0].window == a.window))
+            if not same:
+                raise AssertionError("loopfuse_amd: the two front ends disagree: matcher "
+                                     f"{[m.describe() for m in matches]} vs loop nests {a.describe()}")
     if not matches:
         if _strict():
             raise NotImplementedError(f"loopfuse_amd: no fused-attention pattern in the graph: {reason}")

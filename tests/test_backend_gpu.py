@@ -682,3 +682,49 @@ def test_unlowered_graphs_still_correct(which):
     got = torch.compile(fn, backend=loopfuse_backend, dynamic=True)(*dev_ins)
     tol = 1e-2 if which == "simplified_attn" else 1e-4      # the reference checks that case at rtol 1e-2 too
     torch.testing.assert_close(got.double().cpu(), want, rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize("name", ["c2", "c2_softcap", "c3", "c4", "c5"])
+def test_loop_nest_front_end_on_the_gpu(name, monkeypatch):
+    """LOOPFUSE_FRONTEND=ir: the benchmark configurations' graphs go through the loop-nest front
+    end (per-op nests -> fuse -> online softmax -> block skip -> derived plan) to the HIP kernels
+    and match the oracle."""
+    from loopfuse_amd import workloads
+
+    monkeypatch.setenv("LOOPFUSE_FRONTEND", "ir")
+
+    def mods(s, cap):
+        return s if cap is None else torch.tanh(s / cap) * cap
+
+    def dense(cap, mask, window):
+        def fn(q, k, v):
+            g = q.shape[1] // k.shape[1]
+            if g > 1:
+                k, v = k.repeat_interleave(g, dim=1), v.repeat_interleave(g, dim=1)
+            s = mods(q @ k.transpose(-2, -1) * (q.shape[-1] ** -0.5), cap)
+            if mask == "causal":
+                s = torch.ops.loopfuse.causal_mask(s)
+            elif mask == "sliding":
+                s = torch.ops.loopfuse.sliding_mask(s, window)
+            return torch.softmax(s, dim=-1) @ v
+        return fn
+
+    def paged(Q, Kc, kt, Vc, vt):
+        B, pages = kt.shape
+        P, H, D = Kc.shape[1:]
+        K = torch.ops.loopfuse.paged_load(Kc, kt).reshape(B, pages * P, H, D).transpose(-3, -2)
+        V = torch.ops.loopfuse.paged_load(Vc, vt).reshape(B, pages * P, H, D).transpose(-3, -2)
+        return torch.softmax(Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5), dim=-1) @ V
+
+    w = workloads.make(name, seed=11, B=2, S=640 if name in ("c2", "c2_softcap", "c3") else 1024)
+    before = interface.stats["derived_graphs"]
+    if name == "c5":
+        B, Hq, _, D = w.q.shape
+        Hkv = w.k.shape[2]
+        got = run_fused(paged, (w.q.view(B, Hkv, Hq // Hkv, D), w.k, w.k_table, w.v, w.v_table)).view(B, Hq, 1, D)
+    else:
+        got = run_fused(dense(w.softcap, w.mask, w.window), (w.q, w.k, w.v))
+    assert interface.stats["derived_graphs"] == before + 1, "the loop-nest front end did not derive this graph"
+    want = O.attention_reference(w.q, w.k, w.v, mask=w.mask, window=w.window, softcap=w.softcap,
+                                 k_table=w.k_table, v_table=w.v_table)
+    assert (got - want).abs().max() <= TOL
