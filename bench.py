@@ -249,6 +249,8 @@ def main() -> int:
     ap.add_argument("--torch-sdpa", action="store_true",
                     help="also time torch.nn.functional.scaled_dot_product_attention on the same GPU and inputs "
                          "(config 2 as is; the decode config with its pages gathered into contiguous K/V beforehand)")
+    ap.add_argument("--no-settled", action="store_true",
+                    help="skip the steady-state conditioning legs (for counter runs under rocprofv3, where every launch is slow)")
     ap.add_argument("--no-via-backend", action="store_true",
                     help="skip the legs that time the two headline workloads through torch.compile(backend=loopfuse_backend)")
     ap.add_argument("--mfma-ceiling", action="store_true",
@@ -285,7 +287,7 @@ def main() -> int:
         w = workloads.make(args.workload, seed=0).to(dev)
         o = workloads.run(w)     # first call compiles / loads the code object
         torch.cuda.synchronize()
-        settled = time_settled(lambda i: workloads.run(w, out=o))
+        settled = None if args.no_settled else time_settled(lambda i: workloads.run(w, out=o))
         t, wall = time_gpu(lambda i: workloads.run(w, out=o), args.steps, args.warmup)
         pre = {"workload": args.workload, "sec": t, "wall_sec": wall, "flops": w.flops(), "settled": settled,
                "kernels": lowering.attention.last_launch["kernels"]}
@@ -302,7 +304,7 @@ def main() -> int:
             ws.append(dataclasses.replace(ws[0], k=ws[0].k.clone(), v=ws[0].v.clone()))
         o = workloads.run(ws[0])
         torch.cuda.synchronize()
-        dsettled = time_settled(lambda i: workloads.run(ws[i % nrot], out=o))
+        dsettled = None if args.no_settled else time_settled(lambda i: workloads.run(ws[i % nrot], out=o))
         t, wall = time_gpu(lambda i: workloads.run(ws[i % nrot], out=o), args.steps, args.warmup)
         dec = {"workload": args.decode_workload, "sec": t, "wall_sec": wall, "bytes": base.kv_bytes(), "rotation": nrot,
                "settled": dsettled, "kernels": lowering.attention.last_launch["kernels"]}
@@ -323,9 +325,10 @@ def main() -> int:
                            "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": TRAFFIC_BYTES.get(args.workload),
                            "kernel": "+".join(pre["kernels"]), "us_per_launch": pre["sec"] * 1e6}
         st = pre["settled"]
-        out["settled"] = {"value": pre["flops"] / st["us_per_launch"] / 1e6, "unit": "TFLOP/s",
-                          "frac": pre["flops"] / st["us_per_launch"] / 1e6 / MFMA_BF16_PEAK_TFLOPS, **st,
-                          "protocol": "about 25 ms of untimed launches, then about 100 ms of timed ones (the reference's do_bench)"}
+        if st is not None:
+            out["settled"] = {"value": pre["flops"] / st["us_per_launch"] / 1e6, "unit": "TFLOP/s",
+                              "frac": pre["flops"] / st["us_per_launch"] / 1e6 / MFMA_BF16_PEAK_TFLOPS, **st,
+                              "protocol": "about 25 ms of untimed launches, then about 100 ms of timed ones (the reference's do_bench)"}
     if dec is not None:
         gbs = dec["bytes"] / dec["sec"] / 1e9
         kgbs = dec["bytes"] / dec["kernel_sec"] / 1e9
@@ -336,8 +339,9 @@ def main() -> int:
              "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                           "frac": gbs / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES.get(args.decode_workload),
                           "kernel": "+".join(dec["kernels"]), "us_per_launch": dec["sec"] * 1e6},
-             "settled": {"value": dec["bytes"] / dec["settled"]["us_per_launch"] / 1e3, "unit": "GB/s",
-                         "frac": dec["bytes"] / dec["settled"]["us_per_launch"] / 1e3 / HBM_PEAK_GBS, **dec["settled"]},
+             "settled": None if dec["settled"] is None else
+             {"value": dec["bytes"] / dec["settled"]["us_per_launch"] / 1e3, "unit": "GB/s",
+              "frac": dec["bytes"] / dec["settled"]["us_per_launch"] / 1e3 / HBM_PEAK_GBS, **dec["settled"]},
              "stream_kernel_alone": {"kernel": "+".join(dec["stream_kernels"]), "us_per_launch": dec["kernel_sec"] * 1e6,
                                      "gbs": kgbs, "note": "partials left unmerged, O not written"}}
         if pre is None:
@@ -353,7 +357,7 @@ def main() -> int:
                    "decode_workload": "config 5: paged GQA decode bf16 B64 Hq32/Hkv8 K_len2048 D128 page16"
                    if args.decode_workload == "c5" else args.decode_workload},
     })
-    if not args.no_via_backend and args.only is None and args.workload == "c2" and args.decode_workload == "c5":
+    if not args.no_via_backend and not args.no_settled and args.only is None and args.workload == "c2" and args.decode_workload == "c5":
         out["via_backend"] = via_backend(dev, args.steps, args.warmup)
     if args.mfma_ceiling:
         out["mfma_ceiling"] = mfma_ceiling(dev)
