@@ -150,7 +150,13 @@ class Parser:
             fa = val(a[0])[1] if isinstance(a[0], torch.fx.Node) else (lambda args, c=int(a[0]): c)
             fb = val(a[1])[1] if isinstance(a[1], torch.fx.Node) else (lambda args, c=int(a[1]): c)
             sym = {operator.mul: "*", operator.floordiv: "//", operator.add: "+", operator.sub: "-"}[t]
-            return ("size", (lambda args, f=t, x=fa, y=fb: f(x(args), y(args))), f"({sa}{sym}{sb})", t(ha, hb))
+            fn = None if (fa is None or fb is None) else (lambda args, f=t, x=fa, y=fb: f(x(args), y(args)))
+            return ("size", fn, f"({sa}{sym}{sb})", t(ha, hb))
+        if t is aten.sym_size.int:
+            # extent of a view dimension: only its traced value and text are needed (dims are atoms)
+            v = val(a[0])
+            d = v.dims[a[1] % len(v.dims)]
+            return ("size", None, "*".join(x.size for x in ir.leaves(d)) or "1", math.prod(x.hint for x in ir.leaves(d)) if d else 1)
         # ---- 0-dim values computed from sizes (D ** -0.5 and the like)
         if t is aten.scalar_tensor.default:
             x = a[0]
@@ -207,6 +213,41 @@ class Parser:
         # ---- compute ops
         if t is aten.bmm.default:
             return self.bmm(val(a[0]).instantiate(), val(a[1]).instantiate())
+        if t in (aten.add.Tensor, aten.sub.Tensor, aten.mul.Tensor, aten.div.Tensor) and \
+                isinstance(val(a[0]), View) and isinstance(val(a[1]), View):
+            return self.pointwise2({aten.add.Tensor: "add", aten.sub.Tensor: "sub", aten.mul.Tensor: "mul",
+                                    aten.div.Tensor: "div"}[t], val(a[0]).instantiate(), val(a[1]).instantiate())
+        if t in (aten.add.Tensor, aten.sub.Tensor) and isinstance(val(a[0]), View):
+            y = val(a[1])
+            const: ir.Expr = ir.Scalar(y[1], y[2]) if isinstance(y, tuple) else ir.Const(float(y))
+            v = val(a[0]).instantiate()
+            return self.emit("add", v.dims, [], ir.Bin("add" if t is aten.add.Tensor else "sub", v.read(), const))
+        if t is aten.mm.default:
+            x, y = val(a[0]).instantiate(), val(a[1]).instantiate()
+            ir.unify(x.dims[1], y.dims[0])
+            return self.emit("dot", [x.dims[0], y.dims[1]], [], ir.Dot(x.read(), y.read(), list(x.dims[1])))
+        if t is aten.addmm.default:
+            x, y = val(a[1]).instantiate(), val(a[2]).instantiate()
+            ir.unify(x.dims[1], y.dims[0])
+            prod = self.emit("dot", [x.dims[0], y.dims[1]], [], ir.Dot(x.read(), y.read(), list(x.dims[1])))
+            return self.pointwise2("add", val(a[0]).instantiate(), prod.instantiate())
+        if t is aten.exp.default:
+            v = val(a[0]).instantiate()
+            return self.emit("exp", v.dims, [], ir.Un("exp", v.read()))
+        if t in (aten.max.dim, aten.sum.dim_IntList, aten.amax.default):
+            v = val(a[0]).instantiate()
+            dims = a[1] if isinstance(a[1], (list, tuple)) else [a[1]]
+            dims = [d % len(v.dims) for d in dims]
+            keep = bool(a[2]) if len(a) > 2 else bool(n.kwargs.get("keepdim", False))
+            red = [x for d in dims for x in v.dims[d]]
+            outer = [([] if k in dims else v.dims[k]) for k in range(len(v.dims)) if keep or k not in dims]
+            op = ("add", 0.0) if t is aten.sum.dim_IntList else ("max", float("-inf"))
+            r = self.emit("sum" if op[0] == "add" else "max", outer, red, v.read(), op)
+            return ("tuple", r) if t is aten.max.dim else r
+        if t is operator.getitem and isinstance(val(a[0]), tuple) and val(a[0])[0] == "tuple":
+            if a[1] != 0:
+                raise Unsupported("indices of max are not lowered")
+            return val(a[0])[1]
         if t in (aten.mul.Tensor, aten.div.Tensor):
             x, y = val(a[0]), val(a[1])
             if isinstance(x, View) and not isinstance(y, View):
@@ -269,6 +310,23 @@ class Parser:
         if any(x.hint != 1 for x in flat):
             raise Unsupported("reshape sizes do not multiply out")
         return dataclasses.replace(v, dims=out)
+
+    def pointwise2(self, op: str, x: View, y: View) -> View:
+        """x op y with broadcasting: dims are aligned from the right; where both sides have an extent
+        their index ranges are unified, where one side has none (size 1 / missing) the other's is taken."""
+        n = max(len(x.dims), len(y.dims))
+        xd = [[] for _ in range(n - len(x.dims))] + [list(d) for d in x.dims]
+        yd = [[] for _ in range(n - len(y.dims))] + [list(d) for d in y.dims]
+        out = []
+        for a, b in zip(xd, yd):
+            ha = math.prod(t.hint for t in ir.leaves(a)) if a else 1
+            hb = math.prod(t.hint for t in ir.leaves(b)) if b else 1
+            if ha != 1 and hb != 1:
+                ir.unify(a, b)
+                out.append(a)
+            else:
+                out.append(a if ha != 1 else b)
+        return self.emit(op, out, [], ir.Bin(op, x.read(), y.read()))
 
     def bmm(self, x: View, y: View) -> View:
         # x [bh, m, k] @ y [bh, k, n]

@@ -1,0 +1,148 @@
+"""Run-time side of the generic lowering: compile the emitted kernels with hipRTC through the C
+ABI, solve the run-time extents of the atoms from the argument shapes, allocate temporaries and
+launch (the counterpart of the reference's generated ``launch_kernel_0``,
+``loopfuse/codegen.py:215-298``)."""
+from __future__ import annotations
+
+import ctypes
+import math
+from typing import Sequence
+
+import torch
+
+from . import build, emit, ir, passes
+from .emit import NotLowerable
+
+
+# One thread per output element with sequential inner loops is meant for the small graphs around
+# an attention (epilogues, table look-ups, normalisations); beyond this many inner-loop steps per
+# call the graph is left to the captured ATen ops (rocBLAS for its matmuls).
+MAX_SCALAR_WORK = 1 << 33
+
+
+class GenericProgram:
+    def __init__(self, gm: torch.fx.GraphModule):
+        try:
+            p = build.parse(gm)
+            nests = passes.fuse(p.nests, p.out.buf, keep_contractions=True)
+        except (build.Unsupported, passes.PassError, ValueError) as e:
+            raise NotLowerable(str(e)) from e
+        if any(isinstance(n.stmt, ir.Rescaled) for n in nests):
+            raise NotLowerable("attention nest")
+        self.parsed, self.nests = p, nests
+        out_val = next(n for n in gm.graph.nodes if n.op == "output").args[0]
+        out_val = out_val[0] if isinstance(out_val, (tuple, list)) else out_val
+        self.out_dtype = out_val.meta["val"].dtype
+        # the graph's result must be the last nest's buffer, its dims regrouped in place
+        flat_buf = [a for d in p.out.buf.dims for a in ir.leaves(d) if a.hint != 1]
+        flat_view = [a for d in p.out.dims for a in ir.leaves(d) if a.hint != 1]
+        if len(flat_buf) != len(flat_view) or any(x is not y for x, y in zip(flat_buf, flat_view)):
+            raise NotLowerable("the result is a permuted or broadcast view of what the last nest writes")
+        self.dtypes = {b.name: emit._DT.get(getattr(torch, b.dtype, None), None) for b in p.inputs}
+        if any(v is None for v in self.dtypes.values()):
+            raise NotLowerable("an input dtype the emitted kernels do not read")
+        for n in nests:
+            self.dtypes.setdefault(n.writes().name, 0)               # temporaries are fp32
+        self.dtypes[p.out.buf.name] = emit._DT.get(self.out_dtype, 0)
+        self.kernels = [emit.Emitter(n, self.dtypes, f"lf_gen_{i}").emit() for i, n in enumerate(nests)]
+        self.source = emit.PRELUDE + "\n".join(k.source for k in self.kernels)
+        self._loaded: dict = {}
+
+    @property
+    def code(self) -> str:
+        return self.source
+
+    def _module(self):
+        from .. import lowering, runtime
+        dev = torch.cuda.current_device()
+        if dev not in self._loaded:
+            code, _, _ = runtime.compile_source(self.source, "lf_generic", list(lowering.COMMON_OPTS))
+            mod = runtime.Module(code)
+            self._loaded[dev] = [mod.kernel(k.name) for k in self.kernels]
+        return self._loaded[dev]
+
+    def _solve(self, nest: ir.Nest, bufs: dict, known: dict, syms: dict) -> None:
+        """Run-time extent of every leaf atom of ``nest`` into ``known``: each dimension of a
+        buffer it reads (an argument, or a temporary an earlier nest wrote) is the product of the
+        atoms that index it; atoms that index a dimension whole give values, the rest follows by
+        division (fixed point).  Two atoms whose size is the same symbol of the traced graph
+        (``s74``) have the same extent, whichever nest they belong to: ``syms`` carries those."""
+        eqs = []
+        every = [a for a in ir.leaves(nest.par) + ir.leaves(nest.red)]
+        for e in ir.walk(nest.stmt.value):
+            if isinstance(e, ir.Dot):
+                every += ir.leaves(e.over)
+        for a in every:
+            if a.id not in known and a.hint != 1:
+                if a.size.isdigit():
+                    known[a.id] = int(a.size)
+                elif a.size in syms:
+                    known[a.id] = syms[a.size]
+        for r in ir.reads(nest.stmt.value):
+            t = bufs[r.buf.name]
+            for d, atoms in enumerate(r.idx):
+                if r.gather is not None and r.gather[0] == d:
+                    continue
+                eqs.append(([a for a in ir.leaves(atoms) if not a.broadcast], int(t.shape[d])))
+            if r.gather is not None:
+                tt = bufs[r.gather[1].name]
+                for d, atoms in enumerate(r.gather[2]):
+                    eqs.append((list(ir.leaves(atoms)), int(tt.shape[d])))
+        progress = True
+        while progress:
+            progress = False
+            for atoms, size in eqs:
+                unknown = [a for a in atoms if a.id not in known and a.hint != 1]
+                have = math.prod(known[a.id] for a in atoms if a.id in known)
+                if len(unknown) == 1 and have and size % have == 0:
+                    known[unknown[0].id] = size // have
+                    syms.setdefault(unknown[0].size, size // have)
+                    progress = True
+
+    def run(self, args: Sequence, launchers=None):
+        """One pass over the nests.  ``launchers`` (one callable(blocks, params) per kernel)
+        replaces the HIP launch -- the CPU tests pass a host build of the same source."""
+        tensors = [a for a in args if isinstance(a, torch.Tensor) and a.dim() > 0]
+        if not tensors:
+            raise NotLowerable("no tensor argument")
+        dev = tensors[0].device
+        if any(t.device != dev for t in tensors):
+            raise NotLowerable("arguments on different devices")
+        if launchers is None:
+            if dev.type != "cuda":
+                raise NotLowerable("tensors are not on the GPU")
+            kernels = self._module()
+            launchers = [lambda blocks, prm, fn=fn: fn.launch((blocks, 1, 1), (256, 1, 1), prm) for fn in kernels]
+        ext: dict = {}
+        syms: dict = {name: int(args[i]) for name, i in self.parsed.sizes.items()}
+        work = 0
+        bufs: dict = {b.name: args[b.placeholder] for b in self.parsed.inputs}
+        for nest, k, fn in zip(self.nests, self.kernels, launchers):
+            out = nest.writes()
+            self._solve(nest, bufs, ext, syms)
+            try:
+                shape = [math.prod(1 if a.hint == 1 else ext[a.id] for a in ir.leaves(d)) for d in out.dims]
+            except KeyError as e:
+                raise NotLowerable("an extent could not be derived from the argument shapes") from e
+            dt = self.out_dtype if out is self.parsed.out.buf else torch.float32
+            bufs[out.name] = torch.empty(shape, dtype=dt, device=dev)
+            prm = emit.GenParams()
+            for i, b in enumerate(k.bufs):
+                prm.ptr[i] = bufs[b.name].data_ptr()
+            for i, a in enumerate(k.atoms):
+                prm.n[i] = ext[a.id]
+            for i, (b, d) in enumerate(k.strides):
+                prm.n[len(k.atoms) + i] = bufs[b.name].stride(d)
+            for i, s in enumerate(k.scalars):
+                prm.f[i] = float(s.fn(args))
+            total = math.prod(ext[a.id] for a in k.par)
+            work += total * math.prod(ext[a.id] for a in k.atoms if not any(a is x for x in k.par))
+            if work > MAX_SCALAR_WORK:
+                raise NotLowerable("more scalar work than the plain kernels are meant for")
+            if total:
+                if (total + 255) // 256 >= 1 << 31:
+                    raise NotLowerable("more output elements than one grid dimension holds")
+                fn((total + 255) // 256, prm)
+        res = bufs[self.parsed.out.buf.name]
+        view = [math.prod(1 if a.hint == 1 else ext[a.id] for a in ir.leaves(d)) for d in self.parsed.out.dims]
+        return res.view(view)

@@ -76,9 +76,22 @@ def rename(e: ir.Expr, m: dict) -> ir.Expr:
 
 
 # ---------------------------------------------------------------- fuse
-def fuse(nests: list[Nest], keep: ir.Buffer) -> list[Nest]:
+def _under_dot(e: ir.Expr, buf: ir.Buffer, inside: bool = False) -> bool:
+    """Whether ``buf`` is read inside a contraction of ``e``."""
+    if isinstance(e, ir.Read):
+        return inside and e.buf is buf
+    return any(_under_dot(c, buf, inside or isinstance(e, ir.Dot)) for c in e.children())
+
+
+def fuse(nests: list[Nest], keep: ir.Buffer, keep_contractions: bool = False) -> list[Nest]:
     """Inline every temporary written by a pointwise (``Assign``) nest into its readers and drop
-    its nest; reductions (``Accum``) and the result buffer stay.  Runs to a fixed point."""
+    its nest; reductions (``Accum``) and the result buffer stay.  Runs to a fixed point.
+
+    ``keep_contractions``: a producer that holds a contraction is inlined only into a single
+    pointwise reader (the epilogue of a matmul); where it would be recomputed per element of
+    another contraction or reduction, or by several readers, it stays a temporary.  The
+    attention pipeline inlines everything (its kernels keep the score tile on chip); the plain
+    one-thread-per-element kernels would repeat the contraction instead."""
     nests = list(nests)
     changed = True
     while changed:
@@ -90,6 +103,10 @@ def fuse(nests: list[Nest], keep: ir.Buffer) -> list[Nest]:
             users = [n for n in nests if n is not prod and any(r.buf is buf for r in _stmt_reads(n.stmt))]
             if not users:
                 continue
+            if keep_contractions and any(isinstance(x, ir.Dot) for x in ir.walk(prod.stmt.value)):
+                u = users[0]
+                if len(users) > 1 or not isinstance(u.stmt, ir.Assign) or _under_dot(u.stmt.value, buf):
+                    continue
 
             def inline(x, buf=buf, prod=prod):
                 if isinstance(x, ir.Read) and x.buf is buf:

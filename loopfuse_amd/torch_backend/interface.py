@@ -49,7 +49,7 @@ USE_HARDCODE_KERNEL = os.environ.get("USE_HARDCODE_KERNEL", "0") == "1"
 # "eager_training" = graph traced with gradients enabled (forward or backward half)
 # "refused_signatures" = argument layouts latched as not servable (see optimized_fn)
 stats = {"fused": 0, "eager_graph": 0, "eager_runtime": 0, "eager_training": 0, "compiled_graphs": 0, "matched_graphs": 0,
-         "refused_signatures": 0, "derived_graphs": 0}
+         "refused_signatures": 0, "derived_graphs": 0, "generic_graphs": 0, "fused_generic": 0}
 
 
 def _frontend() -> str:
@@ -175,6 +175,51 @@ def rewrite_graph(gm: torch.fx.GraphModule, matches: list) -> torch.fx.GraphModu
     return fused
 
 
+def _generic_program(gm: torch.fx.GraphModule):
+    """A graph without an attention in it: its loop nests, fused, as one plain HIP kernel per
+    nest (loopfuse_amd/compiler/generic.py) -- what the reference's code generator does for every
+    graph (loopfuse/codegen.py:100-404).  None when the nest builder does not cover the graph or
+    ``LOOPFUSE_GENERIC=0``; then the graph runs as captured."""
+    if os.environ.get("LOOPFUSE_GENERIC", "1") != "1":
+        return None
+    from ..compiler import generic
+    try:
+        prog = generic.GenericProgram(gm)
+    except generic.NotLowerable as e:
+        log.info("generic lowering does not cover this graph: %s", e)
+        return None
+    except Exception as e:                                    # a front-end bug must not take the graph down
+        log.warning("generic lowering failed on this graph (%s: %s); it runs as captured", type(e).__name__, e)
+        return None
+    stats["generic_graphs"] += 1
+    if DEBUG:
+        print("---- loopfuse_amd: no attention in the graph; fused nests ----")
+        print(compiler.ir.show(prog.nests))
+        print(prog.source)
+    out_node = next(n for n in gm.graph.nodes if n.op == "output")
+    as_tuple = isinstance(out_node.args[0], (tuple, list))
+    if CODEGEN_ONLY:
+        return lambda *args: [prog] if as_tuple else prog
+    refused: list = []
+
+    def generic_fn(*args):
+        if not refused:
+            try:
+                out = prog.run(args)
+            except generic.NotLowerable as e:
+                if _strict():
+                    raise
+                refused.append(str(e))
+                log.warning("generic kernels not applicable to this call (%s); the graph runs as captured", e)
+            else:
+                stats["fused_generic"] += 1
+                return (out,) if as_tuple else out
+        stats["eager_runtime"] += 1
+        return gm(*args)
+
+    return generic_fn
+
+
 def loopfuse_compiler(gm: torch.fx.GraphModule, sample_inputs, input_names: list[str] | None = None,
                       symint_names: dict[str, str] | None = None, mode: str | None = None) -> Callable:
     """fw_compiler: ATen graph -> callable over the flat placeholder list."""
@@ -221,6 +266,9 @@ def loopfuse_compiler(gm: torch.fx.GraphModule, sample_inputs, input_names: list
     if not matches:
         if _strict():
             raise NotImplementedError(f"loopfuse_amd: no fused-attention pattern in the graph: {reason}")
+        generic = _generic_program(gm)
+        if generic is not None:
+            return generic
         log.info("graph not recognised (%s); running it unfused", reason)
         if DEBUG:
             print(f"---- loopfuse_amd: no match ({reason}); eager graph ----")
@@ -273,11 +321,22 @@ def loopfuse_compiler(gm: torch.fx.GraphModule, sample_inputs, input_names: list
         return tuple((a.dtype, tuple(a.shape), a.stride(), a.data_ptr() % 16, a.device) if isinstance(a, torch.Tensor) else a
                      for a in args)
 
+    # where the attention kernels refuse a call (fp32 operands, a head dimension they are not
+    # built for), the graph's plain generated kernels serve it if they can, else the captured ops
+    unfused: list = []
+
+    def run_unfused(args):
+        if not unfused:
+            unfused.append(_generic_program(gm) or None)
+        if unfused[0] is not None:
+            return unfused[0](*args)
+        stats["eager_runtime"] += 1
+        return gm(*args)
+
     def optimized_fn(*args):
         sig = signature(args) if refused else None
         if sig is not None and sig in refused:
-            stats["eager_runtime"] += 1
-            return gm(*args)
+            return run_unfused(args)
         try:
             out = fused_gm(*args)
         except lowering.UnsupportedPlan as e:
@@ -289,8 +348,7 @@ def loopfuse_compiler(gm: torch.fx.GraphModule, sample_inputs, input_names: list
             stats["refused_signatures"] += 1
             log.warning("fused path not applicable to this call (%s); calls with these argument layouts run "
                         "the graph unfused", e)
-            stats["eager_runtime"] += 1
-            return gm(*args)
+            return run_unfused(args)
         stats["fused"] += 1
         return out
 

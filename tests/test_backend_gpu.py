@@ -617,12 +617,13 @@ def _softmax64(x):
 
 @pytest.mark.parametrize("which", ["add", "add_2dim", "matmul_add", "matmul_add_3dim", "modified_attn", "softmax_matmul",
                                    "paged_add", "simplified_attn"])
-def test_unlowered_graphs_still_correct(which):
-    """Reference tests/test_accuracy.py:29-82, 172-211, 233-250, 314-333: graphs that are not
-    attention-shaped for this backend (no kernel is lowered for them: they run as captured),
-    plus the modified-attention graph.  Each result is checked against an independent float64
-    computation on the CPU, spelled differently from the compiled function (einsum / explicit
-    exponentials / index loops), not against the same graph run eagerly."""
+def test_graphs_without_attention_run_as_generated_kernels(which):
+    """Reference tests/test_accuracy.py:29-82, 172-211, 233-250, 314-333: graphs with no attention
+    in them (lowered nest by nest to plain generated HIP kernels), plus the modified-attention
+    graph in fp32 (the MFMA kernels take bf16 / fp16 only and refuse it; its generated kernels
+    serve the call).  Each result is checked against an independent
+    float64 computation on the CPU, spelled differently from the compiled function (einsum /
+    explicit exponentials / index loops), not against the same graph run eagerly."""
     f64 = lambda ts: [t.double() if t.is_floating_point() else t for t in ts]
     if which == "add":
         fn = lambda a, b: a + b
@@ -679,9 +680,32 @@ def test_unlowered_graphs_still_correct(which):
     torch._dynamo.reset()
     dev_ins = [t.to(DEV) for t in ins]
     want = ref(*f64(ins))
+    before = dict(interface.stats)
     got = torch.compile(fn, backend=loopfuse_backend, dynamic=True)(*dev_ins)
     tol = 1e-2 if which == "simplified_attn" else 1e-4      # the reference checks that case at rtol 1e-2 too
     torch.testing.assert_close(got.double().cpu(), want, rtol=tol, atol=tol)
+    ran = {k: interface.stats[k] - before[k] for k in ("fused", "fused_generic", "eager_graph", "eager_runtime")}
+    assert ran == {"fused": 0, "fused_generic": 1, "eager_graph": 0, "eager_runtime": 0}, ran
+
+
+def test_generated_kernels_read_bf16_and_follow_new_shapes():
+    """The generated kernels convert on load / store (bf16 in and out, fp32 arithmetic) and take
+    every extent and stride as a run-time argument: one compiled graph serves a second shape and
+    a transposed operand."""
+    fn = lambda a, b, c: a @ b + c
+    torch._dynamo.reset()
+    compiled = torch.compile(fn, backend=loopfuse_backend, dynamic=True)
+    before = dict(interface.stats)
+    for seed, (m, k, n), t in ((1, (64, 32, 48), False), (2, (80, 40, 24), False), (3, (80, 40, 24), True)):
+        a = rand((m, k), torch.bfloat16, seed).to(DEV)
+        b = (rand((n, k), torch.bfloat16, seed + 10).to(DEV).t() if t else rand((k, n), torch.bfloat16, seed + 10).to(DEV))
+        c = rand((m, n), torch.bfloat16, seed + 20).to(DEV)
+        got = compiled(a, b, c)
+        assert got.dtype == torch.bfloat16
+        want = torch.einsum("ik,kj->ij", a.double().cpu(), b.double().cpu()) + c.double().cpu()
+        torch.testing.assert_close(got.double().cpu(), want, rtol=2e-2, atol=2e-2)
+    assert interface.stats["fused_generic"] == before["fused_generic"] + 3
+    assert interface.stats["eager_runtime"] == before["eager_runtime"]
 
 
 @pytest.mark.parametrize("name", ["c2", "c2_softcap", "c3", "c4", "c5"])
