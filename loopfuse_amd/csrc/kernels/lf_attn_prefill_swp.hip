@@ -63,8 +63,9 @@
 // reads in flight (the compiler's own barrier would wait for those too)
 #define LF_BARRIER_VM0() asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory")
 
-// slots per XCD class: (batch, head) pairs of the class, padded to groups of 4, times q-tile pairs
-#define LF_NSLOTS(p, npair) ((((p.B * (p.Hq / LF_HEADS_PER_WG) + 7) / 8 + 3) / 4 * 4) * (npair))
+#ifndef LF_QGROUP
+#define LF_QGROUP 8      /* (batch, head) pairs per group of slots */
+#endif
 
 extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_swp(const LfAttnParams p) {
   __shared__ __attribute__((aligned(16))) lf_elem lds_k[LF_KSLOTS][LF_BN * LF_D];
@@ -76,20 +77,23 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
   const int l32 = lane & 31;
   const int g = lane >> 5;
 
-  // ---- workgroup -> (batch*head, pair of q tiles), as in lf_attn_prefill.hip
+  // ---- workgroup -> (batch*head, q tile).  blockIdx.x % 8 is the XCD (workgroups go to the
+  // XCDs round-robin), so all q tiles of a (batch, head) run on one XCD and share its L2.
+  // Within an XCD class the slots come in groups of LF_QGROUP (batch, head) pairs -- so many
+  // that the resident workgroups of an XCD walk the K/V of few heads at a time -- and within
+  // a group by q tile, the one with the most kv tiles first: workgroups are dispatched in
+  // blockIdx order, so under a causal mask the long tiles start early and the short ones
+  // fill the end of the launch (longest-first list scheduling).
   const int nqt = (p.Sq + LF_BM - 1) / LF_BM;
-  const int npair = (nqt + 1) / 2;
   const int nhv = p.Hq / LF_HEADS_PER_WG;     // head units per batch element (heads, or packs of heads)
   const int nbh = p.B * nhv;
   const int xcd = blockIdx.x & 7;
-  // a workgroup takes slots blockIdx.x/8, + gridDim.x/8, ... of its XCD class (the host
-  // may launch fewer workgroups than slots: the resident set, which then stays)
-  for (int slot = blockIdx.x >> 3; slot < LF_NSLOTS(p, npair); slot += (int)(gridDim.x >> 3)) {
-  const int grp = slot / (4 * npair);
-  const int in_grp = slot % (4 * npair);
-  const int bh = (grp * 4 + (in_grp & 3)) * 8 + xcd;
-  if (bh >= nbh) continue;
-  const int pair = in_grp >> 2;
+  const int slot = blockIdx.x >> 3;
+  const int grp = slot / (LF_QGROUP * nqt);
+  const int in_grp = slot % (LF_QGROUP * nqt);
+  const int bh = (grp * LF_QGROUP + in_grp % LF_QGROUP) * 8 + xcd;
+  if (bh >= nbh) return;     // padding slot of the last group
+  const int slot_qt = nqt - 1 - in_grp / LF_QGROUP;
   const int b = bh / nhv;
 #if LF_GQAPACK
   const int h = (bh % nhv) * LF_GQAPACK + wave % LF_GQAPACK;    // this wave's query head
@@ -425,11 +429,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
         }
       }
     }
-    // the next q tile's prologue overwrites slots other waves may still read ahead from
-    __syncthreads();
   };
 
-  run_q_tile(nqt - 1 - pair);
-  if (pair != nqt - 1 - pair) run_q_tile(pair);
-  }   // slot
+  run_q_tile(slot_qt);
 }

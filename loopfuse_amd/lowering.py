@@ -274,6 +274,9 @@ def _get_scratch(device: torch.device, nfloats: int) -> torch.Tensor:
     return t
 
 
+PREFILL_QGROUP = 8      # LF_QGROUP of lf_attn_prefill_swp.hip (its default)
+
+
 def decode_split(units: int, Sk: int, cus: int = 256, per_cu: int = 2) -> int:
     """Number of KV splits across workgroups.  One workgroup per unit is enough once
     there are ``per_cu`` workgroups per CU (8 resident waves, each with 32 KB of loads
@@ -708,14 +711,18 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         if record_visits:
             visits = torch.zeros((B * heads * nqt, nkt), dtype=torch.uint8, device=q.device)
             P.visits = visits.data_ptr()
-        # 8 XCD classes x (batch*head pairs per class, padded to the kernel's groups of 4) x q tiles
+        # 8 XCD classes x (batch*head pairs per class, padded to the kernel's groups) x q tiles
         per_xcd = (B * heads + 7) // 8
-        # lf_attn_prefill takes two q tiles (heavy + light) per workgroup
-        per_bh = (nqt + 1) // 2
-        grid = 8 * ((per_xcd + 3) // 4 * 4) * per_bh
-        persist = os.environ.get("LOOPFUSE_PREFILL_PERSIST")
-        if family == "prefill_swp" and persist:
-            grid = min(grid, 8 * int(persist))
+        if family == "prefill_swp":
+            # one q tile per workgroup, groups of LF_QGROUP heads, longest q tiles first
+            qgroup = PREFILL_QGROUP
+            for e in spec.extra:
+                if e.startswith("-DLF_QGROUP="):
+                    qgroup = int(e.split("=")[1])
+            grid = 8 * ((per_xcd + qgroup - 1) // qgroup * qgroup) * nqt
+        else:
+            # lf_attn_prefill takes two q tiles (heavy + light) per workgroup, groups of 4 heads
+            grid = 8 * ((per_xcd + 3) // 4 * 4) * ((nqt + 1) // 2)
         get_kernel(spec, spec.entry()).launch((grid, 1, 1), (64 * nw, 1, 1), P)
         _last_launch.set({"kernels": [spec.entry()], "grid": grid, "block": 64 * nw, "q_tile_rows": bm,
                                  "heads_per_workgroup": spec.pack or 1})

@@ -138,9 +138,11 @@ static int run_prefill(const char* dir, const char* file, const char* symbol) {
   p.B = B; p.Hq = H; p.Hkv = H; p.Sq = S; p.Sk = S;
   p.nsplit = 1; p.rows = 1; p.k2_group = 1;
   p.scale = 1.0f / sqrtf((float)D);
-  /* 8 XCD classes x (batch*head pairs per class, in groups of 4) x pairs of 128-row q tiles */
+  /* lf_attn_prefill: 8 XCD classes x (batch*head pairs per class, in groups of 4) x pairs of
+     128-row q tiles; lf_attn_prefill_swp: groups of 8, one q tile per workgroup */
   const unsigned per_xcd = (B * H + 7) / 8, nqt = (S + 127) / 128;
-  const unsigned grid = 8 * ((per_xcd + 3) / 4 * 4) * ((nqt + 1) / 2);
+  const unsigned grid = strcmp(symbol, "lf_attn_prefill_swp") == 0 ? 8 * ((per_xcd + 7) / 8 * 8) * nqt
+                                                                     : 8 * ((per_xcd + 3) / 4 * 4) * ((nqt + 1) / 2);
   void* args[1] = {&p};
   CHECK_LF(lf_launch(fn, grid, 1, 1, 256, 1, 1, 0, NULL, args));
   CHECK_HIP(hipDeviceSynchronize());
