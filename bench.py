@@ -103,6 +103,34 @@ def mfma_ceiling(dev) -> dict:
             c = clk.cpu().view(-1, 2).double()
             res[f"{shape}_{name}"] = {"tflops": iters * 32 * 32768.0 * 4 * nwg / t / 1e12,
                                       "shader_mhz": float((c[:, 0] / c[:, 1]).median() * 100)}
+    res["prefill_kernel"] = prefill_operand_and_shape_rates(dev)
+    return res
+
+
+def prefill_operand_and_shape_rates(dev) -> dict:
+    """The product prefill kernel itself, same instruction stream, on other operands and
+    shapes: config 2 with Q = K = V = 0 (what the operands' switching activity costs), without
+    the mask (what the diagonal tiles and the short q tiles cost), and at S = 8192 with the
+    same number of tokens (what is left of the per-q-tile costs when a q tile runs 130 kv tiles)."""
+    import dataclasses
+
+    import torch
+
+    from loopfuse_amd import workloads
+
+    res = {}
+    for B, S in ((8, 2048), (2, 8192)):
+        for mask in ("causal", None):
+            for data in ("normal", "zeros"):
+                w = dataclasses.replace(workloads.make("c2", seed=0, B=B, S=S), mask=mask)
+                if data == "zeros":
+                    w = dataclasses.replace(w, q=torch.zeros_like(w.q), k=torch.zeros_like(w.k), v=torch.zeros_like(w.v))
+                w = w.to(dev)
+                out = workloads.run(w)
+                r = time_settled(lambda i: workloads.run(w, out=out))
+                flops = 4.0 * B * 32 * S * S * 128 * (0.5 if mask else 1.0)
+                res[f"B{B}_S{S}_{mask or 'nomask'}_{data}"] = {"us_per_launch": r["us_per_launch"],
+                                                               "tflops": flops / r["us_per_launch"] / 1e6}
     return res
 
 
@@ -254,7 +282,8 @@ def main() -> int:
     ap.add_argument("--no-via-backend", action="store_true",
                     help="skip the legs that time the two headline workloads through torch.compile(backend=loopfuse_backend)")
     ap.add_argument("--mfma-ceiling", action="store_true",
-                    help="also run the MFMA-only probe on zeros and on N(0,1) operands (the data-dependent clock ceiling)")
+                    help="also run the MFMA-only probe on zeros and on N(0,1) operands (the data-dependent clock ceiling), and "
+                         "the prefill kernel on zero operands, without the mask and at S = 8192")
     ap.add_argument("--workload", default="c2", help="prefill workload: c2 | c2_softcap | c3 | c2_mask (the causal mask given as a tensor)")
     ap.add_argument("--decode-workload", default="c5", help="decode workload: c5 | c4 | c5_padded | cache4096 (mask tensors: left padding / partly filled cache)")
     args = ap.parse_args()

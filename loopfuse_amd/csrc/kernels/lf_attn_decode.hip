@@ -69,6 +69,270 @@ struct LfDecIds {            // page ids of one step
   long long k, v;
 };
 
+#ifndef LF_COOP
+#define LF_COOP 0            /* 1 (with LF_HEADWAVE, K and V paged, pages of a multiple of 16 tokens, token-major
+                                pools): the workgroup loads each 16-token step of its LF_DW heads as ONE
+                                contiguous block (16 token rows x LF_DW heads x D), every load instruction 1 KB
+                                of consecutive bytes, and hands the rows to the waves through LDS.  Reading
+                                the same bytes head by head -- 256-byte pieces 2 KB apart per wave -- costs
+                                about a tenth of the HBM rate. */
+#endif
+
+#if LF_COOP
+#if !LF_HEADWAVE || LF_PAGED != 3 || LF_BIAS || (LF_PAGE_SIZE % 16) || (LF_PAGE_SIZE_V % 16)
+#error "LF_COOP needs LF_HEADWAVE, paged K and V with pages of a multiple of 16 tokens, and no score bias"
+#endif
+
+struct LfCoopStage {
+  lf_u32x4 k[LF_NJ];
+  lf_u32x4 v[LF_NJ];
+};
+
+// Split decode step, cooperative loads.  Layout of the work as in the kernel below with
+// LF_HEADWAVE: grid = (B * Hkv/LF_DW, nsplit), wave w owns kv head LF_DW*hc + w and writes its
+// own result or partial.  What differs is the way K and V reach the waves:
+//   global -> registers : thread t of the workgroup loads 16-byte pieces t, t + LF_DT, ... of the
+//                         step's block (LF_NJ pieces of K, LF_NJ of V); four steps in flight
+//   registers -> LDS    : the same pieces, rows padded (K +16 B, V +32 B) so that the two read
+//                         patterns below are free of bank conflicts; two buffers alternate,
+//                         one workgroup barrier per step
+//   LDS -> MFMA         : S^T = K Q^T with ds_read_b128 (row = token, 32 d per k-step) on the
+//                         16x16x32 MFMA; O^T += V^T P^T with transposed 8-byte reads on the
+//                         16x16x16 MFMA, whose k extent is the 16 tokens of a step
+extern "C" __global__ void __launch_bounds__(LF_DT, 1) lf_attn_decode(const LfAttnParams p) {
+  constexpr int kRowB = LF_DW * LF_D * 2;            // bytes of one token row over the workgroup's heads
+  constexpr int kPieces = kRowB / 16;                // 16-byte pieces per row
+  constexpr int kKStride = kRowB + 16;               // LDS row strides
+  constexpr int kVStride = kRowB + 32;
+  constexpr int kBufB = 16 * (kKStride + kVStride);
+  static_assert(16 * kPieces == LF_NJ * LF_DT, "a step is LF_NJ pieces per thread");
+  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * kBufB];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int c = lane & 15;      // token of a step (K rows) / query column (MFMA results)
+  const int g = lane >> 4;
+
+  const int z = blockIdx.y;
+  const int chunks = (p.rows + LF_QROWS - 1) / LF_QROWS;   // row chunks per (b, kv head)
+  const int unit = blockIdx.x;
+  const int rc = unit % chunks;
+  const int hchunks = p.Hkv / LF_DW;                        // the host checks Hkv % LF_DW == 0
+  const int hkv0 = ((unit / chunks) % hchunks) * LF_DW;
+  const int hkv = hkv0 + wave;
+  const int b = unit / (chunks * hchunks);
+  const int bh = b * p.Hkv + hkv;
+  const int row0 = rc * LF_QROWS;
+  const int nrows = min(p.rows - row0, LF_QROWS);
+
+  const int tok_begin = z * p.split_len;
+  const int tok_end = min(tok_begin + p.split_len, p.Sk);
+  const int nsteps = (max(tok_end - tok_begin, 0) + 15) / 16;   // the same for every wave of the workgroup
+
+  // ---- B operand of S^T = K Q^T: lane (q = c, g) holds Q[row0 + q][32*j + 8*g .. +7]
+  lf_elem8 qb[LF_NJ];
+  {
+    const lf_elem* qrow = p.q + (long long)b * p.q_sb + (long long)hkv * p.q_sh +
+                          (long long)(row0 + min(c, nrows - 1)) * p.q_ss;
+#pragma unroll
+    for (int j = 0; j < LF_NJ; ++j) {
+      lf_u32x4 raw = *reinterpret_cast<const lf_u32x4*>(qrow + 32 * j + 8 * g);
+      if (c >= nrows) raw = lf_u32x4{0u, 0u, 0u, 0u};
+      qb[j] = __builtin_bit_cast(lf_elem8, raw);
+    }
+  }
+#if LF_SOFTCAP
+  const float sc_in = p.scale / p.softcap;
+  const float cexp = LF_LOG2E;
+#else
+  const float cexp = p.scale * LF_LOG2E;
+#endif
+
+  lf_f32x4 o[LF_NDB];          // O^T: lane (q = c, g) holds d = 16*db + 4*g + i
+#pragma unroll
+  for (int db = 0; db < LF_NDB; ++db) o[db] = lf_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  float mc = LF_NEG_INF;       // exponent offset of column q (same in all 4 lane groups)
+  float l_part = 0.0f;         // this lane's share of the sum
+
+  // ---- loads: piece u of this thread is piece tid + LF_DT*u of the step's block
+  // Page ids: one register holds the ids of 32 steps (lane l: step l % 32 of the chunk, K for
+  // l < 32, V for l >= 32), issue() picks its pair with v_readlane.  The next chunk's register
+  // is loaded 32 steps ahead.  So the loop's only vector memory operations are the K/V loads:
+  // these complete in order, and a table load consumed between them would make the wave wait
+  // for every load in flight.
+  auto load_ids = [&](int st0) -> lf_table_t {
+    const int tok = min(tok_begin + 16 * (st0 + (lane & 31)), p.Sk - 1);   // steps past the end: the last page (never issued)
+    return lane < 32 ? reinterpret_cast<const lf_table_t*>(p.k_table)[(long long)b * p.kt_stride + tok / LF_PAGE_SIZE]
+                     : reinterpret_cast<const lf_table_t*>(p.v_table)[(long long)b * p.vt_stride + tok / LF_PAGE_SIZE_V];
+  };
+  lf_table_t ids_cur = load_ids(0), ids_nxt = load_ids(32);
+  auto id_of = [&](int st, int which) -> long long {
+    const int l = (st & 31) + 32 * which;
+#if LF_TABLE_I64
+    const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(ids_cur & 0xffffffffll), l);
+    const int hi = __builtin_amdgcn_readlane((int)(ids_cur >> 32), l);
+    return ((long long)hi << 32) | lo;
+#else
+    return (long long)__builtin_amdgcn_readlane(ids_cur, l);
+#endif
+  };
+  auto issue = [&](LfCoopStage& sg, int st) {
+    if ((st & 31) == 0 && st > 0) {       // next chunk of ids (workgroup-uniform)
+      ids_cur = ids_nxt;
+      ids_nxt = load_ids(st + 32);
+    }
+    const long long idk = id_of(st, 0), idv = id_of(st, 1);
+    const int tok0 = tok_begin + 16 * st;
+#pragma unroll
+    for (int u = 0; u < LF_NJ; ++u) {
+      const int piece = tid + LF_DT * u;
+      const int tk = min(tok0 + piece / kPieces, p.Sk - 1);  // rows past Sk: clamped, masked later
+      const int within = 8 * (piece % kPieces);              // elements
+      // every byte is read once, whole lines at a time: streaming (non-temporal) loads
+      sg.k[u] = __builtin_nontemporal_load(reinterpret_cast<const lf_u32x4*>(
+          p.k + idk * p.k_sb + (long long)(tk % LF_PAGE_SIZE) * p.k_ss + (long long)hkv0 * p.k_sh + within));
+      sg.v[u] = __builtin_nontemporal_load(reinterpret_cast<const lf_u32x4*>(
+          p.v + idv * p.v_sb + (long long)(tk % LF_PAGE_SIZE_V) * p.v_ss + (long long)hkv0 * p.v_sh + within));
+    }
+  };
+  auto to_lds = [&](const LfCoopStage& sg, int buf) {
+    unsigned char* base = smem + buf * kBufB;
+#pragma unroll
+    for (int u = 0; u < LF_NJ; ++u) {
+      const int piece = tid + LF_DT * u;
+      const int tk = piece / kPieces, within = 16 * (piece % kPieces);
+      *reinterpret_cast<lf_u32x4*>(base + tk * kKStride + within) = sg.k[u];
+      *reinterpret_cast<lf_u32x4*>(base + 16 * kKStride + tk * kVStride + within) = sg.v[u];
+    }
+  };
+
+  // ---- one step (16 tokens) of this wave's head out of LDS buffer `buf`
+  auto consume = [&](int buf, int st) {
+    const unsigned char* kb = smem + buf * kBufB + wave * (LF_D * 2);
+    const unsigned char* vb = kb + 16 * kKStride;
+    lf_f32x4 x4 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int j = 0; j < LF_NJ; ++j) {
+      const lf_u32x4 kf = *reinterpret_cast<const lf_u32x4*>(kb + c * kKStride + 64 * j + 16 * g);
+      x4 = lf_mfma16(__builtin_bit_cast(lf_elem8, kf), qb[j], x4);
+    }
+    // lane (q = c, g): x4[i] is token t0 + i
+    const int t0 = tok_begin + 16 * st + 4 * g;
+    float x[4];
+    float mx = LF_NEG_INF;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float s = x4[i];
+#if LF_SOFTCAP
+      s = p.softcap * lf_tanh(s * sc_in);
+#endif
+      x[i] = (t0 + i < tok_end) ? s * cexp : LF_NEG_INF;
+      mx = fmaxf(mx, x[i]);
+    }
+    if (__builtin_amdgcn_ballot_w64(mx > mc + (float)LF_LAZY_LOG2) != 0ull) {
+      // bring the column's offset up to its max over all four lane groups
+      float mq = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mq = fmaxf(mq, __shfl_xor(mq, 32, 64));
+      const float m_new = fmaxf(mc, mq);
+      const float r = (m_new == LF_NEG_INF) ? 1.0f : lf_exp2(mc - m_new);
+      mc = m_new;
+      l_part *= r;
+#pragma unroll
+      for (int db = 0; db < LF_NDB; ++db) o[db] *= r;
+    }
+    const float m_sub = (mc == LF_NEG_INF) ? 0.0f : mc;
+    lf_elem4 pb;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float e = lf_exp2(x[i] - m_sub);
+      l_part += e;
+      pb[i] = lf_from_float(e);
+    }
+    // O^T += V^T P^T: k-slot i of lane group g is token 4g + i, the order pb is held in.  The
+    // 16 lanes of a group ask for rows 4g .. 4g+3, columns 16db .. +15: lane c supplies the
+    // 8-byte piece (row 4g + c/4, columns +4*(c%4)) and receives column c of the four rows.
+    const int trow = 4 * g + (c >> 2);
+#pragma unroll
+    for (int db = 0; db < LF_NDB; ++db) {
+      const unsigned char* src = vb + trow * kVStride + 2 * (16 * db + 4 * (c & 3));
+      lf_s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_s16x4*)(src));
+      o[db] = lf_mfma16k16(__builtin_bit_cast(lf_elem4, t), pb, o[db]);
+    }
+  };
+
+  // ---- streaming loop: four register stages rotate (static names: four steps per trip)
+  {
+    LfCoopStage s0, s1, s2, s3;
+    // step st: stage -> LDS buffer st & 1, refill the stage with step st + 4, barrier (LDS
+    // writes only: the loads stay in flight), consume.  Buffer st & 1 was last read in step
+    // st - 2, which every wave had left before it arrived at the barrier of step st - 1.
+#define LF_COOP_STEP(sg, st, refill)                                         \
+    {                                                                        \
+      to_lds(sg, (st) & 1);                                                  \
+      if (refill) issue(sg, (st) + 4);                                       \
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");        \
+      consume((st) & 1, (st));                                               \
+    }
+    // The steady state has no condition in it: the compiler counts the loads in flight to
+    // place its waits, and a path on which a refill is skipped would make it wait, on every
+    // path, as if the stage being written were the last one loaded (i.e. for everything).
+    int st = 0;
+    if (nsteps >= 8) {
+      issue(s0, 0);
+      issue(s1, 1);
+      issue(s2, 2);
+      issue(s3, 3);
+      do {
+        LF_COOP_STEP(s0, st, true)
+        LF_COOP_STEP(s1, st + 1, true)
+        LF_COOP_STEP(s2, st + 2, true)
+        LF_COOP_STEP(s3, st + 3, true)
+        st += 4;
+      } while (st + 8 <= nsteps);
+    } else {
+      if (0 < nsteps) issue(s0, 0);
+      if (1 < nsteps) issue(s1, 1);
+      if (2 < nsteps) issue(s2, 2);
+      if (3 < nsteps) issue(s3, 3);
+    }
+    for (; st < nsteps; st += 4) {
+      if (st < nsteps) LF_COOP_STEP(s0, st, st + 4 < nsteps)
+      if (st + 1 < nsteps) LF_COOP_STEP(s1, st + 1, st + 5 < nsteps)
+      if (st + 2 < nsteps) LF_COOP_STEP(s2, st + 2, st + 6 < nsteps)
+      if (st + 3 < nsteps) LF_COOP_STEP(s3, st + 3, st + 7 < nsteps)
+    }
+#undef LF_COOP_STEP
+  }
+
+  // ---- every wave owns its (batch, head): lane (q = c, g) writes d = 16*db + 4*g .. +3 of row q
+  float l_wave = l_part + __shfl_xor(l_part, 16, 64);
+  l_wave += __shfl_xor(l_wave, 32, 64);
+  if (c < nrows) {
+    const int qr = row0 + c;
+    if (p.nsplit == 1) {
+      lf_elem* orow = p.o + (long long)b * p.o_sb + (long long)hkv * p.o_sh + (long long)qr * p.o_ss;
+      const float inv = lf_inv_sum(l_wave);
+#pragma unroll
+      for (int db = 0; db < LF_NDB; ++db) {
+        lf_elem4 w4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w4[e] = lf_from_float(o[db][e] * inv);
+        *reinterpret_cast<lf_elem4*>(orow + 16 * db + 4 * g) = w4;
+      }
+    } else {
+      const long long slot = ((long long)bh * p.rows + qr) * p.nsplit + z;
+#pragma unroll
+      for (int db = 0; db < LF_NDB; ++db)
+        *reinterpret_cast<lf_f32x4*>(&p.part_acc[slot * LF_D + 16 * db + 4 * g]) = o[db];
+      if (g == 0) {
+        p.part_ml[slot * 2 + 0] = mc;            // exponent offset, log2 units
+        p.part_ml[slot * 2 + 1] = l_wave;
+      }
+    }
+  }
+}
+#else   // !LF_COOP
 extern "C" __global__ void __launch_bounds__(LF_DT, 8 / LF_DW) lf_attn_decode(const LfAttnParams p) {
   // One buffer, two lives: wave-private V tiles of the pair being consumed
   // ([LF_DW][2][16*D] elements) during the loop, merge buffer
@@ -439,6 +703,8 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 8 / LF_DW) lf_attn_decode(co
   }
 #endif   // LF_HEADWAVE
 }
+
+#endif  // LF_COOP
 
 // Merge nsplit partial results per query row.  A thread owns 4 consecutive d of one row;
 // block = 256 threads = 1024 / LF_HEAD_DIM rows, grid = ceil(B*Hkv*rows / rows per block).

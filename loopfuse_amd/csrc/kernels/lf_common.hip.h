@@ -179,6 +179,15 @@ __device__ __forceinline__ lf_f32x4 lf_mfma16(lf_elem8 a, lf_elem8 b, lf_f32x4 c
 #endif
 }
 
+// 16x16x16: A lane (row = lane % 16, group = lane / 16) holds k = 4*group .. +3
+__device__ __forceinline__ lf_f32x4 lf_mfma16k16(lf_elem4 a, lf_elem4 b, lf_f32x4 c) {
+#if LF_DTYPE == 0
+  return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(lf_s16x4, a), __builtin_bit_cast(lf_s16x4, b), c, 0, 0, 0);
+#else
+  return __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, c, 0, 0, 0);
+#endif
+}
+
 // Value held by the lane 32 positions away (lane l <-> lane l ^ 32): one
 // v_permlane32_swap (VALU) instead of a round trip through the LDS crossbar.
 __device__ __forceinline__ float lf_swap32(float x) {

@@ -71,6 +71,7 @@ class KernelSpec:
     waves: int = 4         # decode: waves per workgroup
     v_tr: bool = True      # prefill: transposed LDS reads for V
     headwave: bool = False  # decode: one kv head per wave (8 waves) instead of 4 waves sharing a head
+    coop: bool = False     # decode, headwave: the workgroup loads whole 16-token blocks, rows reach the waves through LDS
     denom: bool = False    # prefill: softmax denominator sum + c (c a run-time parameter)
     bias: int = 0          # prefill: bit 0 additive score bias tensor, bit 1 additive output bias tensor, bit 2 unaligned rows
     pack: int = 0          # prefill_swp, grouped-query attention: a workgroup's waves take 2 or 4 heads of one group
@@ -93,6 +94,8 @@ class KernelSpec:
             o += [f"-DLF_PAGE_SIZE_V={self.page_size_v}"]
         if self.family == "decode":
             o += [f"-DLF_DW={self.waves}", f"-DLF_HEADWAVE={int(self.headwave)}"]
+            if self.coop:
+                o += ["-DLF_COOP=1"]
             if self.bias:
                 o += ["-DLF_BIAS=1"]
         elif self.family == "prefill":
@@ -121,7 +124,7 @@ class KernelSpec:
         return (f"lf_{self.family}_t{self.dtype}_d{self.head_dim}_m{self.mask}_c{int(self.softcap)}"
                 f"_p{self.paged}x{self.page_size}i{int(self.table_i64)}_r{self.rows}w{self.waves}v{int(self.v_tr)}h{int(self.headwave)}b{self.bias}n{int(self.denom)}"
                 + (f"_q{self.d2}" if self.d2 else "") + (f"_gp{int(self.pack)}" if self.pack else "") + (f"_pv{self.page_size_v}" if self.page_size_v else "")
-                + ("_z" if self.safe else "")
+                + ("_z" if self.safe else "") + ("_co" if self.coop else "")
                 + "".join("_" + e.replace("-D", "").replace("=", "") for e in self.extra))
 
     def source(self) -> str:
@@ -306,6 +309,17 @@ def _decode_headwave(paged: int, page_size: int, Hkv: int, D: int, P: "AttnParam
     return (paged == 3 and Hkv % 8 == 0 and P.k_sh == D and P.v_sh == D
             and P.k_ss == Hkv * D and P.v_ss == Hkv * D
             and units_hw * max(1, min(8, Sk // 512)) >= cus)
+
+
+def _decode_coop(headwave: bool, page_size: int, page_size_v: int, bias_bits: int, Hkv: int, waves: int) -> bool:
+    """With one kv head per wave the workgroup reads every 16-token block of its 8 heads as one
+    contiguous piece and hands the rows to the waves through LDS (``-DLF_COOP=1``) when a block
+    lies inside a page (pages of a multiple of 16 tokens) and there is no score bias to carry
+    along: a wave that fetches its own head reads 256-byte pieces 2 KB apart, which costs about a
+    tenth of the HBM rate.  LOOPFUSE_DECODE_COOP=0 keeps the per-wave loads."""
+    if os.environ.get("LOOPFUSE_DECODE_COOP", "1") != "1":
+        return False
+    return headwave and page_size % 16 == 0 and not page_size_v and not bias_bits and Hkv % waves == 0
 
 
 def prefill_variant(Sq: int, v_tr: bool = True) -> str:
@@ -763,6 +777,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     P.rows, P.nsplit, P.split_len = rows, nsplit, split_len
     spec = KernelSpec("decode", _DTYPE_CODE[dtype], D, MASK_NONE, plan.softcap is not None, paged,
                       page_size, table_i64, rows=DECODE_QROWS, waves=waves, headwave=headwave, page_size_v=page_size_v,
+                      coop=_decode_coop(headwave, page_size, page_size_v, bias_bits, Hkv, waves),
                       bias=bias_bits, safe=plan.zero_blind_rows and bool(bias_bits),
                       extra=tuple(os.environ.get("LOOPFUSE_KOPTS", "").split()))
     rows_per_block = 1024 // D       # combine kernel: 256 threads, 4 consecutive d each
@@ -774,7 +789,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         runtime.launch_decode_static(get_kernel(spec, "lf_attn_decode"), get_kernel(spec, "lf_attn_decode_combine"), P,
                                      4 * nrow * D, 4 * nrow * 2, (units, nsplit), 64 * spec.waves, combine_grid, 256)
         _last_launch.set({"kernels": ["lf_attn_decode", "lf_attn_decode_combine"], "grid": (units, nsplit),
-                                 "block": 64 * spec.waves, "head_per_wave": headwave, "static_scratch": True})
+                                 "block": 64 * spec.waves, "head_per_wave": headwave, "cooperative_loads": spec.coop,
+                                 "static_scratch": True})
         return out
     if nsplit > 1:
         nrow = B * Hkv * rows * nsplit
@@ -785,5 +801,6 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     if nsplit > 1 and merge_splits:
         get_kernel(spec, "lf_attn_decode_combine").launch((combine_grid, 1, 1), (256, 1, 1), P)
     _last_launch.set({"kernels": ["lf_attn_decode"] + (["lf_attn_decode_combine"] if nsplit > 1 and merge_splits else []),
-                             "grid": (units, nsplit), "block": 64 * spec.waves, "head_per_wave": headwave})
+                             "grid": (units, nsplit), "block": 64 * spec.waves, "head_per_wave": headwave,
+                             "cooperative_loads": spec.coop})
     return out
