@@ -583,17 +583,48 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 8 / LF_DW) lf_attn_decode(co
     i1 = fetch_ids(2 * pr + 1);
     i2 = fetch_ids(2 * (pr + LF_PSTRIDE));
     i3 = fetch_ids(2 * (pr + LF_PSTRIDE) + 1);
-    if (pr < npairs) {
+    // The steady state (both pairs of the trip and both refills exist) has no condition in it:
+    // the compiler places its waits by counting the loads in flight, and a path on which a
+    // refill is skipped would make it wait on every path as if nothing younger were in flight,
+    // i.e. for all loads.  The last trips run below, with the conditions.
+    if (pr + 3 * LF_PSTRIDE < npairs) {
       issue(s0, 2 * pr, i0);
       issue(s1, 2 * pr + 1, i1);
       i0 = fetch_ids(2 * (pr + 2 * LF_PSTRIDE));
       i1 = fetch_ids(2 * (pr + 2 * LF_PSTRIDE) + 1);
-    }
-    if (pr + LF_PSTRIDE < npairs) {
       issue(s2, 2 * (pr + LF_PSTRIDE), i2);
       issue(s3, 2 * (pr + LF_PSTRIDE) + 1, i3);
       i2 = fetch_ids(2 * (pr + 3 * LF_PSTRIDE));
       i3 = fetch_ids(2 * (pr + 3 * LF_PSTRIDE) + 1);
+      do {
+        consume(s0, s1, pr);
+        const int pa = pr + 2 * LF_PSTRIDE;
+        issue(s0, 2 * pa, i0);
+        issue(s1, 2 * pa + 1, i1);
+        i0 = fetch_ids(2 * (pa + 2 * LF_PSTRIDE));
+        i1 = fetch_ids(2 * (pa + 2 * LF_PSTRIDE) + 1);
+        const int pb2 = pr + LF_PSTRIDE;
+        consume(s2, s3, pb2);
+        const int pc = pb2 + 2 * LF_PSTRIDE;
+        issue(s2, 2 * pc, i2);
+        issue(s3, 2 * pc + 1, i3);
+        i2 = fetch_ids(2 * (pc + 2 * LF_PSTRIDE));
+        i3 = fetch_ids(2 * (pc + 2 * LF_PSTRIDE) + 1);
+        pr += 2 * LF_PSTRIDE;
+      } while (pr + 3 * LF_PSTRIDE < npairs);
+    } else {
+      if (pr < npairs) {
+        issue(s0, 2 * pr, i0);
+        issue(s1, 2 * pr + 1, i1);
+        i0 = fetch_ids(2 * (pr + 2 * LF_PSTRIDE));
+        i1 = fetch_ids(2 * (pr + 2 * LF_PSTRIDE) + 1);
+      }
+      if (pr + LF_PSTRIDE < npairs) {
+        issue(s2, 2 * (pr + LF_PSTRIDE), i2);
+        issue(s3, 2 * (pr + LF_PSTRIDE) + 1, i3);
+        i2 = fetch_ids(2 * (pr + 3 * LF_PSTRIDE));
+        i3 = fetch_ids(2 * (pr + 3 * LF_PSTRIDE) + 1);
+      }
     }
     for (; pr < npairs; pr += 2 * LF_PSTRIDE) {
       consume(s0, s1, pr);
