@@ -38,7 +38,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16/fp16, published
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, published
 # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by a plain copy of known
 # size (the rocprofv3 summaries under profiles/); counters cannot be read from inside this process
-TRAFFIC_BYTES = {"c2": (548 + 128) * (1 << 20), "c5": (513 + 4) * (1 << 20)}
+TRAFFIC_BYTES = {"c2": (541 + 128) * (1 << 20), "c5": (513 + 4) * (1 << 20)}
 
 
 def time_gpu(fn, steps: int, warmup: int):
