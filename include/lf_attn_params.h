@@ -30,7 +30,8 @@ typedef struct LfAttnParamsHost {
   const void* k_table;  /* [B, pages] page ids, int32 or int64 (LF_TABLE_I64) */
   const void* v_table;
   float* part_acc;      /* decode split-K scratch: [units, nsplit, rows, D] floats */
-  float* part_ml;       /* decode split-K scratch: [units, nsplit, rows, 2] floats */
+  float* part_ml;       /* decode split-K scratch: [units, nsplit, rows, 2] floats; lf_attn_prefill_swp: optional
+                           output [B, Hq, Sq] floats, the rows' log-sum-exp in log2 units (NULL: not written) */
   unsigned char* visits;/* optional [B*Hq*q_tiles, kv_tiles] visited-tile record, else NULL */
   const void* bias;     /* LF_BIAS & 1: additive score bias [B, Hq, Sq, Sk]; lf_attn_decode -DLF_BIAS=1: [B, Hkv, rows, Sk] */
   const void* obias;    /* LF_BIAS & 2: additive output bias [B, Hq, Sq, D] */

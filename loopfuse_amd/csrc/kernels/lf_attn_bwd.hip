@@ -1,0 +1,337 @@
+// lf_attn_bwd.hip — backward of the fused attention forward (dense K/V, mask none / causal /
+// sliding window, scale; no softcap, no bias) for gfx950.  The reference has no backward
+// (its README lists it as future work); the formulas are the standard ones for
+// O = softmax(scale * Q K^T + mask) V with the row log-sum-exp L kept by the forward:
+//   P = exp(scale * Q K^T - L),  dV = P^T dO,  dP = dO V^T,  delta = rowsum(dO * O),
+//   dS = scale * P * (dP - delta),  dQ = dS K,  dK = dS^T Q.
+// Three kernels, no atomics, every result written once (deterministic):
+//   lf_attn_bwd_delta : delta[b, h, q]
+//   lf_attn_bwd_dkdv  : a workgroup owns 128 keys of one (batch, kv head) -- 4 waves x 32 keys,
+//                       K^T and V^T of its keys in registers as MFMA B operands -- and walks the
+//                       q tiles (64 rows) of the query heads of the group that can see them
+//   lf_attn_bwd_dq    : a workgroup owns 128 query rows of one (batch, head), Q^T and dO^T in
+//                       registers, and walks the kv tiles (64 keys) as the forward does
+// The tiles that are walked go through LDS in the two layouts of lf_prefill_blocks.hip.h: the
+// K layout (ds_read_b128, rows of the tile = MFMA rows) and the V layout (transposed reads,
+// rows of the tile = MFMA k).  As in the forward, the accumulator of the first product is, as
+// held, the B operand of the second, so P and dS never leave registers.
+// L and the exponent are in log2 units (the forward writes L2 = offset + log2(sum)).
+
+struct LfAttnBwdParams {
+  const lf_elem* q;       // [B, Hq, Sq, D]
+  const lf_elem* k;       // [B, Hkv, Sk, D]
+  const lf_elem* v;
+  const lf_elem* o;       // forward output
+  const lf_elem* dout;    // gradient of the output
+  lf_elem* dq;
+  lf_elem* dk;
+  lf_elem* dv;
+  const float* lse;       // [B, Hq, Sq] row log-sum-exp of the scaled, masked scores, log2 units
+  float* delta;           // [B, Hq, Sq] scratch: rowsum(dO * O)
+  long long q_sb, q_sh, q_ss;      // element strides (d stride 1)
+  long long k_sb, k_sh, k_ss;
+  long long v_sb, v_sh, v_ss;
+  long long o_sb, o_sh, o_ss;
+  long long do_sb, do_sh, do_ss;
+  long long dq_sb, dq_sh, dq_ss;
+  long long dk_sb, dk_sh, dk_ss;
+  long long dv_sb, dv_sh, dv_ss;
+  int B, Hq, Hkv, Sq, Sk;
+  int window;
+  float scale;
+};
+
+#define LF_BW_NT 256
+
+// delta[row] = sum_d dO[row][d] * O[row][d]; 16 lanes per row, 8 elements per lane
+extern "C" __global__ void __launch_bounds__(LF_BW_NT) lf_attn_bwd_delta(const LfAttnBwdParams p) {
+  const long long row = (long long)blockIdx.x * (LF_BW_NT / 16) + threadIdx.x / 16;
+  const int piece = threadIdx.x % 16;
+  const long long nrows = (long long)p.B * p.Hq * p.Sq;
+  float s = 0.0f;
+  if (row < nrows && piece < LF_CPR) {
+    const int qi = (int)(row % p.Sq);
+    const int h = (int)((row / p.Sq) % p.Hq);
+    const int b = (int)(row / ((long long)p.Sq * p.Hq));
+    const lf_elem8 ov = *reinterpret_cast<const lf_elem8*>(p.o + b * p.o_sb + h * p.o_sh + qi * p.o_ss + 8 * piece);
+    const lf_elem8 gv = *reinterpret_cast<const lf_elem8*>(p.dout + b * p.do_sb + h * p.do_sh + qi * p.do_ss + 8 * piece);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s += (float)ov[e] * (float)gv[e];
+  }
+  s += __shfl_xor(s, 1, 64);
+  s += __shfl_xor(s, 2, 64);
+  s += __shfl_xor(s, 4, 64);
+  s += __shfl_xor(s, 8, 64);
+  if (row < nrows && piece == 0) p.delta[row] = s;
+}
+
+// 64 rows x D of `src` (rows row0 .. row0+63 of a [rows, D] matrix with row stride `ss`; rows past
+// `nrows` arrive as zeros) into LDS in the K layout (`rm`) and / or the V layout (`tr`)
+__device__ __forceinline__ void lf_bw_stage(const lf_elem* src, long long ss, int row0, int nrows,
+                                            lf_elem* rm, lf_elem* tr, int tid) {
+#pragma unroll
+  for (int u = 0; u < 64 * LF_CPR / LF_BW_NT; ++u) {
+    const int piece = tid + LF_BW_NT * u;
+    const int r = piece / LF_CPR, ch = piece % LF_CPR;
+    lf_u32x4 val = {0u, 0u, 0u, 0u};
+    if (row0 + r < nrows) val = *reinterpret_cast<const lf_u32x4*>(src + (long long)(row0 + r) * ss + 8 * ch);
+    if (rm != nullptr) *reinterpret_cast<lf_u32x4*>(&rm[r * LF_D + 8 * lf_k_phys(r, ch)]) = val;
+    if (tr != nullptr) *reinterpret_cast<lf_u32x4*>(&tr[r * LF_D + 8 * lf_v_phys(r, ch)]) = val;
+  }
+}
+
+// accumulators X^T[d][n] (lane n = lane % 32; element i of block db is d = 32*db + 8*(i/4) + 4*g + i%4)
+// -> rows n of a [rows, D] matrix, 16 bytes per store (the exchange of the forward's epilogue)
+__device__ __forceinline__ void lf_bw_store_rows(const lf_f32x16* acc, lf_elem* row_ptr, bool valid, int g) {
+#pragma unroll
+  for (int db = 0; db < LF_NDB; ++db) {
+    unsigned ch[4][2];
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4) {
+      lf_elem4 w;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) w[e] = lf_from_float(acc[db][4 * i4 + e]);
+      const lf_u32x2 wu = __builtin_bit_cast(lf_u32x2, w);
+      ch[i4][0] = wu[0];
+      ch[i4][1] = wu[1];
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      auto r0 = __builtin_amdgcn_permlane32_swap(ch[2 * j][0], ch[2 * j + 1][0], false, false);
+      auto r1 = __builtin_amdgcn_permlane32_swap(ch[2 * j][1], ch[2 * j + 1][1], false, false);
+      const lf_u32x4 out = {r0[0], r1[0], r0[1], r1[1]};
+      if (valid) *reinterpret_cast<lf_u32x4*>(row_ptr + 32 * db + 16 * j + 8 * g) = out;
+    }
+  }
+}
+
+extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const LfAttnBwdParams p) {
+  __shared__ __attribute__((aligned(16))) lf_elem q_rm[64 * LF_D];
+  __shared__ __attribute__((aligned(16))) lf_elem q_tr[64 * LF_D];
+  __shared__ __attribute__((aligned(16))) lf_elem g_rm[64 * LF_D];     // dO
+  __shared__ __attribute__((aligned(16))) lf_elem g_tr[64 * LF_D];
+  __shared__ __attribute__((aligned(16))) float lse_s[64];
+  __shared__ __attribute__((aligned(16))) float delta_s[64];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31;
+  const int g = lane >> 5;
+
+  const int nkt = (p.Sk + 127) / 128;
+  const int kt = blockIdx.x % nkt;
+  const int bhkv = blockIdx.x / nkt;
+  const int hkv = bhkv % p.Hkv;
+  const int b = bhkv / p.Hkv;
+  const int group = p.Hq / p.Hkv;
+  const int key0 = 128 * kt + 32 * wave;           // first key of this wave
+  const int my_key = key0 + l32;
+  const int nqt = (p.Sq + 63) / 64;
+
+  // K^T and V^T of this lane's key as B operands: d = 16*ks + 8*g .. +7
+  lf_elem8 kf[LF_NKS], vf[LF_NKS];
+  {
+    const int kr = min(my_key, p.Sk - 1);
+    const lf_elem* krow = p.k + (long long)b * p.k_sb + (long long)hkv * p.k_sh + (long long)kr * p.k_ss;
+    const lf_elem* vrow = p.v + (long long)b * p.v_sb + (long long)hkv * p.v_sh + (long long)kr * p.v_ss;
+#pragma unroll
+    for (int ks = 0; ks < LF_NKS; ++ks) {
+      kf[ks] = __builtin_bit_cast(lf_elem8, *reinterpret_cast<const lf_u32x4*>(krow + 16 * ks + 8 * g));
+      vf[ks] = __builtin_bit_cast(lf_elem8, *reinterpret_cast<const lf_u32x4*>(vrow + 16 * ks + 8 * g));
+    }
+  }
+  const float cexp = p.scale * LF_LOG2E;
+
+  lf_f32x16 dk[LF_NDB], dv[LF_NDB];
+#pragma unroll
+  for (int db = 0; db < LF_NDB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) dk[db][i] = dv[db][i] = 0.0f;
+
+  // q tiles (64 rows) that hold a query seeing one of the workgroup's 128 keys
+  int qt_begin = 0, qt_end = nqt;
+#if LF_MASK >= 1
+  qt_begin = (128 * kt) / 64;                                   // q >= key
+#endif
+#if LF_MASK == 2
+  qt_end = min(nqt, (min(128 * kt + 127, p.Sk - 1) + p.window - 1) / 64 + 1);   // q - key < window
+#endif
+
+  for (int gi = 0; gi < group; ++gi) {
+    const int h = hkv * group + gi;
+    const lf_elem* qbase = p.q + (long long)b * p.q_sb + (long long)h * p.q_sh;
+    const lf_elem* gbase = p.dout + (long long)b * p.do_sb + (long long)h * p.do_sh;
+    const long long rbase = ((long long)b * p.Hq + h) * p.Sq;
+    for (int qt = qt_begin; qt < qt_end; ++qt) {
+      const int q0 = 64 * qt;
+      __syncthreads();          // the previous step's reads are done
+      lf_bw_stage(qbase, p.q_ss, q0, p.Sq, q_rm, q_tr, tid);
+      lf_bw_stage(gbase, p.do_ss, q0, p.Sq, g_rm, g_tr, tid);
+      if (tid < 64) {
+        const bool in = q0 + tid < p.Sq;
+        lse_s[tid] = in ? p.lse[rbase + q0 + tid] : __builtin_inff();   // rows past Sq: P = 0
+        delta_s[tid] = in ? p.delta[rbase + q0 + tid] : 0.0f;
+      }
+      __syncthreads();
+
+      bool need = key0 < p.Sk;
+#if LF_MASK >= 1
+      need = need && (q0 + 63 >= key0);
+#endif
+#if LF_MASK == 2
+      need = need && (q0 - min(key0 + 31, p.Sk - 1) < p.window);
+#endif
+      if (!need) continue;      // wave-uniform; the barriers above are reached by every wave
+
+      lf_elem8 pf[LF_NKK], dsf[LF_NKK];
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) {
+        lf_f32x16 s, dp;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[i] = dp[i] = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < LF_NKS; ++ks) {
+          const lf_u32x4 qa = lf_read_k_frag(q_rm, l32, g, ks * LF_NKB + qb);
+          const lf_u32x4 ga = lf_read_k_frag(g_rm, l32, g, ks * LF_NKB + qb);
+          s = lf_mfma32(__builtin_bit_cast(lf_elem8, qa), kf[ks], s);
+          dp = lf_mfma32(__builtin_bit_cast(lf_elem8, ga), vf[ks], dp);
+        }
+        // element i: query q0 + 32*qb + 8*(i/4) + 4*g + i%4, key my_key
+#pragma unroll
+        for (int i4 = 0; i4 < 4; ++i4) {
+          const int ql = 32 * qb + 8 * i4 + 4 * g;
+          const lf_f32x4 l4 = *reinterpret_cast<const lf_f32x4*>(&lse_s[ql]);
+          const lf_f32x4 d4 = *reinterpret_cast<const lf_f32x4*>(&delta_s[ql]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int i = 4 * i4 + e;
+            const bool keep = lf_mask_keep(q0 + ql + e, my_key, p.Sk, p.window);
+            const float pv = keep ? lf_exp2(s[i] * cexp - l4[e]) : 0.0f;
+            const float ds = pv * (dp[i] - d4[e]) * p.scale;
+            pf[2 * qb + i / 8][i % 8] = lf_from_float(pv);
+            dsf[2 * qb + i / 8][i % 8] = lf_from_float(ds);
+          }
+        }
+      }
+      // dV^T += dO^T P, dK^T += Q^T dS (k = the 64 queries of the tile)
+#pragma unroll
+      for (int f = 0; f < LF_NKK * LF_NDB; ++f) {
+        const lf_elem8 ga = lf_read_v_frag_tr(g_tr, lane, g, f);
+        const lf_elem8 qa = lf_read_v_frag_tr(q_tr, lane, g, f);
+        dv[f % LF_NDB] = lf_mfma32(ga, pf[f / LF_NDB], dv[f % LF_NDB]);
+        dk[f % LF_NDB] = lf_mfma32(qa, dsf[f / LF_NDB], dk[f % LF_NDB]);
+      }
+    }
+  }
+
+  const bool valid = my_key < p.Sk;
+  const int kr = min(my_key, p.Sk - 1);
+  lf_bw_store_rows(dk, p.dk + (long long)b * p.dk_sb + (long long)hkv * p.dk_sh + (long long)kr * p.dk_ss, valid, g);
+  lf_bw_store_rows(dv, p.dv + (long long)b * p.dv_sb + (long long)hkv * p.dv_sh + (long long)kr * p.dv_ss, valid, g);
+}
+
+extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dq(const LfAttnBwdParams p) {
+  __shared__ __attribute__((aligned(16))) lf_elem k_rm[64 * LF_D];
+  __shared__ __attribute__((aligned(16))) lf_elem k_tr[64 * LF_D];
+  __shared__ __attribute__((aligned(16))) lf_elem v_rm[64 * LF_D];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31;
+  const int g = lane >> 5;
+
+  const int nqt = (p.Sq + 127) / 128;
+  const int qt = nqt - 1 - (int)(blockIdx.x % nqt);       // long q tiles first
+  const int bh = blockIdx.x / nqt;
+  const int h = bh % p.Hq;
+  const int b = bh / p.Hq;
+  const int hkv = h / (p.Hq / p.Hkv);
+  const int q0 = 128 * qt;
+  const int wq0 = q0 + 32 * wave;
+  const int my_q = wq0 + l32;
+  const int qr = min(my_q, p.Sq - 1);
+  const int nkt = (p.Sk + 63) / 64;
+
+  lf_elem8 qf[LF_NKS], gf[LF_NKS];
+  {
+    const lf_elem* qrow = p.q + (long long)b * p.q_sb + (long long)h * p.q_sh + (long long)qr * p.q_ss;
+    const lf_elem* grow = p.dout + (long long)b * p.do_sb + (long long)h * p.do_sh + (long long)qr * p.do_ss;
+#pragma unroll
+    for (int ks = 0; ks < LF_NKS; ++ks) {
+      qf[ks] = __builtin_bit_cast(lf_elem8, *reinterpret_cast<const lf_u32x4*>(qrow + 16 * ks + 8 * g));
+      gf[ks] = __builtin_bit_cast(lf_elem8, *reinterpret_cast<const lf_u32x4*>(grow + 16 * ks + 8 * g));
+    }
+  }
+  const long long ridx = ((long long)b * p.Hq + h) * p.Sq + qr;
+  const float lse_q = my_q < p.Sq ? p.lse[ridx] : __builtin_inff();
+  const float delta_q = my_q < p.Sq ? p.delta[ridx] : 0.0f;
+  const float cexp = p.scale * LF_LOG2E;
+
+  lf_f32x16 dq[LF_NDB];
+#pragma unroll
+  for (int db = 0; db < LF_NDB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) dq[db][i] = 0.0f;
+
+  int kt_begin = 0, kt_end = nkt;
+  {
+    const int qlast = min(q0 + 128, p.Sq) - 1;
+#if LF_MASK >= 1
+    kt_end = min(nkt, qlast / 64 + 1);
+#endif
+#if LF_MASK == 2
+    const int lo = q0 - p.window + 1;
+    if (lo > 0) kt_begin = lo / 64;
+#endif
+    (void)qlast;
+  }
+  const lf_elem* kbase = p.k + (long long)b * p.k_sb + (long long)hkv * p.k_sh;
+  const lf_elem* vbase = p.v + (long long)b * p.v_sb + (long long)hkv * p.v_sh;
+  for (int kt = kt_begin; kt < kt_end; ++kt) {
+    const int k0 = 64 * kt;
+    __syncthreads();
+    lf_bw_stage(kbase, p.k_ss, k0, p.Sk, k_rm, k_tr, tid);
+    lf_bw_stage(vbase, p.v_ss, k0, p.Sk, v_rm, nullptr, tid);
+    __syncthreads();
+
+    bool need = wq0 < p.Sq;
+#if LF_MASK >= 1
+    need = need && (k0 <= min(wq0 + 31, p.Sq - 1));
+#endif
+#if LF_MASK == 2
+    need = need && (min(k0 + 64, p.Sk) - 1 >= wq0 - p.window + 1);
+#endif
+    if (!need) continue;
+
+    lf_elem8 dsf[LF_NKK];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      lf_f32x16 s, dp;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) s[i] = dp[i] = 0.0f;
+#pragma unroll
+      for (int ks = 0; ks < LF_NKS; ++ks) {
+        const lf_u32x4 ka = lf_read_k_frag(k_rm, l32, g, ks * LF_NKB + kb);
+        const lf_u32x4 va = lf_read_k_frag(v_rm, l32, g, ks * LF_NKB + kb);
+        s = lf_mfma32(__builtin_bit_cast(lf_elem8, ka), qf[ks], s);       // S^T[key][q]
+        dp = lf_mfma32(__builtin_bit_cast(lf_elem8, va), gf[ks], dp);     // dP^T[key][q]
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int j = k0 + 32 * kb + 8 * (i / 4) + 4 * g + (i % 4);
+        const bool keep = lf_mask_keep(my_q, j, p.Sk, p.window);
+        const float pv = keep ? lf_exp2(s[i] * cexp - lse_q) : 0.0f;
+        dsf[2 * kb + i / 8][i % 8] = lf_from_float(pv * (dp[i] - delta_q) * p.scale);
+      }
+    }
+    // dQ^T += K^T dS^T (k = the 64 keys of the tile)
+#pragma unroll
+    for (int f = 0; f < LF_NKK * LF_NDB; ++f) {
+      const lf_elem8 ka = lf_read_v_frag_tr(k_tr, lane, g, f);
+      dq[f % LF_NDB] = lf_mfma32(ka, dsf[f / LF_NDB], dq[f % LF_NDB]);
+    }
+  }
+  lf_bw_store_rows(dq, p.dq + (long long)b * p.dq_sb + (long long)h * p.dq_sh + (long long)qr * p.dq_ss, my_q < p.Sq, g);
+}

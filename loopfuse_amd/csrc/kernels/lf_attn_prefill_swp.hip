@@ -400,6 +400,10 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
     // ---- epilogue: O[q][d] = O^T[d][q] / l.  Element i of block db is
     // d = 32*db + 8*(i/4) + 4*g + i%4.
     const float l_tot = l_run + lf_swap32(l_run);
+    // optional: the row's log-sum-exp of the scaled, masked scores in log2 units (what a
+    // backward pass recomputes the probabilities from); -inf for a row that saw no key
+    if (p.part_ml != nullptr && g == 0 && my_q < p.Sq)
+      p.part_ml[((long long)b * p.Hq + h) * p.Sq + my_q] = mc_ref + __builtin_log2f(l_tot);
     {
       // Lane (q, g) holds, per block db, four 4-value chunks d = 32*db + 8*i4 + 4*g + 0..3.
       // One v_permlane32_swap per register pair trades chunks with the lane that holds

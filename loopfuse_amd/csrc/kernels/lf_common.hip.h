@@ -133,7 +133,8 @@ struct LfAttnParams {
   const void* k_table;       // [B, pages_per_seq] page ids (lf_table_t) when paged
   const void* v_table;
   float* part_acc;           // split-K scratch: [units, nsplit, rows, D]
-  float* part_ml;            // split-K scratch: [units, nsplit, rows, 2] (max, sum)
+  float* part_ml;            // split-K scratch: [units, nsplit, rows, 2] (max, sum); lf_attn_prefill_swp: optional
+                             // output [B, Hq, Sq], the rows' log-sum-exp in log2 units (null: not written)
   unsigned char* visits;     // optional [B*Hq*nqt, nkt] visited-tile record
   const lf_elem* bias;       // LF_BIAS & 1: additive score bias [B, Hq, Sq, Sk] (key stride 1),
                              // added after scale / softcap and before the mask

@@ -59,7 +59,7 @@ class AttnParams(ctypes.Structure):
 class KernelSpec:
     """Compile-time specialisation of one kernel family (= one code object)."""
 
-    family: str            # "prefill" | "decode"
+    family: str            # "prefill" | "prefill_swp" | "decode" | "bwd"
     dtype: int             # 0 bf16, 1 fp16
     head_dim: int          # 64 | 128
     mask: int = MASK_NONE
@@ -110,15 +110,15 @@ class KernelSpec:
 
     def files(self) -> tuple[str, ...]:
         kernel = {"prefill": "lf_attn_prefill.hip", "prefill_swp": "lf_attn_prefill_swp.hip",
-                  "decode": "lf_attn_decode.hip"}[self.family]
+                  "decode": "lf_attn_decode.hip", "bwd": "lf_attn_bwd.hip"}[self.family]
         if self.family == "decode":
             return ("lf_common.hip.h", kernel)
         # the two prefill kernels: their own tuning macros come first (the shared blocks use LF_BN)
         return ("lf_common.hip.h", "lf_prefill_blocks.hip.h", kernel)
 
     def entry(self) -> str:
-        return {"prefill": "lf_attn_prefill",
-                "prefill_swp": "lf_attn_prefill_swp", "decode": "lf_attn_decode"}[self.family]
+        return {"prefill": "lf_attn_prefill", "prefill_swp": "lf_attn_prefill_swp", "decode": "lf_attn_decode",
+                "bwd": "lf_attn_bwd_dq"}[self.family]
 
     def name(self) -> str:
         return (f"lf_{self.family}_t{self.dtype}_d{self.head_dim}_m{self.mask}_c{int(self.softcap)}"
@@ -469,7 +469,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
               score_bias: Optional[torch.Tensor] = None, out_bias: Optional[torch.Tensor] = None,
               choice: Optional[dict] = None, merge_splits: bool = True,
               q2: Optional[torch.Tensor] = None, k2: Optional[torch.Tensor] = None,
-              static_scratch: bool = False):
+              static_scratch: bool = False, lse: Optional[torch.Tensor] = None):
     """Run fused attention on the GPU.
 
     q : [B, Hq, Sq, D];  k, v : [B, Hkv, Sk, D], or page pools [N, P, Hkv, D]
@@ -488,6 +488,9 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     ``lf_launch_decode_static``, whose split-K partials live in a static device array of the
     library -- no device memory is allocated anywhere in the call; a step whose partials exceed
     that array raises ``runtime.ShimError``.
+    ``lse`` (float32 [B, Hq, Sq], contiguous): also write each row's log-sum-exp of the scaled,
+    masked scores, in log2 units -- what ``attention_backward`` recomputes the probabilities
+    from.  Served by ``lf_attn_prefill_swp`` without softcap; anything else raises ``UnsupportedPlan``.
     ``choice`` overrides the launch heuristics (what ``tuned_attention`` searches over):
     ``{"prefill": "swp" | "w32"}``, ``{"head_per_wave": bool, "splits": n}``.
     Returns O [B, Hq, Sq, D] and, with ``record_visits``, the uint8 record of the KV tiles
@@ -737,6 +740,12 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         else:
             # lf_attn_prefill takes two q tiles (heavy + light) per workgroup, groups of 4 heads
             grid = 8 * ((per_xcd + 3) // 4 * 4) * ((nqt + 1) // 2)
+        if lse is not None:
+            if family != "prefill_swp" or plan.softcap is not None or paged:
+                raise UnsupportedPlan("the row log-sum-exp is written by lf_attn_prefill_swp for dense K/V without softcap only")
+            if lse.dtype != torch.float32 or tuple(lse.shape) != (B, Hq, Sq) or not lse.is_contiguous() or lse.device != q.device:
+                raise UnsupportedPlan(f"lse must be a contiguous float32 [{B}, {Hq}, {Sq}] tensor on the device of Q")
+            P.part_ml = lse.data_ptr()
         get_kernel(spec, spec.entry()).launch((grid, 1, 1), (64 * nw, 1, 1), P)
         _last_launch.set({"kernels": [spec.entry()], "grid": grid, "block": 64 * nw, "q_tile_rows": bm,
                                  "heads_per_workgroup": spec.pack or 1})
@@ -744,6 +753,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
 
     if family != "decode":
         raise ValueError(f"unknown kernel family {family!r}")
+    if lse is not None:
+        raise UnsupportedPlan("the decode kernels do not write the row log-sum-exp")
     if mask != MASK_NONE:
         raise UnsupportedPlan("the decode kernel takes no mask")
     # query rows of one unit: the group's heads (Sq == 1) or the Sq rows (group == 1)
@@ -804,3 +815,78 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
                              "grid": (units, nsplit), "block": 64 * spec.waves, "head_per_wave": headwave,
                              "cooperative_loads": spec.coop})
     return out
+
+
+# ---------------------------------------------------------------------------
+# backward (the reference has none: loopfuse README "future work")
+# ---------------------------------------------------------------------------
+class AttnBwdParams(ctypes.Structure):
+    """Mirror of ``struct LfAttnBwdParams`` in csrc/kernels/lf_attn_bwd.hip."""
+
+    _fields_ = (
+        [(n, ctypes.c_void_p) for n in ("q", "k", "v", "o", "dout", "dq", "dk", "dv", "lse", "delta")]
+        + [(f"{t}_{x}", ctypes.c_longlong) for t in ("q", "k", "v", "o", "do", "dq", "dk", "dv") for x in ("sb", "sh", "ss")]
+        + [(n, ctypes.c_int) for n in ("B", "Hq", "Hkv", "Sq", "Sk", "window")]
+        + [("scale", ctypes.c_float)]
+    )
+
+
+def bwd_spec(dtype: torch.dtype, D: int, mask: int) -> KernelSpec:
+    return KernelSpec("bwd", _DTYPE_CODE[dtype], D, mask)
+
+
+def attention_backward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor, lse: torch.Tensor,
+                       dout: torch.Tensor, plan: AttnPlan):
+    """Gradients of ``attention(q, k, v, plan)`` for dense K/V (mask none / causal / sliding, scale;
+    no softcap, bias or paging): returns ``(dq, dk, dv)`` in the operands' dtype.  ``o`` and ``lse``
+    are the forward's output and row log-sum-exp (``attention(..., lse=...)``).  Three launches
+    (csrc/kernels/lf_attn_bwd.hip): delta = rowsum(dO * O); dK and dV, one workgroup per 128 keys of
+    a (batch, kv head); dQ, one workgroup per 128 query rows.  No atomics: results are
+    reproducible bit for bit."""
+    dtype = q.dtype
+    if dtype not in _DTYPE_CODE:
+        raise UnsupportedPlan(f"dtype {dtype} not supported by the MFMA kernels (bf16/fp16 only)")
+    if plan.softcap is not None or plan.k_paged or plan.v_paged or plan.denom_add != 0.0:
+        raise UnsupportedPlan("the backward kernels serve dense K/V without softcap")
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise UnsupportedPlan("Q, K, V must be [B, H, S, D]")
+    B, Hq, Sq, D = q.shape
+    Hkv, Sk = k.shape[1], k.shape[2]
+    if D not in (64, 128) or k.shape != v.shape or k.shape[0] != B or k.shape[3] != D or Hkv < 1 or Hq % Hkv:
+        raise UnsupportedPlan(f"shapes not served: Q {tuple(q.shape)}, K {tuple(k.shape)}, V {tuple(v.shape)}")
+    if Sq < 1 or Sk < 1:
+        raise UnsupportedPlan("empty sequences")
+    if o.shape != q.shape or dout.shape != q.shape or tuple(lse.shape) != (B, Hq, Sq):
+        raise UnsupportedPlan("O, dO must have the shape of Q and lse must be [B, Hq, Sq]")
+    if lse.dtype != torch.float32 or not lse.is_contiguous():
+        raise UnsupportedPlan("lse must be contiguous float32")
+    mask = {None: MASK_NONE, "none": MASK_NONE, "causal": MASK_CAUSAL, "sliding": MASK_SLIDING}.get(plan.mask)
+    if mask is None:
+        raise UnsupportedPlan(f"mask {plan.mask!r} not served")
+    window = int(plan.window or 0)
+    if mask == MASK_SLIDING and window < 1:
+        raise UnsupportedPlan("sliding window must be >= 1")
+    for name, t in (("Q", q), ("K", k), ("V", v), ("O", o), ("dO", dout)):
+        _check_tensor(name, t, dtype)
+    dq = torch.empty((B, Hq, Sq, D), dtype=dtype, device=q.device)
+    dk = torch.empty((B, Hkv, Sk, D), dtype=dtype, device=q.device)
+    dv = torch.empty((B, Hkv, Sk, D), dtype=dtype, device=q.device)
+    delta = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
+    P = AttnBwdParams()
+    for name, t in (("q", q), ("k", k), ("v", v), ("o", o), ("dout", dout), ("dq", dq), ("dk", dk), ("dv", dv),
+                    ("lse", lse), ("delta", delta)):
+        setattr(P, name, t.data_ptr())
+    for pre, t in (("q", q), ("k", k), ("v", v), ("o", o), ("do", dout), ("dq", dq), ("dk", dk), ("dv", dv)):
+        setattr(P, pre + "_sb", t.stride(0))
+        setattr(P, pre + "_sh", t.stride(1))
+        setattr(P, pre + "_ss", t.stride(2))
+    P.B, P.Hq, P.Hkv, P.Sq, P.Sk, P.window = B, Hq, Hkv, Sq, Sk, window
+    P.scale = float(plan.scale)
+    spec = bwd_spec(dtype, D, mask)
+    keep = (q, k, v, o, dout, lse, delta, dq, dk, dv)  # noqa: F841  (tensors stay alive until the launches are queued)
+    rows = B * Hq * Sq
+    get_kernel(spec, "lf_attn_bwd_delta").launch(((rows + 15) // 16, 1, 1), (256, 1, 1), P)
+    get_kernel(spec, "lf_attn_bwd_dkdv").launch((B * Hkv * ((Sk + 127) // 128), 1, 1), (256, 1, 1), P)
+    get_kernel(spec, "lf_attn_bwd_dq").launch((B * Hq * ((Sq + 127) // 128), 1, 1), (256, 1, 1), P)
+    _last_launch.set({"kernels": ["lf_attn_bwd_delta", "lf_attn_bwd_dkdv", "lf_attn_bwd_dq"]})
+    return dq, dk, dv

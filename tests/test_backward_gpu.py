@@ -1,0 +1,89 @@
+"""Backward of the fused attention (lf_attn_bwd.hip) against torch autograd on an fp32 eager
+graph of the same attention (float64 accumulation of the reference values), through
+``lowering.attention(..., lse=...)`` and ``lowering.attention_backward``.
+
+The reference has no backward (its README lists it as future work), so there is no reference
+test to mirror; the cases follow its forward matrix: masks none / causal / sliding, grouped
+query heads, ragged lengths, both dtypes and head dims."""
+import math
+
+import pytest
+import torch
+
+from loopfuse_amd import lowering
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _ref(q, k, v, dout, mask, window, scale):
+    """O and the gradients from autograd on the eager graph, in float64."""
+    q, k, v = (t.double().detach().requires_grad_(True) for t in (q, k, v))
+    g = q.shape[1] // k.shape[1]
+    kk, vv = k.repeat_interleave(g, dim=1), v.repeat_interleave(g, dim=1)
+    s = q @ kk.transpose(-2, -1) * scale
+    Sq, Sk = s.shape[-2:]
+    i = torch.arange(Sq, device=s.device)[:, None]
+    j = torch.arange(Sk, device=s.device)[None, :]
+    keep = torch.ones(Sq, Sk, dtype=torch.bool, device=s.device)
+    if mask in ("causal", "sliding"):
+        keep &= j <= i
+    if mask == "sliding":
+        keep &= (i - j) < window
+    s = s.masked_fill(~keep, float("-inf"))
+    lse2 = torch.logsumexp(s, dim=-1) / math.log(2.0)
+    o = torch.softmax(s, dim=-1) @ vv
+    o.backward(dout.double())
+    return o.detach(), lse2.detach(), q.grad, k.grad, v.grad
+
+
+CASES = [
+    # B, Hq, Hkv, Sq, Sk, D, mask, window, dtype
+    (2, 4, 4, 256, 256, 128, "causal", 0, torch.bfloat16),
+    (2, 4, 4, 256, 256, 128, None, 0, torch.bfloat16),
+    (1, 8, 2, 320, 320, 128, "causal", 0, torch.bfloat16),          # grouped query heads
+    (1, 4, 4, 200, 200, 64, "causal", 0, torch.float16),            # ragged, D 64
+    (1, 4, 2, 384, 384, 128, "sliding", 100, torch.bfloat16),
+    (1, 2, 2, 192, 333, 64, None, 0, torch.bfloat16),               # Sq != Sk
+    (1, 2, 1, 130, 130, 128, "sliding", 7, torch.float16),
+]
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,mask,window,dtype", CASES)
+def test_backward_matches_autograd(B, Hq, Hkv, Sq, Sk, D, mask, window, dtype):
+    g = torch.Generator().manual_seed(Sq * 7 + Sk + D)
+    q, k, v = (torch.randn(shape, generator=g).to(dtype).to(DEV)
+               for shape in ((B, Hq, Sq, D), (B, Hkv, Sk, D), (B, Hkv, Sk, D)))
+    dout = torch.randn((B, Hq, Sq, D), generator=g).to(dtype).to(DEV)
+    scale = D ** -0.5
+    plan = lowering.AttnPlan(mask=mask, window=window, scale=scale)
+    lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=DEV)
+    o = lowering.attention(q, k, v, plan, lse=lse)
+    o_ref, lse_ref, dq_ref, dk_ref, dv_ref = _ref(q, k, v, dout, mask, window, scale)
+    tol = 2e-2 if dtype == torch.bfloat16 else 5e-3
+    assert (o.double() - o_ref).abs().max().item() <= tol
+    torch.testing.assert_close(lse.double(), lse_ref, rtol=1e-3, atol=2e-3)
+    dq, dk, dv = lowering.attention_backward(q, k, v, o, lse, dout, plan)
+    assert dq.dtype == dtype and dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape
+    # gradients are sums of up to Sq (dK, dV: times the group) rounded products: tolerance relative to their size
+    for name, got, want in (("dq", dq, dq_ref), ("dk", dk, dk_ref), ("dv", dv, dv_ref)):
+        err = (got.double() - want).abs().max().item()
+        bound = (4e-2 if dtype == torch.bfloat16 else 1e-2) * max(1.0, want.abs().max().item())
+        assert err <= bound, f"{name}: max abs err {err} > {bound}"
+        rel = ((got.double() - want).norm() / want.norm()).item()
+        assert rel <= (2e-2 if dtype == torch.bfloat16 else 4e-3), f"{name}: relative error {rel}"
+
+
+def test_backward_is_reproducible_and_refuses_what_it_does_not_serve():
+    g = torch.Generator().manual_seed(5)
+    q, k, v, dout = (torch.randn((1, 2, 256, 128), generator=g).to(torch.bfloat16).to(DEV) for _ in range(4))
+    plan = lowering.AttnPlan(mask="causal", scale=128 ** -0.5)
+    lse = torch.empty((1, 2, 256), dtype=torch.float32, device=DEV)
+    o = lowering.attention(q, k, v, plan, lse=lse)
+    a = lowering.attention_backward(q, k, v, o, lse, dout, plan)
+    b = lowering.attention_backward(q, k, v, o, lse, dout, plan)
+    assert all(torch.equal(x, y) for x, y in zip(a, b))          # no atomics: bit for bit
+    with pytest.raises(lowering.UnsupportedPlan):
+        lowering.attention_backward(q, k, v, o, lse, dout, lowering.AttnPlan(mask="causal", scale=0.1, softcap=30.0))
+    with pytest.raises(lowering.UnsupportedPlan):
+        lowering.attention(q, k, v, lowering.AttnPlan(mask="causal", scale=0.1, softcap=30.0), lse=lse)
