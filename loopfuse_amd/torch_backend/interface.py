@@ -49,7 +49,8 @@ USE_HARDCODE_KERNEL = os.environ.get("USE_HARDCODE_KERNEL", "0") == "1"
 # "eager_training" = graph traced with gradients enabled (forward or backward half)
 # "refused_signatures" = argument layouts latched as not servable (see optimized_fn)
 stats = {"fused": 0, "eager_graph": 0, "eager_runtime": 0, "eager_training": 0, "compiled_graphs": 0, "matched_graphs": 0,
-         "refused_signatures": 0, "derived_graphs": 0, "generic_graphs": 0, "fused_generic": 0}
+         "refused_signatures": 0, "derived_graphs": 0, "generic_graphs": 0, "fused_generic": 0,
+         "training_graphs": 0, "fused_training": 0}
 
 
 def _frontend() -> str:
@@ -106,19 +107,86 @@ def loopfuse_backend(gm: torch.fx.GraphModule, sample_inputs, mode="max-autotune
         # AOTAutograd is about to trace a forward + backward pair: the forward graph must
         # hand the probabilities to the backward graph, which a fused forward never forms
         global _warned_training
+        fused = _training_graph(gm, sample_inputs)
+        if fused is not None:
+            return fused
         if _strict():
-            raise NotImplementedError("loopfuse_amd: the attention kernels are forward-only and this graph is "
-                                      "traced with gradients enabled")
+            raise NotImplementedError("loopfuse_amd: this graph is traced with gradients enabled and the kernels are "
+                                      "forward-only for it (its attention is not one the backward kernels serve, or "
+                                      "its tensors are not on the GPU)")
         if not _warned_training:
             _warned_training = True
-            log.warning("loopfuse_amd: graph traced with gradients enabled (an input requires grad); the attention "
-                        "kernels are forward-only, so this graph runs unfused.  Wrap inference in torch.no_grad().")
+            log.warning("loopfuse_amd: graph traced with gradients enabled (an input requires grad) and its attention "
+                        "is not one the backward kernels serve, so this graph runs unfused.  Wrap inference in "
+                        "torch.no_grad().")
         return aot_module_simplified(gm, sample_inputs, fw_compiler=_unfused_compiler)
     compiler = partial(loopfuse_compiler, input_names=get_input_names(gm), **kwargs)
     return aot_module_simplified(gm, sample_inputs, fw_compiler=compiler)
 
 
 _warned_training = False
+
+
+def _training_graph(gm: torch.fx.GraphModule, sample_inputs):
+    """A graph traced with gradients enabled: trace its forward to ATen once (for the matcher only),
+    and when every attention found is one the backward kernels serve, hand AOTAutograd that graph
+    with the attentions replaced by ``training.fused_call_train`` -- differentiable views around
+    the custom op ``loopfuse_amd::attention_fwd``, whose registered formula is the HIP backward.
+    None when the graph has to run unfused.  The forward trace bakes the traced sizes into the view
+    ops it keeps, so under dynamic shapes only a graph that is nothing but its attentions is taken."""
+    from torch.fx.experimental.proxy_tensor import make_fx
+
+    from . import training
+
+    if os.environ.get("LOOPFUSE_TRAINING", "1") != "1":
+        return None
+    if not all(t.is_cuda for t in sample_inputs if isinstance(t, torch.Tensor)):
+        return None                                          # the kernels run on the GPU only: CPU graphs stay unfused
+    try:
+        with torch.no_grad():
+            aten_gm = make_fx(gm, tracing_mode="real", _allow_non_fake_inputs=True)(*sample_inputs)
+        matches = capture.match_attention(aten_gm)
+    except capture.NoMatch as e:
+        log.info("training graph: no attention found (%s)", e)
+        return None
+    except Exception as e:                                   # tracing a user graph a second way may fail in ways of its own
+        log.info("training graph: forward trace for the matcher failed (%s: %s)", type(e).__name__, e)
+        return None
+    if not matches:
+        return None
+    for m in matches:
+        vals = [n.meta.get("val") for n in m.inputs]
+        why = training.trainable(m, lambda i: vals[i])
+        if why:
+            if _strict():
+                raise NotImplementedError(f"loopfuse_amd: no backward kernel for this attention ({why})")
+            log.info("training graph: attention runs unfused (%s)", why)
+            return None
+    rewritten = rewrite_graph(aten_gm, matches, call=training.fused_call_train)
+    dynamic = any(isinstance(a, torch.SymInt) for a in sample_inputs)
+    others = [n for n in rewritten.graph.nodes if n.op == "call_function" and n.target is not training.fused_call_train]
+    if dynamic and others:
+        log.info("training graph: other operations beside the attention under dynamic shapes; running unfused")
+        return None
+    stats["training_graphs"] += 1
+    if DEBUG:
+        print("---- loopfuse_amd: graph traced for training, attentions fused ----")
+        for m in matches:
+            print(m.describe())
+        print(rewritten.code)
+    return aot_module_simplified(rewritten, sample_inputs, fw_compiler=_training_compiler, bw_compiler=_training_compiler)
+
+
+def _training_compiler(gm: torch.fx.GraphModule, sample_inputs) -> Callable:
+    """fw_compiler / bw_compiler of a fused training graph: the graphs hold the custom ops
+    (``loopfuse_amd::attention_fwd`` / ``attention_bwd``) and run as they are."""
+    stats["compiled_graphs"] += 1
+
+    def run(*args):
+        stats["fused_training"] += 1
+        return gm(*args)
+
+    return make_boxed_func(run)
 
 
 def _unfused_compiler(gm: torch.fx.GraphModule, sample_inputs) -> Callable:
@@ -146,9 +214,10 @@ def _fused_call(match, *vals):
     return match.run(vals)
 
 
-def rewrite_graph(gm: torch.fx.GraphModule, matches: list) -> torch.fx.GraphModule:
+def rewrite_graph(gm: torch.fx.GraphModule, matches: list, call=None) -> torch.fx.GraphModule:
     """A copy of ``gm`` in which every matched attention output is produced by one
-    ``_fused_call`` node; what only fed the unfused chain is dropped."""
+    ``_fused_call`` node (or ``call``); what only fed the unfused chain is dropped."""
+    call = call or _fused_call
     new_graph = torch.fx.Graph()
     val_map: dict = {}
     out = new_graph.graph_copy(gm.graph, val_map)
@@ -163,8 +232,8 @@ def rewrite_graph(gm: torch.fx.GraphModule, matches: list) -> torch.fx.GraphModu
         with new_graph.inserting_after(old):
             attr = new_graph.get_attr(name)
         with new_graph.inserting_after(attr):
-            call = new_graph.call_function(_fused_call, (attr, *[val_map[n] for n in m.inputs]))
-        old.replace_all_uses_with(call)
+            node = new_graph.call_function(call, (attr, *[val_map[n] for n in m.inputs]))
+        old.replace_all_uses_with(node)
     new_graph.eliminate_dead_code()
     try:
         fused = torch.fx.GraphModule(gm, new_graph)
