@@ -65,18 +65,31 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT) lf_attn_bwd_delta(const L
   if (row < nrows && piece == 0) p.delta[row] = s;
 }
 
-// 64 rows x D of `src` (rows row0 .. row0+63 of a [rows, D] matrix with row stride `ss`; rows past
-// `nrows` arrive as zeros) into LDS in the K layout (`rm`) and / or the V layout (`tr`)
-__device__ __forceinline__ void lf_bw_stage(const lf_elem* src, long long ss, int row0, int nrows,
-                                            lf_elem* rm, lf_elem* tr, int tid) {
+// A 64-row tile of a [rows, D] matrix (row stride `ss`) on its way into LDS: LF_BW_NP 16-byte
+// pieces per thread.  Loads and LDS writes are separate steps so that the loads of the next
+// tile travel while the current one is being consumed; rows past `nrows` arrive as zeros.
+#define LF_BW_NP (64 * LF_CPR / LF_BW_NT)
+struct LfBwTile {
+  lf_u32x4 piece[LF_BW_NP];
+};
+__device__ __forceinline__ void lf_bw_load(LfBwTile& t, const lf_elem* src, long long ss, int row0, int nrows, int tid) {
 #pragma unroll
-  for (int u = 0; u < 64 * LF_CPR / LF_BW_NT; ++u) {
+  for (int u = 0; u < LF_BW_NP; ++u) {
     const int piece = tid + LF_BW_NT * u;
     const int r = piece / LF_CPR, ch = piece % LF_CPR;
-    lf_u32x4 val = {0u, 0u, 0u, 0u};
-    if (row0 + r < nrows) val = *reinterpret_cast<const lf_u32x4*>(src + (long long)(row0 + r) * ss + 8 * ch);
-    if (rm != nullptr) *reinterpret_cast<lf_u32x4*>(&rm[r * LF_D + 8 * lf_k_phys(r, ch)]) = val;
-    if (tr != nullptr) *reinterpret_cast<lf_u32x4*>(&tr[r * LF_D + 8 * lf_v_phys(r, ch)]) = val;
+    t.piece[u] = lf_u32x4{0u, 0u, 0u, 0u};
+    if (row0 + r < nrows) t.piece[u] = *reinterpret_cast<const lf_u32x4*>(src + (long long)(row0 + r) * ss + 8 * ch);
+  }
+}
+// into the K layout (`rm`: ds_read_b128, tile rows = MFMA rows) and / or the V layout (`tr`:
+// transposed reads, tile rows = MFMA k)
+__device__ __forceinline__ void lf_bw_store(const LfBwTile& t, lf_elem* rm, lf_elem* tr, int tid) {
+#pragma unroll
+  for (int u = 0; u < LF_BW_NP; ++u) {
+    const int piece = tid + LF_BW_NT * u;
+    const int r = piece / LF_CPR, ch = piece % LF_CPR;
+    if (rm != nullptr) *reinterpret_cast<lf_u32x4*>(&rm[r * LF_D + 8 * lf_k_phys(r, ch)]) = t.piece[u];
+    if (tr != nullptr) *reinterpret_cast<lf_u32x4*>(&tr[r * LF_D + 8 * lf_v_phys(r, ch)]) = t.piece[u];
   }
 }
 
@@ -158,70 +171,83 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
   qt_end = min(nqt, (min(128 * kt + 127, p.Sk - 1) + p.window - 1) / 64 + 1);   // q - key < window
 #endif
 
-  for (int gi = 0; gi < group; ++gi) {
-    const int h = hkv * group + gi;
-    const lf_elem* qbase = p.q + (long long)b * p.q_sb + (long long)h * p.q_sh;
-    const lf_elem* gbase = p.dout + (long long)b * p.do_sb + (long long)h * p.do_sh;
-    const long long rbase = ((long long)b * p.Hq + h) * p.Sq;
-    for (int qt = qt_begin; qt < qt_end; ++qt) {
-      const int q0 = 64 * qt;
-      __syncthreads();          // the previous step's reads are done
-      lf_bw_stage(qbase, p.q_ss, q0, p.Sq, q_rm, q_tr, tid);
-      lf_bw_stage(gbase, p.do_ss, q0, p.Sq, g_rm, g_tr, tid);
-      if (tid < 64) {
-        const bool in = q0 + tid < p.Sq;
-        lse_s[tid] = in ? p.lse[rbase + q0 + tid] : __builtin_inff();   // rows past Sq: P = 0
-        delta_s[tid] = in ? p.delta[rbase + q0 + tid] : 0.0f;
-      }
-      __syncthreads();
+  // the steps of this workgroup: query heads of the group x q tiles, one flat sequence; the
+  // global loads of step it + 1 are issued before step it is computed
+  const int ntq = max(qt_end - qt_begin, 0);
+  const int nsteps = group * ntq;
+  LfBwTile tq, tg;
+  float r_lse = 0.0f, r_delta = 0.0f;
+  auto issue = [&](int it) {
+    const int h = hkv * group + it / ntq;
+    const int q0 = 64 * (qt_begin + it % ntq);
+    lf_bw_load(tq, p.q + (long long)b * p.q_sb + (long long)h * p.q_sh, p.q_ss, q0, p.Sq, tid);
+    lf_bw_load(tg, p.dout + (long long)b * p.do_sb + (long long)h * p.do_sh, p.do_ss, q0, p.Sq, tid);
+    if (tid < 64) {
+      const long long r = ((long long)b * p.Hq + h) * p.Sq + q0 + tid;
+      const bool in = q0 + tid < p.Sq;
+      r_lse = in ? p.lse[r] : __builtin_inff();            // rows past Sq: P = 0
+      r_delta = in ? p.delta[r] : 0.0f;
+    }
+  };
+  if (nsteps > 0) issue(0);
+  for (int it = 0; it < nsteps; ++it) {
+    const int q0 = 64 * (qt_begin + it % ntq);
+    __syncthreads();            // the previous step's reads are done
+    lf_bw_store(tq, q_rm, q_tr, tid);
+    lf_bw_store(tg, g_rm, g_tr, tid);
+    if (tid < 64) {
+      lse_s[tid] = r_lse;
+      delta_s[tid] = r_delta;
+    }
+    __syncthreads();
+    if (it + 1 < nsteps) issue(it + 1);
 
-      bool need = key0 < p.Sk;
+    bool need = key0 < p.Sk;
 #if LF_MASK >= 1
-      need = need && (q0 + 63 >= key0);
+    need = need && (q0 + 63 >= key0);
 #endif
 #if LF_MASK == 2
-      need = need && (q0 - min(key0 + 31, p.Sk - 1) < p.window);
+    need = need && (q0 - min(key0 + 31, p.Sk - 1) < p.window);
 #endif
-      if (!need) continue;      // wave-uniform; the barriers above are reached by every wave
+    if (!need) continue;        // wave-uniform; the barriers above are reached by every wave
 
-      lf_elem8 pf[LF_NKK], dsf[LF_NKK];
+    lf_elem8 pf[LF_NKK], dsf[LF_NKK];
 #pragma unroll
-      for (int qb = 0; qb < 2; ++qb) {
-        lf_f32x16 s, dp;
+    for (int qb = 0; qb < 2; ++qb) {
+      lf_f32x16 s, dp;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s[i] = dp[i] = 0.0f;
+      for (int i = 0; i < 16; ++i) s[i] = dp[i] = 0.0f;
 #pragma unroll
-        for (int ks = 0; ks < LF_NKS; ++ks) {
-          const lf_u32x4 qa = lf_read_k_frag(q_rm, l32, g, ks * LF_NKB + qb);
-          const lf_u32x4 ga = lf_read_k_frag(g_rm, l32, g, ks * LF_NKB + qb);
-          s = lf_mfma32(__builtin_bit_cast(lf_elem8, qa), kf[ks], s);
-          dp = lf_mfma32(__builtin_bit_cast(lf_elem8, ga), vf[ks], dp);
-        }
-        // element i: query q0 + 32*qb + 8*(i/4) + 4*g + i%4, key my_key
+      for (int ks = 0; ks < LF_NKS; ++ks) {
+        const lf_u32x4 qa = lf_read_k_frag(q_rm, l32, g, ks * LF_NKB + qb);
+        const lf_u32x4 ga = lf_read_k_frag(g_rm, l32, g, ks * LF_NKB + qb);
+        s = lf_mfma32(__builtin_bit_cast(lf_elem8, qa), kf[ks], s);
+        dp = lf_mfma32(__builtin_bit_cast(lf_elem8, ga), vf[ks], dp);
+      }
+      // element i: query q0 + 32*qb + 8*(i/4) + 4*g + i%4, key my_key
 #pragma unroll
-        for (int i4 = 0; i4 < 4; ++i4) {
-          const int ql = 32 * qb + 8 * i4 + 4 * g;
-          const lf_f32x4 l4 = *reinterpret_cast<const lf_f32x4*>(&lse_s[ql]);
-          const lf_f32x4 d4 = *reinterpret_cast<const lf_f32x4*>(&delta_s[ql]);
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const int ql = 32 * qb + 8 * i4 + 4 * g;
+        const lf_f32x4 l4 = *reinterpret_cast<const lf_f32x4*>(&lse_s[ql]);
+        const lf_f32x4 d4 = *reinterpret_cast<const lf_f32x4*>(&delta_s[ql]);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int i = 4 * i4 + e;
-            const bool keep = lf_mask_keep(q0 + ql + e, my_key, p.Sk, p.window);
-            const float pv = keep ? lf_exp2(s[i] * cexp - l4[e]) : 0.0f;
-            const float ds = pv * (dp[i] - d4[e]) * p.scale;
-            pf[2 * qb + i / 8][i % 8] = lf_from_float(pv);
-            dsf[2 * qb + i / 8][i % 8] = lf_from_float(ds);
-          }
+        for (int e = 0; e < 4; ++e) {
+          const int i = 4 * i4 + e;
+          const bool keep = lf_mask_keep(q0 + ql + e, my_key, p.Sk, p.window);
+          const float pv = keep ? lf_exp2(s[i] * cexp - l4[e]) : 0.0f;
+          const float ds = pv * (dp[i] - d4[e]) * p.scale;
+          pf[2 * qb + i / 8][i % 8] = lf_from_float(pv);
+          dsf[2 * qb + i / 8][i % 8] = lf_from_float(ds);
         }
       }
-      // dV^T += dO^T P, dK^T += Q^T dS (k = the 64 queries of the tile)
+    }
+    // dV^T += dO^T P, dK^T += Q^T dS (k = the 64 queries of the tile)
 #pragma unroll
-      for (int f = 0; f < LF_NKK * LF_NDB; ++f) {
-        const lf_elem8 ga = lf_read_v_frag_tr(g_tr, lane, g, f);
-        const lf_elem8 qa = lf_read_v_frag_tr(q_tr, lane, g, f);
-        dv[f % LF_NDB] = lf_mfma32(ga, pf[f / LF_NDB], dv[f % LF_NDB]);
-        dk[f % LF_NDB] = lf_mfma32(qa, dsf[f / LF_NDB], dk[f % LF_NDB]);
-      }
+    for (int f = 0; f < LF_NKK * LF_NDB; ++f) {
+      const lf_elem8 ga = lf_read_v_frag_tr(g_tr, lane, g, f);
+      const lf_elem8 qa = lf_read_v_frag_tr(q_tr, lane, g, f);
+      dv[f % LF_NDB] = lf_mfma32(ga, pf[f / LF_NDB], dv[f % LF_NDB]);
+      dk[f % LF_NDB] = lf_mfma32(qa, dsf[f / LF_NDB], dk[f % LF_NDB]);
     }
   }
 
@@ -289,12 +315,21 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dq(const L
   }
   const lf_elem* kbase = p.k + (long long)b * p.k_sb + (long long)hkv * p.k_sh;
   const lf_elem* vbase = p.v + (long long)b * p.v_sb + (long long)hkv * p.v_sh;
+  LfBwTile tk, tv;
+  if (kt_begin < kt_end) {
+    lf_bw_load(tk, kbase, p.k_ss, 64 * kt_begin, p.Sk, tid);
+    lf_bw_load(tv, vbase, p.v_ss, 64 * kt_begin, p.Sk, tid);
+  }
   for (int kt = kt_begin; kt < kt_end; ++kt) {
     const int k0 = 64 * kt;
     __syncthreads();
-    lf_bw_stage(kbase, p.k_ss, k0, p.Sk, k_rm, k_tr, tid);
-    lf_bw_stage(vbase, p.v_ss, k0, p.Sk, v_rm, nullptr, tid);
+    lf_bw_store(tk, k_rm, k_tr, tid);
+    lf_bw_store(tv, v_rm, nullptr, tid);
     __syncthreads();
+    if (kt + 1 < kt_end) {      // the next tile's loads travel during this tile's products
+      lf_bw_load(tk, kbase, p.k_ss, k0 + 64, p.Sk, tid);
+      lf_bw_load(tv, vbase, p.v_ss, k0 + 64, p.Sk, tid);
+    }
 
     bool need = wq0 < p.Sq;
 #if LF_MASK >= 1
