@@ -134,6 +134,28 @@ def prefill_operand_and_shape_rates(dev) -> dict:
     return res
 
 
+def backward_leg(dev) -> dict:
+    """Forward (with the row log-sum-exp written) and backward of config 2, steady state.  The
+    backward counts 2.5 times the forward's flop (five matrix products against two), the usual
+    convention; it is not part of the headline metric -- the reference has no backward."""
+    import torch
+
+    from loopfuse_amd import lowering, workloads
+
+    w = workloads.make("c2", seed=0).to(dev)
+    plan = lowering.AttnPlan(mask=w.mask, window=w.window, scale=w.scale)
+    lse = torch.empty(w.q.shape[:-1], dtype=torch.float32, device=dev)
+    o = lowering.attention(w.q, w.k, w.v, plan, lse=lse)
+    dout = torch.randn_like(o)
+    fwd = time_settled(lambda i: lowering.attention(w.q, w.k, w.v, plan, lse=lse, out=o))
+    bwd = time_settled(lambda i: lowering.attention_backward(w.q, w.k, w.v, o, lse, dout, plan), 25.0, 200.0)
+    flop = w.flops()
+    return {"workload": "config 2 (causal bf16 B8 H32 S2048 D128)",
+            "forward_with_lse_us": fwd["us_per_launch"], "forward_tflops": flop / fwd["us_per_launch"] / 1e6,
+            "backward_us": bwd["us_per_launch"], "backward_tflops": 2.5 * flop / bwd["us_per_launch"] / 1e6,
+            "kernels": "lf_attn_bwd_delta+lf_attn_bwd_dkdv+lf_attn_bwd_dq"}
+
+
 def via_backend(dev, steps: int, warmup: int) -> dict:
     """The two headline workloads through the drop-in path: the reference's own graph
     spellings (tests/benchmark.py:78-84 causal prefill, 400-406 paged GQA decode with the
@@ -284,6 +306,8 @@ def main() -> int:
     ap.add_argument("--mfma-ceiling", action="store_true",
                     help="also run the MFMA-only probe on zeros and on N(0,1) operands (the data-dependent clock ceiling), and "
                          "the prefill kernel on zero operands, without the mask and at S = 8192")
+    ap.add_argument("--backward", action="store_true",
+                    help="also time the forward with its log-sum-exp output and the backward kernels on config 2")
     ap.add_argument("--workload", default="c2", help="prefill workload: c2 | c2_softcap | c3 | c2_mask (the causal mask given as a tensor)")
     ap.add_argument("--decode-workload", default="c5", help="decode workload: c5 | c4 | c5_padded | cache4096 (mask tensors: left padding / partly filled cache)")
     args = ap.parse_args()
@@ -390,6 +414,8 @@ def main() -> int:
         out["via_backend"] = via_backend(dev, args.steps, args.warmup)
     if args.mfma_ceiling:
         out["mfma_ceiling"] = mfma_ceiling(dev)
+    if args.backward:
+        out["backward"] = backward_leg(dev)
     if args.torch_sdpa:
         out["torch_sdpa"] = torch_sdpa(args, dev)
     if not args.no_cpu_baseline:
