@@ -65,17 +65,19 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT) lf_attn_bwd_delta(const L
   if (row < nrows && piece == 0) p.delta[row] = s;
 }
 
-// A 64-row tile of a [rows, D] matrix (row stride `ss`) on its way into LDS: LF_BW_NP 16-byte
-// pieces per thread.  Loads and LDS writes are separate steps so that the loads of the next
-// tile travel while the current one is being consumed; rows past `nrows` arrive as zeros.
-#define LF_BW_NP (64 * LF_CPR / LF_BW_NT)
+// A 64-row tile of a [rows, D] matrix (row stride `ss`) on its way into LDS: 64 * LF_CPR / NT
+// 16-byte pieces per thread of a workgroup of NT threads.  Loads and LDS writes are separate
+// steps so that the loads of the next tile travel while the current one is being consumed;
+// rows past `nrows` arrive as zeros.
+template <int NT>
 struct LfBwTile {
-  lf_u32x4 piece[LF_BW_NP];
+  lf_u32x4 piece[64 * LF_CPR / NT];
 };
-__device__ __forceinline__ void lf_bw_load(LfBwTile& t, const lf_elem* src, long long ss, int row0, int nrows, int tid) {
+template <int NT>
+__device__ __forceinline__ void lf_bw_load(LfBwTile<NT>& t, const lf_elem* src, long long ss, int row0, int nrows, int tid) {
 #pragma unroll
-  for (int u = 0; u < LF_BW_NP; ++u) {
-    const int piece = tid + LF_BW_NT * u;
+  for (int u = 0; u < 64 * LF_CPR / NT; ++u) {
+    const int piece = tid + NT * u;
     const int r = piece / LF_CPR, ch = piece % LF_CPR;
     t.piece[u] = lf_u32x4{0u, 0u, 0u, 0u};
     if (row0 + r < nrows) t.piece[u] = *reinterpret_cast<const lf_u32x4*>(src + (long long)(row0 + r) * ss + 8 * ch);
@@ -83,15 +85,22 @@ __device__ __forceinline__ void lf_bw_load(LfBwTile& t, const lf_elem* src, long
 }
 // into the K layout (`rm`: ds_read_b128, tile rows = MFMA rows) and / or the V layout (`tr`:
 // transposed reads, tile rows = MFMA k)
-__device__ __forceinline__ void lf_bw_store(const LfBwTile& t, lf_elem* rm, lf_elem* tr, int tid) {
+template <int NT>
+__device__ __forceinline__ void lf_bw_store(const LfBwTile<NT>& t, lf_elem* rm, lf_elem* tr, int tid) {
 #pragma unroll
-  for (int u = 0; u < LF_BW_NP; ++u) {
-    const int piece = tid + LF_BW_NT * u;
+  for (int u = 0; u < 64 * LF_CPR / NT; ++u) {
+    const int piece = tid + NT * u;
     const int r = piece / LF_CPR, ch = piece % LF_CPR;
     if (rm != nullptr) *reinterpret_cast<lf_u32x4*>(&rm[r * LF_D + 8 * lf_k_phys(r, ch)]) = t.piece[u];
     if (tr != nullptr) *reinterpret_cast<lf_u32x4*>(&tr[r * LF_D + 8 * lf_v_phys(r, ch)]) = t.piece[u];
   }
 }
+
+// Fragment read-ahead of the two product loops (LDS reads in flight ahead of the MFMA that
+// consumes them; the order of reads and MFMAs is pinned with scheduling barriers, left to
+// itself the compiler issues read, wait, MFMA one after the other)
+#define LF_BW_PF1 3      /* first products: pairs of K-layout fragments */
+#define LF_BW_PF2 4      /* second products: V-layout fragments */
 
 // accumulators X^T[d][n] (lane n = lane % 32; element i of block db is d = 32*db + 8*(i/4) + 4*g + i%4)
 // -> rows n of a [rows, D] matrix, 16 bytes per store (the exchange of the forward's epilogue)
@@ -175,7 +184,7 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
   // global loads of step it + 1 are issued before step it is computed
   const int ntq = max(qt_end - qt_begin, 0);
   const int nsteps = group * ntq;
-  LfBwTile tq, tg;
+  LfBwTile<LF_BW_NT> tq, tg;
   float r_lse = 0.0f, r_delta = 0.0f;
   auto issue = [&](int it) {
     const int h = hkv * group + it / ntq;
@@ -217,12 +226,22 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
       lf_f32x16 s, dp;
 #pragma unroll
       for (int i = 0; i < 16; ++i) s[i] = dp[i] = 0.0f;
+      lf_u32x4 qa[LF_NKS], ga[LF_NKS];
+#pragma unroll
+      for (int ks = 0; ks < LF_BW_PF1; ++ks) {
+        qa[ks] = lf_read_k_frag(q_rm, l32, g, ks * LF_NKB + qb);
+        ga[ks] = lf_read_k_frag(g_rm, l32, g, ks * LF_NKB + qb);
+      }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ks = 0; ks < LF_NKS; ++ks) {
-        const lf_u32x4 qa = lf_read_k_frag(q_rm, l32, g, ks * LF_NKB + qb);
-        const lf_u32x4 ga = lf_read_k_frag(g_rm, l32, g, ks * LF_NKB + qb);
-        s = lf_mfma32(__builtin_bit_cast(lf_elem8, qa), kf[ks], s);
-        dp = lf_mfma32(__builtin_bit_cast(lf_elem8, ga), vf[ks], dp);
+        if (ks + LF_BW_PF1 < LF_NKS) {
+          qa[ks + LF_BW_PF1] = lf_read_k_frag(q_rm, l32, g, (ks + LF_BW_PF1) * LF_NKB + qb);
+          ga[ks + LF_BW_PF1] = lf_read_k_frag(g_rm, l32, g, (ks + LF_BW_PF1) * LF_NKB + qb);
+        }
+        s = lf_mfma32(__builtin_bit_cast(lf_elem8, qa[ks]), kf[ks], s);
+        dp = lf_mfma32(__builtin_bit_cast(lf_elem8, ga[ks]), vf[ks], dp);
+        __builtin_amdgcn_sched_barrier(0);
       }
       // element i: query q0 + 32*qb + 8*(i/4) + 4*g + i%4, key my_key
 #pragma unroll
@@ -242,12 +261,25 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
       }
     }
     // dV^T += dO^T P, dK^T += Q^T dS (k = the 64 queries of the tile)
+    {
+      constexpr int kNF = LF_NKK * LF_NDB;
+      lf_elem8 gt[kNF], qt2[kNF];
 #pragma unroll
-    for (int f = 0; f < LF_NKK * LF_NDB; ++f) {
-      const lf_elem8 ga = lf_read_v_frag_tr(g_tr, lane, g, f);
-      const lf_elem8 qa = lf_read_v_frag_tr(q_tr, lane, g, f);
-      dv[f % LF_NDB] = lf_mfma32(ga, pf[f / LF_NDB], dv[f % LF_NDB]);
-      dk[f % LF_NDB] = lf_mfma32(qa, dsf[f / LF_NDB], dk[f % LF_NDB]);
+      for (int f = 0; f < LF_BW_PF2; ++f) {
+        gt[f] = lf_read_v_frag_tr(g_tr, lane, g, f);
+        qt2[f] = lf_read_v_frag_tr(q_tr, lane, g, f);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int f = 0; f < kNF; ++f) {
+        if (f + LF_BW_PF2 < kNF) {
+          gt[f + LF_BW_PF2] = lf_read_v_frag_tr(g_tr, lane, g, f + LF_BW_PF2);
+          qt2[f + LF_BW_PF2] = lf_read_v_frag_tr(q_tr, lane, g, f + LF_BW_PF2);
+        }
+        dv[f % LF_NDB] = lf_mfma32(gt[f], pf[f / LF_NDB], dv[f % LF_NDB]);
+        dk[f % LF_NDB] = lf_mfma32(qt2[f], dsf[f / LF_NDB], dk[f % LF_NDB]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
   }
 
@@ -315,7 +347,7 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dq(const L
   }
   const lf_elem* kbase = p.k + (long long)b * p.k_sb + (long long)hkv * p.k_sh;
   const lf_elem* vbase = p.v + (long long)b * p.v_sb + (long long)hkv * p.v_sh;
-  LfBwTile tk, tv;
+  LfBwTile<LF_BW_NT> tk, tv;
   if (kt_begin < kt_end) {
     lf_bw_load(tk, kbase, p.k_ss, 64 * kt_begin, p.Sk, tid);
     lf_bw_load(tv, vbase, p.v_ss, 64 * kt_begin, p.Sk, tid);
@@ -346,12 +378,22 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dq(const L
       lf_f32x16 s, dp;
 #pragma unroll
       for (int i = 0; i < 16; ++i) s[i] = dp[i] = 0.0f;
+      lf_u32x4 ka[LF_NKS], va[LF_NKS];
+#pragma unroll
+      for (int ks = 0; ks < LF_BW_PF1; ++ks) {
+        ka[ks] = lf_read_k_frag(k_rm, l32, g, ks * LF_NKB + kb);
+        va[ks] = lf_read_k_frag(v_rm, l32, g, ks * LF_NKB + kb);
+      }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ks = 0; ks < LF_NKS; ++ks) {
-        const lf_u32x4 ka = lf_read_k_frag(k_rm, l32, g, ks * LF_NKB + kb);
-        const lf_u32x4 va = lf_read_k_frag(v_rm, l32, g, ks * LF_NKB + kb);
-        s = lf_mfma32(__builtin_bit_cast(lf_elem8, ka), qf[ks], s);       // S^T[key][q]
-        dp = lf_mfma32(__builtin_bit_cast(lf_elem8, va), gf[ks], dp);     // dP^T[key][q]
+        if (ks + LF_BW_PF1 < LF_NKS) {
+          ka[ks + LF_BW_PF1] = lf_read_k_frag(k_rm, l32, g, (ks + LF_BW_PF1) * LF_NKB + kb);
+          va[ks + LF_BW_PF1] = lf_read_k_frag(v_rm, l32, g, (ks + LF_BW_PF1) * LF_NKB + kb);
+        }
+        s = lf_mfma32(__builtin_bit_cast(lf_elem8, ka[ks]), qf[ks], s);       // S^T[key][q]
+        dp = lf_mfma32(__builtin_bit_cast(lf_elem8, va[ks]), gf[ks], dp);     // dP^T[key][q]
+        __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
@@ -362,10 +404,18 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dq(const L
       }
     }
     // dQ^T += K^T dS^T (k = the 64 keys of the tile)
+    {
+      constexpr int kNF = LF_NKK * LF_NDB;
+      lf_elem8 kt2[kNF];
 #pragma unroll
-    for (int f = 0; f < LF_NKK * LF_NDB; ++f) {
-      const lf_elem8 ka = lf_read_v_frag_tr(k_tr, lane, g, f);
-      dq[f % LF_NDB] = lf_mfma32(ka, dsf[f / LF_NDB], dq[f % LF_NDB]);
+      for (int f = 0; f < LF_BW_PF2; ++f) kt2[f] = lf_read_v_frag_tr(k_tr, lane, g, f);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int f = 0; f < kNF; ++f) {
+        if (f + LF_BW_PF2 < kNF) kt2[f + LF_BW_PF2] = lf_read_v_frag_tr(k_tr, lane, g, f + LF_BW_PF2);
+        dq[f % LF_NDB] = lf_mfma32(kt2[f], dsf[f / LF_NDB], dq[f % LF_NDB]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
   }
   lf_bw_store_rows(dq, p.dq + (long long)b * p.dq_sb + (long long)h * p.dq_sh + (long long)qr * p.dq_ss, my_q < p.Sq, g);

@@ -203,3 +203,16 @@ def test_work_bound_sends_large_graphs_to_the_captured_ops(tmp_path, monkeypatch
     monkeypatch.setattr(generic, "MAX_SCALAR_WORK", 100)
     with pytest.raises(emit.NotLowerable, match="scalar work"):
         prog.run(args, launchers=_host_build(prog, tmp_path))
+
+
+def test_codegen_only_hands_back_the_generated_source(monkeypatch):
+    """CODEGEN_ONLY (reference interface.py:615-622): a graph without an attention returns its
+    generic program; ``.code`` is the HIP source that would be compiled."""
+    from loopfuse_amd import loopfuse_backend
+    from loopfuse_amd.torch_backend import interface
+
+    monkeypatch.setattr(interface, "CODEGEN_ONLY", True)
+    torch._dynamo.reset()
+    prg = torch.compile(lambda a, b, c: a @ b + c, backend=loopfuse_backend, dynamic=True)(
+        _r(16, 8), _r(8, 12, seed=1), _r(16, 12, seed=2))
+    assert prg.code.count("__global__") == 1 and "lf_gen_0" in prg.code and "LfGenParams" in prg.code
