@@ -160,3 +160,42 @@ def test_training_graph_with_an_unserved_attention_stays_unfused():
     assert interface.stats["training_graphs"] == before["training_graphs"]
     assert interface.stats["eager_training"] > before["eager_training"]
     assert leaves[0].grad is not None and torch.isfinite(leaves[0].grad.float()).all()
+
+
+def test_module_with_projections_trains_with_the_fused_attention():
+    """A block with parameters (qkv projection, attention, output projection) compiled with
+    static shapes and called outside ``torch.no_grad()``: the attention in the middle runs the
+    fused forward and backward, the projections around it stay ATen ops, and the parameter
+    gradients match the uncompiled module."""
+    from loopfuse_amd import loopfuse_backend
+    from loopfuse_amd.torch_backend import interface, training
+
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            torch.manual_seed(0)
+            self.qkv = torch.nn.Linear(256, 3 * 256, bias=False)
+            self.out = torch.nn.Linear(256, 256, bias=False)
+
+        def forward(self, x):
+            B, S, E = x.shape
+            q, k, v = (t.view(B, S, 4, 64).transpose(1, 2) for t in self.qkv(x).chunk(3, dim=-1))
+            a = torch.softmax(torch.ops.loopfuse.causal_mask(q @ k.transpose(-2, -1) * 0.125), dim=-1) @ v
+            return self.out(a.transpose(1, 2).reshape(B, S, E))
+
+    m = Block().to(DEV).to(torch.bfloat16)
+    x = (torch.randn((2, 192, 256), generator=torch.Generator().manual_seed(3)) * 0.5).to(torch.bfloat16).to(DEV)
+    torch._dynamo.reset()
+    before, ops_before = dict(interface.stats), dict(training.counters)
+    y = torch.compile(m, backend=loopfuse_backend)(x)
+    y.float().square().mean().backward()
+    got = {n: p.grad.float().clone() for n, p in m.named_parameters()}
+    m.zero_grad()
+    y_ref = m(x)
+    y_ref.float().square().mean().backward()
+    assert interface.stats["training_graphs"] == before["training_graphs"] + 1
+    assert training.counters["fwd"] == ops_before["fwd"] + 1 and training.counters["bwd"] == ops_before["bwd"] + 1
+    assert (y.float() - y_ref.float()).abs().max() <= 2e-2
+    for n, p in m.named_parameters():
+        ref = p.grad.float()
+        assert ((got[n] - ref).norm() / ref.norm()).item() <= 3e-2, n
