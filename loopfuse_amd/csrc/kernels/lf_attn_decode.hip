@@ -45,6 +45,14 @@
                                 then reads whole pages front to back.  No merge between waves; every
                                 wave writes its own result (nsplit == 1) or partial. */
 #endif
+#ifndef LF_ROWLOAD
+#define LF_ROWLOAD 0         /* 1 (register-staged path, no score bias, K/V dense or in pages of a multiple of 16
+                                tokens): a load instruction reads whole rows -- 64 / (D/8) tokens x D elements,
+                                every 128-byte line in one piece -- with non-temporal loads, and K goes through a
+                                wave-private LDS tile like V.  Lane (token c, 64-byte quarter) loads, which are the
+                                MFMA operand layout, touch half a line per instruction; with non-temporal loads
+                                they would fetch every line twice. */
+#endif
 #define LF_PSTRIDE (LF_HEADWAVE ? 1 : LF_DW)   /* distance between the pairs of steps of one wave */
 #define LF_DT (LF_DW * 64)
 #define LF_D LF_HEAD_DIM
@@ -337,7 +345,7 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 8 / LF_DW) lf_attn_decode(co
   // One buffer, two lives: wave-private V tiles of the pair being consumed
   // ([LF_DW][2][16*D] elements) during the loop, merge buffer
   // ([LF_DW][16][LF_OSTRIDE] floats) after it.
-  constexpr int kVBytes = LF_DW * 2 * 16 * LF_D * 2;
+  constexpr int kVBytes = LF_DW * 2 * 16 * LF_D * 2 * (LF_ROWLOAD ? 2 : 1);   // wave-private V (and K) tiles of a pair
   constexpr int kOBytes = LF_DW * LF_QROWS * LF_OSTRIDE * 4;
   __shared__ __attribute__((aligned(16))) unsigned char smem[kVBytes > kOBytes ? kVBytes : kOBytes];
 #if !LF_HEADWAVE
@@ -459,6 +467,27 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 8 / LF_DW) lf_attn_decode(co
                             (long long)(row0 + min(c, nrows - 1)) * p.bias_sq;
 #endif
   auto issue = [&](LfDecStage& sg, int st, const LfDecIds& id) {
+#if LF_ROWLOAD
+    // load u of the step: tokens kTokPerLoad*u .. +kTokPerLoad-1, lane = (token, 16-byte piece of its row)
+    constexpr int kCpr = LF_D / 8, kTokPerLoad = 64 / kCpr;
+    static_assert(kTokPerLoad * LF_NJ == 16, "LF_NJ loads cover the 16 tokens of a step");
+    const int lt = lane / kCpr, piece = lane % kCpr;
+#pragma unroll
+    for (int u = 0; u < LF_NJ; ++u) {
+      const int tok = min(step_tok0(st) + kTokPerLoad * u + lt, p.Sk - 1);   // clamp: masked later, never out of bounds
+      const lf_elem *kp, *vp;
+      if (kPagedK)
+        kp = p.k + id.k * p.k_sb + (long long)(tok % LF_PAGE_SIZE) * p.k_ss + (long long)hkv * p.k_sh;
+      else
+        kp = p.k + (long long)b * p.k_sb + (long long)hkv * p.k_sh + (long long)tok * p.k_ss;
+      if (kPagedV)
+        vp = p.v + id.v * p.v_sb + (long long)(tok % LF_PAGE_SIZE_V) * p.v_ss + (long long)hkv * p.v_sh;
+      else
+        vp = p.v + (long long)b * p.v_sb + (long long)hkv * p.v_sh + (long long)tok * p.v_ss;
+      sg.k[u] = __builtin_nontemporal_load(reinterpret_cast<const lf_u32x4*>(kp + 8 * piece));
+      sg.v[u] = __builtin_nontemporal_load(reinterpret_cast<const lf_u32x4*>(vp + 8 * piece));
+    }
+#else
     const int tok = min(step_tok0(st) + c, p.Sk - 1);      // clamp: masked later, never out of bounds
     const lf_elem *kp, *vp;
     if (kPagedK)
@@ -473,6 +502,7 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 8 / LF_DW) lf_attn_decode(co
     for (int j = 0; j < LF_NJ; ++j) sg.k[j] = *reinterpret_cast<const lf_u32x4*>(kp + 32 * j);
 #pragma unroll
     for (int j = 0; j < LF_NJ; ++j) sg.v[j] = *reinterpret_cast<const lf_u32x4*>(vp + 32 * j);
+#endif
 #if LF_BIAS
     {
       // keys past Sk read clamped positions: their scores are masked in consume()
@@ -487,7 +517,27 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 8 / LF_DW) lf_attn_decode(co
 #endif
   };
 
-  lf_elem* my_v = reinterpret_cast<lf_elem*>(smem) + wave * 2 * 16 * LF_D;
+  lf_elem* my_v = reinterpret_cast<lf_elem*>(smem) + wave * 2 * 16 * LF_D * (LF_ROWLOAD ? 2 : 1);
+#if LF_ROWLOAD
+  lf_elem* my_k = my_v + 2 * 16 * LF_D;
+  // rows as loaded -> the wave-private tiles of step hsel: V with the chunk swizzle of the
+  // transposed reads below, K with chunk ^ (row & (chunks - 1)) so that the 16 rows one
+  // ds_read_b128 of a fragment touches lie on different banks
+  auto stash_kv = [&](const LfDecStage& sg, int hsel) {
+    constexpr int kCpr = LF_D / 8, kTokPerLoad = 64 / kCpr;
+    const int lt = lane / kCpr, piece = lane % kCpr;
+#pragma unroll
+    for (int u = 0; u < LF_NJ; ++u) {
+      const int row = kTokPerLoad * u + lt;
+      *reinterpret_cast<lf_u32x4*>(&my_v[hsel * 16 * LF_D + row * LF_D + 8 * (piece ^ (2 * (row & 3)))]) = sg.v[u];
+      *reinterpret_cast<lf_u32x4*>(&my_k[hsel * 16 * LF_D + row * LF_D + 8 * (piece ^ (row & (kCpr - 1)))]) = sg.k[u];
+    }
+  };
+  auto k_frag = [&](int hsel, int j) {      // A operand of k-step j: lane (token c, g) holds d = 32 j + 8 g .. +7
+    constexpr int kCpr = LF_D / 8;
+    return *reinterpret_cast<const lf_u32x4*>(&my_k[hsel * 16 * LF_D + c * LF_D + 8 * ((4 * j + g) ^ (c & (kCpr - 1)))]);
+  };
+#endif
   // V rows of a step -> wave-private LDS tile hsel (row = token c, 16-byte chunk
   // 4j+g, chunk index XORed with 2*(row&3) so that the 4 rows a transposed read
   // touches sit on different banks)
@@ -502,6 +552,15 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 8 / LF_DW) lf_attn_decode(co
   // ---- one pair of steps (32 tokens)
   auto consume = [&](const LfDecStage& sa, const LfDecStage& sb, int pr) {
     lf_f32x4 xa = {0.0f, 0.0f, 0.0f, 0.0f}, xb = {0.0f, 0.0f, 0.0f, 0.0f};
+#if LF_ROWLOAD
+    stash_kv(sa, 0);
+    stash_kv(sb, 1);
+#pragma unroll
+    for (int j = 0; j < LF_NJ; ++j) {
+      xa = lf_mfma16(__builtin_bit_cast(lf_elem8, k_frag(0, j)), qb[j], xa);
+      xb = lf_mfma16(__builtin_bit_cast(lf_elem8, k_frag(1, j)), qb[j], xb);
+    }
+#else
 #pragma unroll
     for (int j = 0; j < LF_NJ; ++j) {
       xa = lf_mfma16(__builtin_bit_cast(lf_elem8, sa.k[j]), qb[j], xa);
@@ -509,6 +568,7 @@ extern "C" __global__ void __launch_bounds__(LF_DT, 8 / LF_DW) lf_attn_decode(co
     }
     stash_v(sa, 0);
     stash_v(sb, 1);
+#endif
 
     // lane (q = c, g): xa[i] is token t0 + i, xb[i] token t0 + 16 + i
     const int t0 = step_tok0(2 * pr) + 4 * g;

@@ -72,6 +72,7 @@ class KernelSpec:
     v_tr: bool = True      # prefill: transposed LDS reads for V
     headwave: bool = False  # decode: one kv head per wave (8 waves) instead of 4 waves sharing a head
     coop: bool = False     # decode, headwave: the workgroup loads whole 16-token blocks, rows reach the waves through LDS
+    rowload: bool = False  # decode, register-staged path: whole-row non-temporal loads, K through a wave-private LDS tile
     denom: bool = False    # prefill: softmax denominator sum + c (c a run-time parameter)
     bias: int = 0          # prefill: bit 0 additive score bias tensor, bit 1 additive output bias tensor, bit 2 unaligned rows
     pack: int = 0          # prefill_swp, grouped-query attention: a workgroup's waves take 2 or 4 heads of one group
@@ -96,6 +97,8 @@ class KernelSpec:
             o += [f"-DLF_DW={self.waves}", f"-DLF_HEADWAVE={int(self.headwave)}"]
             if self.coop:
                 o += ["-DLF_COOP=1"]
+            if self.rowload:
+                o += ["-DLF_ROWLOAD=1"]
             if self.bias:
                 o += ["-DLF_BIAS=1"]
         elif self.family == "prefill":
@@ -124,7 +127,7 @@ class KernelSpec:
         return (f"lf_{self.family}_t{self.dtype}_d{self.head_dim}_m{self.mask}_c{int(self.softcap)}"
                 f"_p{self.paged}x{self.page_size}i{int(self.table_i64)}_r{self.rows}w{self.waves}v{int(self.v_tr)}h{int(self.headwave)}b{self.bias}n{int(self.denom)}"
                 + (f"_q{self.d2}" if self.d2 else "") + (f"_gp{int(self.pack)}" if self.pack else "") + (f"_pv{self.page_size_v}" if self.page_size_v else "")
-                + ("_z" if self.safe else "") + ("_co" if self.coop else "")
+                + ("_z" if self.safe else "") + ("_co" if self.coop else "") + ("_rl" if self.rowload else "")
                 + "".join("_" + e.replace("-D", "").replace("=", "") for e in self.extra))
 
     def source(self) -> str:
@@ -320,6 +323,16 @@ def _decode_coop(headwave: bool, page_size: int, page_size_v: int, bias_bits: in
     if os.environ.get("LOOPFUSE_DECODE_COOP", "1") != "1":
         return False
     return headwave and page_size % 16 == 0 and not page_size_v and not bias_bits and Hkv % waves == 0
+
+
+def _decode_rowload(paged: int, page_size: int, page_size_v: int, bias_bits: int) -> bool:
+    """The register-staged decode path reads whole rows (every 128-byte line in one piece) with
+    non-temporal loads and passes K through a wave-private LDS tile (``-DLF_ROWLOAD=1``) when a
+    16-token step lies inside one page (or K/V are dense) and there is no score bias.
+    LOOPFUSE_DECODE_ROWLOAD=0 keeps the loads in MFMA operand layout."""
+    if os.environ.get("LOOPFUSE_DECODE_ROWLOAD", "1") != "1" or bias_bits:
+        return False
+    return not paged or (page_size % 16 == 0 and (page_size_v or page_size) % 16 == 0)
 
 
 def prefill_variant(Sq: int, v_tr: bool = True) -> str:
@@ -788,7 +801,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     P.rows, P.nsplit, P.split_len = rows, nsplit, split_len
     spec = KernelSpec("decode", _DTYPE_CODE[dtype], D, MASK_NONE, plan.softcap is not None, paged,
                       page_size, table_i64, rows=DECODE_QROWS, waves=waves, headwave=headwave, page_size_v=page_size_v,
-                      coop=_decode_coop(headwave, page_size, page_size_v, bias_bits, Hkv, waves),
+                      coop=(coop := _decode_coop(headwave, page_size, page_size_v, bias_bits, Hkv, waves)),
+                      rowload=not coop and _decode_rowload(paged, page_size, page_size_v, bias_bits),
                       bias=bias_bits, safe=plan.zero_blind_rows and bool(bias_bits),
                       extra=tuple(os.environ.get("LOOPFUSE_KOPTS", "").split()))
     rows_per_block = 1024 // D       # combine kernel: 256 threads, 4 consecutive d each
