@@ -42,6 +42,9 @@ struct LfAttnBwdParams {
 };
 
 #define LF_BW_NT 256
+#ifndef LF_BW_DQ_NT
+#define LF_BW_DQ_NT 512     /* threads of lf_attn_bwd_dq: 8 waves x 32 query rows, two waves per SIMD */
+#endif
 
 // delta[row] = sum_d dO[row][d] * O[row][d]; 16 lanes per row, 8 elements per lane
 extern "C" __global__ void __launch_bounds__(LF_BW_NT) lf_attn_bwd_delta(const LfAttnBwdParams p) {
@@ -65,36 +68,27 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT) lf_attn_bwd_delta(const L
   if (row < nrows && piece == 0) p.delta[row] = s;
 }
 
-// A 64-row tile of a [rows, D] matrix (row stride `ss`) on its way into LDS: 64 * LF_CPR / NT
-// 16-byte pieces per thread of a workgroup of NT threads.  Loads and LDS writes are separate
-// steps so that the loads of the next tile travel while the current one is being consumed;
-// rows past `nrows` arrive as zeros.
+// A 64-row tile of a [rows, D] matrix goes global -> LDS directly (buffer_load ... lds, the
+// forward's staging): per pass the workgroup's NT threads move NT / LF_CPR whole rows, a wave
+// 64 lanes x 16 B that land contiguously; the XOR swizzle of the K layout (`tr` false:
+// ds_read_b128, tile rows = MFMA rows) or of the V layout (`tr` true: transposed reads, tile
+// rows = MFMA k) is applied on the global side.  `rs` covers rows 0 .. nrows-1 of the matrix
+// (row stride `rowb` bytes): rows past the end get an offset beyond it and arrive as zeros.
+// Not tracked by the compiler's wait counters: callers wait with s_waitcnt vmcnt(0).
 template <int NT>
-struct LfBwTile {
-  lf_u32x4 piece[64 * LF_CPR / NT];
-};
-template <int NT>
-__device__ __forceinline__ void lf_bw_load(LfBwTile<NT>& t, const lf_elem* src, long long ss, int row0, int nrows, int tid) {
+__device__ __forceinline__ void lf_bw_dma_tile(const lf_u32x4& rs, unsigned rowb, int row0, lf_elem* tile, bool tr,
+                                               int tid, int wave) {
+  constexpr int kRowsPerPass = NT / LF_CPR, kRowsPerWave = 64 / LF_CPR;
+  const int srow = tid / LF_CPR, sch = tid % LF_CPR;
 #pragma unroll
-  for (int u = 0; u < 64 * LF_CPR / NT; ++u) {
-    const int piece = tid + NT * u;
-    const int r = piece / LF_CPR, ch = piece % LF_CPR;
-    t.piece[u] = lf_u32x4{0u, 0u, 0u, 0u};
-    if (row0 + r < nrows) t.piece[u] = *reinterpret_cast<const lf_u32x4*>(src + (long long)(row0 + r) * ss + 8 * ch);
+  for (int ps = 0; ps < 64 / kRowsPerPass; ++ps) {
+    const int r = kRowsPerPass * ps + srow;
+    const unsigned off = (unsigned)(row0 + r) * rowb + 16u * (unsigned)(tr ? lf_v_phys(r, sch) : lf_k_phys(r, sch));
+    lf_dma_to_lds(rs, off, &tile[(kRowsPerPass * ps + kRowsPerWave * wave) * LF_D]);
   }
 }
-// into the K layout (`rm`: ds_read_b128, tile rows = MFMA rows) and / or the V layout (`tr`:
-// transposed reads, tile rows = MFMA k)
-template <int NT>
-__device__ __forceinline__ void lf_bw_store(const LfBwTile<NT>& t, lf_elem* rm, lf_elem* tr, int tid) {
-#pragma unroll
-  for (int u = 0; u < 64 * LF_CPR / NT; ++u) {
-    const int piece = tid + NT * u;
-    const int r = piece / LF_CPR, ch = piece % LF_CPR;
-    if (rm != nullptr) *reinterpret_cast<lf_u32x4*>(&rm[r * LF_D + 8 * lf_k_phys(r, ch)]) = t.piece[u];
-    if (tr != nullptr) *reinterpret_cast<lf_u32x4*>(&tr[r * LF_D + 8 * lf_v_phys(r, ch)]) = t.piece[u];
-  }
-}
+// wait for this wave's direct loads and LDS writes, then meet the other waves
+#define LF_BW_BARRIER() asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory")
 
 // Fragment read-ahead of the two product loops (LDS reads in flight ahead of the MFMA that
 // consumes them; the order of reads and MFMAs is pinned with scheduling barriers, left to
@@ -128,12 +122,10 @@ __device__ __forceinline__ void lf_bw_store_rows(const lf_f32x16* acc, lf_elem* 
 }
 
 extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const LfAttnBwdParams p) {
-  __shared__ __attribute__((aligned(16))) lf_elem q_rm[64 * LF_D];
-  __shared__ __attribute__((aligned(16))) lf_elem q_tr[64 * LF_D];
-  __shared__ __attribute__((aligned(16))) lf_elem g_rm[64 * LF_D];     // dO
-  __shared__ __attribute__((aligned(16))) lf_elem g_tr[64 * LF_D];
-  __shared__ __attribute__((aligned(16))) float lse_s[64];
-  __shared__ __attribute__((aligned(16))) float delta_s[64];
+  // two stages of: Q tile in both layouts, dO tile in both layouts, L and delta of the 64 rows
+  __shared__ __attribute__((aligned(16))) lf_elem tiles[2][4][64 * LF_D];
+  __shared__ __attribute__((aligned(16))) float lse_st[2][64];
+  __shared__ __attribute__((aligned(16))) float delta_st[2][64];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -181,35 +173,51 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
 #endif
 
   // the steps of this workgroup: query heads of the group x q tiles, one flat sequence; the
-  // global loads of step it + 1 are issued before step it is computed
+  // direct loads of step it + 1 fill the other stage while step it is computed
   const int ntq = max(qt_end - qt_begin, 0);
   const int nsteps = group * ntq;
-  LfBwTile<LF_BW_NT> tq, tg;
+  const unsigned q_bytes = (unsigned)(((long long)(p.Sq - 1) * p.q_ss + LF_D) * 2);
+  const unsigned g_bytes = (unsigned)(((long long)(p.Sq - 1) * p.do_ss + LF_D) * 2);
+  const int wave_u = wave;
   float r_lse = 0.0f, r_delta = 0.0f;
-  auto issue = [&](int it) {
+  auto issue = [&](int it, int st) {
     const int h = hkv * group + it / ntq;
     const int q0 = 64 * (qt_begin + it % ntq);
-    lf_bw_load(tq, p.q + (long long)b * p.q_sb + (long long)h * p.q_sh, p.q_ss, q0, p.Sq, tid);
-    lf_bw_load(tg, p.dout + (long long)b * p.do_sb + (long long)h * p.do_sh, p.do_ss, q0, p.Sq, tid);
-    if (tid < 64) {
+    const lf_u32x4 q_rs = lf_make_buffer(p.q + (long long)b * p.q_sb + (long long)h * p.q_sh, q_bytes);
+    const lf_u32x4 g_rs = lf_make_buffer(p.dout + (long long)b * p.do_sb + (long long)h * p.do_sh, g_bytes);
+    lf_bw_dma_tile<LF_BW_NT>(q_rs, (unsigned)p.q_ss * 2u, q0, tiles[st][0], false, tid, wave_u);
+    lf_bw_dma_tile<LF_BW_NT>(q_rs, (unsigned)p.q_ss * 2u, q0, tiles[st][1], true, tid, wave_u);
+    lf_bw_dma_tile<LF_BW_NT>(g_rs, (unsigned)p.do_ss * 2u, q0, tiles[st][2], false, tid, wave_u);
+    lf_bw_dma_tile<LF_BW_NT>(g_rs, (unsigned)p.do_ss * 2u, q0, tiles[st][3], true, tid, wave_u);
+    if (tid < 64) {            // into registers now, into the stage just before the barrier that opens it
       const long long r = ((long long)b * p.Hq + h) * p.Sq + q0 + tid;
       const bool in = q0 + tid < p.Sq;
-      r_lse = in ? p.lse[r] : __builtin_inff();            // rows past Sq: P = 0
+      r_lse = in ? p.lse[r] : __builtin_inff();                      // rows past Sq: P = 0
       r_delta = in ? p.delta[r] : 0.0f;
     }
   };
-  if (nsteps > 0) issue(0);
-  for (int it = 0; it < nsteps; ++it) {
-    const int q0 = 64 * (qt_begin + it % ntq);
-    __syncthreads();            // the previous step's reads are done
-    lf_bw_store(tq, q_rm, q_tr, tid);
-    lf_bw_store(tg, g_rm, g_tr, tid);
+  auto publish = [&](int st) {
     if (tid < 64) {
-      lse_s[tid] = r_lse;
-      delta_s[tid] = r_delta;
+      lse_st[st][tid] = r_lse;
+      delta_st[st][tid] = r_delta;
     }
-    __syncthreads();
-    if (it + 1 < nsteps) issue(it + 1);
+  };
+  if (nsteps > 0) {
+    issue(0, 0);
+    publish(0);
+  }
+  LF_BW_BARRIER();
+  for (int it = 0; it < nsteps; ++it) {
+    const int st = it & 1;
+    const int q0 = 64 * (qt_begin + it % ntq);
+    const lf_elem* q_rm = tiles[st][0];
+    const lf_elem* q_tr = tiles[st][1];
+    const lf_elem* g_rm = tiles[st][2];
+    const lf_elem* g_tr = tiles[st][3];
+    const float* lse_s = lse_st[st];
+    const float* delta_s = delta_st[st];
+    // the other stage was last read in step it - 1, which every wave left at the barrier below
+    if (it + 1 < nsteps) issue(it + 1, st ^ 1);
 
     bool need = key0 < p.Sk;
 #if LF_MASK >= 1
@@ -218,7 +226,7 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
 #if LF_MASK == 2
     need = need && (q0 - min(key0 + 31, p.Sk - 1) < p.window);
 #endif
-    if (!need) continue;        // wave-uniform; the barriers above are reached by every wave
+    if (need) {                 // wave-uniform
 
     lf_elem8 pf[LF_NKK], dsf[LF_NKK];
 #pragma unroll
@@ -281,6 +289,9 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+    }   // need
+    if (it + 1 < nsteps) publish(st ^ 1);
+    LF_BW_BARRIER();            // the next stage has landed; every wave is done with this one
   }
 
   const bool valid = my_key < p.Sk;
@@ -289,10 +300,9 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
   lf_bw_store_rows(dv, p.dv + (long long)b * p.dv_sb + (long long)hkv * p.dv_sh + (long long)kr * p.dv_ss, valid, g);
 }
 
-extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dq(const LfAttnBwdParams p) {
-  __shared__ __attribute__((aligned(16))) lf_elem k_rm[64 * LF_D];
-  __shared__ __attribute__((aligned(16))) lf_elem k_tr[64 * LF_D];
-  __shared__ __attribute__((aligned(16))) lf_elem v_rm[64 * LF_D];
+extern "C" __global__ void __launch_bounds__(LF_BW_DQ_NT, LF_BW_DQ_NT / 256) lf_attn_bwd_dq(const LfAttnBwdParams p) {
+  // two stages of: K tile in both layouts, V tile in the K layout
+  __shared__ __attribute__((aligned(16))) lf_elem tiles[2][3][64 * LF_D];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -300,13 +310,14 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dq(const L
   const int l32 = lane & 31;
   const int g = lane >> 5;
 
-  const int nqt = (p.Sq + 127) / 128;
+  constexpr int kBM = LF_BW_DQ_NT / 2;                    // query rows of a workgroup
+  const int nqt = (p.Sq + kBM - 1) / kBM;
   const int qt = nqt - 1 - (int)(blockIdx.x % nqt);       // long q tiles first
   const int bh = blockIdx.x / nqt;
   const int h = bh % p.Hq;
   const int b = bh / p.Hq;
   const int hkv = h / (p.Hq / p.Hkv);
-  const int q0 = 128 * qt;
+  const int q0 = kBM * qt;
   const int wq0 = q0 + 32 * wave;
   const int my_q = wq0 + l32;
   const int qr = min(my_q, p.Sq - 1);
@@ -335,7 +346,7 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dq(const L
 
   int kt_begin = 0, kt_end = nkt;
   {
-    const int qlast = min(q0 + 128, p.Sq) - 1;
+    const int qlast = min(q0 + kBM, p.Sq) - 1;
 #if LF_MASK >= 1
     kt_end = min(nkt, qlast / 64 + 1);
 #endif
@@ -347,21 +358,22 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dq(const L
   }
   const lf_elem* kbase = p.k + (long long)b * p.k_sb + (long long)hkv * p.k_sh;
   const lf_elem* vbase = p.v + (long long)b * p.v_sb + (long long)hkv * p.v_sh;
-  LfBwTile<LF_BW_NT> tk, tv;
-  if (kt_begin < kt_end) {
-    lf_bw_load(tk, kbase, p.k_ss, 64 * kt_begin, p.Sk, tid);
-    lf_bw_load(tv, vbase, p.v_ss, 64 * kt_begin, p.Sk, tid);
-  }
+  const lf_u32x4 k_rs = lf_make_buffer(kbase, (unsigned)(((long long)(p.Sk - 1) * p.k_ss + LF_D) * 2));
+  const lf_u32x4 v_rs = lf_make_buffer(vbase, (unsigned)(((long long)(p.Sk - 1) * p.v_ss + LF_D) * 2));
+  auto issue = [&](int kt, int st) {
+    lf_bw_dma_tile<LF_BW_DQ_NT>(k_rs, (unsigned)p.k_ss * 2u, 64 * kt, tiles[st][0], false, tid, wave);
+    lf_bw_dma_tile<LF_BW_DQ_NT>(k_rs, (unsigned)p.k_ss * 2u, 64 * kt, tiles[st][1], true, tid, wave);
+    lf_bw_dma_tile<LF_BW_DQ_NT>(v_rs, (unsigned)p.v_ss * 2u, 64 * kt, tiles[st][2], false, tid, wave);
+  };
+  if (kt_begin < kt_end) issue(kt_begin, 0);
+  LF_BW_BARRIER();
   for (int kt = kt_begin; kt < kt_end; ++kt) {
     const int k0 = 64 * kt;
-    __syncthreads();
-    lf_bw_store(tk, k_rm, k_tr, tid);
-    lf_bw_store(tv, v_rm, nullptr, tid);
-    __syncthreads();
-    if (kt + 1 < kt_end) {      // the next tile's loads travel during this tile's products
-      lf_bw_load(tk, kbase, p.k_ss, k0 + 64, p.Sk, tid);
-      lf_bw_load(tv, vbase, p.v_ss, k0 + 64, p.Sk, tid);
-    }
+    const int st = (kt - kt_begin) & 1;
+    const lf_elem* k_rm = tiles[st][0];
+    const lf_elem* k_tr = tiles[st][1];
+    const lf_elem* v_rm = tiles[st][2];
+    if (kt + 1 < kt_end) issue(kt + 1, st ^ 1);     // fills the stage every wave left at the last barrier
 
     bool need = wq0 < p.Sq;
 #if LF_MASK >= 1
@@ -370,7 +382,7 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dq(const L
 #if LF_MASK == 2
     need = need && (min(k0 + 64, p.Sk) - 1 >= wq0 - p.window + 1);
 #endif
-    if (!need) continue;
+    if (need) {
 
     lf_elem8 dsf[LF_NKK];
 #pragma unroll
@@ -417,6 +429,8 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dq(const L
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+    }   // need
+    LF_BW_BARRIER();
   }
   lf_bw_store_rows(dq, p.dq + (long long)b * p.dq_sb + (long long)h * p.dq_sh + (long long)qr * p.dq_ss, my_q < p.Sq, g);
 }

@@ -845,8 +845,15 @@ class AttnBwdParams(ctypes.Structure):
     )
 
 
+def bwd_dq_threads(mask: int) -> int:
+    """Workgroup size of lf_attn_bwd_dq: 8 waves (256 query rows, two waves per SIMD on one K/V
+    tile stream) except under a sliding window, where a 256-row tile walks too many kv tiles
+    that only part of its rows can see."""
+    return 256 if mask == MASK_SLIDING else 512
+
+
 def bwd_spec(dtype: torch.dtype, D: int, mask: int) -> KernelSpec:
-    return KernelSpec("bwd", _DTYPE_CODE[dtype], D, mask)
+    return KernelSpec("bwd", _DTYPE_CODE[dtype], D, mask, extra=(f"-DLF_BW_DQ_NT={bwd_dq_threads(mask)}",))
 
 
 def attention_backward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor, lse: torch.Tensor,
@@ -882,6 +889,11 @@ def attention_backward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: tor
         raise UnsupportedPlan("sliding window must be >= 1")
     for name, t in (("Q", q), ("K", k), ("V", v), ("O", o), ("dO", dout)):
         _check_tensor(name, t, dtype)
+    # the tiles travel global -> LDS with 32-bit byte offsets inside one (batch, head) span, rows
+    # past the end addressed too (and range-checked to zeros)
+    for name, t, S in (("Q", q, Sq), ("dO", dout, Sq), ("K", k, Sk), ("V", v, Sk)):
+        if t.stride(2) < D or (S + 64) * t.stride(2) * 2 + 2 * D >= (1 << 32):
+            raise UnsupportedPlan(f"{name}: row stride {t.stride(2)} not served by the backward kernels' direct loads")
     dq = torch.empty((B, Hq, Sq, D), dtype=dtype, device=q.device)
     dk = torch.empty((B, Hkv, Sk, D), dtype=dtype, device=q.device)
     dv = torch.empty((B, Hkv, Sk, D), dtype=dtype, device=q.device)
@@ -901,6 +913,7 @@ def attention_backward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: tor
     rows = B * Hq * Sq
     get_kernel(spec, "lf_attn_bwd_delta").launch(((rows + 15) // 16, 1, 1), (256, 1, 1), P)
     get_kernel(spec, "lf_attn_bwd_dkdv").launch((B * Hkv * ((Sk + 127) // 128), 1, 1), (256, 1, 1), P)
-    get_kernel(spec, "lf_attn_bwd_dq").launch((B * Hq * ((Sq + 127) // 128), 1, 1), (256, 1, 1), P)
+    nt = bwd_dq_threads(mask)
+    get_kernel(spec, "lf_attn_bwd_dq").launch((B * Hq * ((Sq + nt // 2 - 1) // (nt // 2)), 1, 1), (nt, 1, 1), P)
     _last_launch.set({"kernels": ["lf_attn_bwd_delta", "lf_attn_bwd_dkdv", "lf_attn_bwd_dq"]})
     return dq, dk, dv
