@@ -56,6 +56,43 @@ typedef struct LfAttnParamsHost {
   float denom_add;            /* LF_DENOM: softmax denominator is sum + denom_add */
 } LfAttnParamsHost;
 
+/*
+ * Parameter block of the backward kernels lf_attn_bwd_delta, lf_attn_bwd_dkdv and
+ * lf_attn_bwd_dq (loopfuse_amd/csrc/kernels/lf_attn_bwd.hip, `struct LfAttnBwdParams`;
+ * loopfuse_amd/lowering.py::AttnBwdParams is the ctypes mirror).  The three kernels take
+ * the same block and run in that order on one stream.  The reference has no backward:
+ * its backend traces inference graphs only (reference loopfuse/torch_backend/interface.py:600-621).
+ */
+typedef struct LfAttnBwdParamsHost {
+  const void* q;        /* Q [B, Hq, Sq, D] */
+  const void* k;        /* K [B, Hkv, Sk, D] */
+  const void* v;
+  const void* o;        /* the forward's output */
+  const void* dout;     /* gradient of the output */
+  void* dq;
+  void* dk;             /* [B, Hkv, Sk, D]: summed over the query heads of a group */
+  void* dv;
+  const float* lse;     /* [B, Hq, Sq] row log-sum-exp of the scaled, masked scores in log2 units (part_ml of the forward) */
+  float* delta;         /* [B, Hq, Sq] scratch, written by lf_attn_bwd_delta */
+  int64_t q_sb, q_sh, q_ss;
+  int64_t k_sb, k_sh, k_ss;
+  int64_t v_sb, v_sh, v_ss;
+  int64_t o_sb, o_sh, o_ss;
+  int64_t do_sb, do_sh, do_ss;
+  int64_t dq_sb, dq_sh, dq_ss;
+  int64_t dk_sb, dk_sh, dk_ss;
+  int64_t dv_sb, dv_sh, dv_ss;
+  int32_t B, Hq, Hkv, Sq, Sk;
+  int32_t window;       /* sliding-window width (LF_MASK == 2) */
+  float scale;
+} LfAttnBwdParamsHost;
+
+#ifdef __cplusplus
+static_assert(sizeof(LfAttnBwdParamsHost) == 304, "LfAttnBwdParamsHost must match the device struct");
+#else
+_Static_assert(sizeof(LfAttnBwdParamsHost) == 304, "LfAttnBwdParamsHost must match the device struct");
+#endif
+
 #ifdef __cplusplus
 static_assert(sizeof(LfAttnParamsHost) == 376, "LfAttnParamsHost must match the device struct");
 }

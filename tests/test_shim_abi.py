@@ -78,29 +78,34 @@ def test_params_struct_layout():
     assert ctypes.sizeof(AttnParams) == 376
 
 
-def test_c_header_matches_the_ctypes_mirror_and_the_device_struct(tmp_path):
-    """include/lf_attn_params.h (C hosts), lowering.AttnParams (ctypes) and struct
-    LfAttnParams (device) list the same fields at the same offsets."""
+@pytest.mark.parametrize("host,mirror,device,source", [
+    ("LfAttnParamsHost", "AttnParams", "LfAttnParams", "lf_common.hip.h"),
+    ("LfAttnBwdParamsHost", "AttnBwdParams", "LfAttnBwdParams", "lf_attn_bwd.hip"),
+])
+def test_c_header_matches_the_ctypes_mirror_and_the_device_struct(tmp_path, host, mirror, device, source):
+    """include/lf_attn_params.h (C hosts), the ctypes structure of lowering.py and the device
+    struct list the same fields at the same offsets."""
     import subprocess
 
-    from loopfuse_amd.lowering import AttnParams
+    from loopfuse_amd import lowering
 
-    names = [n for n, _ in AttnParams._fields_]
+    mirror = getattr(lowering, mirror)
+    names = [n for n, _ in mirror._fields_]
     prog = "#include <stdio.h>\n#include <stddef.h>\n#include \"lf_attn_params.h\"\nint main(void) {\n"
     for n in names:
-        prog += f'  printf("{n} %zu\\n", offsetof(LfAttnParamsHost, {n}));\n'
-    prog += '  printf("sizeof %zu\\n", sizeof(LfAttnParamsHost));\n  return 0;\n}\n'
+        prog += f'  printf("{n} %zu\\n", offsetof({host}, {n}));\n'
+    prog += f'  printf("sizeof %zu\\n", sizeof({host}));\n  return 0;\n}}\n'
     src = tmp_path / "off.c"
     src.write_text(prog)
     exe = tmp_path / "off"
     subprocess.run(["gcc", "-std=c11", "-I" + os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
     out = dict(line.split() for line in subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.splitlines())
     for n in names:
-        assert int(out[n]) == getattr(AttnParams, n).offset, n
-    assert int(out["sizeof"]) == ctypes.sizeof(AttnParams)
+        assert int(out[n]) == getattr(mirror, n).offset, n
+    assert int(out["sizeof"]) == ctypes.sizeof(mirror)
     # the device struct declares the same field names in the same order
-    dev = open(os.path.join(ROOT, "loopfuse_amd", "csrc", "kernels", "lf_common.hip.h")).read()
-    body = dev[dev.index("struct LfAttnParams {"):]
+    dev = open(os.path.join(ROOT, "loopfuse_amd", "csrc", "kernels", source)).read()
+    body = dev[dev.index("struct %s {" % device):]
     body = re.sub(r"//[^\n]*", "", body[:body.index("};")])
     fields = []
     for decl in body.split("{", 1)[1].split(";"):
