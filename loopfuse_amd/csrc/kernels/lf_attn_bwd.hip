@@ -76,25 +76,66 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT) lf_attn_bwd_delta(const L
 // (row stride `rowb` bytes): rows past the end get an offset beyond it and arrive as zeros.
 // Not tracked by the compiler's wait counters: callers wait with s_waitcnt vmcnt(0).
 template <int NT>
-__device__ __forceinline__ void lf_bw_dma_tile(const lf_u32x4& rs, unsigned rowb, int row0, lf_elem* tile, bool tr,
-                                               int tid, int wave) {
+__device__ __forceinline__ void lf_bw_dma_piece(const lf_u32x4& rs, unsigned rowb, int row0, lf_elem* tile, bool tr,
+                                                int ps, int tid, int wave) {
   constexpr int kRowsPerPass = NT / LF_CPR, kRowsPerWave = 64 / LF_CPR;
   const int srow = tid / LF_CPR, sch = tid % LF_CPR;
-#pragma unroll
-  for (int ps = 0; ps < 64 / kRowsPerPass; ++ps) {
-    const int r = kRowsPerPass * ps + srow;
-    const unsigned off = (unsigned)(row0 + r) * rowb + 16u * (unsigned)(tr ? lf_v_phys(r, sch) : lf_k_phys(r, sch));
-    lf_dma_to_lds(rs, off, &tile[(kRowsPerPass * ps + kRowsPerWave * wave) * LF_D]);
-  }
+  const int r = kRowsPerPass * ps + srow;
+  const unsigned off = (unsigned)(row0 + r) * rowb + 16u * (unsigned)(tr ? lf_v_phys(r, sch) : lf_k_phys(r, sch));
+  lf_dma_to_lds(rs, off, &tile[(kRowsPerPass * ps + kRowsPerWave * wave) * LF_D]);
 }
-// wait for this wave's direct loads and LDS writes, then meet the other waves
-#define LF_BW_BARRIER() asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory")
+template <int NT>
+__device__ __forceinline__ void lf_bw_dma_tile(const lf_u32x4& rs, unsigned rowb, int row0, lf_elem* tile, bool tr,
+                                               int tid, int wave) {
+#pragma unroll
+  for (int ps = 0; ps < 64 * LF_CPR / NT; ++ps) lf_bw_dma_piece<NT>(rs, rowb, row0, tile, tr, ps, tid, wave);
+}
+// wait for this wave's direct loads and LDS writes, then meet the other waves.  The wait is the
+// builtin, not inline asm, so that the compiler's wait-counter pass sees that nothing is
+// outstanding afterwards: otherwise it waits again inside the step -- for the operands loaded
+// before the loop and before overwriting a register a tracked load wrote -- with vmcnt values
+// that also drain the direct loads of the next stage just issued (0x0070: vmcnt(0) lgkmcnt(0))
+#define LF_BW_BARRIER()                      \
+  do {                                       \
+    asm volatile("" ::: "memory");           \
+    __builtin_amdgcn_s_waitcnt(0x0070);      \
+    __builtin_amdgcn_s_barrier();            \
+    asm volatile("" ::: "memory");           \
+  } while (0)
 
 // Fragment read-ahead of the two product loops (LDS reads in flight ahead of the MFMA that
 // consumes them; the order of reads and MFMAs is pinned with scheduling barriers, left to
 // itself the compiler issues read, wait, MFMA one after the other)
 #define LF_BW_PF1 3      /* first products: pairs of K-layout fragments */
 #define LF_BW_PF2 4      /* second products: V-layout fragments */
+
+// MFMAs of lf_attn_bwd_dkdv with the register file of every operand spelled out.  At one wave per
+// SIMD the kernel has 512 registers per lane, and the compiler then gives every MFMA an AGPR
+// destination while keeping what it computes with in VGPRs: left to it, the loop carries hundreds
+// of v_accvgpr moves per step.  Here dK^T / dV^T (written in the loop, read after it) and the
+// loop-invariant K^T / V^T operands live in AGPRs, S^T / dP^T (read by the VALU right away) in VGPRs.
+// What the compiler would otherwise see to: an MFMA result may be read 12 wait states after the MFMA
+// was issued at the earliest (LF_BW_MFMA_DRAIN), and a VGPR written by the VALU may be an MFMA
+// operand 2 wait states later (LF_BW_VALU_SETTLE); back-to-back MFMAs on one accumulator need nothing.
+#if LF_DTYPE == 0
+#define LF_BW_MFMA "v_mfma_f32_32x32x16_bf16"
+#else
+#define LF_BW_MFMA "v_mfma_f32_32x32x16_f16"
+#endif
+#define LF_BW_MFMA_DRAIN "s_nop 9\n\ts_nop 9"
+#define LF_BW_VALU_SETTLE "s_nop 1"
+// c (VGPRs) = a (VGPRs) x b (AGPRs)
+__device__ __forceinline__ void lf_bw_mfma_first(lf_f32x16& c, const lf_u32x4& a, const lf_u32x4& b) {
+  asm volatile(LF_BW_MFMA " %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
+}
+// c (VGPRs) += a (VGPRs) x b (AGPRs)
+__device__ __forceinline__ void lf_bw_mfma_vva(lf_f32x16& c, const lf_u32x4& a, const lf_u32x4& b) {
+  asm volatile(LF_BW_MFMA " %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+}
+// c (AGPRs) += a (VGPRs) x b (VGPRs)
+__device__ __forceinline__ void lf_bw_mfma_avv(lf_f32x16& c, const lf_u32x4& a, const lf_u32x4& b) {
+  asm volatile(LF_BW_MFMA " %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
 
 // accumulators X^T[d][n] (lane n = lane % 32; element i of block db is d = 32*db + 8*(i/4) + 4*g + i%4)
 // -> rows n of a [rows, D] matrix, 16 bytes per store (the exchange of the forward's epilogue)
@@ -143,25 +184,29 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
   const int my_key = key0 + l32;
   const int nqt = (p.Sq + 63) / 64;
 
-  // K^T and V^T of this lane's key as B operands: d = 16*ks + 8*g .. +7
-  lf_elem8 kf[LF_NKS], vf[LF_NKS];
+  // K^T and V^T of this lane's key as B operands (d = 16*ks + 8*g .. +7), parked in AGPRs
+  lf_u32x4 kf[LF_NKS], vf[LF_NKS];
   {
     const int kr = min(my_key, p.Sk - 1);
     const lf_elem* krow = p.k + (long long)b * p.k_sb + (long long)hkv * p.k_sh + (long long)kr * p.k_ss;
     const lf_elem* vrow = p.v + (long long)b * p.v_sb + (long long)hkv * p.v_sh + (long long)kr * p.v_ss;
 #pragma unroll
     for (int ks = 0; ks < LF_NKS; ++ks) {
-      kf[ks] = __builtin_bit_cast(lf_elem8, *reinterpret_cast<const lf_u32x4*>(krow + 16 * ks + 8 * g));
-      vf[ks] = __builtin_bit_cast(lf_elem8, *reinterpret_cast<const lf_u32x4*>(vrow + 16 * ks + 8 * g));
+      kf[ks] = *reinterpret_cast<const lf_u32x4*>(krow + 16 * ks + 8 * g);
+      vf[ks] = *reinterpret_cast<const lf_u32x4*>(vrow + 16 * ks + 8 * g);
     }
+#pragma unroll
+    for (int ks = 0; ks < LF_NKS; ++ks) asm volatile("" : "+a"(kf[ks]), "+a"(vf[ks]));
   }
   const float cexp = p.scale * LF_LOG2E;
 
   lf_f32x16 dk[LF_NDB], dv[LF_NDB];
 #pragma unroll
-  for (int db = 0; db < LF_NDB; ++db)
+  for (int db = 0; db < LF_NDB; ++db) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) dk[db][i] = dv[db][i] = 0.0f;
+    asm volatile("" : "+a"(dk[db]), "+a"(dv[db]));
+  }
 
   // q tiles (64 rows) that hold a query seeing one of the workgroup's 128 keys
   int qt_begin = 0, qt_end = nqt;
@@ -173,28 +218,36 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
 #endif
 
   // the steps of this workgroup: query heads of the group x q tiles, one flat sequence; the
-  // direct loads of step it + 1 fill the other stage while step it is computed
+  // direct loads of step it + 1 fill the other stage while step it is computed, one load after
+  // every pair of MFMAs of the first products (a wave owes LF_CPR loads per step, and that many
+  // pairs there are: the loads go through the CU's one texture path at 64 bytes per cycle, issued
+  // in one go they hold up the wave for as long as a quarter of its MFMAs take)
   const int ntq = max(qt_end - qt_begin, 0);
   const int nsteps = group * ntq;
   const unsigned q_bytes = (unsigned)(((long long)(p.Sq - 1) * p.q_ss + LF_D) * 2);
   const unsigned g_bytes = (unsigned)(((long long)(p.Sq - 1) * p.do_ss + LF_D) * 2);
   const int wave_u = wave;
+  constexpr int kPasses = 64 * LF_CPR / LF_BW_NT;      // loads of a wave per tile
+  static_assert(4 * kPasses == 2 * LF_NKS, "one direct load per pair of MFMAs of the first products");
   float r_lse = 0.0f, r_delta = 0.0f;
-  auto issue = [&](int it, int st) {
+  lf_u32x4 q_rs, g_rs;        // rows of Q and dO of the step being loaded (zero bytes: nothing to load)
+  int q0_next = 0;
+  auto aim = [&](int it, bool real) {
     const int h = hkv * group + it / ntq;
-    const int q0 = 64 * (qt_begin + it % ntq);
-    const lf_u32x4 q_rs = lf_make_buffer(p.q + (long long)b * p.q_sb + (long long)h * p.q_sh, q_bytes);
-    const lf_u32x4 g_rs = lf_make_buffer(p.dout + (long long)b * p.do_sb + (long long)h * p.do_sh, g_bytes);
-    lf_bw_dma_tile<LF_BW_NT>(q_rs, (unsigned)p.q_ss * 2u, q0, tiles[st][0], false, tid, wave_u);
-    lf_bw_dma_tile<LF_BW_NT>(q_rs, (unsigned)p.q_ss * 2u, q0, tiles[st][1], true, tid, wave_u);
-    lf_bw_dma_tile<LF_BW_NT>(g_rs, (unsigned)p.do_ss * 2u, q0, tiles[st][2], false, tid, wave_u);
-    lf_bw_dma_tile<LF_BW_NT>(g_rs, (unsigned)p.do_ss * 2u, q0, tiles[st][3], true, tid, wave_u);
+    q0_next = 64 * (qt_begin + it % ntq);
+    q_rs = lf_make_buffer(p.q + (long long)b * p.q_sb + (long long)h * p.q_sh, real ? q_bytes : 0u);
+    g_rs = lf_make_buffer(p.dout + (long long)b * p.do_sb + (long long)h * p.do_sh, real ? g_bytes : 0u);
     if (tid < 64) {            // into registers now, into the stage just before the barrier that opens it
-      const long long r = ((long long)b * p.Hq + h) * p.Sq + q0 + tid;
-      const bool in = q0 + tid < p.Sq;
+      const long long r = ((long long)b * p.Hq + h) * p.Sq + q0_next + tid;
+      const bool in = real && q0_next + tid < p.Sq;
       r_lse = in ? p.lse[r] : __builtin_inff();                      // rows past Sq: P = 0
       r_delta = in ? p.delta[r] : 0.0f;
     }
+  };
+  auto issue_piece = [&](int st, int j) {      // load j of LF_CPR: tile j / kPasses (Q, Q, dO, dO), pass j % kPasses
+    const int t = j / kPasses;
+    lf_bw_dma_piece<LF_BW_NT>(t < 2 ? q_rs : g_rs, (unsigned)(t < 2 ? p.q_ss : p.do_ss) * 2u, q0_next, tiles[st][t],
+                              (t & 1) != 0, j % kPasses, tid, wave_u);
   };
   auto publish = [&](int st) {
     if (tid < 64) {
@@ -203,7 +256,9 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
     }
   };
   if (nsteps > 0) {
-    issue(0, 0);
+    aim(0, true);
+#pragma unroll
+    for (int j = 0; j < LF_CPR; ++j) issue_piece(0, j);
     publish(0);
   }
   LF_BW_BARRIER();
@@ -216,8 +271,9 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
     const lf_elem* g_tr = tiles[st][3];
     const float* lse_s = lse_st[st];
     const float* delta_s = delta_st[st];
-    // the other stage was last read in step it - 1, which every wave left at the barrier below
-    if (it + 1 < nsteps) issue(it + 1, st ^ 1);
+    // the other stage was last read in step it - 1, which every wave left at the barrier below;
+    // after the last step the loads still go out, against an empty range: they fetch nothing
+    aim(min(it + 1, nsteps - 1), it + 1 < nsteps);
 
     bool need = key0 < p.Sk;
 #if LF_MASK >= 1
@@ -228,12 +284,10 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
 #endif
     if (need) {                 // wave-uniform
 
-    lf_elem8 pf[LF_NKK], dsf[LF_NKK];
+    lf_u32x4 pf[LF_NKK], dsf[LF_NKK];
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
       lf_f32x16 s, dp;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) s[i] = dp[i] = 0.0f;
       lf_u32x4 qa[LF_NKS], ga[LF_NKS];
 #pragma unroll
       for (int ks = 0; ks < LF_BW_PF1; ++ks) {
@@ -247,52 +301,72 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
           qa[ks + LF_BW_PF1] = lf_read_k_frag(q_rm, l32, g, (ks + LF_BW_PF1) * LF_NKB + qb);
           ga[ks + LF_BW_PF1] = lf_read_k_frag(g_rm, l32, g, (ks + LF_BW_PF1) * LF_NKB + qb);
         }
-        s = lf_mfma32(__builtin_bit_cast(lf_elem8, qa[ks]), kf[ks], s);
-        dp = lf_mfma32(__builtin_bit_cast(lf_elem8, ga[ks]), vf[ks], dp);
+        if (ks == 0) {
+          lf_bw_mfma_first(s, qa[ks], kf[ks]);
+          lf_bw_mfma_first(dp, ga[ks], vf[ks]);
+        } else {
+          lf_bw_mfma_vva(s, qa[ks], kf[ks]);
+          lf_bw_mfma_vva(dp, ga[ks], vf[ks]);
+        }
+        issue_piece(st ^ 1, LF_NKS * qb + ks);
         __builtin_amdgcn_sched_barrier(0);
       }
+      asm volatile(LF_BW_MFMA_DRAIN : "+v"(s), "+v"(dp));
       // element i: query q0 + 32*qb + 8*(i/4) + 4*g + i%4, key my_key
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
         const int ql = 32 * qb + 8 * i4 + 4 * g;
         const lf_f32x4 l4 = *reinterpret_cast<const lf_f32x4*>(&lse_s[ql]);
         const lf_f32x4 d4 = *reinterpret_cast<const lf_f32x4*>(&delta_s[ql]);
+        lf_elem4 pw, dw;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int i = 4 * i4 + e;
           const bool keep = lf_mask_keep(q0 + ql + e, my_key, p.Sk, p.window);
           const float pv = keep ? lf_exp2(s[i] * cexp - l4[e]) : 0.0f;
           const float ds = pv * (dp[i] - d4[e]) * p.scale;
-          pf[2 * qb + i / 8][i % 8] = lf_from_float(pv);
-          dsf[2 * qb + i / 8][i % 8] = lf_from_float(ds);
+          pw[e] = lf_from_float(pv);
+          dw[e] = lf_from_float(ds);
         }
+        const lf_u32x2 pu = __builtin_bit_cast(lf_u32x2, pw), du = __builtin_bit_cast(lf_u32x2, dw);
+        pf[2 * qb + i4 / 2][2 * (i4 % 2)] = pu[0];
+        pf[2 * qb + i4 / 2][2 * (i4 % 2) + 1] = pu[1];
+        dsf[2 * qb + i4 / 2][2 * (i4 % 2)] = du[0];
+        dsf[2 * qb + i4 / 2][2 * (i4 % 2) + 1] = du[1];
       }
     }
     // dV^T += dO^T P, dK^T += Q^T dS (k = the 64 queries of the tile)
     {
       constexpr int kNF = LF_NKK * LF_NDB;
-      lf_elem8 gt[kNF], qt2[kNF];
+      lf_u32x4 gt[kNF], qt2[kNF];
 #pragma unroll
       for (int f = 0; f < LF_BW_PF2; ++f) {
-        gt[f] = lf_read_v_frag_tr(g_tr, lane, g, f);
-        qt2[f] = lf_read_v_frag_tr(q_tr, lane, g, f);
+        gt[f] = __builtin_bit_cast(lf_u32x4, lf_read_v_frag_tr(g_tr, lane, g, f));
+        qt2[f] = __builtin_bit_cast(lf_u32x4, lf_read_v_frag_tr(q_tr, lane, g, f));
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
+      for (int kk = 0; kk < LF_NKK; ++kk) asm volatile(LF_BW_VALU_SETTLE : "+v"(pf[kk]), "+v"(dsf[kk]));
+#pragma unroll
       for (int f = 0; f < kNF; ++f) {
         if (f + LF_BW_PF2 < kNF) {
-          gt[f + LF_BW_PF2] = lf_read_v_frag_tr(g_tr, lane, g, f + LF_BW_PF2);
-          qt2[f + LF_BW_PF2] = lf_read_v_frag_tr(q_tr, lane, g, f + LF_BW_PF2);
+          gt[f + LF_BW_PF2] = __builtin_bit_cast(lf_u32x4, lf_read_v_frag_tr(g_tr, lane, g, f + LF_BW_PF2));
+          qt2[f + LF_BW_PF2] = __builtin_bit_cast(lf_u32x4, lf_read_v_frag_tr(q_tr, lane, g, f + LF_BW_PF2));
         }
-        dv[f % LF_NDB] = lf_mfma32(gt[f], pf[f / LF_NDB], dv[f % LF_NDB]);
-        dk[f % LF_NDB] = lf_mfma32(qt2[f], dsf[f / LF_NDB], dk[f % LF_NDB]);
+        lf_bw_mfma_avv(dv[f % LF_NDB], gt[f], pf[f / LF_NDB]);
+        lf_bw_mfma_avv(dk[f % LF_NDB], qt2[f], dsf[f / LF_NDB]);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    }   // need
+    } else {
+#pragma unroll
+      for (int j = 0; j < LF_CPR; ++j) issue_piece(st ^ 1, j);
+    }
     if (it + 1 < nsteps) publish(st ^ 1);
     LF_BW_BARRIER();            // the next stage has landed; every wave is done with this one
   }
+#pragma unroll
+  for (int db = 0; db < LF_NDB; ++db) asm volatile(LF_BW_MFMA_DRAIN : "+a"(dk[db]), "+a"(dv[db]));
 
   const bool valid = my_key < p.Sk;
   const int kr = min(my_key, p.Sk - 1);
