@@ -76,19 +76,19 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT) lf_attn_bwd_delta(const L
 // (row stride `rowb` bytes): rows past the end get an offset beyond it and arrive as zeros.
 // Not tracked by the compiler's wait counters: callers wait with s_waitcnt vmcnt(0).
 template <int NT>
-__device__ __forceinline__ void lf_bw_dma_piece(const lf_u32x4& rs, unsigned rowb, int row0, lf_elem* tile, bool tr,
-                                                int ps, int tid, int wave) {
-  constexpr int kRowsPerPass = NT / LF_CPR, kRowsPerWave = 64 / LF_CPR;
+__device__ __forceinline__ unsigned lf_bw_dma_lane_off(unsigned rowb, bool tr, int tid) {
+  // byte offset of this lane's 16 bytes in the first pass of a tile that starts at row 0; the
+  // swizzles repeat every 16 rows and a pass is a multiple of 16 rows, so every pass adds rows only
   const int srow = tid / LF_CPR, sch = tid % LF_CPR;
-  const int r = kRowsPerPass * ps + srow;
-  const unsigned off = (unsigned)(row0 + r) * rowb + 16u * (unsigned)(tr ? lf_v_phys(r, sch) : lf_k_phys(r, sch));
-  lf_dma_to_lds(rs, off, &tile[(kRowsPerPass * ps + kRowsPerWave * wave) * LF_D]);
+  return (unsigned)srow * rowb + 16u * (unsigned)(tr ? lf_v_phys(srow, sch) : lf_k_phys(srow, sch));
 }
 template <int NT>
-__device__ __forceinline__ void lf_bw_dma_tile(const lf_u32x4& rs, unsigned rowb, int row0, lf_elem* tile, bool tr,
-                                               int tid, int wave) {
-#pragma unroll
-  for (int ps = 0; ps < 64 * LF_CPR / NT; ++ps) lf_bw_dma_piece<NT>(rs, rowb, row0, tile, tr, ps, tid, wave);
+__device__ __forceinline__ void lf_bw_dma_piece(const lf_u32x4& rs, unsigned rowb, int row0, lf_elem* tile,
+                                                unsigned lane_off, int ps, int wave) {
+  constexpr int kRowsPerPass = NT / LF_CPR, kRowsPerWave = 64 / LF_CPR;
+  static_assert(kRowsPerPass % 16 == 0, "a pass must keep the swizzle phase");
+  const unsigned off = (unsigned)(row0 + kRowsPerPass * ps) * rowb + lane_off;
+  lf_dma_to_lds(rs, off, &tile[(kRowsPerPass * ps + kRowsPerWave * wave) * LF_D]);
 }
 // wait for this wave's direct loads and LDS writes, then meet the other waves.  The wait is the
 // builtin, not inline asm, so that the compiler's wait-counter pass sees that nothing is
@@ -108,6 +108,7 @@ __device__ __forceinline__ void lf_bw_dma_tile(const lf_u32x4& rs, unsigned rowb
 // itself the compiler issues read, wait, MFMA one after the other)
 #define LF_BW_PF1 3      /* first products: pairs of K-layout fragments */
 #define LF_BW_PF2 4      /* second products: V-layout fragments */
+#define LF_BW_DQ_PF1 2   /* lf_attn_bwd_dq, first products: 3 do not fit its 256 registers */
 
 // MFMAs of lf_attn_bwd_dkdv with the register file of every operand spelled out.  At one wave per
 // SIMD the kernel has 512 registers per lane, and the compiler then gives every MFMA an AGPR
@@ -135,6 +136,32 @@ __device__ __forceinline__ void lf_bw_mfma_vva(lf_f32x16& c, const lf_u32x4& a, 
 // c (AGPRs) += a (VGPRs) x b (VGPRs)
 __device__ __forceinline__ void lf_bw_mfma_avv(lf_f32x16& c, const lf_u32x4& a, const lf_u32x4& b) {
   asm volatile(LF_BW_MFMA " %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+
+// lf_attn_bwd_dq in its 8-wave form runs two waves per SIMD on 256 registers: the compiler then uses
+// no AGPRs and its own MFMAs are as good; the 4-wave form has 512 and gets the explicit ones
+#if LF_BW_DQ_NT == 256
+#define LF_BW_DQ_ASM 1
+#else
+#define LF_BW_DQ_ASM 0
+#endif
+__device__ __forceinline__ void lf_bw_dq_mfma_s(lf_f32x16& c, const lf_u32x4& a, const lf_u32x4& b, bool first) {
+#if LF_BW_DQ_ASM
+  if (first) lf_bw_mfma_first(c, a, b); else lf_bw_mfma_vva(c, a, b);
+#else
+  if (first) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) c[i] = 0.0f;
+  }
+  c = lf_mfma32(__builtin_bit_cast(lf_elem8, a), __builtin_bit_cast(lf_elem8, b), c);
+#endif
+}
+__device__ __forceinline__ void lf_bw_dq_mfma_acc(lf_f32x16& c, const lf_u32x4& a, const lf_u32x4& b) {
+#if LF_BW_DQ_ASM
+  lf_bw_mfma_avv(c, a, b);
+#else
+  c = lf_mfma32(__builtin_bit_cast(lf_elem8, a), __builtin_bit_cast(lf_elem8, b), c);
+#endif
 }
 
 // accumulators X^T[d][n] (lane n = lane % 32; element i of block db is d = 32*db + 8*(i/4) + 4*g + i%4)
@@ -244,10 +271,14 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
       r_delta = in ? p.delta[r] : 0.0f;
     }
   };
+  const unsigned lane_off[4] = {lf_bw_dma_lane_off<LF_BW_NT>((unsigned)p.q_ss * 2u, false, tid),
+                                lf_bw_dma_lane_off<LF_BW_NT>((unsigned)p.q_ss * 2u, true, tid),
+                                lf_bw_dma_lane_off<LF_BW_NT>((unsigned)p.do_ss * 2u, false, tid),
+                                lf_bw_dma_lane_off<LF_BW_NT>((unsigned)p.do_ss * 2u, true, tid)};
   auto issue_piece = [&](int st, int j) {      // load j of LF_CPR: tile j / kPasses (Q, Q, dO, dO), pass j % kPasses
     const int t = j / kPasses;
     lf_bw_dma_piece<LF_BW_NT>(t < 2 ? q_rs : g_rs, (unsigned)(t < 2 ? p.q_ss : p.do_ss) * 2u, q0_next, tiles[st][t],
-                              (t & 1) != 0, j % kPasses, tid, wave_u);
+                              lane_off[t], j % kPasses, wave_u);
   };
   auto publish = [&](int st) {
     if (tid < 64) {
@@ -397,15 +428,19 @@ extern "C" __global__ void __launch_bounds__(LF_BW_DQ_NT, LF_BW_DQ_NT / 256) lf_
   const int qr = min(my_q, p.Sq - 1);
   const int nkt = (p.Sk + 63) / 64;
 
-  lf_elem8 qf[LF_NKS], gf[LF_NKS];
+  lf_u32x4 qf[LF_NKS], gf[LF_NKS];
   {
     const lf_elem* qrow = p.q + (long long)b * p.q_sb + (long long)h * p.q_sh + (long long)qr * p.q_ss;
     const lf_elem* grow = p.dout + (long long)b * p.do_sb + (long long)h * p.do_sh + (long long)qr * p.do_ss;
 #pragma unroll
     for (int ks = 0; ks < LF_NKS; ++ks) {
-      qf[ks] = __builtin_bit_cast(lf_elem8, *reinterpret_cast<const lf_u32x4*>(qrow + 16 * ks + 8 * g));
-      gf[ks] = __builtin_bit_cast(lf_elem8, *reinterpret_cast<const lf_u32x4*>(grow + 16 * ks + 8 * g));
+      qf[ks] = *reinterpret_cast<const lf_u32x4*>(qrow + 16 * ks + 8 * g);
+      gf[ks] = *reinterpret_cast<const lf_u32x4*>(grow + 16 * ks + 8 * g);
     }
+#if LF_BW_DQ_ASM
+#pragma unroll
+    for (int ks = 0; ks < LF_NKS; ++ks) asm volatile("" : "+a"(qf[ks]), "+a"(gf[ks]));
+#endif
   }
   const long long ridx = ((long long)b * p.Hq + h) * p.Sq + qr;
   const float lse_q = my_q < p.Sq ? p.lse[ridx] : __builtin_inff();
@@ -414,9 +449,13 @@ extern "C" __global__ void __launch_bounds__(LF_BW_DQ_NT, LF_BW_DQ_NT / 256) lf_
 
   lf_f32x16 dq[LF_NDB];
 #pragma unroll
-  for (int db = 0; db < LF_NDB; ++db)
+  for (int db = 0; db < LF_NDB; ++db) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) dq[db][i] = 0.0f;
+#if LF_BW_DQ_ASM
+    asm volatile("" : "+a"(dq[db]));
+#endif
+  }
 
   int kt_begin = 0, kt_end = nkt;
   {
@@ -434,12 +473,25 @@ extern "C" __global__ void __launch_bounds__(LF_BW_DQ_NT, LF_BW_DQ_NT / 256) lf_
   const lf_elem* vbase = p.v + (long long)b * p.v_sb + (long long)hkv * p.v_sh;
   const lf_u32x4 k_rs = lf_make_buffer(kbase, (unsigned)(((long long)(p.Sk - 1) * p.k_ss + LF_D) * 2));
   const lf_u32x4 v_rs = lf_make_buffer(vbase, (unsigned)(((long long)(p.Sk - 1) * p.v_ss + LF_D) * 2));
-  auto issue = [&](int kt, int st) {
-    lf_bw_dma_tile<LF_BW_DQ_NT>(k_rs, (unsigned)p.k_ss * 2u, 64 * kt, tiles[st][0], false, tid, wave);
-    lf_bw_dma_tile<LF_BW_DQ_NT>(k_rs, (unsigned)p.k_ss * 2u, 64 * kt, tiles[st][1], true, tid, wave);
-    lf_bw_dma_tile<LF_BW_DQ_NT>(v_rs, (unsigned)p.v_ss * 2u, 64 * kt, tiles[st][2], false, tid, wave);
+  // the direct loads of tile kt + 1 go out one by one behind MFMA pairs of the first products of
+  // tile kt (a wave owes 3 * kPasses per tile); past the last tile they go out against an empty
+  // range and fetch nothing
+  constexpr int kPasses = 64 * LF_CPR / LF_BW_DQ_NT;
+  constexpr int kLoads = 3 * kPasses;
+  static_assert(kLoads <= 2 * LF_NKS, "one direct load per pair of MFMAs of the first products");
+  lf_u32x4 k_cur = k_rs, v_cur = v_rs;
+  const unsigned lane_off[3] = {lf_bw_dma_lane_off<LF_BW_DQ_NT>((unsigned)p.k_ss * 2u, false, tid),
+                                lf_bw_dma_lane_off<LF_BW_DQ_NT>((unsigned)p.k_ss * 2u, true, tid),
+                                lf_bw_dma_lane_off<LF_BW_DQ_NT>((unsigned)p.v_ss * 2u, false, tid)};
+  auto issue_piece = [&](int kt, int st, int j) {      // tile j / kPasses (K, K transposed, V), pass j % kPasses
+    const int t = j / kPasses;
+    lf_bw_dma_piece<LF_BW_DQ_NT>(t < 2 ? k_cur : v_cur, (unsigned)(t < 2 ? p.k_ss : p.v_ss) * 2u, 64 * kt, tiles[st][t],
+                                 lane_off[t], j % kPasses, wave);
   };
-  if (kt_begin < kt_end) issue(kt_begin, 0);
+  if (kt_begin < kt_end) {
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) issue_piece(kt_begin, 0, j);
+  }
   LF_BW_BARRIER();
   for (int kt = kt_begin; kt < kt_end; ++kt) {
     const int k0 = 64 * kt;
@@ -447,7 +499,11 @@ extern "C" __global__ void __launch_bounds__(LF_BW_DQ_NT, LF_BW_DQ_NT / 256) lf_
     const lf_elem* k_rm = tiles[st][0];
     const lf_elem* k_tr = tiles[st][1];
     const lf_elem* v_rm = tiles[st][2];
-    if (kt + 1 < kt_end) issue(kt + 1, st ^ 1);     // fills the stage every wave left at the last barrier
+    if (kt + 1 >= kt_end) k_cur[2] = v_cur[2] = 0u;   // the other stage is free: every wave left it at the last barrier
+#if !LF_BW_DQ_ASM      // 8 waves: a wave owes few loads and has no registers to spare for their offsets
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) issue_piece(kt + 1, st ^ 1, j);
+#endif
 
     bool need = wq0 < p.Sq;
 #if LF_MASK >= 1
@@ -458,53 +514,83 @@ extern "C" __global__ void __launch_bounds__(LF_BW_DQ_NT, LF_BW_DQ_NT / 256) lf_
 #endif
     if (need) {
 
-    lf_elem8 dsf[LF_NKK];
+    lf_u32x4 dsf[LF_NKK];
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
       lf_f32x16 s, dp;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) s[i] = dp[i] = 0.0f;
       lf_u32x4 ka[LF_NKS], va[LF_NKS];
 #pragma unroll
-      for (int ks = 0; ks < LF_BW_PF1; ++ks) {
+      for (int ks = 0; ks < LF_BW_DQ_PF1; ++ks) {
         ka[ks] = lf_read_k_frag(k_rm, l32, g, ks * LF_NKB + kb);
         va[ks] = lf_read_k_frag(v_rm, l32, g, ks * LF_NKB + kb);
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ks = 0; ks < LF_NKS; ++ks) {
-        if (ks + LF_BW_PF1 < LF_NKS) {
-          ka[ks + LF_BW_PF1] = lf_read_k_frag(k_rm, l32, g, (ks + LF_BW_PF1) * LF_NKB + kb);
-          va[ks + LF_BW_PF1] = lf_read_k_frag(v_rm, l32, g, (ks + LF_BW_PF1) * LF_NKB + kb);
+        if (ks + LF_BW_DQ_PF1 < LF_NKS) {
+          ka[ks + LF_BW_DQ_PF1] = lf_read_k_frag(k_rm, l32, g, (ks + LF_BW_DQ_PF1) * LF_NKB + kb);
+          va[ks + LF_BW_DQ_PF1] = lf_read_k_frag(v_rm, l32, g, (ks + LF_BW_DQ_PF1) * LF_NKB + kb);
         }
-        s = lf_mfma32(__builtin_bit_cast(lf_elem8, ka[ks]), qf[ks], s);       // S^T[key][q]
-        dp = lf_mfma32(__builtin_bit_cast(lf_elem8, va[ks]), gf[ks], dp);     // dP^T[key][q]
+        lf_bw_dq_mfma_s(s, ka[ks], qf[ks], ks == 0);         // S^T[key][q]
+        lf_bw_dq_mfma_s(dp, va[ks], gf[ks], ks == 0);        // dP^T[key][q]
+#if LF_BW_DQ_ASM
+        if (LF_NKS * kb + ks < kLoads) issue_piece(kt + 1, st ^ 1, LF_NKS * kb + ks);
+#endif
         __builtin_amdgcn_sched_barrier(0);
       }
+#if LF_BW_DQ_ASM
+      asm volatile(LF_BW_MFMA_DRAIN : "+v"(s), "+v"(dp));
+#endif
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int j = k0 + 32 * kb + 8 * (i / 4) + 4 * g + (i % 4);
-        const bool keep = lf_mask_keep(my_q, j, p.Sk, p.window);
-        const float pv = keep ? lf_exp2(s[i] * cexp - lse_q) : 0.0f;
-        dsf[2 * kb + i / 8][i % 8] = lf_from_float(pv * (dp[i] - delta_q) * p.scale);
+      for (int i4 = 0; i4 < 4; ++i4) {
+        lf_elem4 dw;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int i = 4 * i4 + e;
+          const int j = k0 + 32 * kb + 8 * i4 + 4 * g + e;
+          const bool keep = lf_mask_keep(my_q, j, p.Sk, p.window);
+          const float pv = keep ? lf_exp2(s[i] * cexp - lse_q) : 0.0f;
+          dw[e] = lf_from_float(pv * (dp[i] - delta_q) * p.scale);
+        }
+        const lf_u32x2 du = __builtin_bit_cast(lf_u32x2, dw);
+        dsf[2 * kb + i4 / 2][2 * (i4 % 2)] = du[0];
+        dsf[2 * kb + i4 / 2][2 * (i4 % 2) + 1] = du[1];
       }
     }
     // dQ^T += K^T dS^T (k = the 64 keys of the tile)
     {
       constexpr int kNF = LF_NKK * LF_NDB;
-      lf_elem8 kt2[kNF];
+      lf_u32x4 kt2[kNF];
+      // the addresses of the transposed reads are formed again in every step: held across the
+      // first products they do not fit the 256 registers of a wave and end up in scratch memory
+      int lane_r = lane;
+      asm volatile("" : "+v"(lane_r));
+      const int g_r = lane_r >> 5;
 #pragma unroll
-      for (int f = 0; f < LF_BW_PF2; ++f) kt2[f] = lf_read_v_frag_tr(k_tr, lane, g, f);
+      for (int f = 0; f < LF_BW_PF2; ++f) kt2[f] = __builtin_bit_cast(lf_u32x4, lf_read_v_frag_tr(k_tr, lane_r, g_r, f));
       __builtin_amdgcn_sched_barrier(0);
+#if LF_BW_DQ_ASM
+#pragma unroll
+      for (int kk = 0; kk < LF_NKK; ++kk) asm volatile(LF_BW_VALU_SETTLE : "+v"(dsf[kk]));
+#endif
 #pragma unroll
       for (int f = 0; f < kNF; ++f) {
-        if (f + LF_BW_PF2 < kNF) kt2[f + LF_BW_PF2] = lf_read_v_frag_tr(k_tr, lane, g, f + LF_BW_PF2);
-        dq[f % LF_NDB] = lf_mfma32(kt2[f], dsf[f / LF_NDB], dq[f % LF_NDB]);
+        if (f + LF_BW_PF2 < kNF) kt2[f + LF_BW_PF2] = __builtin_bit_cast(lf_u32x4, lf_read_v_frag_tr(k_tr, lane_r, g_r, f + LF_BW_PF2));
+        lf_bw_dq_mfma_acc(dq[f % LF_NDB], kt2[f], dsf[f / LF_NDB]);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    }   // need
+    } else {
+#if LF_BW_DQ_ASM
+#pragma unroll
+      for (int j = 0; j < kLoads; ++j) issue_piece(kt + 1, st ^ 1, j);
+#endif
+    }
     LF_BW_BARRIER();
   }
+#if LF_BW_DQ_ASM
+#pragma unroll
+  for (int db = 0; db < LF_NDB; ++db) asm volatile(LF_BW_MFMA_DRAIN : "+a"(dq[db]));
+#endif
   lf_bw_store_rows(dq, p.dq + (long long)b * p.dq_sb + (long long)h * p.dq_sh + (long long)qr * p.dq_ss, my_q < p.Sq, g);
 }
