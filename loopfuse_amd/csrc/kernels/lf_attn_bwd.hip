@@ -42,6 +42,18 @@ struct LfAttnBwdParams {
 };
 
 #define LF_BW_NT 256
+// Is the score with (query - key) = t kept?  Callers fold the bound of the key sequence into t.
+__device__ __forceinline__ bool lf_bw_keep(int t, int window) {
+#if LF_MASK == 0
+  (void)window;
+  return t > -(1 << 29);
+#elif LF_MASK == 1
+  (void)window;
+  return t >= 0;
+#else
+  return (unsigned)t < (unsigned)window;
+#endif
+}
 #ifndef LF_BW_DQ_NT
 #define LF_BW_DQ_NT 512     /* threads of lf_attn_bwd_dq: 8 waves x 32 query rows, two waves per SIMD */
 #endif
@@ -286,39 +298,57 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
       delta_st[st][tid] = r_delta;
     }
   };
-  if (nsteps > 0) {
-    aim(0, true);
-#pragma unroll
-    for (int j = 0; j < LF_CPR; ++j) issue_piece(0, j);
-    publish(0);
-  }
-  LF_BW_BARRIER();
-  for (int it = 0; it < nsteps; ++it) {
-    const int st = it & 1;
-    const int q0 = 64 * (qt_begin + it % ntq);
+  // One step of a wave: S^T and dP^T of 32 keys x 64 queries in two blocks of 32 queries, P and dS,
+  // then dV^T += dO^T P and dK^T += Q^T dS.  With one wave per SIMD nothing else fills the matrix
+  // pipe while the wave computes P and dS, so the step is written as four phases of 16 MFMAs with
+  // that arithmetic placed between them: first products of block 0 | first products of block 1 with
+  // P, dS of block 0 | second products over block 0's queries with P, dS of block 1 | second
+  // products over block 1's queries.  dS is kept without the factor `scale`, which multiplies dK once
+  // at the end.
+  auto step = [&](bool masked, int st, int q0) {
+    // query minus key of element (qb, i4, e) is rel + 32*qb + 8*i4 + e; a key past Sk fails every test
+    const int rel = my_key < p.Sk ? q0 + 4 * g - my_key : -(1 << 30);
     const lf_elem* q_rm = tiles[st][0];
     const lf_elem* q_tr = tiles[st][1];
     const lf_elem* g_rm = tiles[st][2];
     const lf_elem* g_tr = tiles[st][3];
     const float* lse_s = lse_st[st];
     const float* delta_s = delta_st[st];
-    // the other stage was last read in step it - 1, which every wave left at the barrier below;
-    // after the last step the loads still go out, against an empty range: they fetch nothing
-    aim(min(it + 1, nsteps - 1), it + 1 < nsteps);
-
-    bool need = key0 < p.Sk;
-#if LF_MASK >= 1
-    need = need && (q0 + 63 >= key0);
-#endif
-#if LF_MASK == 2
-    need = need && (q0 - min(key0 + 31, p.Sk - 1) < p.window);
-#endif
-    if (need) {                 // wave-uniform
-
+    constexpr int kNF = LF_NKK * LF_NDB;
     lf_u32x4 pf[LF_NKK], dsf[LF_NKK];
+    lf_f32x16 s[2], dp[2];
+    // P and dS of the four queries (qb, i4): elements 4*i4 .. +3 of the accumulators, query
+    // q0 + 32*qb + 8*i4 + 4*g + e, key my_key
+    auto soft4 = [&](int qb, int i4) {
+      const int ql = 32 * qb + 8 * i4 + 4 * g;
+      const lf_f32x4 l4 = *reinterpret_cast<const lf_f32x4*>(&lse_s[ql]);
+      const lf_f32x4 d4 = *reinterpret_cast<const lf_f32x4*>(&delta_s[ql]);
+      lf_elem4 pw, dw;
+      float pv[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int i = 4 * i4 + e;
+        pv[e] = lf_exp2(s[qb][i] * cexp - l4[e]);
+      }
+      if (masked) {             // wave-uniform: most steps of a workgroup lie below the diagonal
+#pragma unroll
+        for (int e = 0; e < 4; ++e) pv[e] = lf_bw_keep(rel + 32 * qb + 8 * i4 + e, p.window) ? pv[e] : 0.0f;
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int i = 4 * i4 + e;
+        pw[e] = lf_from_float(pv[e]);
+        dw[e] = lf_from_float(pv[e] * (dp[qb][i] - d4[e]));
+      }
+      const lf_u32x2 pu = __builtin_bit_cast(lf_u32x2, pw), du = __builtin_bit_cast(lf_u32x2, dw);
+      pf[2 * qb + i4 / 2][2 * (i4 % 2)] = pu[0];
+      pf[2 * qb + i4 / 2][2 * (i4 % 2) + 1] = pu[1];
+      dsf[2 * qb + i4 / 2][2 * (i4 % 2)] = du[0];
+      dsf[2 * qb + i4 / 2][2 * (i4 % 2) + 1] = du[1];
+    };
+    // phases 1 and 2
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
-      lf_f32x16 s, dp;
       lf_u32x4 qa[LF_NKS], ga[LF_NKS];
 #pragma unroll
       for (int ks = 0; ks < LF_BW_PF1; ++ks) {
@@ -333,42 +363,20 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
           ga[ks + LF_BW_PF1] = lf_read_k_frag(g_rm, l32, g, (ks + LF_BW_PF1) * LF_NKB + qb);
         }
         if (ks == 0) {
-          lf_bw_mfma_first(s, qa[ks], kf[ks]);
-          lf_bw_mfma_first(dp, ga[ks], vf[ks]);
+          lf_bw_mfma_first(s[qb], qa[ks], kf[ks]);
+          lf_bw_mfma_first(dp[qb], ga[ks], vf[ks]);
         } else {
-          lf_bw_mfma_vva(s, qa[ks], kf[ks]);
-          lf_bw_mfma_vva(dp, ga[ks], vf[ks]);
+          lf_bw_mfma_vva(s[qb], qa[ks], kf[ks]);
+          lf_bw_mfma_vva(dp[qb], ga[ks], vf[ks]);
         }
         issue_piece(st ^ 1, LF_NKS * qb + ks);
+        if (qb == 1 && ks * 4 % LF_NKS == 0) soft4(0, ks * 4 / LF_NKS);      // 4 groups over the LF_NKS pairs
         __builtin_amdgcn_sched_barrier(0);
       }
-      asm volatile(LF_BW_MFMA_DRAIN : "+v"(s), "+v"(dp));
-      // element i: query q0 + 32*qb + 8*(i/4) + 4*g + i%4, key my_key
-#pragma unroll
-      for (int i4 = 0; i4 < 4; ++i4) {
-        const int ql = 32 * qb + 8 * i4 + 4 * g;
-        const lf_f32x4 l4 = *reinterpret_cast<const lf_f32x4*>(&lse_s[ql]);
-        const lf_f32x4 d4 = *reinterpret_cast<const lf_f32x4*>(&delta_s[ql]);
-        lf_elem4 pw, dw;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int i = 4 * i4 + e;
-          const bool keep = lf_mask_keep(q0 + ql + e, my_key, p.Sk, p.window);
-          const float pv = keep ? lf_exp2(s[i] * cexp - l4[e]) : 0.0f;
-          const float ds = pv * (dp[i] - d4[e]) * p.scale;
-          pw[e] = lf_from_float(pv);
-          dw[e] = lf_from_float(ds);
-        }
-        const lf_u32x2 pu = __builtin_bit_cast(lf_u32x2, pw), du = __builtin_bit_cast(lf_u32x2, dw);
-        pf[2 * qb + i4 / 2][2 * (i4 % 2)] = pu[0];
-        pf[2 * qb + i4 / 2][2 * (i4 % 2) + 1] = pu[1];
-        dsf[2 * qb + i4 / 2][2 * (i4 % 2)] = du[0];
-        dsf[2 * qb + i4 / 2][2 * (i4 % 2) + 1] = du[1];
-      }
+      asm volatile(LF_BW_MFMA_DRAIN : "+v"(s[qb]), "+v"(dp[qb]));
     }
-    // dV^T += dO^T P, dK^T += Q^T dS (k = the 64 queries of the tile)
+    // phases 3 and 4
     {
-      constexpr int kNF = LF_NKK * LF_NDB;
       lf_u32x4 gt[kNF], qt2[kNF];
 #pragma unroll
       for (int f = 0; f < LF_BW_PF2; ++f) {
@@ -377,18 +385,54 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int kk = 0; kk < LF_NKK; ++kk) asm volatile(LF_BW_VALU_SETTLE : "+v"(pf[kk]), "+v"(dsf[kk]));
-#pragma unroll
       for (int f = 0; f < kNF; ++f) {
+        if (f % (kNF / 2) == 0) {
+#pragma unroll
+          for (int kk = 0; kk < LF_NKK / 2; ++kk)
+            asm volatile(LF_BW_VALU_SETTLE : "+v"(pf[f / (kNF / 2) * (LF_NKK / 2) + kk]), "+v"(dsf[f / (kNF / 2) * (LF_NKK / 2) + kk]));
+        }
         if (f + LF_BW_PF2 < kNF) {
           gt[f + LF_BW_PF2] = __builtin_bit_cast(lf_u32x4, lf_read_v_frag_tr(g_tr, lane, g, f + LF_BW_PF2));
           qt2[f + LF_BW_PF2] = __builtin_bit_cast(lf_u32x4, lf_read_v_frag_tr(q_tr, lane, g, f + LF_BW_PF2));
         }
         lf_bw_mfma_avv(dv[f % LF_NDB], gt[f], pf[f / LF_NDB]);
         lf_bw_mfma_avv(dk[f % LF_NDB], qt2[f], dsf[f / LF_NDB]);
+        if (f < kNF / 2 && f * 8 % kNF == 0) soft4(1, f * 8 / kNF);              // 4 groups over the first kNF / 2 pairs
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+  };
+  if (nsteps > 0) {
+    aim(0, true);
+#pragma unroll
+    for (int j = 0; j < LF_CPR; ++j) issue_piece(0, j);
+    publish(0);
+  }
+  LF_BW_BARRIER();
+  for (int it = 0; it < nsteps; ++it) {
+    const int st = it & 1;
+    const int q0 = 64 * (qt_begin + it % ntq);
+    // the other stage was last read in step it - 1, which every wave left at the barrier below;
+    // after the last step the loads still go out, against an empty range: they fetch nothing
+    aim(min(it + 1, nsteps - 1), it + 1 < nsteps);
+
+    bool need = key0 < p.Sk;
+#if LF_MASK >= 1
+    need = need && (q0 + 63 >= key0);
+#endif
+#if LF_MASK == 2
+    need = need && (q0 - min(key0 + 31, p.Sk - 1) < p.window);
+#endif
+    if (need) {                 // wave-uniform
+      // are all 32 x 64 scores of this wave kept?  Then the step runs without the mask arithmetic
+      bool full = key0 + 31 < p.Sk;
+#if LF_MASK >= 1
+      full = full && (key0 + 31 <= q0);
+#endif
+#if LF_MASK == 2
+      full = full && (q0 + 63 - key0 < p.window);
+#endif
+      step(!full, st, q0);
     } else {
 #pragma unroll
       for (int j = 0; j < LF_CPR; ++j) issue_piece(st ^ 1, j);
@@ -398,6 +442,10 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
   }
 #pragma unroll
   for (int db = 0; db < LF_NDB; ++db) asm volatile(LF_BW_MFMA_DRAIN : "+a"(dk[db]), "+a"(dv[db]));
+#pragma unroll
+  for (int db = 0; db < LF_NDB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) dk[db][i] *= p.scale;
 
   const bool valid = my_key < p.Sk;
   const int kr = min(my_key, p.Sk - 1);
