@@ -561,6 +561,15 @@ extern "C" __global__ void __launch_bounds__(LF_BW_DQ_NT, LF_BW_DQ_NT / 256) lf_
     need = need && (min(k0 + 64, p.Sk) - 1 >= wq0 - p.window + 1);
 #endif
     if (need) {
+    // are all 64 x 32 scores of this wave kept?  Then the tile runs without the mask arithmetic
+    bool full = k0 + 63 < p.Sk;
+#if LF_MASK >= 1
+    full = full && (k0 + 63 <= wq0);
+#endif
+#if LF_MASK == 2
+    full = full && (wq0 + 31 - k0 < p.window);
+#endif
+    const bool masked = !full;
 
     lf_u32x4 dsf[LF_NKK];
 #pragma unroll
@@ -592,14 +601,18 @@ extern "C" __global__ void __launch_bounds__(LF_BW_DQ_NT, LF_BW_DQ_NT / 256) lf_
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
         lf_elem4 dw;
+        float pv[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int i = 4 * i4 + e;
-          const int j = k0 + 32 * kb + 8 * i4 + 4 * g + e;
-          const bool keep = lf_mask_keep(my_q, j, p.Sk, p.window);
-          const float pv = keep ? lf_exp2(s[i] * cexp - lse_q) : 0.0f;
-          dw[e] = lf_from_float(pv * (dp[i] - delta_q) * p.scale);
+        for (int e = 0; e < 4; ++e) pv[e] = lf_exp2(s[4 * i4 + e] * cexp - lse_q);
+        if (masked) {           // wave-uniform: most tiles of a q tile lie below the diagonal
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int j = k0 + 32 * kb + 8 * i4 + 4 * g + e;
+            pv[e] = (j < p.Sk && lf_bw_keep(my_q - j, p.window)) ? pv[e] : 0.0f;
+          }
         }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) dw[e] = lf_from_float(pv[e] * (dp[4 * i4 + e] - delta_q));   // dS without `scale`
         const lf_u32x2 du = __builtin_bit_cast(lf_u32x2, dw);
         dsf[2 * kb + i4 / 2][2 * (i4 % 2)] = du[0];
         dsf[2 * kb + i4 / 2][2 * (i4 % 2) + 1] = du[1];
@@ -640,5 +653,9 @@ extern "C" __global__ void __launch_bounds__(LF_BW_DQ_NT, LF_BW_DQ_NT / 256) lf_
 #pragma unroll
   for (int db = 0; db < LF_NDB; ++db) asm volatile(LF_BW_MFMA_DRAIN : "+a"(dq[db]));
 #endif
+#pragma unroll
+  for (int db = 0; db < LF_NDB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) dq[db][i] *= p.scale;
   lf_bw_store_rows(dq, p.dq + (long long)b * p.dq_sb + (long long)h * p.dq_sh + (long long)qr * p.dq_ss, my_q < p.Sq, g);
 }
