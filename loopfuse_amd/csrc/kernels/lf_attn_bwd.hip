@@ -42,6 +42,9 @@ struct LfAttnBwdParams {
 };
 
 #define LF_BW_NT 256
+#ifndef LF_BW_GROUP
+#define LF_BW_GROUP 4      /* (batch, kv head) pairs of one XCD whose workgroups are dispatched together */
+#endif
 // Is the score with (query - key) = t kept?  Callers fold the bound of the key sequence into t.
 __device__ __forceinline__ bool lf_bw_keep(int t, int window) {
 #if LF_MASK == 0
@@ -214,8 +217,15 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
   const int g = lane >> 5;
 
   const int nkt = (p.Sk + 127) / 128;
-  const int kt = blockIdx.x % nkt;
-  const int bhkv = blockIdx.x / nkt;
+  // Workgroup ids with equal id % 8 run on one XCD.  All key blocks of a (batch, kv head) go to one
+  // XCD, so the Q / dO tiles they all walk are fetched into one L2, once; within an XCD the ids come
+  // in groups of LF_BW_GROUP (batch, kv head) pairs and, inside a group, by key block, the ones with
+  // the most steps under a causal mask first.  The grid is padded to whole groups.
+  const int slot = blockIdx.x / 8;
+  const int in_grp = slot % (LF_BW_GROUP * nkt);
+  const int kt = in_grp / LF_BW_GROUP;
+  const int bhkv = (slot / (LF_BW_GROUP * nkt) * LF_BW_GROUP + in_grp % LF_BW_GROUP) * 8 + (int)(blockIdx.x % 8);
+  if (bhkv >= p.B * p.Hkv) return;
   const int hkv = bhkv % p.Hkv;
   const int b = bhkv / p.Hkv;
   const int group = p.Hq / p.Hkv;
@@ -465,11 +475,18 @@ extern "C" __global__ void __launch_bounds__(LF_BW_DQ_NT, LF_BW_DQ_NT / 256) lf_
 
   constexpr int kBM = LF_BW_DQ_NT / 2;                    // query rows of a workgroup
   const int nqt = (p.Sq + kBM - 1) / kBM;
-  const int qt = nqt - 1 - (int)(blockIdx.x % nqt);       // long q tiles first
-  const int bh = blockIdx.x / nqt;
-  const int h = bh % p.Hq;
-  const int b = bh / p.Hq;
-  const int hkv = h / (p.Hq / p.Hkv);
+  // As in lf_attn_bwd_dkdv: the q tiles of all query heads of a (batch, kv head) run on one XCD
+  // and share its K / V tiles there; inside a group of LF_BW_GROUP pairs the long q tiles come first.
+  const int nrow = (p.Hq / p.Hkv) * nqt;                  // (query head of the group, q tile) per pair
+  const int slot = blockIdx.x / 8;
+  const int in_grp = slot % (LF_BW_GROUP * nrow);
+  const int row = in_grp / LF_BW_GROUP;
+  const int bhkv = (slot / (LF_BW_GROUP * nrow) * LF_BW_GROUP + in_grp % LF_BW_GROUP) * 8 + (int)(blockIdx.x % 8);
+  if (bhkv >= p.B * p.Hkv) return;
+  const int qt = nqt - 1 - row / (p.Hq / p.Hkv);
+  const int hkv = bhkv % p.Hkv;
+  const int b = bhkv / p.Hkv;
+  const int h = hkv * (p.Hq / p.Hkv) + row % (p.Hq / p.Hkv);
   const int q0 = kBM * qt;
   const int wq0 = q0 + 32 * wave;
   const int my_q = wq0 + l32;

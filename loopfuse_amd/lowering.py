@@ -281,6 +281,7 @@ def _get_scratch(device: torch.device, nfloats: int) -> torch.Tensor:
 
 
 PREFILL_QGROUP = 8      # LF_QGROUP of lf_attn_prefill_swp.hip (its default)
+BWD_GROUP = 4           # LF_BW_GROUP of lf_attn_bwd.hip (its default)
 
 
 def decode_split(units: int, Sk: int, cus: int = 256, per_cu: int = 2) -> int:
@@ -912,8 +913,16 @@ def attention_backward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: tor
     keep = (q, k, v, o, dout, lse, delta, dq, dk, dv)  # noqa: F841  (tensors stay alive until the launches are queued)
     rows = B * Hq * Sq
     get_kernel(spec, "lf_attn_bwd_delta").launch(((rows + 15) // 16, 1, 1), (256, 1, 1), P)
-    get_kernel(spec, "lf_attn_bwd_dkdv").launch((B * Hkv * ((Sk + 127) // 128), 1, 1), (256, 1, 1), P)
+    # 8 XCD classes x (batch, kv head) pairs per class, padded to the kernels' groups, x the
+    # workgroups of a pair (key blocks; query heads of the group x q tiles)
+    grp = BWD_GROUP
+    for e in spec.extra:
+        if e.startswith("-DLF_BW_GROUP="):
+            grp = int(e.split("=")[1])
+    pairs = ((B * Hkv + 7) // 8 + grp - 1) // grp * grp
+    get_kernel(spec, "lf_attn_bwd_dkdv").launch((8 * pairs * ((Sk + 127) // 128), 1, 1), (256, 1, 1), P)
     nt = bwd_dq_threads(mask)
-    get_kernel(spec, "lf_attn_bwd_dq").launch((B * Hq * ((Sq + nt // 2 - 1) // (nt // 2)), 1, 1), (nt, 1, 1), P)
+    get_kernel(spec, "lf_attn_bwd_dq").launch((8 * pairs * (Hq // Hkv) * ((Sq + nt // 2 - 1) // (nt // 2)), 1, 1),
+                                              (nt, 1, 1), P)
     _last_launch.set({"kernels": ["lf_attn_bwd_delta", "lf_attn_bwd_dkdv", "lf_attn_bwd_dq"]})
     return dq, dk, dv
