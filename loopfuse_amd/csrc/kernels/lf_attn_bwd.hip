@@ -133,12 +133,16 @@ __device__ __forceinline__ void lf_bw_dma_piece(const lf_u32x4& rs, unsigned row
 // What the compiler would otherwise see to: an MFMA result may be read 12 wait states after the MFMA
 // was issued at the earliest (LF_BW_MFMA_DRAIN), and a VGPR written by the VALU may be an MFMA
 // operand 2 wait states later (LF_BW_VALU_SETTLE); back-to-back MFMAs on one accumulator need nothing.
+// What it cannot see to at all: a register copy or a spill of its own placed right behind one of these
+// MFMAs would read the accumulator too early.  The live ranges are laid out so that it has no reason
+// for either, and tests/test_kernel_codegen.py checks the generated code for it.
 #if LF_DTYPE == 0
 #define LF_BW_MFMA "v_mfma_f32_32x32x16_bf16"
 #else
 #define LF_BW_MFMA "v_mfma_f32_32x32x16_f16"
 #endif
 #define LF_BW_MFMA_DRAIN "s_nop 9\n\ts_nop 9"
+#define LF_BW_MFMA_DRAIN_LAST "s_nop 15\n\ts_nop 15\n\ts_nop 15"     /* behind the last MFMAs issued: one may still wait for the pipe */
 #define LF_BW_VALU_SETTLE "s_nop 1"
 // c (VGPRs) = a (VGPRs) x b (AGPRs)
 __device__ __forceinline__ void lf_bw_mfma_first(lf_f32x16& c, const lf_u32x4& a, const lf_u32x4& b) {
@@ -451,7 +455,7 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
     LF_BW_BARRIER();            // the next stage has landed; every wave is done with this one
   }
 #pragma unroll
-  for (int db = 0; db < LF_NDB; ++db) asm volatile(LF_BW_MFMA_DRAIN : "+a"(dk[db]), "+a"(dv[db]));
+  for (int db = 0; db < LF_NDB; ++db) asm volatile(LF_BW_MFMA_DRAIN_LAST : "+a"(dk[db]), "+a"(dv[db]));
 #pragma unroll
   for (int db = 0; db < LF_NDB; ++db)
 #pragma unroll
@@ -668,7 +672,7 @@ extern "C" __global__ void __launch_bounds__(LF_BW_DQ_NT, LF_BW_DQ_NT / 256) lf_
   }
 #if LF_BW_DQ_ASM
 #pragma unroll
-  for (int db = 0; db < LF_NDB; ++db) asm volatile(LF_BW_MFMA_DRAIN : "+a"(dq[db]));
+  for (int db = 0; db < LF_NDB; ++db) asm volatile(LF_BW_MFMA_DRAIN_LAST : "+a"(dq[db]));
 #endif
 #pragma unroll
   for (int db = 0; db < LF_NDB; ++db)
