@@ -149,7 +149,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
     } else {
       off = k_doff + (unsigned)(kt * LF_BN + kRowsPerPass * ps) * k_rowb;
     }
-    dma(k_rsq, off, &lds_k[sl][(kRowsPerPass * ps + kRowsPerWave * wave) * LF_D]);
+    dma(k_rsq, off, &lds_k[sl][(kRowsPerPass * ps + kRowsPerWave * wave_u) * LF_D]);
   };
   auto dma_v_pass = [&](int kt, int sl, int ps, unsigned pg) {
     unsigned off;
@@ -160,7 +160,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
     } else {
       off = v_doff + (unsigned)(kt * LF_BN + kRowsPerPass * ps) * v_rowb;
     }
-    dma(v_rsq, off, &lds_v[sl][(kRowsPerPass * ps + kRowsPerWave * wave) * LF_D]);
+    dma(v_rsq, off, &lds_v[sl][(kRowsPerPass * ps + kRowsPerWave * wave_u) * LF_D]);
   };
 
 #if LF_SOFTCAP
