@@ -140,7 +140,9 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
   const unsigned v_doff = (unsigned)(kPagedV ? srow % (64 / LF_CPR) : srow) * v_rowb + 16u * (unsigned)lf_v_phys(srow, sch);
   auto dma = [&](const lf_u32x4& rs, unsigned voff, const lf_elem* lds_row0) { lf_dma_to_lds(rs, voff, lds_row0); };
   // pg: page_off() of the pass (paged operands only; fetched a tile ahead by the caller)
-  auto dma_k_pass = [&](int kt, int sl, int ps, unsigned pg) {
+  // `rs`: k_rsq / v_rsq, or the same with an empty range for a tile past the last one (nothing is
+  // fetched then; the slot it would fill is free)
+  auto dma_k_pass = [&](const lf_u32x4& rs, int kt, int sl, int ps, unsigned pg) {
     unsigned off;
     if (kPagedK) {
       const int tokw = kt * LF_BN + kRowsPerPass * ps + kRowsPerWave * wave_u;     // first row of this wave's load
@@ -149,9 +151,9 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
     } else {
       off = k_doff + (unsigned)(kt * LF_BN + kRowsPerPass * ps) * k_rowb;
     }
-    dma(k_rsq, off, &lds_k[sl][(kRowsPerPass * ps + kRowsPerWave * wave_u) * LF_D]);
+    dma(rs, off, &lds_k[sl][(kRowsPerPass * ps + kRowsPerWave * wave_u) * LF_D]);
   };
-  auto dma_v_pass = [&](int kt, int sl, int ps, unsigned pg) {
+  auto dma_v_pass = [&](const lf_u32x4& rs, int kt, int sl, int ps, unsigned pg) {
     unsigned off;
     if (kPagedV) {
       const int tokw = kt * LF_BN + kRowsPerPass * ps + kRowsPerWave * wave_u;
@@ -160,7 +162,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
     } else {
       off = v_doff + (unsigned)(kt * LF_BN + kRowsPerPass * ps) * v_rowb;
     }
-    dma(v_rsq, off, &lds_v[sl][(kRowsPerPass * ps + kRowsPerWave * wave_u) * LF_D]);
+    dma(rs, off, &lds_v[sl][(kRowsPerPass * ps + kRowsPerWave * wave_u) * LF_D]);
   };
 
 #if LF_SOFTCAP
@@ -241,9 +243,9 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
       }
 #pragma unroll
       for (int ps = 0; ps < LF_NPASS; ++ps) {
-        dma_k_pass(kt_begin, 0, ps, k0pg[ps]);
-        if (kt_begin + 1 < kt_end) dma_k_pass(kt_begin + 1, 1, ps, k1pg[ps]);
-        dma_v_pass(kt_begin, 0, ps, v0pg[ps]);
+        dma_k_pass(k_rsq, kt_begin, 0, ps, k0pg[ps]);
+        if (kt_begin + 1 < kt_end) dma_k_pass(k_rsq, kt_begin + 1, 1, ps, k1pg[ps]);
+        dma_v_pass(v_rsq, kt_begin, 0, ps, v0pg[ps]);
       }
     }
     LF_BARRIER_VM0();
@@ -260,14 +262,15 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
       const lf_elem* knext = lds_k[ks_nxt];
       const lf_elem* vbuf = lds_v[rel & 1];
       const int vs_ld = (rel + 1) & 1;                                 // slot V(kt+1) is loaded into
-      // direct load number d of this tile: K(kt+2) passes, then V(kt+1) passes
-      // (tiles past the last one are not fetched: wave-uniform tests)
+      // direct load number d of this tile: K(kt+2) passes, then V(kt+1) passes.  Tiles past the
+      // last one are asked for with an empty range instead of a test per load: a branch between the
+      // MFMAs ends the compiler's knowledge of what is in flight
+      lf_u32x4 k_cur = k_rsq, v_cur = v_rsq;
+      if (kt + 2 >= kt_end) k_cur[2] = 0u;
+      if (kt + 1 >= kt_end) v_cur[2] = 0u;
       auto dma_step = [&](int d) {
-        if (d < LF_NPASS) {
-          if (kt + 2 < kt_end) dma_k_pass(kt + 2, ks_ld, d, kpg[d]);
-        } else if (kt + 1 < kt_end) {
-          dma_v_pass(kt + 1, vs_ld, d - LF_NPASS, vpg[d - LF_NPASS]);
-        }
+        if (d < LF_NPASS) dma_k_pass(k_cur, kt + 2, ks_ld, d, kpg[d]);
+        else dma_v_pass(v_cur, kt + 1, vs_ld, d - LF_NPASS, vpg[d - LF_NPASS]);
       };
       // page offsets for the next tile's loads (table reads: in flight during this tile)
       unsigned kpg_n[LF_NPASS], vpg_n[LF_NPASS];
