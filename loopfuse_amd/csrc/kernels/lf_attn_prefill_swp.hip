@@ -73,7 +73,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // in a scalar register: what derives from it stays scalar
   const int l32 = lane & 31;
   const int g = lane >> 5;
 
@@ -123,7 +123,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
   const unsigned k_bytes = kPagedK ? (unsigned)(p.k_span * 2) : (unsigned)(((long long)(p.Sk - 1) * p.k_ss + LF_D) * 2);
   const unsigned v_bytes = kPagedV ? (unsigned)(p.v_span * 2) : (unsigned)(((long long)(p.Sk - 1) * p.v_ss + LF_D) * 2);
   const unsigned k_rowb = (unsigned)p.k_ss * 2u, v_rowb = (unsigned)p.v_ss * 2u;
-  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const int wave_u = wave;
   // page id (as a byte offset of the page + this kv head) for the rows of this wave in
   // pass ps of tile kt; tiles / rows past Sk re-use the last page (their rows are zeroed)
   auto page_off = [&](int which, int kt, int ps) -> unsigned {
