@@ -74,6 +74,53 @@ def test_backward_matches_autograd(B, Hq, Hkv, Sq, Sk, D, mask, window, dtype):
         assert rel <= (2e-2 if dtype == torch.bfloat16 else 4e-3), f"{name}: relative error {rel}"
 
 
+def _ref_head_fp32(q, k, v, dout, mask, window, scale):
+    """Reference for one (batch, kv head): q, dout [G, Sq, D] (the G query heads of the group), k, v
+    [Sk, D], all on the GPU; fp32 autograd on the dense graph.  Returns dq [G, Sq, D], dk, dv [Sk, D]."""
+    q, k, v = (t.float().detach().requires_grad_(True) for t in (q, k, v))
+    s = q @ k.t() * scale
+    Sq, Sk = s.shape[-2:]
+    i = torch.arange(Sq, device=s.device)[:, None]
+    j = torch.arange(Sk, device=s.device)[None, :]
+    keep = torch.ones(Sq, Sk, dtype=torch.bool, device=s.device)
+    if mask in ("causal", "sliding"):
+        keep &= j <= i
+    if mask == "sliding":
+        keep &= (i - j) < window
+    o = torch.softmax(s.masked_fill(~keep, float("-inf")), dim=-1) @ v
+    o.backward(dout.float())
+    return q.grad, k.grad, v.grad
+
+
+@pytest.mark.parametrize("name,Hkv,mask,window", [("config 2", 32, "causal", 0), ("config 3 without its softcap", 8, "sliding", 256)])
+def test_backward_full_size_every_head(name, Hkv, mask, window):
+    """The benchmark shapes (B8 Hq32 S2048 D128 bf16) at full size: every gradient element of every
+    (batch, head) against fp32 autograd on the dense graph, evaluated on the GPU one kv head at a time."""
+    B, Hq, S, D = 8, 32, 2048, 128
+    G = Hq // Hkv
+    g = torch.Generator().manual_seed(17)
+    q = torch.randn((B, Hq, S, D), generator=g).to(torch.bfloat16).to(DEV)
+    k = torch.randn((B, Hkv, S, D), generator=g).to(torch.bfloat16).to(DEV)
+    v = torch.randn((B, Hkv, S, D), generator=g).to(torch.bfloat16).to(DEV)
+    dout = torch.randn((B, Hq, S, D), generator=g).to(torch.bfloat16).to(DEV)
+    scale = D ** -0.5
+    plan = lowering.AttnPlan(mask=mask, window=window, scale=scale)
+    lse = torch.empty((B, Hq, S), dtype=torch.float32, device=DEV)
+    o = lowering.attention(q, k, v, plan, lse=lse)
+    dq, dk, dv = lowering.attention_backward(q, k, v, o, lse, dout, plan)
+    worst = {"dq": 0.0, "dk": 0.0, "dv": 0.0}
+    for b in range(B):
+        for hk in range(Hkv):
+            hs = slice(hk * G, (hk + 1) * G)
+            rq, rk, rv = _ref_head_fp32(q[b, hs], k[b, hk], v[b, hk], dout[b, hs], mask, window, scale)
+            for nm, got, want in (("dq", dq[b, hs], rq), ("dk", dk[b, hk], rk), ("dv", dv[b, hk], rv)):
+                rel = ((got.float() - want).norm() / want.norm()).item()
+                err = (got.float() - want).abs().max().item() / max(1.0, want.abs().max().item())
+                worst[nm] = max(worst[nm], rel)
+                assert rel <= 2e-2 and err <= 4e-2, f"{name} {nm} batch {b} kv head {hk}: relative {rel}, max abs {err}"
+    assert all(w > 0.0 for w in worst.values())       # the comparison saw data
+
+
 def test_backward_is_reproducible_and_refuses_what_it_does_not_serve():
     g = torch.Generator().manual_seed(5)
     q, k, v, dout = (torch.randn((1, 2, 256, 128), generator=g).to(torch.bfloat16).to(DEV) for _ in range(4))
