@@ -85,6 +85,7 @@ typedef struct LfAttnBwdParamsHost {
   int32_t B, Hq, Hkv, Sq, Sk;
   int32_t window;       /* sliding-window width (LF_MASK == 2) */
   float scale;
+  float softcap;        /* LF_SOFTCAP: cap of cap * tanh(s / cap) */
 } LfAttnBwdParamsHost;
 
 #ifdef __cplusplus

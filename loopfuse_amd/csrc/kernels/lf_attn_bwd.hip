@@ -1,9 +1,11 @@
 // lf_attn_bwd.hip — backward of the fused attention forward (dense K/V, mask none / causal /
-// sliding window, scale; no softcap, no bias) for gfx950.  The reference has no backward
+// sliding window, scale, optional softcap; no bias) for gfx950.  The reference has no backward
 // (its README lists it as future work); the formulas are the standard ones for
 // O = softmax(scale * Q K^T + mask) V with the row log-sum-exp L kept by the forward:
 //   P = exp(scale * Q K^T - L),  dV = P^T dO,  dP = dO V^T,  delta = rowsum(dO * O),
 //   dS = scale * P * (dP - delta),  dQ = dS K,  dK = dS^T Q.
+// With a softcap (LF_SOFTCAP) the scores are T = cap * tanh(scale * Q K^T / cap), P = exp(T - L), and
+// dS picks up the derivative of the cap: dS = scale * (1 - tanh^2) * P * (dP - delta).
 // Three kernels, no atomics, every result written once (deterministic):
 //   lf_attn_bwd_delta : delta[b, h, q]
 //   lf_attn_bwd_dkdv  : a workgroup owns 128 keys of one (batch, kv head) -- 4 waves x 32 keys,
@@ -39,6 +41,7 @@ struct LfAttnBwdParams {
   int B, Hq, Hkv, Sq, Sk;
   int window;
   float scale;
+  float softcap;          // LF_SOFTCAP: cap of cap * tanh(s / cap)
 };
 
 #define LF_BW_NT 256
@@ -251,7 +254,12 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
 #pragma unroll
     for (int ks = 0; ks < LF_NKS; ++ks) asm volatile("" : "+a"(kf[ks]), "+a"(vf[ks]));
   }
+#if LF_SOFTCAP
+  const float sc_exp = p.scale / p.softcap * (2.0f * LF_LOG2E);   // 2^(s * sc_exp) = e^(2x)
+  const float cexp = p.softcap * LF_LOG2E;                        // exponent of P: tanh x * cexp - L
+#else
   const float cexp = p.scale * LF_LOG2E;
+#endif
 
   lf_f32x16 dk[LF_NDB], dv[LF_NDB];
 #pragma unroll
@@ -339,10 +347,20 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
       const lf_f32x4 d4 = *reinterpret_cast<const lf_f32x4*>(&delta_s[ql]);
       lf_elem4 pw, dw;
       float pv[4];
+#if LF_SOFTCAP
+      float dcap[4];           // 1 - tanh^2
+#endif
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int i = 4 * i4 + e;
+#if LF_SOFTCAP
+        const float r = __builtin_amdgcn_rcpf(1.0f + lf_exp2(s[qb][i] * sc_exp));     // 1 / (e^(2x) + 1), x = s * scale / cap
+        const float th = 1.0f - 2.0f * r;                                               // tanh x
+        pv[e] = lf_exp2(th * cexp - l4[e]);
+        dcap[e] = 4.0f * r * (1.0f - r);
+#else
         pv[e] = lf_exp2(s[qb][i] * cexp - l4[e]);
+#endif
       }
       if (masked) {             // wave-uniform: most steps of a workgroup lie below the diagonal
 #pragma unroll
@@ -352,7 +370,11 @@ extern "C" __global__ void __launch_bounds__(LF_BW_NT, 1) lf_attn_bwd_dkdv(const
       for (int e = 0; e < 4; ++e) {
         const int i = 4 * i4 + e;
         pw[e] = lf_from_float(pv[e]);
+#if LF_SOFTCAP
+        dw[e] = lf_from_float(pv[e] * (dp[qb][i] - d4[e]) * dcap[e]);
+#else
         dw[e] = lf_from_float(pv[e] * (dp[qb][i] - d4[e]));
+#endif
       }
       const lf_u32x2 pu = __builtin_bit_cast(lf_u32x2, pw), du = __builtin_bit_cast(lf_u32x2, dw);
       pf[2 * qb + i4 / 2][2 * (i4 % 2)] = pu[0];
@@ -514,7 +536,12 @@ extern "C" __global__ void __launch_bounds__(LF_BW_DQ_NT, LF_BW_DQ_NT / 256) lf_
   const long long ridx = ((long long)b * p.Hq + h) * p.Sq + qr;
   const float lse_q = my_q < p.Sq ? p.lse[ridx] : __builtin_inff();
   const float delta_q = my_q < p.Sq ? p.delta[ridx] : 0.0f;
+#if LF_SOFTCAP
+  const float sc_exp = p.scale / p.softcap * (2.0f * LF_LOG2E);   // 2^(s * sc_exp) = e^(2x)
+  const float cexp = p.softcap * LF_LOG2E;                        // exponent of P: tanh x * cexp - L
+#else
   const float cexp = p.scale * LF_LOG2E;
+#endif
 
   lf_f32x16 dq[LF_NDB];
 #pragma unroll
@@ -623,8 +650,18 @@ extern "C" __global__ void __launch_bounds__(LF_BW_DQ_NT, LF_BW_DQ_NT / 256) lf_
       for (int i4 = 0; i4 < 4; ++i4) {
         lf_elem4 dw;
         float pv[4];
+#if LF_SOFTCAP
+        float dcap[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float r = __builtin_amdgcn_rcpf(1.0f + lf_exp2(s[4 * i4 + e] * sc_exp));
+          pv[e] = lf_exp2((1.0f - 2.0f * r) * cexp - lse_q);
+          dcap[e] = 4.0f * r * (1.0f - r);
+        }
+#else
 #pragma unroll
         for (int e = 0; e < 4; ++e) pv[e] = lf_exp2(s[4 * i4 + e] * cexp - lse_q);
+#endif
         if (masked) {           // wave-uniform: most tiles of a q tile lie below the diagonal
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
@@ -633,7 +670,13 @@ extern "C" __global__ void __launch_bounds__(LF_BW_DQ_NT, LF_BW_DQ_NT / 256) lf_
           }
         }
 #pragma unroll
-        for (int e = 0; e < 4; ++e) dw[e] = lf_from_float(pv[e] * (dp[4 * i4 + e] - delta_q));   // dS without `scale`
+        for (int e = 0; e < 4; ++e) {
+#if LF_SOFTCAP
+          dw[e] = lf_from_float(pv[e] * (dp[4 * i4 + e] - delta_q) * dcap[e]);
+#else
+          dw[e] = lf_from_float(pv[e] * (dp[4 * i4 + e] - delta_q));   // dS without `scale`
+#endif
+        }
         const lf_u32x2 du = __builtin_bit_cast(lf_u32x2, dw);
         dsf[2 * kb + i4 / 2][2 * (i4 % 2)] = du[0];
         dsf[2 * kb + i4 / 2][2 * (i4 % 2) + 1] = du[1];

@@ -406,7 +406,12 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
     // optional: the row's log-sum-exp of the scaled, masked scores in log2 units (what a
     // backward pass recomputes the probabilities from); -inf for a row that saw no key
     if (p.part_ml != nullptr && g == 0 && my_q < p.Sq)
+#if LF_SOFTCAP
+      // the kernel's scores are the capped ones minus the cap: the cap comes back in here
+      p.part_ml[((long long)b * p.Hq + h) * p.Sq + my_q] = mc_ref + __builtin_log2f(l_tot) + p.softcap * LF_LOG2E;
+#else
       p.part_ml[((long long)b * p.Hq + h) * p.Sq + my_q] = mc_ref + __builtin_log2f(l_tot);
+#endif
     {
       // Lane (q, g) holds, per block db, four 4-value chunks d = 32*db + 8*i4 + 4*g + 0..3.
       // One v_permlane32_swap per register pair trades chunks with the lane that holds

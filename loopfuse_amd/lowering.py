@@ -504,7 +504,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     that array raises ``runtime.ShimError``.
     ``lse`` (float32 [B, Hq, Sq], contiguous): also write each row's log-sum-exp of the scaled,
     masked scores, in log2 units -- what ``attention_backward`` recomputes the probabilities
-    from.  Served by ``lf_attn_prefill_swp`` without softcap; anything else raises ``UnsupportedPlan``.
+    from.  Served by ``lf_attn_prefill_swp`` (dense K/V); anything else raises ``UnsupportedPlan``.
     ``choice`` overrides the launch heuristics (what ``tuned_attention`` searches over):
     ``{"prefill": "swp" | "w32"}``, ``{"head_per_wave": bool, "splits": n}``.
     Returns O [B, Hq, Sq, D] and, with ``record_visits``, the uint8 record of the KV tiles
@@ -755,8 +755,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
             # lf_attn_prefill takes two q tiles (heavy + light) per workgroup, groups of 4 heads
             grid = 8 * ((per_xcd + 3) // 4 * 4) * ((nqt + 1) // 2)
         if lse is not None:
-            if family != "prefill_swp" or plan.softcap is not None or paged:
-                raise UnsupportedPlan("the row log-sum-exp is written by lf_attn_prefill_swp for dense K/V without softcap only")
+            if family != "prefill_swp" or paged:
+                raise UnsupportedPlan("the row log-sum-exp is written by lf_attn_prefill_swp for dense K/V only")
             if lse.dtype != torch.float32 or tuple(lse.shape) != (B, Hq, Sq) or not lse.is_contiguous() or lse.device != q.device:
                 raise UnsupportedPlan(f"lse must be a contiguous float32 [{B}, {Hq}, {Sq}] tensor on the device of Q")
             P.part_ml = lse.data_ptr()
@@ -842,25 +842,26 @@ class AttnBwdParams(ctypes.Structure):
         [(n, ctypes.c_void_p) for n in ("q", "k", "v", "o", "dout", "dq", "dk", "dv", "lse", "delta")]
         + [(f"{t}_{x}", ctypes.c_longlong) for t in ("q", "k", "v", "o", "do", "dq", "dk", "dv") for x in ("sb", "sh", "ss")]
         + [(n, ctypes.c_int) for n in ("B", "Hq", "Hkv", "Sq", "Sk", "window")]
-        + [("scale", ctypes.c_float)]
+        + [("scale", ctypes.c_float), ("softcap", ctypes.c_float)]
     )
 
 
-def bwd_dq_threads(mask: int) -> int:
+def bwd_dq_threads(mask: int, softcap: bool = False) -> int:
     """Workgroup size of lf_attn_bwd_dq: 8 waves (256 query rows, two waves per SIMD on one K/V
     tile stream) except under a sliding window, where a 256-row tile walks too many kv tiles
-    that only part of its rows can see."""
-    return 256 if mask == MASK_SLIDING else 512
+    that only part of its rows can see, and with a softcap, whose extra values do not fit the
+    256 registers a wave has at two per SIMD."""
+    return 256 if mask == MASK_SLIDING or softcap else 512
 
 
-def bwd_spec(dtype: torch.dtype, D: int, mask: int) -> KernelSpec:
-    return KernelSpec("bwd", _DTYPE_CODE[dtype], D, mask, extra=(f"-DLF_BW_DQ_NT={bwd_dq_threads(mask)}",))
+def bwd_spec(dtype: torch.dtype, D: int, mask: int, softcap: bool = False) -> KernelSpec:
+    return KernelSpec("bwd", _DTYPE_CODE[dtype], D, mask, softcap, extra=(f"-DLF_BW_DQ_NT={bwd_dq_threads(mask, softcap)}",))
 
 
 def attention_backward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor, lse: torch.Tensor,
                        dout: torch.Tensor, plan: AttnPlan):
-    """Gradients of ``attention(q, k, v, plan)`` for dense K/V (mask none / causal / sliding, scale;
-    no softcap, bias or paging): returns ``(dq, dk, dv)`` in the operands' dtype.  ``o`` and ``lse``
+    """Gradients of ``attention(q, k, v, plan)`` for dense K/V (mask none / causal / sliding, scale,
+    softcap; no bias or paging): returns ``(dq, dk, dv)`` in the operands' dtype.  ``o`` and ``lse``
     are the forward's output and row log-sum-exp (``attention(..., lse=...)``).  Three launches
     (csrc/kernels/lf_attn_bwd.hip): delta = rowsum(dO * O); dK and dV, one workgroup per 128 keys of
     a (batch, kv head); dQ, one workgroup per 128 query rows.  No atomics: results are
@@ -868,8 +869,13 @@ def attention_backward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: tor
     dtype = q.dtype
     if dtype not in _DTYPE_CODE:
         raise UnsupportedPlan(f"dtype {dtype} not supported by the MFMA kernels (bf16/fp16 only)")
-    if plan.softcap is not None or plan.k_paged or plan.v_paged or plan.denom_add != 0.0:
-        raise UnsupportedPlan("the backward kernels serve dense K/V without softcap")
+    if plan.k_paged or plan.v_paged or plan.denom_add != 0.0:
+        raise UnsupportedPlan("the backward kernels serve dense K/V and the plain softmax denominator")
+    softcap = None
+    if plan.softcap is not None:
+        softcap = abs(float(plan.softcap))
+        if not (softcap > 0.0) or not math.isfinite(softcap):
+            raise UnsupportedPlan("softcap must be finite and non-zero")
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise UnsupportedPlan("Q, K, V must be [B, H, S, D]")
     B, Hq, Sq, D = q.shape
@@ -909,7 +915,8 @@ def attention_backward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: tor
         setattr(P, pre + "_ss", t.stride(2))
     P.B, P.Hq, P.Hkv, P.Sq, P.Sk, P.window = B, Hq, Hkv, Sq, Sk, window
     P.scale = float(plan.scale)
-    spec = bwd_spec(dtype, D, mask)
+    P.softcap = softcap if softcap is not None else 0.0
+    spec = bwd_spec(dtype, D, mask, softcap is not None)
     keep = (q, k, v, o, dout, lse, delta, dq, dk, dv)  # noqa: F841  (tensors stay alive until the launches are queued)
     rows = B * Hq * Sq
     get_kernel(spec, "lf_attn_bwd_delta").launch(((rows + 15) // 16, 1, 1), (256, 1, 1), P)
@@ -921,7 +928,7 @@ def attention_backward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: tor
             grp = int(e.split("=")[1])
     pairs = ((B * Hkv + 7) // 8 + grp - 1) // grp * grp
     get_kernel(spec, "lf_attn_bwd_dkdv").launch((8 * pairs * ((Sk + 127) // 128), 1, 1), (256, 1, 1), P)
-    nt = bwd_dq_threads(mask)
+    nt = bwd_dq_threads(mask, softcap is not None)
     get_kernel(spec, "lf_attn_bwd_dq").launch((8 * pairs * (Hq // Hkv) * ((Sq + nt // 2 - 1) // (nt // 2)), 1, 1),
                                               (nt, 1, 1), P)
     _last_launch.set({"kernels": ["lf_attn_bwd_delta", "lf_attn_bwd_dkdv", "lf_attn_bwd_dq"]})

@@ -32,48 +32,51 @@ def _rows(t: torch.Tensor) -> torch.Tensor:
 
 @torch.library.custom_op("loopfuse_amd::attention_fwd", mutates_args=())
 def attention_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: int, window: int,
-                  scale: float) -> tuple[torch.Tensor, torch.Tensor]:
+                  scale: float, softcap: float) -> tuple[torch.Tensor, torch.Tensor]:
     """O [B, Hq, Sq, D] and the rows' log-sum-exp [B, Hq, Sq] (float32, log2 units)."""
     if not q.is_cuda:
         raise RuntimeError("loopfuse_amd: attention_fwd needs tensors on the GPU; the HIP path has no CPU fallback")
-    plan = lowering.AttnPlan(mask=_MASK_NAME[mask], window=int(window), scale=float(scale))
+    plan = lowering.AttnPlan(mask=_MASK_NAME[mask], window=int(window), scale=float(scale),
+                             softcap=float(softcap) if softcap else None)       # 0: no cap
     lse = torch.empty(q.shape[:-1], dtype=torch.float32, device=q.device)
     counters["fwd"] += 1
     return lowering.attention(_rows(q), _rows(k), _rows(v), plan, lse=lse), lse
 
 
 @attention_fwd.register_fake
-def _(q, k, v, mask, window, scale):
+def _(q, k, v, mask, window, scale, softcap):
     return q.new_empty(q.shape), q.new_empty(q.shape[:-1], dtype=torch.float32)
 
 
 @torch.library.custom_op("loopfuse_amd::attention_bwd", mutates_args=())
 def attention_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor, lse: torch.Tensor,
-                  dout: torch.Tensor, mask: int, window: int, scale: float) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+                  dout: torch.Tensor, mask: int, window: int, scale: float,
+                  softcap: float) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     if not q.is_cuda:
         raise RuntimeError("loopfuse_amd: attention_bwd needs tensors on the GPU; the HIP path has no CPU fallback")
-    plan = lowering.AttnPlan(mask=_MASK_NAME[mask], window=int(window), scale=float(scale))
+    plan = lowering.AttnPlan(mask=_MASK_NAME[mask], window=int(window), scale=float(scale),
+                             softcap=float(softcap) if softcap else None)
     counters["bwd"] += 1
     return lowering.attention_backward(_rows(q), _rows(k), _rows(v), _rows(o), lse.contiguous(), _rows(dout), plan)
 
 
 @attention_bwd.register_fake
-def _(q, k, v, o, lse, dout, mask, window, scale):
+def _(q, k, v, o, lse, dout, mask, window, scale, softcap):
     return q.new_empty(q.shape), k.new_empty(k.shape), v.new_empty(v.shape)
 
 
 def _setup(ctx, inputs, output):
-    q, k, v, mask, window, scale = inputs
+    q, k, v, mask, window, scale, softcap = inputs
     o, lse = output
     ctx.save_for_backward(q, k, v, o, lse)
-    ctx.consts = (mask, window, scale)
+    ctx.consts = (mask, window, scale, softcap)
 
 
 def _backward(ctx, d_o, d_lse):
     q, k, v, o, lse = ctx.saved_tensors
-    mask, window, scale = ctx.consts
-    dq, dk, dv = attention_bwd(q, k, v, o, lse, d_o, mask, window, scale)
-    return dq, dk, dv, None, None, None
+    mask, window, scale, softcap = ctx.consts
+    dq, dk, dv = attention_bwd(q, k, v, o, lse, d_o, mask, window, scale, softcap)
+    return dq, dk, dv, None, None, None, None
 
 
 attention_fwd.register_autograd(_backward, setup_context=_setup)
@@ -84,8 +87,8 @@ def trainable(match, dtype_of) -> str:
     ``dtype_of(i)`` / shapes come from the traced values of the match's inputs."""
     if match.k.paged or match.v.paged:
         return "paged K/V"
-    if match.has_tanh or match.base2 or match.denom_add or match.q2 is not None:
-        return "softcap / explicit softmax / two-part scores"
+    if match.base2 or match.denom_add or match.q2 is not None:
+        return "explicit softmax / two-part scores"
     if match.bias is not None or match.out_bias is not None:
         return "additive biases"
     if match.out_order or match.zero_blind_rows:
@@ -119,7 +122,8 @@ def fused_call_train(match, *vals):
 
     plan = match.plan_for(vals)
     out, _ = torch.ops.loopfuse_amd.attention_fwd(view(match.q), view(match.k), view(match.v),
-                                                  _MASK_CODE[plan.mask], plan.window, plan.scale)
+                                                  _MASK_CODE[plan.mask], plan.window, plan.scale,
+                                                  float(plan.softcap) if plan.softcap is not None else 0.0)
     if match.out_rank == 3:
         out = out.reshape(out.shape[0] * out.shape[1], out.shape[2], out.shape[3])
     return out

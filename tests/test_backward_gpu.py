@@ -16,12 +16,14 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def _ref(q, k, v, dout, mask, window, scale):
+def _ref(q, k, v, dout, mask, window, scale, softcap=None):
     """O and the gradients from autograd on the eager graph, in float64."""
     q, k, v = (t.double().detach().requires_grad_(True) for t in (q, k, v))
     g = q.shape[1] // k.shape[1]
     kk, vv = k.repeat_interleave(g, dim=1), v.repeat_interleave(g, dim=1)
     s = q @ kk.transpose(-2, -1) * scale
+    if softcap is not None:
+        s = softcap * torch.tanh(s / softcap)
     Sq, Sk = s.shape[-2:]
     i = torch.arange(Sq, device=s.device)[:, None]
     j = torch.arange(Sk, device=s.device)[None, :]
@@ -121,6 +123,33 @@ def test_backward_full_size_every_head(name, Hkv, mask, window):
     assert all(w > 0.0 for w in worst.values())       # the comparison saw data
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,mask,window,dtype,cap,qscale", [
+    (1, 4, 4, 256, 256, 128, "causal", 0, torch.bfloat16, 30.0, 1.0),
+    (1, 8, 2, 320, 320, 128, "sliding", 96, torch.bfloat16, 30.0, 1.0),
+    (1, 2, 2, 200, 333, 64, None, 0, torch.float16, 2.0, 3.0),          # a cap that bites: |scores| reach several caps
+    (1, 2, 1, 130, 130, 64, "causal", 0, torch.float16, -5.0, 2.0),      # cap given with a minus sign
+])
+def test_backward_with_softcap_matches_autograd(B, Hq, Hkv, Sq, Sk, D, mask, window, dtype, cap, qscale):
+    g = torch.Generator().manual_seed(Sq * 5 + Sk + D)
+    q = (torch.randn((B, Hq, Sq, D), generator=g) * qscale).to(dtype).to(DEV)
+    k, v = (torch.randn((B, Hkv, Sk, D), generator=g).to(dtype).to(DEV) for _ in range(2))
+    dout = torch.randn((B, Hq, Sq, D), generator=g).to(dtype).to(DEV)
+    scale = D ** -0.5
+    plan = lowering.AttnPlan(mask=mask, window=window, scale=scale, softcap=cap)
+    lse = torch.empty((B, Hq, Sq), dtype=torch.float32, device=DEV)
+    o = lowering.attention(q, k, v, plan, lse=lse)
+    o_ref, lse_ref, dq_ref, dk_ref, dv_ref = _ref(q, k, v, dout, mask, window, scale, cap)
+    tol = 2e-2 if dtype == torch.bfloat16 else 5e-3
+    assert (o.double() - o_ref).abs().max().item() <= tol
+    torch.testing.assert_close(lse.double(), lse_ref, rtol=1e-3, atol=4e-3)
+    dq, dk, dv = lowering.attention_backward(q, k, v, o, lse, dout, plan)
+    for name, got, want in (("dq", dq, dq_ref), ("dk", dk, dk_ref), ("dv", dv, dv_ref)):
+        rel = ((got.double() - want).norm() / want.norm()).item()
+        assert rel <= (2e-2 if dtype == torch.bfloat16 else 5e-3), f"{name}: relative error {rel}"
+        err = (got.double() - want).abs().max().item()
+        assert err <= (4e-2 if dtype == torch.bfloat16 else 1e-2) * max(1.0, want.abs().max().item()), f"{name}: max abs err {err}"
+
+
 def test_backward_is_reproducible_and_refuses_what_it_does_not_serve():
     g = torch.Generator().manual_seed(5)
     q, k, v, dout = (torch.randn((1, 2, 256, 128), generator=g).to(torch.bfloat16).to(DEV) for _ in range(4))
@@ -131,9 +160,9 @@ def test_backward_is_reproducible_and_refuses_what_it_does_not_serve():
     b = lowering.attention_backward(q, k, v, o, lse, dout, plan)
     assert all(torch.equal(x, y) for x, y in zip(a, b))          # no atomics: bit for bit
     with pytest.raises(lowering.UnsupportedPlan):
-        lowering.attention_backward(q, k, v, o, lse, dout, lowering.AttnPlan(mask="causal", scale=0.1, softcap=30.0))
+        lowering.attention_backward(q, k, v, o, lse, dout, lowering.AttnPlan(mask="causal", scale=0.1, denom_add=1.0))
     with pytest.raises(lowering.UnsupportedPlan):
-        lowering.attention(q, k, v, lowering.AttnPlan(mask="causal", scale=0.1, softcap=30.0), lse=lse)
+        lowering.attention_backward(q, k, v, o, lse, dout, lowering.AttnPlan(mask="causal", scale=0.1, softcap=0.0))
 
 
 # ---- through torch.compile(backend=loopfuse_backend): graphs traced for training
@@ -154,6 +183,13 @@ def _train_case(name):
         q, k, v = (t.transpose(1, 2) for t in (q, k, v))
         return (torch.softmax(q @ k.transpose(-2, -1) * 0.125, dim=-1) @ v).transpose(1, 2)
 
+    def capped(q, k, v):                # config 2 + softcap as the reference spells it (tests/benchmark.py:142-147)
+        s = q @ k.transpose(-2, -1) * (q.shape[-1] ** -0.5)
+        s = 30.0 * torch.tanh(s / 30.0)
+        return torch.softmax(torch.ops.loopfuse.causal_mask(s), dim=-1) @ v
+
+    if name == "capped":
+        return capped, [(1, 4, 256, 128)] * 3, "causal", 0
     if name == "causal":
         return causal, [(2, 4, 256, 128)] * 3, "causal", 0
     if name == "sliding_gqa":
@@ -161,7 +197,7 @@ def _train_case(name):
     return plain_bshd, [(2, 192, 4, 64)] * 3, None, 0
 
 
-@pytest.mark.parametrize("name", ["causal", "sliding_gqa", "plain_bshd"])
+@pytest.mark.parametrize("name", ["causal", "sliding_gqa", "plain_bshd", "capped"])
 def test_training_graph_runs_the_fused_forward_and_backward(name):
     """``torch.compile(backend=loopfuse_backend)`` on a function whose inputs require grad: the
     forward and the backward graph both run the HIP kernels (counted), and the gradients match
@@ -193,16 +229,16 @@ def test_training_graph_with_an_unserved_attention_stays_unfused():
     from loopfuse_amd import loopfuse_backend
     from loopfuse_amd.torch_backend import interface
 
-    def capped(q, k, v):
-        s = q @ k.transpose(-2, -1) * (q.shape[-1] ** -0.5)
-        s = torch.tanh(s / 30.0) * 30.0
+    def biased(q, k, v, bias):          # an additive score bias: fused for inference, no backward kernel
+        s = q @ k.transpose(-2, -1) * (q.shape[-1] ** -0.5) + bias
         return torch.softmax(torch.ops.loopfuse.causal_mask(s), dim=-1) @ v
 
     leaves = [torch.randn((1, 2, 128, 64), generator=torch.Generator().manual_seed(s)).to(torch.bfloat16).to(DEV).requires_grad_(True)
               for s in range(3)]
+    bias = torch.randn((1, 2, 128, 128), generator=torch.Generator().manual_seed(9)).to(torch.bfloat16).to(DEV)
     torch._dynamo.reset()
     before = dict(interface.stats)
-    out = torch.compile(capped, backend=loopfuse_backend)(*leaves)
+    out = torch.compile(biased, backend=loopfuse_backend)(*leaves, bias)
     out.sum().backward()
     assert interface.stats["training_graphs"] == before["training_graphs"]
     assert interface.stats["eager_training"] > before["eager_training"]

@@ -70,6 +70,8 @@ SPECS = [
     lowering.bwd_spec(torch.float16, 64, lowering.MASK_NONE),
     lowering.bwd_spec(torch.bfloat16, 128, lowering.MASK_SLIDING),     # 4-wave dQ kernel
     lowering.bwd_spec(torch.float16, 64, lowering.MASK_SLIDING),
+    lowering.bwd_spec(torch.bfloat16, 128, lowering.MASK_CAUSAL, True),     # with softcap
+    lowering.bwd_spec(torch.float16, 128, lowering.MASK_SLIDING, True),
 ]
 
 
