@@ -66,6 +66,9 @@
 #ifndef LF_QGROUP
 #define LF_QGROUP 8      /* (batch, head) pairs per group of slots */
 #endif
+#ifndef LF_SPLIT_EXP
+#define LF_SPLIT_EXP (!LF_SOFTCAP)     /* second key block's exponentials between the MFMAs of the first (config 2: -0.7 %; no gain with a softcap) */
+#endif
 
 extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_swp(const LfAttnParams p) {
   __shared__ __attribute__((aligned(16))) lf_elem lds_k[LF_KSLOTS][LF_BN * LF_D];
@@ -359,15 +362,23 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
         const float mc_sub = (mc_ref == LF_NEG_INF) ? 0.0f : mc_ref;
         float rs = 0.0f;
         lf_elem8 pf[LF_NKK];
+        // probabilities of the tile's key block kb, elements [i0, i1)
+        auto exp_block = [&](int kb, int i0, int i1) {
 #pragma unroll
-        for (int kb = 0; kb < LF_NKB; ++kb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
+          for (int i = i0; i < i1; ++i) {
             const float e = lf_exp2(s[kb][i] * cexp - mc_sub);
             rs += e;
             pf[2 * kb + i / 8][i % 8] = lf_from_float(e);
           }
-        l_run += rs;
+        };
+#if LF_SPLIT_EXP
+        // the exponentials of the second key block go between the MFMAs that consume the first:
+        // the wave keeps the matrix pipe busy during half of its own softmax
+        exp_block(0, 0, 16);
+#else
+#pragma unroll
+        for (int kb = 0; kb < LF_NKB; ++kb) exp_block(kb, 0, 16);
+#endif
 
         // ---- O^T += V^T P^T; the last steps also read the first fragments of K(kt+1)
 #if LF_SETPRIO
@@ -379,8 +390,12 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
           if (f + LF_VPF < LF_NFV) vf[f + LF_VPF] = v_frag(vbuf, f + LF_VPF);
           if (f >= LF_NFV - LF_KPF) kpre[f - (LF_NFV - LF_KPF)] = k_frag(knext, f - (LF_NFV - LF_KPF));
           o[f % LF_NDB] = lf_mfma32(vf[f], pf[f / LF_NDB], o[f % LF_NDB]);
+#if LF_SPLIT_EXP
+          if (f < LF_NFV / 2) exp_block(1, f * 32 / LF_NFV, (f + 1) * 32 / LF_NFV);
+#endif
           __builtin_amdgcn_sched_barrier(0);
         }
+        l_run += rs;
 #if LF_SETPRIO
         __builtin_amdgcn_s_setprio(0);
 #endif
