@@ -206,32 +206,11 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
     const bool wave_has_rows = wq0 < p.Sq;
     const int my_q = wq0 + l32;
 
-    // Q^T fragments (B operand): lane holds row my_q, d = 16*ks + 8*g .. +7.
-    lf_elem8 qf[LF_NKS];
-    {
-      const lf_elem* qrow = p.q + (long long)b * p.q_sb + (long long)h * p.q_sh +
-                            (long long)min(my_q, p.Sq - 1) * p.q_ss;
-#pragma unroll
-      for (int ks = 0; ks < LF_NKS; ++ks)
-        qf[ks] = __builtin_bit_cast(lf_elem8, *reinterpret_cast<const lf_u32x4*>(qrow + 16 * ks + 8 * g));
-    }
-    // the compiler waits for the Q loads here (a use it can see) and all older vector
-    // memory operations are drained, so its bookkeeping is clear before the direct
-    // loads, which it does not track, start
-#pragma unroll
-    for (int ks = 0; ks < LF_NKS; ++ks) asm volatile("" :: "v"(qf[ks]));
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-
-    lf_f32x16 o[LF_NDB];
-#pragma unroll
-    for (int db = 0; db < LF_NDB; ++db)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) o[db][i] = 0.0f;
-    float mc_ref = LF_NEG_INF;   // exponent offset of this query, log2 units (a lagging running max)
-    float l_run = 0.0f;          // this lane's share of the running sum
-
-    // ---- prologue: K(begin), K(begin+1), V(begin) resident; first K fragments in flight
-    // paged operands: page offsets of the passes issued during the coming tile (K two
+    // ---- prologue: K(begin), K(begin+1), V(begin) resident; first K fragments in flight.
+    // The direct loads go out before the Q fetch, so the q tile pays one memory latency
+    // instead of two (the memory counter retires in order: the compiler's wait for the Q
+    // registers, which counts only the loads it knows, also covers the older direct loads).
+    // Paged operands: page offsets of the passes issued during the coming tile (K two
     // tiles ahead, V one tile ahead), fetched a tile before they are needed
     unsigned kpg[LF_NPASS], vpg[LF_NPASS];
     {
@@ -251,6 +230,30 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
         dma_v_pass(v_rsq, kt_begin, 0, ps, v0pg[ps]);
       }
     }
+    // Q^T fragments (B operand): lane holds row my_q, d = 16*ks + 8*g .. +7.
+    lf_elem8 qf[LF_NKS];
+    {
+      const lf_elem* qrow = p.q + (long long)b * p.q_sb + (long long)h * p.q_sh +
+                            (long long)min(my_q, p.Sq - 1) * p.q_ss;
+#pragma unroll
+      for (int ks = 0; ks < LF_NKS; ++ks)
+        qf[ks] = __builtin_bit_cast(lf_elem8, *reinterpret_cast<const lf_u32x4*>(qrow + 16 * ks + 8 * g));
+    }
+    // the compiler waits for the Q loads here (a use it can see) and all older vector
+    // memory operations are drained, so its bookkeeping is clear before the direct
+    // loads of the tile loop, which it does not track, start
+#pragma unroll
+    for (int ks = 0; ks < LF_NKS; ++ks) asm volatile("" :: "v"(qf[ks]));
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    lf_f32x16 o[LF_NDB];
+#pragma unroll
+    for (int db = 0; db < LF_NDB; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[db][i] = 0.0f;
+    float mc_ref = LF_NEG_INF;   // exponent offset of this query, log2 units (a lagging running max)
+    float l_run = 0.0f;          // this lane's share of the running sum
+
     LF_BARRIER_VM0();
     lf_u32x4 kpre[LF_KPF];
 #pragma unroll
