@@ -48,6 +48,9 @@ CASES = [
     (1, 4, 2, 384, 384, 128, "sliding", 100, torch.bfloat16),
     (1, 2, 2, 192, 333, 64, None, 0, torch.bfloat16),               # Sq != Sk
     (1, 2, 1, 130, 130, 128, "sliding", 7, torch.float16),
+    (3, 6, 3, 593, 593, 128, "causal", 0, torch.bfloat16),          # odd length; 9 (batch, kv head) pairs: padded slot groups
+    (1, 3, 3, 1000, 1500, 64, None, 0, torch.float16),              # many tiles, Sq != Sk, neither a tile multiple
+    (2, 4, 1, 700, 700, 128, "sliding", 4096, torch.bfloat16),      # window wider than the sequence; four query heads per kv head
 ]
 
 
