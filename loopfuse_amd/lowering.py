@@ -682,7 +682,9 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     family = force_family
     if family is None:
         few = (Sq == 1 and group <= 64) or (group == 1 and Sq <= 16)
-        family = "decode" if (mask == MASK_NONE and few and Sk >= 16) else "prefill"
+        # a caller that wants the row log-sum-exp (a forward that a backward will follow) gets the
+        # prefill kernel, which writes it; the decode kernels do not
+        family = "decode" if (mask == MASK_NONE and few and Sk >= 16 and lse is None) else "prefill"
     keep = (q, k, v, out, kt, vt, score_bias, out_bias, q2, k2)  # noqa: F841  (tensors stay alive until the launch is queued)
 
     if family == "prefill" and not bias_bits and plan.denom_add == 0.0 and not d2:
