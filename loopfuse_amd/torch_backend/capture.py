@@ -94,6 +94,7 @@ class Stage:
     mask: Optional[str] = None
     window: Any = 0                # int or fx.Node (SymInt)
     bias: Optional[tuple] = None       # (Ids, stage shape when added): additive score bias, before the mask
+    bias_keep: int = 0                 # the "bias" is a boolean tensor: +1 True = visible, -1 True = masked (filled with -inf)
     out_bias: Optional[tuple] = None   # (Ids, stage shape when added): additive output bias
     # explicit softmax written with loopfuse.scan_max (reference tests/test_attention.py:95-125):
     uid: int = 0                       # set when scan_max is applied to this value
@@ -181,6 +182,7 @@ class BiasOperand:
 
     index: int
     dims: tuple                    # per logical dim (b, h, row, col): source dim it walks, or None (broadcast)
+    keep: int = 0                  # a boolean mask instead of an additive term: +1 True = visible, -1 True = masked
 
 
 @dataclasses.dataclass
@@ -289,10 +291,18 @@ class AttentionMatch:
             t = t.clone(memory_format=torch.contiguous_format)
         return t, None
 
-    def _bias_view(self, bo: Optional[BiasOperand], vals, shape):
+    def _bias_view(self, bo: Optional[BiasOperand], vals, shape, dtype=None):
         if bo is None:
             return None
         t = vals[bo.index]
+        if bo.keep:
+            # a boolean mask written with masked_fill / where: the kernels take it as the additive
+            # term 0 / -inf (of the mask's own, possibly broadcast, shape; tiles that are all -inf
+            # are never walked)
+            if t.dtype != torch.bool:
+                raise lowering.UnsupportedPlan("the mask is not the boolean tensor seen at trace time")
+            t = torch.zeros(t.shape, dtype=dtype or torch.float32, device=t.device).masked_fill_(
+                t if bo.keep < 0 else ~t, float("-inf"))
         strides = tuple(0 if d is None else t.stride(d) for d in bo.dims)
         for size, d in zip(shape, bo.dims):
             if d is not None and t.shape[d] != size:
@@ -340,7 +350,7 @@ class AttentionMatch:
         run = lowering.tuned_attention if self.tune else lowering.attention
         given = {"out": self.empty_out(vals, q.dtype, q.device)} if self.out_order else {}
         out = run(q, k, v, self.plan_for(vals), kt, vt, **given,
-                                 score_bias=self._bias_view(self.bias, vals, (B, Hq, Sq, Sk)),
+                                 score_bias=self._bias_view(self.bias, vals, (B, Hq, Sq, Sk), q.dtype),
                                  out_bias=self._bias_view(self.out_bias, vals, (B, Hq, Sq, D)),
                                  **self._second_product(vals))
         if self.out_rank == 3:
@@ -781,6 +791,22 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
     def is_number(x) -> bool:
         return isinstance(x, (int, float)) and not isinstance(x, bool)
 
+    def is_neg_inf(x) -> bool:
+        return (is_number(x) and x == float("-inf")) or (isinstance(x, Scalar) and x.expr == ("lit", float("-inf")))
+
+    def is_bool(ids) -> bool:
+        val = ids.src.node.meta.get("val") if isinstance(ids, Ids) and ids.src.kind == "node" else None
+        return isinstance(val, torch.Tensor) and val.dtype == torch.bool
+
+    def bool_mask(st, ids, keep):
+        """Scores whose masked elements are filled with -inf according to a boolean tensor: taken as
+        an additive 0 / -inf term (only -inf commutes with that reading: a finite fill value replaces
+        the score, it does not add to it)."""
+        if not (isinstance(st, Stage) and st.kind == "scores" and st.mask is None and st.bias is None and st.uid == 0
+                and st.sm == "" and st.lay is None):
+            raise _Skip("boolean mask on scores that already carry a mask or a bias")
+        return dataclasses.replace(st, bias=(ids, st.shape), bias_keep=keep)
+
     def meta_view(target, shape, args, kwargs):
         m = torch.empty(shape, device="meta")
         return tuple(target(m, *args, **kwargs).shape)
@@ -946,6 +972,11 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
                     raise _Skip("QK^T shapes disagree")
                 shape = tuple(qi.t.shape[:-1]) + (ki.t.shape[-1],)
                 return Stage("scores", shape, qi, ki, mat=(shape[-2], shape[-1]))
+            if tgt is aten.where.self and len(a) == 3 and is_bool(first):
+                # where(keep, scores, -inf) / where(masked, -inf, scores): a mask given as a boolean tensor
+                pos = 1 if isinstance(a[1], Stage) else (2 if isinstance(a[2], Stage) else 0)
+                if pos and is_neg_inf(a[3 - pos]):
+                    return bool_mask(a[pos], first, +1 if pos == 1 else -1)
             raise _Skip(f"op on a tensor view: {tgt}")
 
         # -- the attention pipeline
@@ -1066,6 +1097,11 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
                     return dataclasses.replace(st, has_tanh=True)
                 if tgt is torch.ops.loopfuse.causal_mask.default and st.mask is None:
                     return dataclasses.replace(st, mask="causal")
+                if tgt in (aten.masked_fill.Scalar, aten.masked_fill.Tensor) and len(a) == 3 and isinstance(a[1], Ids) \
+                        and is_bool(a[1]) and is_neg_inf(a[2]):
+                    return bool_mask(st, a[1], -1)          # scores.masked_fill(masked, -inf)
+                if tgt is aten.full_like.default and len(a) > 1 and is_neg_inf(a[1]):
+                    return Scalar(node, float("-inf"), ("lit", float("-inf")))     # the other branch of a where()
                 if tgt is torch.ops.loopfuse.sliding_mask.default and st.mask is None:
                     w = node.args[1]
                     return dataclasses.replace(st, mask="sliding", window=w if isinstance(w, torch.fx.Node) else int(a[1]))
@@ -1199,7 +1235,7 @@ def _build_match(out_node: torch.fx.Node, st: Stage) -> AttentionMatch:
     bias_op = obias_op = None
     if st.bias is not None:
         n, dims = _fit_bias(st.bias, (qshape[0], qshape[1], qshape[2], sk))
-        bias_op = BiasOperand(slot(n), dims)
+        bias_op = BiasOperand(slot(n), dims, st.bias_keep)
     if st.out_bias is not None:
         n, dims = _fit_bias(st.out_bias, qshape)
         obias_op = BiasOperand(slot(n), dims)

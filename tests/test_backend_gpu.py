@@ -329,6 +329,54 @@ def test_attention_inside_a_transformer_block():
     assert (got - want).abs().max() <= 4 * TOL and (got - want).abs().mean() <= 4e-3
 
 
+@pytest.mark.parametrize("which", ["buffer_eq_zero", "arange_where", "key_padding_decode", "band"])
+def test_boolean_masks_written_by_hand(which):
+    """``masked_fill`` / ``where`` with a boolean tensor and -inf (a causal buffer cut to the sequence as in
+    the common GPT module, index comparisons built in the graph, a key-padding mask on a decode step, a
+    symmetric band): fused, the mask travelling as a 0 / -inf score term."""
+    import math
+    ninf = float("-inf")
+    if which == "buffer_eq_zero":
+        def fn(x, wqkv, wo, buf):
+            B, T, E = x.shape
+            q, k, v = ((x @ w).view(B, T, 8, E // 8).transpose(1, 2) for w in wqkv.unbind(0))
+            att = (q @ k.transpose(-2, -1)) * (1.0 / math.sqrt(k.size(-1)))
+            att = att.masked_fill(buf[:, :, :T, :T] == 0, ninf)
+            y = torch.softmax(att, dim=-1) @ v
+            return y.transpose(1, 2).contiguous().view(B, T, E) @ wo
+        ins = (rand((2, 593, 512), seed=1), rand((3, 512, 512), seed=2) * 0.04, rand((512, 512), seed=3) * 0.04,
+               torch.tril(torch.ones(1024, 1024)).view(1, 1, 1024, 1024))
+        ins = tuple(t.to(torch.bfloat16) if i < 3 else t for i, t in enumerate(ins))
+    elif which == "arange_where":
+        def fn(q, k, v):
+            s = q @ k.transpose(-2, -1) * q.shape[-1] ** -0.5
+            i = torch.arange(q.shape[-2], device=q.device)[:, None]
+            j = torch.arange(k.shape[-2], device=q.device)[None, :]
+            return torch.softmax(torch.where((j <= i) & (i - j < 100), s, ninf), -1) @ v
+        ins = tuple(rand((2, 4, 700, 128), seed=s) for s in (1, 2, 3))
+    elif which == "key_padding_decode":
+        def fn(q, k, v, pad):
+            s = q @ k.transpose(-2, -1) * q.shape[-1] ** -0.5
+            return torch.softmax(s.masked_fill(pad[:, None, None, :], ninf), -1) @ v
+        pad = torch.zeros(8, 1024, dtype=torch.bool)
+        for b in range(8):
+            pad[b, 200 + 100 * b:] = True
+        ins = (rand((8, 8, 1, 128), seed=1), rand((8, 8, 1024, 128), seed=2), rand((8, 8, 1024, 128), seed=3), pad)
+    else:
+        def fn(q, k, v):
+            s = q @ k.transpose(-2, -1) * q.shape[-1] ** -0.5
+            i = torch.arange(q.shape[-2], device=q.device)[:, None]
+            j = torch.arange(k.shape[-2], device=q.device)[None, :]
+            return torch.softmax(s.masked_fill((i - j).abs() >= 64, ninf), -1) @ v
+        ins = (rand((1, 4, 300, 64), seed=1), rand((1, 4, 420, 64), seed=2), rand((1, 4, 420, 64), seed=3))
+    got = run_fused(fn, ins)
+    (m,) = interface.last_matches
+    assert m.mask is None and m.bias is not None and m.bias.keep in (1, -1)
+    want = fn(*[t.to(DEV).float() if t.dtype == torch.bfloat16 else t.to(DEV) for t in ins]).float().cpu()   # eager, fp32
+    assert torch.isfinite(got).all()
+    assert (got - want).abs().max() <= (4 * TOL if which == "buffer_eq_zero" else TOL)
+
+
 @pytest.mark.parametrize("which", ["causal", "gqa_decode", "scale_rect", "module", "bool_mask", "float_mask"])
 @pytest.mark.parametrize("dynamic", [True, False])
 def test_torch_fused_attention_calls_are_taken_over(which, dynamic):

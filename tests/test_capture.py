@@ -426,6 +426,83 @@ def test_rewritten_graphs_compute_the_same(which, monkeypatch):
         torch.testing.assert_close(g, w, rtol=2e-4, atol=2e-4)
 
 
+@pytest.mark.parametrize("which", ["buffer_eq_zero", "tril_in_graph", "arange_where", "where_full_like",
+                                   "where_masked_first", "key_padding", "band_not_causal"])
+def test_boolean_masks_written_by_hand_are_fused(which, monkeypatch):
+    """Masks spelled with ``masked_fill`` / ``where`` on a boolean tensor (a registered buffer cut to
+    the sequence, ``ones().tril()``, ``arange`` comparisons, a key-padding mask), filled with -inf:
+    the attention is fused with the mask as a 0 / -inf score term, whatever shape the mask has."""
+    monkeypatch.setattr(capture.AttentionMatch, "run", _oracle_run)
+    f32 = lambda *shape, seed=0: torch.randn(*shape, generator=torch.Generator().manual_seed(seed))
+    S, Sk, D = 24, 40, 64
+    ninf = float("-inf")
+    q, k, v = f32(2, 3, S, D), f32(2, 3, S, D, seed=1), f32(2, 3, S, D, seed=2)
+    kr, vr = f32(2, 3, Sk, D, seed=3), f32(2, 3, Sk, D, seed=4)
+    if which == "buffer_eq_zero":
+        def fn(q, k, v, buf):                  # the mask of a 64-token context cut to the sequence at hand
+            T = q.shape[-2]
+            att = (q @ k.transpose(-2, -1)) * (1.0 / math.sqrt(k.size(-1)))
+            return torch.softmax(att.masked_fill(buf[:, :, :T, :T] == 0, ninf), dim=-1) @ v
+        ins = (q, k, v, torch.tril(torch.ones(64, 64)).view(1, 1, 64, 64))
+    elif which == "tril_in_graph":
+        def fn(q, k, v):                       # bottom-right aligned on a rectangular problem
+            s = q @ k.transpose(-2, -1) * q.shape[-1] ** -0.5
+            m = torch.ones(q.shape[-2], k.shape[-2], dtype=torch.bool).tril(diagonal=k.shape[-2] - q.shape[-2])
+            return torch.softmax(s.masked_fill(~m, ninf), -1) @ v
+        ins = (q, kr, vr)
+    elif which == "arange_where":
+        def fn(q, k, v):
+            s = q @ k.transpose(-2, -1) * q.shape[-1] ** -0.5
+            i, j = torch.arange(q.shape[-2])[:, None], torch.arange(k.shape[-2])[None, :]
+            return torch.softmax(torch.where(j <= i, s, ninf), -1) @ v
+        ins = (q, k, v)
+    elif which == "where_full_like":
+        def fn(q, k, v, m):
+            s = q @ k.transpose(-2, -1) * q.shape[-1] ** -0.5
+            return torch.softmax(torch.where(m, s, torch.full_like(s, ninf)), -1) @ v
+        ins = (q, k, v, torch.ones(S, S, dtype=torch.bool).tril())
+    elif which == "where_masked_first":
+        def fn(q, k, v, m):
+            s = q @ k.transpose(-2, -1) * q.shape[-1] ** -0.5
+            return torch.softmax(torch.where(m, ninf, s), -1) @ v
+        ins = (q, k, v, torch.ones(S, S, dtype=torch.bool).triu(diagonal=1))
+    elif which == "key_padding":
+        def fn(q, k, v, pad):                  # [B, Sk] True = padding
+            s = q @ k.transpose(-2, -1) * q.shape[-1] ** -0.5
+            return torch.softmax(s.masked_fill(pad[:, None, None, :], ninf), -1) @ v
+        pad = torch.zeros(2, Sk, dtype=torch.bool)
+        pad[0, 30:] = True
+        pad[1, 17:] = True
+        ins = (q, kr, vr, pad)
+    else:
+        def fn(q, k, v):                       # a symmetric band: neither of the two mask flags
+            s = q @ k.transpose(-2, -1) * q.shape[-1] ** -0.5
+            i, j = torch.arange(q.shape[-2])[:, None], torch.arange(k.shape[-2])[None, :]
+            return torch.softmax(s.masked_fill((i - j).abs() >= 5, ninf), -1) @ v
+        ins = (q, k, v)
+    torch._dynamo.reset()
+    before = dict(interface.stats)
+    with torch.no_grad():
+        got = torch.compile(fn, backend=loopfuse_amd.loopfuse_backend, dynamic=True)(*ins)
+    assert interface.stats["fused"] == before["fused"] + 1
+    (m,) = interface.last_matches
+    assert m.mask is None and m.bias is not None and m.bias.keep in (1, -1)
+    torch.testing.assert_close(got, fn(*ins), rtol=2e-4, atol=2e-4)
+
+
+@pytest.mark.parametrize("fill", [-1e9, 0.0, torch.finfo(torch.float32).min])
+def test_finite_fill_values_are_not_taken_for_masks(fill):
+    """A finite fill value replaces the score; only -inf can be read as an additive term (a row whose
+    keys are all filled differs otherwise), so these graphs run as captured."""
+    def fn(q, k, v, m):
+        s = q @ k.transpose(-2, -1) * q.shape[-1] ** -0.5
+        return torch.softmax(s.masked_fill(~m, fill), -1) @ v
+    f32 = lambda *shape, seed=0: torch.randn(*shape, generator=torch.Generator().manual_seed(seed))
+    ins = (f32(1, 2, 24, 64), f32(1, 2, 24, 64, seed=1), f32(1, 2, 24, 64, seed=2), torch.ones(24, 24, dtype=torch.bool).tril())
+    box = capture_graph(fn, ins)
+    assert "match" not in box
+
+
 def test_backend_on_cpu_tensors_runs_graph_unfused():
     """CPU tensors have no HIP path: the compiled function must still be correct (it
     runs the captured graph) and must say so in the stats."""
