@@ -39,6 +39,7 @@ from typing import Any, Optional
 import torch
 
 from .. import lowering
+from . import index_masks
 
 aten = torch.ops.aten
 prims = torch.ops.prims
@@ -798,13 +799,23 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
         val = ids.src.node.meta.get("val") if isinstance(ids, Ids) and ids.src.kind == "node" else None
         return isinstance(val, torch.Tensor) and val.dtype == torch.bool
 
-    def bool_mask(st, ids, keep):
-        """Scores whose masked elements are filled with -inf according to a boolean tensor: taken as
+    def bool_mask(st, ids, keep, mask_node):
+        """Scores whose masked elements are filled with -inf according to a boolean tensor.  A mask the
+        graph builds from indices alone (tril of ones, arange comparisons) that comes out as the causal
+        triangle or a causal window becomes the kernels' mask flag; any other boolean tensor is taken as
         an additive 0 / -inf term (only -inf commutes with that reading: a finite fill value replaces
         the score, it does not add to it)."""
         if not (isinstance(st, Stage) and st.kind == "scores" and st.mask is None and st.bias is None and st.uid == 0
                 and st.sm == "" and st.lay is None):
             raise _Skip("boolean mask on scores that already carry a mask or a bias")
+        pred = sym.get(mask_node) if isinstance(mask_node, torch.fx.Node) else None
+        if isinstance(pred, index_masks.Pred):
+            lo_hi = index_masks.band(pred, keep)
+            if lo_hi is not None and lo_hi[0] == 0:
+                if lo_hi[1] == math.inf:
+                    return dataclasses.replace(st, mask="causal")
+                if lo_hi[1] >= 0:
+                    return dataclasses.replace(st, mask="sliding", window=int(lo_hi[1]) + 1)
         return dataclasses.replace(st, bias=(ids, st.shape), bias_keep=keep)
 
     def meta_view(target, shape, args, kwargs):
@@ -813,6 +824,7 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
 
     matches: list = []
     reasons: list = []
+    sym: dict = {}
     finalised: dict = {}
     uid_box = [0]
 
@@ -976,7 +988,7 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
                 # where(keep, scores, -inf) / where(masked, -inf, scores): a mask given as a boolean tensor
                 pos = 1 if isinstance(a[1], Stage) else (2 if isinstance(a[2], Stage) else 0)
                 if pos and is_neg_inf(a[3 - pos]):
-                    return bool_mask(a[pos], first, +1 if pos == 1 else -1)
+                    return bool_mask(a[pos], first, +1 if pos == 1 else -1, node.args[0])
             raise _Skip(f"op on a tensor view: {tgt}")
 
         # -- the attention pipeline
@@ -1099,7 +1111,7 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
                     return dataclasses.replace(st, mask="causal")
                 if tgt in (aten.masked_fill.Scalar, aten.masked_fill.Tensor) and len(a) == 3 and isinstance(a[1], Ids) \
                         and is_bool(a[1]) and is_neg_inf(a[2]):
-                    return bool_mask(st, a[1], -1)          # scores.masked_fill(masked, -inf)
+                    return bool_mask(st, a[1], -1, node.args[1])          # scores.masked_fill(masked, -inf)
                 if tgt is aten.full_like.default and len(a) > 1 and is_neg_inf(a[1]):
                     return Scalar(node, float("-inf"), ("lit", float("-inf")))     # the other branch of a where()
                 if tgt is torch.ops.loopfuse.sliding_mask.default and st.mask is None:
@@ -1132,6 +1144,7 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
             raise NoMatch("graph has constant tensors")
         if node.op != "call_function":
             raise NoMatch(f"unsupported node kind {node.op}")
+        sym[node] = index_masks.step(node, sym)       # masks built from indices alone, as predicates
         a = arg(node.args)
         kw = arg(node.kwargs)
         first = a[0] if a else None

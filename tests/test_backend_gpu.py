@@ -371,7 +371,10 @@ def test_boolean_masks_written_by_hand(which):
         ins = (rand((1, 4, 300, 64), seed=1), rand((1, 4, 420, 64), seed=2), rand((1, 4, 420, 64), seed=3))
     got = run_fused(fn, ins)
     (m,) = interface.last_matches
-    assert m.mask is None and m.bias is not None and m.bias.keep in (1, -1)
+    if which == "arange_where":        # built from indices alone: recognised as a causal window, no mask tensor at all
+        assert m.mask == "sliding" and m.window == 100 and m.bias is None
+    else:
+        assert m.mask is None and m.bias is not None and m.bias.keep in (1, -1)
     want = fn(*[t.to(DEV).float() if t.dtype == torch.bfloat16 else t.to(DEV) for t in ins]).float().cpu()   # eager, fp32
     assert torch.isfinite(got).all()
     assert (got - want).abs().max() <= (4 * TOL if which == "buffer_eq_zero" else TOL)

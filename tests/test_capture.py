@@ -486,7 +486,10 @@ def test_boolean_masks_written_by_hand_are_fused(which, monkeypatch):
         got = torch.compile(fn, backend=loopfuse_amd.loopfuse_backend, dynamic=True)(*ins)
     assert interface.stats["fused"] == before["fused"] + 1
     (m,) = interface.last_matches
-    assert m.mask is None and m.bias is not None and m.bias.keep in (1, -1)
+    if which == "arange_where":            # a mask built from indices alone that is the causal triangle: a flag
+        assert m.mask == "causal" and m.bias is None
+    else:
+        assert m.mask is None and m.bias is not None and m.bias.keep in (1, -1)
     torch.testing.assert_close(got, fn(*ins), rtol=2e-4, atol=2e-4)
 
 
