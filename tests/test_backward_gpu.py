@@ -191,6 +191,14 @@ def _train_case(name):
         s = 30.0 * torch.tanh(s / 30.0)
         return torch.softmax(torch.ops.loopfuse.causal_mask(s), dim=-1) @ v
 
+    def tril_by_hand(q, k, v):          # the common GPT module: the triangle built in the graph, filled with -inf
+        T = q.shape[-2]
+        att = (q @ k.transpose(-2, -1)) * (1.0 / math.sqrt(k.size(-1)))
+        att = att.masked_fill(torch.tril(torch.ones(T, T, device=q.device)).view(1, 1, T, T) == 0, float("-inf"))
+        return torch.softmax(att, dim=-1) @ v
+
+    if name == "tril_by_hand":
+        return tril_by_hand, [(2, 4, 300, 64)] * 3, "causal", 0
     if name == "capped":
         return capped, [(1, 4, 256, 128)] * 3, "causal", 0
     if name == "causal":
@@ -200,7 +208,7 @@ def _train_case(name):
     return plain_bshd, [(2, 192, 4, 64)] * 3, None, 0
 
 
-@pytest.mark.parametrize("name", ["causal", "sliding_gqa", "plain_bshd", "capped"])
+@pytest.mark.parametrize("name", ["causal", "sliding_gqa", "plain_bshd", "capped", "tril_by_hand"])
 def test_training_graph_runs_the_fused_forward_and_backward(name):
     """``torch.compile(backend=loopfuse_backend)`` on a function whose inputs require grad: the
     forward and the backward graph both run the HIP kernels (counted), and the gradients match
