@@ -689,6 +689,17 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
         if h is None:
             hints[s] = 8
     sizes = _stand_in_sizes(hints)
+    # a symbol that some shape divides (x.chunk(3, -1) of a dynamic width: (s + 2) // 3) keeps its traced
+    # value: an arbitrary stand-in would not divide the same way (down to a dim of 0)
+    for n in graph.nodes:
+        val = n.meta.get("val")
+        for t in (val if isinstance(val, (tuple, list)) else (val,)):
+            for d in (t.shape if isinstance(t, torch.Tensor) else (t,)):
+                if isinstance(d, torch.SymInt) and any(
+                        type(e).__name__ in ("FloorDiv", "CleanDiv", "CeilDiv", "Mod", "PythonMod", "ModularIndexing", "floor")
+                        for e in sympy.preorder_traversal(d.node.expr)):
+                    for sym_ in d.node.expr.free_symbols:
+                        sizes[sym_] = hints[sym_]
 
     # Static dims normally keep their values (a head dim of 128 marked static).  A graph
     # traced with static shapes at real sizes would need id tensors of the real size: then
@@ -738,7 +749,10 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
 
     def concrete(d) -> int:
         if isinstance(d, torch.SymInt):
-            return int(d.node.expr.subs(sizes))
+            v = int(d.node.expr.subs(sizes))
+            if v < 0 or (v == 0 and _hint(d) != 0):
+                raise NoMatch("stand-in sizes do not reproduce the traced shapes")
+            return v
         d = int(d)
         if d in fmap:
             return fmap[d]

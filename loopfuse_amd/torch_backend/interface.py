@@ -50,7 +50,7 @@ USE_HARDCODE_KERNEL = os.environ.get("USE_HARDCODE_KERNEL", "0") == "1"
 # "refused_signatures" = argument layouts latched as not servable (see optimized_fn)
 stats = {"fused": 0, "eager_graph": 0, "eager_runtime": 0, "eager_training": 0, "compiled_graphs": 0, "matched_graphs": 0,
          "refused_signatures": 0, "derived_graphs": 0, "generic_graphs": 0, "fused_generic": 0,
-         "training_graphs": 0, "fused_training": 0}
+         "training_graphs": 0, "fused_training": 0, "match_errors": 0}
 
 
 def _frontend() -> str:
@@ -322,6 +322,11 @@ def loopfuse_compiler(gm: torch.fx.GraphModule, sample_inputs, input_names: list
         except capture.NoMatch as e:
             matches = []
             reason = str(e)
+        except Exception as e:                     # a front-end bug must not take the graph down: it runs as captured
+            log.warning("attention matching failed on this graph (%s: %s); it runs as captured", type(e).__name__, e)
+            stats["match_errors"] += 1
+            matches = []
+            reason = f"{type(e).__name__}: {e}"
         else:
             reason = ""
         if frontend == "check" and derived is not None:

@@ -506,6 +506,45 @@ def test_finite_fill_values_are_not_taken_for_masks(fill):
     assert "match" not in box
 
 
+def test_dynamic_width_split_into_heads(monkeypatch):
+    """``qkv.chunk(3, -1)`` of a tensor whose width is a symbol: head dim (s + 2) // 12.  The stand-in
+    sizes must divide as the traced ones do (an arbitrary stand-in once gave a head dim of 0)."""
+    monkeypatch.setattr(capture.AttentionMatch, "run", _oracle_run)
+    B, N, H, D = 2, 24, 4, 64
+
+    def fn(qkv):
+        q, k, v = qkv.chunk(3, dim=-1)
+        sh = lambda t: t.view(B, N, H, D).transpose(1, 2)
+        return F.scaled_dot_product_attention(sh(q), sh(k), sh(v), is_causal=True).transpose(1, 2).reshape(B, N, H * D)
+
+    import torch.nn.functional as F
+    x = torch.randn(B, N, 3 * H * D, generator=torch.Generator().manual_seed(0))
+    torch._dynamo.reset()
+    before = dict(interface.stats)
+    with torch.no_grad():
+        got = torch.compile(fn, backend=loopfuse_amd.loopfuse_backend, dynamic=True)(x)
+    assert interface.stats["fused"] == before["fused"] + 1 and interface.stats["match_errors"] == before["match_errors"]
+    torch.testing.assert_close(got, fn(x), rtol=2e-4, atol=2e-4)
+
+
+def test_an_error_inside_the_matcher_leaves_the_graph_running(monkeypatch):
+    """The backend never fails a compilation because its own pattern matching broke: the graph runs
+    as captured and the event is counted."""
+    def boom(gm):
+        raise ZeroDivisionError("0.0 cannot be raised to a negative power")
+    monkeypatch.setattr(capture, "match_attention", boom)
+
+    def fn(q, k, v):
+        return torch.softmax(torch.ops.loopfuse.causal_mask(q @ k.transpose(-2, -1) * 0.125), -1) @ v
+    ins = [torch.randn(1, 2, 16, 64, generator=torch.Generator().manual_seed(s)) for s in range(3)]
+    torch._dynamo.reset()
+    before = dict(interface.stats)
+    with torch.no_grad():
+        got = torch.compile(fn, backend=loopfuse_amd.loopfuse_backend, dynamic=True)(*ins)
+    assert interface.stats["match_errors"] == before["match_errors"] + 1 and interface.stats["fused"] == before["fused"]
+    torch.testing.assert_close(got, fn(*ins))
+
+
 def test_backend_on_cpu_tensors_runs_graph_unfused():
     """CPU tensors have no HIP path: the compiled function must still be correct (it
     runs the captured graph) and must say so in the stats."""
