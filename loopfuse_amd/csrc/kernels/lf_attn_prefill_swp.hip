@@ -61,6 +61,11 @@
 
 // workgroup barrier that waits for this wave's direct-to-LDS loads but leaves LDS
 // reads in flight (the compiler's own barrier would wait for those too)
+#ifndef LF_BIAS
+#define LF_BIAS 0        /* 1: additive score bias [B, Hq, Sq, Sk] (a mask given as a tensor) with the tile classes
+                            that lf_bias_classify wrote into p.part_acc: dead tiles at either end of a q tile's
+                            range are not walked, all-zero tiles cost nothing, the others add their values */
+#endif
 #define LF_BARRIER_VM0() asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory")
 
 #ifndef LF_QGROUP
@@ -196,6 +201,31 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
       if (lo > 0) kt_begin = lo / LF_BN;
     }
 #endif
+#if LF_BIAS
+    // tile classes of the bias for this (batch, head, q tile): broadcast dims of the bias collapse
+    const int nhh = p.bias_sh ? p.Hq : 1;
+    const int cunit = ((p.bias_sb ? b : 0) * nhh + (p.bias_sh ? h : 0)) * nqt + qt;
+    const lf_cint* ccls = reinterpret_cast<const lf_cint*>(reinterpret_cast<unsigned long long>(p.part_acc)) +
+                          (long long)cunit * nkt;
+    {
+      // the q tile's range shrinks to its first .. last tile that is not dead (every wave scans for
+      // itself, 64 tiles per step: no exchange needed)
+      const int* vcls = reinterpret_cast<const int*>(p.part_acc) + (long long)cunit * nkt;
+      int lo = kt_end, hi = kt_begin;
+      for (int t0 = kt_begin; t0 < kt_end; t0 += 64) {
+        const int t = t0 + lane;
+        const unsigned long long live = __builtin_amdgcn_ballot_w64(t < kt_end && vcls[min(t, kt_end - 1)] != 0);
+        if (live != 0ull) {
+          lo = min(lo, t0 + (int)__builtin_ctzll(live));
+          hi = t0 + 64 - (int)__builtin_clzll(live);
+        }
+      }
+      kt_begin = min(lo, kt_end);
+      kt_end = max(hi, kt_begin);
+      kt_begin = __builtin_amdgcn_readfirstlane(kt_begin);
+      kt_end = __builtin_amdgcn_readfirstlane(kt_end);
+    }
+#endif
     if (p.visits != nullptr && tid == 0) {
       for (int kt = kt_begin; kt < kt_end; ++kt)
         p.visits[((long long)bh * nqt + qt) * nkt + kt] = 1;
@@ -298,6 +328,26 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
       full = full && (wq0 + 31 - k0 < p.window);
 #endif
 
+#if LF_BIAS
+      // class 2: the tile's bias values are requested before the S^T products.  Element i of block kb is
+      // key j = k0 + 32*kb + 8*(i/4) + 4*g + i%4 of row my_q: four consecutive keys per 8-byte load
+      // class 0 inside the range (a dead tile between live ones): staged like any tile, not computed
+      const int tile_class = (int)ccls[kt];
+      need = need && tile_class != 0;
+      const bool biased = need && tile_class == 2;
+      lf_u32x2 bias_v[LF_NKB][4];
+      if (biased) {
+        const lf_elem* brow = p.bias + (long long)b * p.bias_sb + (long long)h * p.bias_sh +
+                              (long long)min(my_q, p.Sq - 1) * p.bias_sq;
+#pragma unroll
+        for (int kb = 0; kb < LF_NKB; ++kb)
+#pragma unroll
+          for (int i4 = 0; i4 < 4; ++i4) {
+            const int j0 = k0 + 32 * kb + 8 * i4 + 4 * g;
+            bias_v[kb][i4] = *reinterpret_cast<const lf_u32x2*>(brow + min(j0, p.Sk - 4));
+          }
+      }
+#endif
       if (need) {
         // ---- S^T = K Q^T; the two accumulator chains alternate
         lf_f32x16 s[LF_NKB];
@@ -327,6 +377,26 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
 
         // ---- score modifications and mask; element i of block kb is kv index
         // j = k0 + 32*kb + 8*(i/4) + 4*g + i%4, query my_q.
+#if LF_BIAS
+        if (biased) {
+          // x = scale * s + bias: the scores stay in units of 1 / scale, so the bias is divided by it
+          const float inv_scale = 1.0f / p.scale;
+#pragma unroll
+          for (int kb = 0; kb < LF_NKB; ++kb)
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
+              const int j0 = k0 + 32 * kb + 8 * i4 + 4 * g;
+              const lf_elem4 bv = __builtin_bit_cast(lf_elem4, bias_v[kb][i4]);
+              // a tile that ends past Sk was read from Sk - 4: keys beyond Sk are masked below anyway
+              const int sh = j0 - min(j0, p.Sk - 4);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                const float bval = lf_bias_value(sh == 0 ? bv[e] : bv[min(e + sh, 3)]);
+                s[kb][4 * i4 + e] += bval * inv_scale;
+              }
+            }
+        }
+#endif
 #if LF_SOFTCAP
 #pragma unroll
         for (int kb = 0; kb < LF_NKB; ++kb)
@@ -435,7 +505,11 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
       // One v_permlane32_swap per register pair trades chunks with the lane that holds
       // the other half of the same row, so that each lane owns 8 consecutive d's and
       // writes them with one 16-byte store (32 contiguous bytes per row and instruction).
+#if LF_SAFE
+      const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;      // a row that saw no key gives zeros
+#else
       const float inv = 1.0f / l_tot;
+#endif
       lf_elem* orow = p.o + (long long)b * p.o_sb + (long long)h * p.o_sh +
                       (long long)min(my_q, p.Sq - 1) * p.o_ss;
 #pragma unroll

@@ -68,6 +68,7 @@ typedef float lf_f32x4 __attribute__((ext_vector_type(4)));
 typedef float lf_f32x16 __attribute__((ext_vector_type(16)));
 typedef unsigned int lf_u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int lf_u32x2 __attribute__((ext_vector_type(2)));
+typedef const int __attribute__((address_space(4))) lf_cint;   /* read-only table entries fetched with scalar loads */
 
 #if LF_TABLE_I64
 typedef long long lf_table_t;
@@ -132,7 +133,7 @@ struct LfAttnParams {
   lf_elem* o;
   const void* k_table;       // [B, pages_per_seq] page ids (lf_table_t) when paged
   const void* v_table;
-  float* part_acc;           // split-K scratch: [units, nsplit, rows, D]
+  float* part_acc;           // split-K scratch: [units, nsplit, rows, D]; prefill_swp with LF_BIAS: the bias tile classes (int32)
   float* part_ml;            // split-K scratch: [units, nsplit, rows, 2] (max, sum); lf_attn_prefill_swp: optional
                              // output [B, Hq, Sq], the rows' log-sum-exp in log2 units (null: not written)
   unsigned char* visits;     // optional [B*Hq*nqt, nkt] visited-tile record

@@ -105,8 +105,11 @@ class KernelSpec:
             o += [f"-DLF_V_TR={int(self.v_tr)}", f"-DLF_BIAS={self.bias}", f"-DLF_DENOM={int(self.denom)}"]
             if self.d2:
                 o += [f"-DLF_D2={self.d2}"]
-        elif self.family == "prefill_swp" and self.pack:
-            o += [f"-DLF_GQAPACK={int(self.pack)}"]
+        elif self.family == "prefill_swp":
+            if self.pack:
+                o += [f"-DLF_GQAPACK={int(self.pack)}"]
+            if self.bias:
+                o += ["-DLF_BIAS=1"]
         if self.safe:
             o += ["-DLF_SAFE=1"]
         return o + list(self.extra)
@@ -117,6 +120,9 @@ class KernelSpec:
         if self.family == "decode":
             return ("lf_common.hip.h", kernel)
         # the two prefill kernels: their own tuning macros come first (the shared blocks use LF_BN)
+        if self.family == "prefill_swp" and self.bias:
+            # one code object holds the attention kernel and the kernel that classifies the bias tiles for it
+            return ("lf_common.hip.h", "lf_prefill_blocks.hip.h", kernel, "lf_bias_classify.hip")
         return ("lf_common.hip.h", "lf_prefill_blocks.hip.h", kernel)
 
     def entry(self) -> str:
@@ -689,6 +695,14 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
 
     if family == "prefill" and not bias_bits and plan.denom_add == 0.0 and not d2:
         family = {"swp": "prefill_swp", "w32": "prefill"}.get(choice.get("prefill"), None) or prefill_variant(Sq, v_tr)
+    # a score bias with 8-byte aligned rows and nothing else special: the direct-to-LDS kernel with the bias
+    # classified tile by tile first (lf_bias_classify) -- what a mask given as a tensor needs
+    bias_tiles = (family == "prefill" and bias_bits == 1 and plan.denom_add == 0.0 and not d2 and softcap is None
+                  and lse is None and Sk >= 4 and (Sk + 63) // 64 <= 65535 * 4 and B * Hq <= 65535
+                  and os.environ.get("LOOPFUSE_BIAS_TILES", "1") == "1" and choice.get("prefill") != "w32"
+                  and prefill_variant(Sq, v_tr) == "prefill_swp")
+    if bias_tiles:
+        family = "prefill_swp"
     if family == "prefill_swp":
         # direct-to-LDS staging addresses memory with 32-bit byte offsets.  Dense operands:
         # offsets inside one (batch, kv head) span; the kernel also addresses up to three
@@ -723,12 +737,14 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         # group over the same query rows and share every K/V tile in LDS
         pack = 0
         if family == "prefill_swp" and group % 2 == 0 and not any(e.startswith("-DLF_NW=") for e in extra) and \
-                choice.get("pack", os.environ.get("LOOPFUSE_GQAPACK", "1") == "1"):
-            pack = 4 if group % 4 == 0 else 2
+                choice.get("pack", os.environ.get("LOOPFUSE_GQAPACK", "1") == "1") and not bias_bits:
+            pack = 4 if group % 4 == 0 else 2          # (the bias tile classes are per 128-row q tile of one head)
+        if family == "prefill_swp" and bias_bits and not bias_tiles:
+            family = "prefill"                          # swp was refused above (spans): the register-staged kernel
         spec = KernelSpec(family, _DTYPE_CODE[dtype], D, mask, plan.softcap is not None, paged,
                           page_size, table_i64, v_tr=v_tr if family == "prefill" else True, bias=bias_bits,
                           denom=plan.denom_add != 0.0, d2=d2, page_size_v=page_size_v, pack=pack, extra=extra,
-                          safe=plan.zero_blind_rows and bool(bias_bits & 1) and family == "prefill")
+                          safe=plan.zero_blind_rows and bool(bias_bits & 1))
         bm, bn = TILE_SHAPES[family]
         nw = 4
         for e in spec.extra:                    # tuning: -DLF_NW=8 doubles the q tile
@@ -762,8 +778,17 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
             if lse.dtype != torch.float32 or tuple(lse.shape) != (B, Hq, Sq) or not lse.is_contiguous() or lse.device != q.device:
                 raise UnsupportedPlan(f"lse must be a contiguous float32 [{B}, {Hq}, {Sq}] tensor on the device of Q")
             P.part_ml = lse.data_ptr()
+        names = [spec.entry()]
+        if family == "prefill_swp" and bias_bits:
+            # tile classes of the bias, once per distinct (batch, head) it holds: int32 [units][kv tiles]
+            nb_, nh_ = (B if P.bias_sb else 1), (Hq if P.bias_sh else 1)
+            table = torch.empty((nb_ * nh_ * nqt * nkt,), dtype=torch.int32, device=q.device)
+            keep += (table,)
+            P.part_acc = table.data_ptr()
+            get_kernel(spec, "lf_bias_classify").launch((nqt, nb_ * nh_, (nkt + 3) // 4), (256, 1, 1), P)
+            names.insert(0, "lf_bias_classify")
         get_kernel(spec, spec.entry()).launch((grid, 1, 1), (64 * nw, 1, 1), P)
-        _last_launch.set({"kernels": [spec.entry()], "grid": grid, "block": 64 * nw, "q_tile_rows": bm,
+        _last_launch.set({"kernels": names, "grid": grid, "block": 64 * nw, "q_tile_rows": bm,
                                  "heads_per_workgroup": spec.pack or 1})
         return (out, visits) if record_visits else out
 

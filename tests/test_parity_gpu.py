@@ -797,18 +797,24 @@ def _mask_bias(kind, Sq, Sk, dtype, seed=0):
 @pytest.mark.parametrize("S,D", [(593, 64), (1300, 128)])
 def test_mask_tensors_skip_dead_tiles_without_changing_the_result(dtype, kind, S, D, monkeypatch):
     """Mask tensors are biases of 0 / -inf; KV tiles that are -inf for a whole q tile are left
-    out of the loop.  The result must equal the oracle's and, bit for bit, the result of the
-    same kernel walking every tile."""
+    out of the loop.  Both kernels that serve them -- the direct-to-LDS kernel on classified tiles
+    (default) and the register-staged one with its list of live tiles -- must equal the oracle, and
+    the latter, bit for bit, the result of the same kernel walking every tile."""
     q, k, v = (rand((2, 3, S, D), dtype, s) for s in (1, 2, 3))
     bias = _mask_bias(kind, S, S, dtype)[None, None].expand(2, 1, S, S).contiguous()
     plan = lowering.AttnPlan(scale=D ** -0.5)
     on = [t.to(dev()) for t in (q, k, v, bias)]
-    got = lowering.attention(*on[:3], plan, score_bias=on[3])
     want = O.attention_reference(q, k, v, score_bias=bias.float())
+    got = lowering.attention(*on[:3], plan, score_bias=on[3])
+    assert lowering.attention.last_launch["kernels"] == ["lf_bias_classify", "lf_attn_prefill_swp"]
     assert (got.float().cpu() - want).abs().max().item() <= TOL[dtype]
+    monkeypatch.setenv("LOOPFUSE_BIAS_TILES", "0")
+    staged = lowering.attention(*on[:3], plan, score_bias=on[3])
+    assert lowering.attention.last_launch["kernels"] == ["lf_attn_prefill"]
+    assert (staged.float().cpu() - want).abs().max().item() <= TOL[dtype]
     monkeypatch.setenv("LOOPFUSE_KOPTS", "-DLF_LIVE_LIST=0")
     every_tile = lowering.attention(*on[:3], plan, score_bias=on[3])
-    assert torch.equal(got, every_tile)
+    assert torch.equal(staged, every_tile)
 
 
 def test_mask_tensor_with_rows_that_see_nothing():
@@ -950,9 +956,64 @@ def test_rows_that_see_nothing_give_zeros_when_asked(shape):
     assert torch.isnan(want[blind]).all()
     for zero in (False, True):
         got = lowering.attention(*on[:3], lowering.AttnPlan(scale=D ** -0.5, zero_blind_rows=zero), score_bias=on[3], **kw).float().cpu()
-        assert lowering.attention.last_launch["kernels"][0] == ("lf_attn_prefill" if shape == "prefill" else "lf_attn_decode")
+        assert lowering.attention.last_launch["kernels"] == (["lf_bias_classify", "lf_attn_prefill_swp"] if shape == "prefill"
+                                                            else ["lf_attn_decode"] + ["lf_attn_decode_combine"] * (shape == "decode_split"))
         assert (got[blind] == 0).all() if zero else torch.isnan(got[blind]).all()
         assert (got[~blind] - want[~blind]).abs().max().item() <= TOL[torch.bfloat16]
+
+
+@pytest.mark.parametrize("i", range(10))
+def test_bias_tile_classes(i, monkeypatch):
+    """The direct-to-LDS kernel with the bias classified tile by tile (lf_bias_classify): the tiles
+    it walks are each q tile's first .. last block that is not all -inf (brute force over the bias),
+    and its output equals the oracle's and the register-staged bias kernel's.  Leading, trailing and
+    interior dead blocks, zero blocks, blocks of real values, lengths that are no multiple of 4, 64 or
+    128, every broadcast form, rows that see nothing."""
+    g = torch.Generator().manual_seed(7000 + i)
+    ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    pick = lambda xs: xs[ri(0, len(xs) - 1)]
+    dt, D = pick([torch.bfloat16, torch.float16]), pick([64, 128])
+    B, H = ri(1, 2), pick([1, 3])
+    Sq, Sk = pick([17, 100, 128, 129, 300, 515]), pick([4, 63, 64, 65, 130, 333, 700, 1101])    # (up to 16 rows: decode kernels)
+    bshape = [pick([1, B]), pick([1, H]), pick([1, Sq, Sq]), Sk]
+    bias = torch.randn(bshape, generator=g) * 0.5 if pick([False, True]) else torch.zeros(bshape)
+    bias[..., :ri(0, Sk // 2)] = float("-inf")                       # leading dead keys
+    bias[..., Sk - ri(0, Sk // 3):] = float("-inf")                  # trailing dead keys
+    for _ in range(ri(0, 4)):                                        # holes, some wider than a tile
+        c0 = ri(0, Sk - 1)
+        r0 = ri(0, bshape[2] - 1)
+        bias[..., r0:r0 + ri(1, 300), c0:c0 + ri(1, 300)] = float("-inf")
+    if pick([False, True]) and Sk > 200:
+        bias[..., 100:164] = 0.0                                      # a whole zero tile
+    bias = bias.to(dt)
+    q, k, v = rand((B, H, Sq, D), dt, 7100 + i), rand((B, H, Sk, D), dt, 7200 + i), rand((B, H, Sk, D), dt, 7300 + i)
+    print("bias tile case", i, dict(dt=dt, D=D, B=B, H=H, Sq=Sq, Sk=Sk, bshape=bshape), flush=True)
+    on = [t.to(dev()) for t in (q, k, v, bias)]
+    plan = lowering.AttnPlan(scale=D ** -0.5)
+    got, visits = lowering.attention(*on[:3], plan, score_bias=on[3], record_visits=True)
+    assert lowering.attention.last_launch["kernels"] == ["lf_bias_classify", "lf_attn_prefill_swp"]
+    # walked tiles against brute force
+    nqt, nkt = (Sq + 127) // 128, (Sk + 63) // 64
+    full = bias.float().expand(B, H, Sq, Sk)
+    want_vis = torch.zeros(B * H * nqt, nkt, dtype=torch.uint8)
+    for bh in range(B * H):
+        for qt in range(nqt):
+            blk = full[bh // H, bh % H, 128 * qt:128 * qt + 128]
+            live = [kt for kt in range(nkt) if not torch.isinf(blk[:, 64 * kt:64 * kt + 64]).all()]
+            if live:
+                want_vis[bh * nqt + qt, live[0]:live[-1] + 1] = 1
+    assert torch.equal(visits.cpu(), want_vis)
+    # values against the oracle and the other kernel
+    want = O.attention_reference(q, k, v, score_bias=bias.float())
+    blind = torch.isnan(want).any(-1)
+    gotc = got.float().cpu()
+    assert torch.isnan(gotc[blind]).all()
+    assert (gotc[~blind] - want[~blind]).abs().max().item() <= TOL[dt] if (~blind).any() else True
+    monkeypatch.setenv("LOOPFUSE_BIAS_TILES", "0")
+    other = lowering.attention(*on[:3], plan, score_bias=on[3]).float().cpu()
+    assert lowering.attention.last_launch["kernels"] == ["lf_attn_prefill"]
+    assert torch.equal(torch.isnan(other), torch.isnan(gotc))
+    assert (other[~blind] - gotc[~blind]).abs().max().item() <= TOL[dt] if (~blind).any() else True
 
 
 def _mask_sweep_case(i):
