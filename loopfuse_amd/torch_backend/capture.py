@@ -1155,7 +1155,16 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
             consume(node.all_input_nodes)
             continue
         if node.op == "get_attr":
-            raise NoMatch("graph has constant tensors")
+            # a constant tensor of the graph (torch.tensor([...]) in the traced function): a value that is
+            # simply there, like the result of an ordinary op
+            val = node.meta.get("val")
+            if not isinstance(val, torch.Tensor):
+                try:
+                    val = getattr(gm, node.target)
+                except AttributeError:
+                    val = None
+            env[node] = fresh_ids(node, val) if isinstance(val, torch.Tensor) else None
+            continue
         if node.op != "call_function":
             raise NoMatch(f"unsupported node kind {node.op}")
         sym[node] = index_masks.step(node, sym)       # masks built from indices alone, as predicates

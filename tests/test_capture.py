@@ -527,6 +527,26 @@ def test_dynamic_width_split_into_heads(monkeypatch):
     torch.testing.assert_close(got, fn(x), rtol=2e-4, atol=2e-4)
 
 
+def test_constant_tensors_in_the_graph_do_not_stop_the_fusion(monkeypatch):
+    """``torch.tensor([...])`` inside the traced function becomes an attribute of the graph; the
+    attention beside it is fused all the same, and a constant can be one of its operands (a bias)."""
+    monkeypatch.setattr(capture.AttentionMatch, "run", _oracle_run)
+    outer = torch.linspace(-1.0, 1.0, 24)              # one value per key
+
+    def fn(q, k, v):
+        s = q @ k.transpose(-2, -1) * 0.125 + outer[None, None, None, :]
+        out = torch.softmax(torch.ops.loopfuse.causal_mask(s), -1) @ v
+        return out * torch.tensor([1.0, 2.0, 3.0])[None, :, None, None]
+
+    ins = [torch.randn(2, 3, 24, 64, generator=torch.Generator().manual_seed(s)) for s in range(3)]
+    torch._dynamo.reset()
+    before = dict(interface.stats)
+    with torch.no_grad():
+        got = torch.compile(fn, backend=loopfuse_amd.loopfuse_backend, dynamic=True)(*ins)
+    assert interface.stats["fused"] == before["fused"] + 1
+    torch.testing.assert_close(got, fn(*ins), rtol=2e-4, atol=2e-4)
+
+
 def test_an_error_inside_the_matcher_leaves_the_graph_running(monkeypatch):
     """The backend never fails a compilation because its own pattern matching broke: the graph runs
     as captured and the event is counted."""
