@@ -91,8 +91,8 @@ def trainable(match, dtype_of) -> str:
         return "explicit softmax / two-part scores"
     if match.bias is not None or match.out_bias is not None:
         return "additive biases"
-    if match.out_order or match.zero_blind_rows:
-        return "an attention taken over from F.scaled_dot_product_attention"
+    # (an attention taken over from F.scaled_dot_product_attention asks for zeros in rows that see no key:
+    # without a mask tensor -- refused above -- there is no such row, so the flag changes nothing here)
     if match.late_factors:
         return "factors applied after the mask"
     val = dtype_of(match.q.index)
@@ -124,6 +124,13 @@ def fused_call_train(match, *vals):
     out, _ = torch.ops.loopfuse_amd.attention_fwd(view(match.q), view(match.k), view(match.v),
                                                   _MASK_CODE[plan.mask], plan.window, plan.scale,
                                                   float(plan.softcap) if plan.softcap is not None else 0.0)
+    if match.out_order:
+        # the traced graph goes on with the output's memory order (torch's fused attention ops return
+        # [B, H, S, D] values stored as [B, S, H, D], and a view may rely on it): same values, that order
+        inv = [0] * 4
+        for pos, dim in enumerate(match.out_order):
+            inv[dim] = pos
+        out = out.permute(match.out_order).contiguous().permute(inv)
     if match.out_rank == 3:
         out = out.reshape(out.shape[0] * out.shape[1], out.shape[2], out.shape[3])
     return out

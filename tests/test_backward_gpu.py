@@ -256,11 +256,16 @@ def test_training_graph_with_an_unserved_attention_stays_unfused():
     assert leaves[0].grad is not None and torch.isfinite(leaves[0].grad.float()).all()
 
 
-def test_module_with_projections_trains_with_the_fused_attention():
+@pytest.mark.parametrize("spelling", ["mask_op", "sdpa_view", "sdpa_gqa"])
+def test_module_with_projections_trains_with_the_fused_attention(spelling):
     """A block with parameters (qkv projection, attention, output projection) compiled with
     static shapes and called outside ``torch.no_grad()``: the attention in the middle runs the
     fused forward and backward, the projections around it stay ATen ops, and the parameter
-    gradients match the uncompiled module."""
+    gradients match the uncompiled module.  The attention spelled with the reference's mask op, or
+    as ``F.scaled_dot_product_attention(is_causal=True)`` whose output is viewed without a copy
+    (the view relies on the op's [B, S, H, D] memory order), also with grouped kv heads."""
+    import torch.nn.functional as F
+
     from loopfuse_amd import loopfuse_backend
     from loopfuse_amd.torch_backend import interface, training
 
@@ -268,14 +273,20 @@ def test_module_with_projections_trains_with_the_fused_attention():
         def __init__(self):
             super().__init__()
             torch.manual_seed(0)
-            self.qkv = torch.nn.Linear(256, 3 * 256, bias=False)
+            self.kvh = 2 if spelling == "sdpa_gqa" else 4
+            self.qkv = torch.nn.Linear(256, 256 + 2 * 64 * self.kvh, bias=False)
             self.out = torch.nn.Linear(256, 256, bias=False)
 
         def forward(self, x):
             B, S, E = x.shape
-            q, k, v = (t.view(B, S, 4, 64).transpose(1, 2) for t in self.qkv(x).chunk(3, dim=-1))
-            a = torch.softmax(torch.ops.loopfuse.causal_mask(q @ k.transpose(-2, -1) * 0.125), dim=-1) @ v
-            return self.out(a.transpose(1, 2).reshape(B, S, E))
+            q, k, v = self.qkv(x).split([256, 64 * self.kvh, 64 * self.kvh], dim=-1)
+            q = q.view(B, S, 4, 64).transpose(1, 2)
+            k, v = (t.view(B, S, self.kvh, 64).transpose(1, 2) for t in (k, v))
+            if spelling == "mask_op":
+                a = torch.softmax(torch.ops.loopfuse.causal_mask(q @ k.transpose(-2, -1) * 0.125), dim=-1) @ v
+                return self.out(a.transpose(1, 2).reshape(B, S, E))
+            a = F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=spelling == "sdpa_gqa")
+            return self.out(a.transpose(1, 2).view(B, S, E))
 
     m = Block().to(DEV).to(torch.bfloat16)
     x = (torch.randn((2, 192, 256), generator=torch.Generator().manual_seed(3)) * 0.5).to(torch.bfloat16).to(DEV)
