@@ -377,10 +377,21 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
 
         // ---- score modifications and mask; element i of block kb is kv index
         // j = k0 + 32*kb + 8*(i/4) + 4*g + i%4, query my_q.
+#if LF_SOFTCAP
+#pragma unroll
+        for (int kb = 0; kb < LF_NKB; ++kb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) s[kb][i] = __builtin_amdgcn_rcpf(-1.0f - lf_exp2(s[kb][i] * sc_exp));   // -r
+#endif
 #if LF_BIAS
         if (biased) {
-          // x = scale * s + bias: the scores stay in units of 1 / scale, so the bias is divided by it
+          // x = scale * s + bias: the scores stay in units of 1 / scale, so the bias is divided by it; capped
+          // scores are held as -r with c * tanh = c - 2 c r: there the unit is 2 c
+#if LF_SOFTCAP
+          const float inv_scale = 0.5f / p.softcap;
+#else
           const float inv_scale = 1.0f / p.scale;
+#endif
 #pragma unroll
           for (int kb = 0; kb < LF_NKB; ++kb)
 #pragma unroll
@@ -396,12 +407,6 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
               }
             }
         }
-#endif
-#if LF_SOFTCAP
-#pragma unroll
-        for (int kb = 0; kb < LF_NKB; ++kb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) s[kb][i] = __builtin_amdgcn_rcpf(-1.0f - lf_exp2(s[kb][i] * sc_exp));   // -r
 #endif
         if (!full) {
 #pragma unroll

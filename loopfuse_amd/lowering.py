@@ -697,7 +697,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         family = {"swp": "prefill_swp", "w32": "prefill"}.get(choice.get("prefill"), None) or prefill_variant(Sq, v_tr)
     # a score bias with 8-byte aligned rows and nothing else special: the direct-to-LDS kernel with the bias
     # classified tile by tile first (lf_bias_classify) -- what a mask given as a tensor needs
-    bias_tiles = (family == "prefill" and bias_bits == 1 and plan.denom_add == 0.0 and not d2 and softcap is None
+    bias_tiles = (family == "prefill" and bias_bits == 1 and plan.denom_add == 0.0 and not d2
                   and lse is None and Sk >= 4 and (Sk + 63) // 64 <= 65535 * 4 and B * Hq <= 65535
                   and os.environ.get("LOOPFUSE_BIAS_TILES", "1") == "1" and choice.get("prefill") != "w32"
                   and prefill_variant(Sq, v_tr) == "prefill_swp")

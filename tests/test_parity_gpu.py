@@ -962,7 +962,7 @@ def test_rows_that_see_nothing_give_zeros_when_asked(shape):
         assert (got[~blind] - want[~blind]).abs().max().item() <= TOL[torch.bfloat16]
 
 
-@pytest.mark.parametrize("i", range(10))
+@pytest.mark.parametrize("i", range(14))
 def test_bias_tile_classes(i, monkeypatch):
     """The direct-to-LDS kernel with the bias classified tile by tile (lf_bias_classify): the tiles
     it walks are each q tile's first .. last block that is not all -inf (brute force over the bias),
@@ -987,9 +987,10 @@ def test_bias_tile_classes(i, monkeypatch):
         bias[..., 100:164] = 0.0                                      # a whole zero tile
     bias = bias.to(dt)
     q, k, v = rand((B, H, Sq, D), dt, 7100 + i), rand((B, H, Sk, D), dt, 7200 + i), rand((B, H, Sk, D), dt, 7300 + i)
-    print("bias tile case", i, dict(dt=dt, D=D, B=B, H=H, Sq=Sq, Sk=Sk, bshape=bshape), flush=True)
+    cap = pick([None, None, 5.0, 30.0])
+    print("bias tile case", i, dict(dt=dt, D=D, B=B, H=H, Sq=Sq, Sk=Sk, bshape=bshape, softcap=cap), flush=True)
     on = [t.to(dev()) for t in (q, k, v, bias)]
-    plan = lowering.AttnPlan(scale=D ** -0.5)
+    plan = lowering.AttnPlan(scale=D ** -0.5, softcap=cap)
     got, visits = lowering.attention(*on[:3], plan, score_bias=on[3], record_visits=True)
     assert lowering.attention.last_launch["kernels"] == ["lf_bias_classify", "lf_attn_prefill_swp"]
     # walked tiles against brute force
@@ -1004,7 +1005,7 @@ def test_bias_tile_classes(i, monkeypatch):
                 want_vis[bh * nqt + qt, live[0]:live[-1] + 1] = 1
     assert torch.equal(visits.cpu(), want_vis)
     # values against the oracle and the other kernel
-    want = O.attention_reference(q, k, v, score_bias=bias.float())
+    want = O.attention_reference(q, k, v, score_bias=bias.float(), softcap=cap)
     blind = torch.isnan(want).any(-1)
     gotc = got.float().cpu()
     assert torch.isnan(gotc[blind]).all()
