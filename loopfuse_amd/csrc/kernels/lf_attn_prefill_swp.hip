@@ -184,8 +184,47 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
   const float cexp = p.scale * LF_LOG2E;
 #endif
 
-  auto k_frag = [&](const lf_elem* kbuf, int f) { return lf_read_k_frag(kbuf, l32, g, f); };
-  auto v_frag = [&](const lf_elem* vbuf, int f) { return lf_read_v_frag_tr(vbuf, lane, g, f); };
+  // Fragment addresses inside a tile.  The XOR swizzles (lf_k_phys, lf_v_phys) depend on the lane and on
+  // which 16-dim step (K) / 32-dim block (V) a fragment belongs to, not on its row block: per lane there
+  // are LF_NKS + LF_NDB distinct byte offsets, kept in registers for the whole kernel (laundered through
+  // an empty asm so that they are not recomputed per read); every read is then one of them + the tile's
+  // slot + a constant that fits the instruction's offset field.
+  unsigned kb_off[LF_NKS], vb_off[LF_NDB];
+#pragma unroll
+  for (int ks = 0; ks < LF_NKS; ++ks) {
+    kb_off[ks] = (unsigned)(l32 * LF_D * 2 + 16 * lf_k_phys(l32, 2 * ks + g));
+    asm volatile("" : "+v"(kb_off[ks]));
+  }
+#pragma unroll
+  for (int db = 0; db < LF_NDB; ++db) {
+    const int j16 = lane & 15, dh = (lane >> 4) & 1, row0 = 4 * g + (j16 >> 2);
+    const int col = 32 * db + 16 * dh + 4 * (j16 & 3);
+    vb_off[db] = (unsigned)(row0 * LF_D * 2 + 16 * lf_v_phys(row0, col / 8) + 2 * (col % 8));
+    asm volatile("" : "+v"(vb_off[db]));
+  }
+  // K fragment f = (16-dim step ks, 32-row block kb): rows 32*kb + l32, as lf_read_k_frag
+  auto k_frag = [&](const lf_elem* kbuf, int f) {
+    const int ks = f / LF_NKB, kb = f % LF_NKB;
+    const char* base = reinterpret_cast<const char*>(kbuf) + kb_off[ks];
+    return *reinterpret_cast<const lf_u32x4*>(base + kb * 32 * LF_D * 2);
+  };
+  // V^T fragment f = (16-key step kk, 32-dim block db), two transposed 8-byte reads, as lf_read_v_frag_tr
+  auto v_frag = [&](const lf_elem* vbuf, int f) {
+    const int kk = f / LF_NDB, db = f % LF_NDB;
+    const char* base = reinterpret_cast<const char*>(vbuf) + vb_off[db];
+    lf_elem8 a;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const char* src = base + (16 * kk + 8 * half) * LF_D * 2;
+      lf_s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_s16x4*)(src));
+      lf_elem4 te = __builtin_bit_cast(lf_elem4, t);
+      a[4 * half + 0] = te[0];
+      a[4 * half + 1] = te[1];
+      a[4 * half + 2] = te[2];
+      a[4 * half + 3] = te[3];
+    }
+    return a;
+  };
 
   auto run_q_tile = [&](const int qt) {
     const int q0 = qt * LF_BM;
