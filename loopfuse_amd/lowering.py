@@ -648,7 +648,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
             t = t.expand(B, Hq, Sq, last)
         except RuntimeError:
             raise UnsupportedPlan(f"{what} does not broadcast to [{B}, {Hq}, {Sq}, {last}]")
-        if t.stride(3) != 1:
+        if t.stride(3) != 1 and t.shape[3] != 1:
             raise UnsupportedPlan(f"{what} needs last-dim stride 1")
         if t.data_ptr() % 8 or any(st % 4 for n, st in zip(t.shape[:3], t.stride()[:3]) if n > 1):
             bias_bits |= 4          # rows not 8-byte aligned: element loads

@@ -1133,7 +1133,9 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
                     return dataclasses.replace(st, mask="sliding", window=w if isinstance(w, torch.fx.Node) else int(a[1]))
                 if tgt is aten._softmax.default:
                     dim = a[1]
-                    if dim not in (-1, len(st.shape) - 1) or a[2]:
+                    # (a[2], half_to_float: the probabilities of fp16 scores come out in fp32 -- what
+                    # softmax(..., dtype=torch.float32) traces to; a cast like any other to the matcher)
+                    if dim not in (-1, len(st.shape) - 1):
                         raise _Skip("softmax not over the key dimension")
                     return dataclasses.replace(st, kind="probs")
                 raise _Skip(f"unsupported score modification: {tgt}")

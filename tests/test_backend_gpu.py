@@ -329,6 +329,22 @@ def test_attention_inside_a_transformer_block():
     assert (got - want).abs().max() <= 4 * TOL and (got - want).abs().mean() <= 4e-3
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_softmax_asked_for_in_float32(dtype):
+    """``F.softmax(scores, dim=-1, dtype=torch.float32).to(q.dtype)``, the decoder layers' spelling: for
+    fp16 scores on the GPU it traces to ``_softmax(..., half_to_float=True)``, for bf16 to a cast and a
+    plain softmax; both are the fused attention."""
+    import torch.nn.functional as F
+
+    def fn(q, k, v):
+        s = torch.ops.loopfuse.causal_mask(q @ k.transpose(-2, -1) * q.shape[-1] ** -0.5)
+        return F.softmax(s, dim=-1, dtype=torch.float32).to(q.dtype) @ v
+
+    Q, K, V = (rand((2, 4, 300, 64), dtype=dtype, seed=s) for s in (1, 2, 3))
+    got = run_fused(fn, (Q, K, V))
+    assert (got - O.attention_reference(Q, K, V, mask="causal")).abs().max() <= (TOL if dtype == torch.bfloat16 else 5e-3)
+
+
 @pytest.mark.parametrize("which", ["buffer_eq_zero", "arange_where", "key_padding_decode", "band"])
 def test_boolean_masks_written_by_hand(which):
     """``masked_fill`` / ``where`` with a boolean tensor and -inf (a causal buffer cut to the sequence as in
