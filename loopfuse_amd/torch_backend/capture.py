@@ -304,9 +304,22 @@ class AttentionMatch:
                 raise lowering.UnsupportedPlan("the mask is not the boolean tensor seen at trace time")
             t = torch.zeros(t.shape, dtype=dtype or torch.float32, device=t.device).masked_fill_(
                 t if bo.keep < 0 else ~t, float("-inf"))
-        strides = tuple(0 if d is None else t.stride(d) for d in bo.dims)
-        for size, d in zip(shape, bo.dims):
-            if d is not None and t.shape[d] != size:
+        # ("merged", k) / ("inner", k): batch and heads share source dim k ([B*H, ..], what baddbmm takes)
+        def stride_of(d):
+            if d is None:
+                return 0
+            if isinstance(d, tuple):
+                return t.stride(d[1]) * (shape[1] if d[0] == "merged" else 1)
+            return t.stride(d)
+
+        strides = tuple(stride_of(d) for d in bo.dims)
+        for i, (size, d) in enumerate(zip(shape, bo.dims)):
+            if isinstance(d, tuple):
+                want = shape[0] * shape[1] if bo.dims[0] is not None else shape[1]
+                ok = t.shape[d[1]] == want
+            else:
+                ok = d is None or t.shape[d] == size
+            if not ok:
                 raise lowering.UnsupportedPlan("bias does not have the shape seen at trace time")
         return torch.as_strided(t, tuple(shape), strides, t.storage_offset())
 
@@ -484,6 +497,18 @@ def _fit_bias(entry: tuple, logical: tuple):
             dims.append(None)
             continue
         cand = [k for k in range(len(shape)) if cstride[k] == step and shape[k] == n]
+        if not cand and d == 0:
+            # batch and heads merged into one source dim ([B*H, Sq, Sk], what baddbmm takes): the batch walks
+            # that dim in steps of the head count
+            merged = [k for k in range(len(shape)) if cstride[k] * logical[1] == step and shape[k] == n * logical[1]]
+            if merged:
+                dims.append(("merged", merged[0]))
+                recon = recon + (torch.arange(n) * step).view([n, 1, 1, 1])
+                continue
+        if not cand and d == 1:
+            inner = [k for k in range(len(shape)) if cstride[k] == step and shape[k] == n * logical[0]]
+            if inner and dims and dims[0] in (None, ("merged", inner[0])):
+                cand = [("inner", inner[0])]        # the heads' share of a merged [B*H] dim
         if not cand:
             raise NoMatch("bias is not a permuted / broadcast view of one tensor")
         dims.append(cand[0])
@@ -998,6 +1023,25 @@ def _match_attention(gm: torch.fx.GraphModule) -> list:
                     raise _Skip("QK^T shapes disagree")
                 shape = tuple(qi.t.shape[:-1]) + (ki.t.shape[-1],)
                 return Stage("scores", shape, qi, ki, mat=(shape[-2], shape[-1]))
+            if tgt is aten.baddbmm.default and len(a) == 3 and isinstance(a[1], Ids) and isinstance(a[2], Ids):
+                # beta * bias + alpha * (Q K^T): the score product of the decoders that spell it with baddbmm on a
+                # tensor of zeros (or on a bias); alpha is the scale
+                qi, ki = a[1], a[2]
+                beta, alpha = kw.get("beta", 1), kw.get("alpha", 1)
+                if qi.t.dim() != 3 or ki.t.dim() != 3 or qi.t.shape[0] != ki.t.shape[0] or qi.t.shape[-1] != ki.t.shape[-2]:
+                    raise _Skip("baddbmm operands are not a batched Q K^T")
+                if not is_number(beta) or not (is_number(alpha) or isinstance(alpha, Scalar)):
+                    raise _Skip("baddbmm factors not understood")
+                shape = tuple(qi.t.shape[:-1]) + (ki.t.shape[-1],)
+                st = Stage("scores", shape, qi, ki, mat=(shape[-2], shape[-1]))
+                raw = node.kwargs.get("alpha", 1)
+                if isinstance(alpha, Scalar) or isinstance(raw, torch.fx.Node) or float(alpha) != 1.0:
+                    st.factors = [alpha if isinstance(alpha, Scalar) else (raw if isinstance(raw, torch.fx.Node) else float(alpha))]
+                if sym.get(node.args[0]) is index_masks.ZERO or beta == 0:
+                    return st
+                if beta != 1:
+                    raise _Skip("baddbmm with a scaled bias")
+                return dataclasses.replace(st, bias=(first, shape))
             if tgt is aten.where.self and len(a) == 3 and is_bool(first):
                 # where(keep, scores, -inf) / where(masked, -inf, scores): a mask given as a boolean tensor
                 pos = 1 if isinstance(a[1], Stage) else (2 if isinstance(a[2], Stage) else 0)

@@ -80,6 +80,16 @@ class Pred:
         return Pred(a.clauses + b.clauses, False)
 
 
+class _Zero:
+    """A tensor of zeros (``torch.zeros(...)`` and views of it): as an additive term it is nothing."""
+
+    def __repr__(self):
+        return "ZERO"
+
+
+ZERO = _Zero()
+
+
 def _is_int(x) -> bool:
     return isinstance(x, int) and not isinstance(x, bool)
 
@@ -151,9 +161,16 @@ def step(node: torch.fx.Node, sym: dict):
     if t in (aten.ones.default, aten.ones_like.default) or \
             (t in (aten.full.default, aten.full_like.default) and len(args) > 1 and args[1] in (1, 1.0, True)):
         return Pred(())                                       # true everywhere
+    if t in (aten.zeros.default, aten.zeros_like.default) or \
+            (t in (aten.full.default, aten.full_like.default) and len(args) > 1 and args[1] in (0, 0.0) and args[1] is not False):
+        return ZERO
     if not args:
         return None
     x = val(args[0])
+    if x is ZERO:
+        views = _IDENTITY | {aten.unsqueeze.default, aten.slice.Tensor, aten.view.default, aten.reshape.default,
+                             aten._unsafe_view.default, aten.transpose.int, aten.permute.default, aten.squeeze.dim}
+        return ZERO if t in views else None
     if t in _CMP:
         a, b = x, val(args[1])
         if isinstance(a, Pred) and b in (0, 0.0, False) and _CMP[t] in ("eq", "ne"):

@@ -329,6 +329,31 @@ def test_attention_inside_a_transformer_block():
     assert (got - want).abs().max() <= 4 * TOL and (got - want).abs().mean() <= 4e-3
 
 
+@pytest.mark.parametrize("which", ["on_zeros", "alibi"])
+def test_scores_spelled_with_baddbmm(which):
+    """The decoders that merge batch and heads and take the scores from ``torch.baddbmm``: on a tensor of
+    zeros (GPT-NeoX) -- read as zeros from the graph, no bias at all -- or on an ALiBi term of shape
+    [B*H, 1, S] (BLOOM, Falcon), which becomes the kernels' score bias with batch and heads sharing a dim."""
+    B, H, S, D = 2, 8, 333, 64
+
+    def fn(q, k, v, alibi):
+        bs, nh, ql, hd = q.shape
+        qq, kk = q.reshape(bs * nh, ql, hd), k.reshape(bs * nh, ql, hd)
+        base = torch.zeros(bs * nh, ql, ql, dtype=q.dtype, device=q.device) if which == "on_zeros" else alibi
+        scores = torch.baddbmm(base, qq, kk.transpose(1, 2), beta=1.0, alpha=hd ** -0.5).view(bs, nh, ql, ql)
+        w = torch.softmax(torch.ops.loopfuse.causal_mask(scores), dim=-1, dtype=torch.float32).to(q.dtype)
+        return torch.matmul(w, v)
+
+    q, k, v = (rand((B, H, S, D), seed=s) for s in (1, 2, 3))
+    slopes = 2.0 ** -torch.arange(1, H + 1).float()
+    alibi = (slopes[:, None, None] * torch.arange(S).float()[None, None, :]).repeat(B, 1, 1).to(torch.bfloat16)   # [B*H, 1, S]
+    got = run_fused(fn, (q, k, v, alibi))
+    (m,) = interface.last_matches
+    assert m.mask == "causal" and (m.bias is not None) == (which == "alibi")
+    bias = None if which == "on_zeros" else alibi.float().view(B, H, 1, S).expand(B, H, S, S)
+    assert (got - O.attention_reference(q, k, v, mask="causal", score_bias=bias)).abs().max() <= TOL
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_softmax_asked_for_in_float32(dtype):
     """``F.softmax(scores, dim=-1, dtype=torch.float32).to(q.dtype)``, the decoder layers' spelling: for

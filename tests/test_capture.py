@@ -506,6 +506,37 @@ def test_finite_fill_values_are_not_taken_for_masks(fill):
     assert "match" not in box
 
 
+@pytest.mark.parametrize("which", ["on_zeros", "on_a_bias", "beta_zero", "scaled_bias"])
+def test_scores_spelled_with_baddbmm(which, monkeypatch):
+    """``torch.baddbmm(zeros, q, k^T, beta=1, alpha=scale)`` on operands merged to [B*H, S, D] (the
+    GPT-NeoX / Falcon spelling): the zeros are read as such from the graph and dropped, a real tensor
+    becomes the score bias, a bias scaled by beta stays unfused."""
+    monkeypatch.setattr(capture.AttentionMatch, "run", _oracle_run)
+    f32 = lambda *shape, seed=0: torch.randn(*shape, generator=torch.Generator().manual_seed(seed))
+    B, H, S, D = 2, 3, 24, 64
+
+    def fn(q, k, v, bias):
+        bs, nh, ql, hd = q.shape
+        qq, kk = q.view(bs * nh, ql, hd), k.view(bs * nh, k.size(-2), hd)
+        base = torch.zeros(bs * nh, ql, k.size(-2), dtype=q.dtype) if which in ("on_zeros", "beta_zero") else bias
+        beta = {"on_zeros": 1.0, "on_a_bias": 1.0, "beta_zero": 0.0, "scaled_bias": 0.5}[which]
+        scores = torch.baddbmm(base, qq, kk.transpose(1, 2), beta=beta, alpha=hd ** -0.5).view(bs, nh, ql, -1)
+        w = torch.softmax(torch.ops.loopfuse.causal_mask(scores), dim=-1)
+        return torch.matmul(w, v)
+
+    ins = (f32(B, H, S, D), f32(B, H, S, D, seed=1), f32(B, H, S, D, seed=2), f32(B * H, S, S, seed=3))
+    torch._dynamo.reset()
+    before = dict(interface.stats)
+    with torch.no_grad():
+        got = torch.compile(fn, backend=loopfuse_amd.loopfuse_backend, dynamic=True)(*ins)
+    fused = interface.stats["fused"] - before["fused"]
+    assert fused == (0 if which == "scaled_bias" else 1)
+    if fused:
+        (m,) = interface.last_matches
+        assert m.mask == "causal" and (m.bias is not None) == (which == "on_a_bias")
+    torch.testing.assert_close(got, fn(*ins), rtol=2e-4, atol=2e-4)
+
+
 def test_dynamic_width_split_into_heads(monkeypatch):
     """``qkv.chunk(3, -1)`` of a tensor whose width is a symbol: head dim (s + 2) // 12.  The stand-in
     sizes must divide as the traced ones do (an arbitrary stand-in once gave a head dim of 0)."""
