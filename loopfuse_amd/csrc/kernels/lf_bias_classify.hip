@@ -17,7 +17,7 @@
 // top-right corners are both masked, or both zero, are read in full.
 //
 // Grid (q tiles, batches' * heads', groups of 4 kv tiles), 256 threads: one wave per block,
-// 32 eight-byte loads per lane in batches of 8.  Needs bias rows that start on 8-byte
+// 32 eight-byte loads per lane, all in flight together.  Needs bias rows that start on 8-byte
 // boundaries (p.bias_sq and the strides multiples of 4) and Sk >= 4.
 //
 // The reference has no counterpart: its mask ops are index predicates
@@ -54,34 +54,31 @@ extern "C" __global__ __launch_bounds__(256) void lf_bias_classify(const LfAttnP
     const int j = k0 + 4 * (lane & 15), r4 = lane >> 4;
     const bool whole = j + 3 <= klast;
     const int jload = min(j, p.Sk - 4);        // the chunk that would run past Sk is read from Sk - 4 (and not used)
-    for (int it0 = 0; it0 < LF_BC_BM / 4; it0 += 8) {
-      lf_u32x2 w[8];
+    // all 32 loads of the lane go out before the first is looked at: one memory latency per block
+    lf_u32x2 w[LF_BC_BM / 4];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int q = min(q0 + 4 * (it0 + u) + r4, qlast);      // rows past the end re-read the last one
-        w[u] = *reinterpret_cast<const lf_u32x2*>(base + (long long)q * p.bias_sq + jload);
-      }
-      if (whole) {
+    for (int u = 0; u < LF_BC_BM / 4; ++u) {
+      const int q = min(q0 + 4 * u + r4, qlast);      // rows past the end re-read the last one
+      w[u] = *reinterpret_cast<const lf_u32x2*>(base + (long long)q * p.bias_sq + jload);
+    }
+    if (whole) {
 #pragma unroll
-        for (int u = 0; u < 8; ++u)
+      for (int u = 0; u < LF_BC_BM / 4; ++u)
 #pragma unroll
-          for (int e = 0; e < 2; ++e) {
-            dead = dead && lf_bias_masked2(w[u][e]);
-            zero = zero && is_zero(w[u][e] & 0xffffu) && is_zero(w[u][e] >> 16);
-          }
-      } else if (j <= klast) {
-        // the chunk that holds key Sk - 1: element by element
-        for (int u = 0; u < 8; ++u) {
-          const int q = min(q0 + 4 * (it0 + u) + r4, qlast);
-          for (int e = 0; j + e <= klast; ++e) {
-            const unsigned b16 = bits(q, j + e);
-            dead = dead && lf_bias_masked(b16);
-            zero = zero && is_zero(b16);
-          }
+        for (int e = 0; e < 2; ++e) {
+          dead = dead && lf_bias_masked2(w[u][e]);
+          zero = zero && is_zero(w[u][e] & 0xffffu) && is_zero(w[u][e] >> 16);
+        }
+    } else if (j <= klast) {
+      // the chunk that holds key Sk - 1: element by element
+      for (int u = 0; u < LF_BC_BM / 4; ++u) {
+        const int q = min(q0 + 4 * u + r4, qlast);
+        for (int e = 0; j + e <= klast; ++e) {
+          const unsigned b16 = bits(q, j + e);
+          dead = dead && lf_bias_masked(b16);
+          zero = zero && is_zero(b16);
         }
       }
-      // a block that is neither any more needs no further reads (wave-uniform exit)
-      if (__builtin_amdgcn_ballot_w64(dead) != ~0ull && __builtin_amdgcn_ballot_w64(zero) != ~0ull) break;
     }
   }
   const bool all_dead = __builtin_amdgcn_ballot_w64(dead) == ~0ull;
