@@ -6,7 +6,8 @@
 // (nothing of the block is visible: the attention kernel does not compute it, and does not
 // walk it at either end of a q tile's range) or all zero (the block needs no bias at all);
 // only the few blocks on the edge of the visible region mix values.  This kernel reads the
-// bias once per distinct (batch, head) it holds and writes, per q tile of 128 rows and kv
+// bias once per distinct (batch, head) it holds and writes, per q tile (128 rows; 64 or 32 when the
+// attention kernel packs query heads, which it does only for a bias shared by all heads) and kv
 // tile of 64 keys,
 //
 //   class[unit][kv tile] = 0 dead | 1 zero | 2 mixed                (int32)
@@ -23,8 +24,8 @@
 // The reference has no counterpart: its mask ops are index predicates
 // (loopfuse/torch_backend/ops.py:675-751) and a mask given as data is not skipped over.
 
-#define LF_BC_BM 128
-#define LF_BC_BN 64
+#define LF_BC_BM LF_BM      /* rows of the attention kernel's q tile: 128, or 64 / 32 with packed query heads */
+#define LF_BC_BN LF_BN
 
 extern "C" __global__ __launch_bounds__(256) void lf_bias_classify(const LfAttnParams p) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -50,11 +51,11 @@ extern "C" __global__ __launch_bounds__(256) void lf_bias_classify(const LfAttnP
   bool dead = lf_bias_masked(bl) && lf_bias_masked(tr);
   bool zero = is_zero(bl) && is_zero(tr);
   if (dead || zero) {
-    // lane = (row in a group of 4, 4-key chunk): 8-byte loads, 32 groups of 4 rows cover 128 rows
+    // lane = (row in a group of 4, 4-key chunk): 8-byte loads, LF_BC_BM / 4 groups of 4 rows cover the tile
     const int j = k0 + 4 * (lane & 15), r4 = lane >> 4;
     const bool whole = j + 3 <= klast;
     const int jload = min(j, p.Sk - 4);        // the chunk that would run past Sk is read from Sk - 4 (and not used)
-    // all 32 loads of the lane go out before the first is looked at: one memory latency per block
+    // all loads of the lane go out before the first is looked at: one memory latency per block
     lf_u32x2 w[LF_BC_BM / 4];
 #pragma unroll
     for (int u = 0; u < LF_BC_BM / 4; ++u) {

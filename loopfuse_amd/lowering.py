@@ -737,8 +737,10 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         # group over the same query rows and share every K/V tile in LDS
         pack = 0
         if family == "prefill_swp" and group % 2 == 0 and not any(e.startswith("-DLF_NW=") for e in extra) and \
-                choice.get("pack", os.environ.get("LOOPFUSE_GQAPACK", "1") == "1") and not bias_bits:
-            pack = 4 if group % 4 == 0 else 2          # (the bias tile classes are per 128-row q tile of one head)
+                choice.get("pack", os.environ.get("LOOPFUSE_GQAPACK", "1") == "1") and (not bias_bits or P.bias_sh == 0):
+            # (with a score bias only when all heads share it: the tile classes are then the same for the
+            # packed heads of a workgroup)
+            pack = 4 if group % 4 == 0 else 2
         if family == "prefill_swp" and bias_bits and not bias_tiles:
             family = "prefill"                          # swp was refused above (spans): the register-staged kernel
         spec = KernelSpec(family, _DTYPE_CODE[dtype], D, mask, plan.softcap is not None, paged,

@@ -1017,6 +1017,29 @@ def test_bias_tile_classes(i, monkeypatch):
     assert (other[~blind] - gotc[~blind]).abs().max().item() <= TOL[dt] if (~blind).any() else True
 
 
+@pytest.mark.parametrize("per_head", [False, True])
+@pytest.mark.parametrize("group", [2, 4])
+def test_bias_tiles_with_grouped_query_heads(group, per_head):
+    """A mask shared by all heads keeps the packing of query heads (q tiles of 32 or 64 rows, classes at
+    that granularity); a bias that differs per head runs one head per workgroup.  Both equal the oracle."""
+    B, Hkv, Sq, Sk, D = 2, 2, 300, 333, 128
+    Hq = Hkv * group
+    q, k, v = rand((B, Hq, Sq, D), torch.bfloat16, 1), rand((B, Hkv, Sk, D), torch.bfloat16, 2), rand((B, Hkv, Sk, D), torch.bfloat16, 3)
+    i, j = torch.arange(Sq)[:, None], torch.arange(Sk)[None, :]
+    keep = (j <= i + 33) & (i + 33 - j < 100)
+    bias = torch.zeros(B, Hq if per_head else 1, Sq, Sk).masked_fill(~keep, float("-inf"))
+    bias[1, :, :, 150:170] = float("-inf")                       # a hole in the second sequence
+    if per_head:
+        bias = bias + (torch.arange(Hq).float()[None, :, None, None] * 0.01 * (j - i)).masked_fill(~keep, 0.0)
+    bias = bias.to(torch.bfloat16)
+    on = [t.to(dev()) for t in (q, k, v, bias)]
+    got = lowering.attention(*on[:3], lowering.AttnPlan(scale=D ** -0.5), score_bias=on[3]).float().cpu()
+    assert lowering.attention.last_launch["kernels"] == ["lf_bias_classify", "lf_attn_prefill_swp"]
+    assert lowering.attention.last_launch["heads_per_workgroup"] == (1 if per_head else group)
+    want = O.attention_reference(q, k, v, score_bias=bias.float())
+    assert (got - want).abs().max().item() <= TOL[torch.bfloat16]
+
+
 def _mask_sweep_case(i):
     """Case i of a seeded sweep over score biases that hold -inf regions (mask tensors)."""
     g = torch.Generator().manual_seed(5000 + i)
