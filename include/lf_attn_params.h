@@ -32,7 +32,7 @@ typedef struct LfAttnParamsHost {
   float* part_acc;      /* decode split-K scratch: [units, nsplit, rows, D] floats; lf_attn_prefill_swp -DLF_BIAS=1 and
                            lf_bias_classify: int32 [units', kv tiles of 64] tile classes of the score bias (written by
                            lf_bias_classify, launched first with the same block; units' = distinct (batch, head) of the
-                           bias x q tiles of 128 rows) */
+                           bias x q tiles of the attention kernel) */
   float* part_ml;       /* decode split-K scratch: [units, nsplit, rows, 2] floats; lf_attn_prefill_swp: optional
                            output [B, Hq, Sq] floats, the rows' log-sum-exp in log2 units (NULL: not written) */
   unsigned char* visits;/* optional [B*Hq*q_tiles, kv_tiles] visited-tile record, else NULL */
