@@ -448,12 +448,26 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
         }
 #endif
         if (!full) {
+          // key j = k0 + 4*g + c with the compile-time c = 32*kb + 8*(i/4) + i%4: the bound j < Sk and the
+          // causal j <= my_q fold into one per-lane limit, so an element costs one compare against an
+          // inline constant (the window, i - j < w, a second one)
+          int hi = p.Sk - 1 - k0 - 4 * g;
+#if LF_MASK >= 1
+          hi = min(hi, my_q - k0 - 4 * g);
+#endif
+#if LF_MASK == 2
+          const int lo = my_q - k0 - 4 * g - p.window;       // c > lo
+#endif
 #pragma unroll
           for (int kb = 0; kb < LF_NKB; ++kb)
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-              const int j = k0 + 32 * kb + 8 * (i / 4) + 4 * g + (i % 4);
-              const bool ok = lf_mask_keep(my_q, j, p.Sk, p.window);
+              const int c = 32 * kb + 8 * (i / 4) + (i % 4);
+#if LF_MASK == 2
+              const bool ok = c <= hi && c > lo;
+#else
+              const bool ok = c <= hi;
+#endif
               s[kb][i] = ok ? s[kb][i] : LF_NEG_INF;
             }
         }
