@@ -483,12 +483,16 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
         if (__builtin_amdgcn_ballot_w64(mxc > mc_ref + (float)LF_LAZY_LOG2) != 0ull) {
           const float mc_new = fmaxf(mc_ref, mxc);
           const float r = (mc_new == LF_NEG_INF) ? 1.0f : lf_exp2(mc_ref - mc_new);
+          // no row of the wave has seen a key yet (the first tile of a q tile): O and l are still zero
+          const bool fresh = __builtin_amdgcn_ballot_w64(mc_ref != LF_NEG_INF) == 0ull;
           mc_ref = mc_new;
-          l_run *= r;
+          if (!fresh) {
+            l_run *= r;
 #pragma unroll
-          for (int db = 0; db < LF_NDB; ++db)
+            for (int db = 0; db < LF_NDB; ++db)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) o[db][i] *= r;
+              for (int i = 0; i < 16; ++i) o[db][i] *= r;
+          }
         }
         const float mc_sub = (mc_ref == LF_NEG_INF) ? 0.0f : mc_ref;
         float rs = 0.0f;
