@@ -29,7 +29,7 @@ from __future__ import annotations
 import logging
 import os
 from functools import partial
-from typing import Any, Callable
+from typing import Callable
 
 import torch
 from torch._functorch.aot_autograd import aot_module_simplified, make_boxed_func

@@ -2,7 +2,6 @@
 of every node the tracker claims to understand is compared, element by element, with the tensor
 the node really produces; and the front end turns such masks into the kernels' causal / window flag
 exactly when the visible set is ``0 <= i - j [<= w - 1]``."""
-import itertools
 
 import pytest
 import torch
