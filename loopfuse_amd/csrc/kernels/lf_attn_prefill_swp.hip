@@ -478,7 +478,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
         for (int kb = 0; kb < LF_NKB; ++kb)
 #pragma unroll
           for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kb][i]);
-        mx = fmaxf(mx, lf_swap32(mx));
+        mx = lf_max_halves(mx);
         const float mxc = mx * cexp;
         if (__builtin_amdgcn_ballot_w64(mxc > mc_ref + (float)LF_LAZY_LOG2) != 0ull) {
           const float mc_new = fmaxf(mc_ref, mxc);

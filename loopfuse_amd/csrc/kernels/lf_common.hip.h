@@ -202,6 +202,15 @@ __device__ __forceinline__ float lf_swap32(float x) {
   return __builtin_bit_cast(float, other);
 }
 
+// max(x of this lane, x of lane ^ 32) in every lane.  After v_permlane32_swap of two copies of x one register
+// holds the lower half's values in both halves and the other the upper half's: their maximum is the answer
+// without a select.  Inline asm: written with the builtin, the compiler keeps the swap and drops the maximum.
+__device__ __forceinline__ float lf_max_halves(float x) {
+  float a = x, b = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  return fmaxf(a, b);
+}
+
 __device__ __forceinline__ float lf_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // tanh(x) = 1 - 2 / (2^(2 x log2 e) + 1); exact limits at +-inf.
