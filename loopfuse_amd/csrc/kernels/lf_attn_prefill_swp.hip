@@ -321,6 +321,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
 #pragma unroll
       for (int i = 0; i < 16; ++i) o[db][i] = 0.0f;
     float mc_ref = LF_NEG_INF;   // exponent offset of this query, log2 units (a lagging running max)
+    float mc_sub = 0.0f;         // what the exponentials subtract: mc_ref, or 0 while it is still -inf
     float l_run = 0.0f;          // this lane's share of the running sum
 
     LF_BARRIER_VM0();
@@ -486,6 +487,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
           // no row of the wave has seen a key yet (the first tile of a q tile): O and l are still zero
           const bool fresh = __builtin_amdgcn_ballot_w64(mc_ref != LF_NEG_INF) == 0ull;
           mc_ref = mc_new;
+          mc_sub = (mc_new == LF_NEG_INF) ? 0.0f : mc_new;
           if (!fresh) {
             l_run *= r;
 #pragma unroll
@@ -494,7 +496,6 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
               for (int i = 0; i < 16; ++i) o[db][i] *= r;
           }
         }
-        const float mc_sub = (mc_ref == LF_NEG_INF) ? 0.0f : mc_ref;
         float rs = 0.0f;
         lf_elem8 pf[LF_NKK];
         // probabilities of the tile's key block kb, elements [i0, i1)
