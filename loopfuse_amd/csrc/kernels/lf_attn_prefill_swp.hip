@@ -58,6 +58,12 @@
 #define LF_NPASS (LF_BN * LF_CPR / LF_NT)
 #define LF_NFK (LF_NKS * LF_NKB)      /* MFMAs (= K fragments) of S^T per tile */
 #define LF_NFV (LF_NKK * LF_NDB)      /* MFMAs (= V fragments) of O^T per tile */
+#if LF_KPF > LF_NFK || LF_KPF > LF_NFV || LF_VPF > LF_NFK || LF_VPF > LF_NFV
+#error "the fragment read-ahead (LF_KPF, LF_VPF) cannot exceed the fragments of a tile"
+#endif
+#ifndef LF_WPE
+#define LF_WPE (8 / LF_NW)     /* waves per SIMD the register budget is sized for (= workgroups per CU for 4 waves) */
+#endif
 
 // workgroup barrier that waits for this wave's direct-to-LDS loads but leaves LDS
 // reads in flight (the compiler's own barrier would wait for those too)
@@ -68,16 +74,27 @@
 #endif
 #define LF_BARRIER_VM0() asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory")
 
+#define LF_CAPPOLY (LF_SOFTCAP && !LF_BIAS)   /* polynomial fast path of the softcap (below) */
+#ifndef LF_CAP_TERMS
+#define LF_CAP_TERMS 1   /* terms of the polynomial that is fused into the exponent (1 or 2) */
+#endif
+/* minimax fits of tanh(x)/x - 1 in x^2: one term on |x| <= 0.15 (absolute error of tanh 1.4e-6), two terms on
+   |x| <= 0.4 (2.1e-6) */
+#define LF_CAP1_X0 0.15f
+#define LF_CAP1_B1 (-0.3307545f)
+#define LF_CAP2_X0 0.4f
+#define LF_CAP2_B1 (-0.33269722f)
+#define LF_CAP2_B2 0.12145087f
 #ifndef LF_QGROUP
 #define LF_QGROUP 8      /* (batch, head) pairs per group of slots */
 #endif
 #ifndef LF_SPLIT_EXP
-#define LF_SPLIT_EXP (!LF_SOFTCAP)     /* second key block's exponentials between the MFMAs of the first (config 2: -0.7 %; no gain with a softcap) */
+#define LF_SPLIT_EXP (!LF_SOFTCAP || !LF_BIAS)     /* second key block's exponentials between the MFMAs of the first (config 2: -0.7 %; no gain with a softcap) */
 #endif
 
-extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_swp(const LfAttnParams p) {
-  __shared__ __attribute__((aligned(16))) lf_elem lds_k[LF_KSLOTS][LF_BN * LF_D];
-  __shared__ __attribute__((aligned(16))) lf_elem lds_v[LF_VSLOTS][LF_BN * LF_D];
+extern "C" __global__ void __launch_bounds__(LF_NT, LF_WPE) lf_attn_prefill_swp(const LfAttnParams p) {
+  // one array, K slots first
+  __shared__ __attribute__((aligned(16))) lf_elem lds_all[(LF_KSLOTS + LF_VSLOTS) * LF_BN * LF_D];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -146,7 +163,10 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
   // per-lane part of the offset: dense = row inside the pass, paged = row inside the wave's load
   const unsigned k_doff = (unsigned)(kPagedK ? srow % (64 / LF_CPR) : srow) * k_rowb + 16u * (unsigned)lf_k_phys(srow, sch);
   const unsigned v_doff = (unsigned)(kPagedV ? srow % (64 / LF_CPR) : srow) * v_rowb + 16u * (unsigned)lf_v_phys(srow, sch);
-  auto dma = [&](const lf_u32x4& rs, unsigned voff, const lf_elem* lds_row0) { lf_dma_to_lds(rs, voff, lds_row0); };
+  // LDS byte addresses of the slots' rows as integers (scalar arithmetic on the constant base)
+  const unsigned lds0 = lf_lds_addr(lds_all);
+  auto k_row_addr = [&](int sl, int row) { return lds0 + (unsigned)((sl * LF_BN + row) * LF_D * 2); };
+  auto v_row_addr = [&](int sl, int row) { return lds0 + (unsigned)(((LF_KSLOTS + sl) * LF_BN + row) * LF_D * 2); };
   // pg: page_off() of the pass (paged operands only; fetched a tile ahead by the caller)
   // `rs`: k_rsq / v_rsq, or the same with an empty range for a tile past the last one (nothing is
   // fetched then; the slot it would fill is free)
@@ -159,7 +179,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
     } else {
       off = k_doff + (unsigned)(kt * LF_BN + kRowsPerPass * ps) * k_rowb;
     }
-    dma(rs, off, &lds_k[sl][(kRowsPerPass * ps + kRowsPerWave * wave_u) * LF_D]);
+    lf_dma_to_lds_at(rs, off, k_row_addr(sl, kRowsPerPass * ps + kRowsPerWave * wave_u));
   };
   auto dma_v_pass = [&](const lf_u32x4& rs, int kt, int sl, int ps, unsigned pg) {
     unsigned off;
@@ -170,11 +190,36 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
     } else {
       off = v_doff + (unsigned)(kt * LF_BN + kRowsPerPass * ps) * v_rowb;
     }
-    dma(rs, off, &lds_v[sl][(kRowsPerPass * ps + kRowsPerWave * wave_u) * LF_D]);
+    lf_dma_to_lds_at(rs, off, v_row_addr(sl, kRowsPerPass * ps + kRowsPerWave * wave_u));
   };
 
-#if LF_SOFTCAP
-  // capped score c*tanh(x) = c - 2c*r with r = 1 / (e^(2x) + 1), x = s*scale/c.  The
+#if LF_CAPPOLY
+  // Capped score c*tanh(x), x = s*scale/c, in log2 units.  Three forms, chosen per wave and tile (uniformly):
+  //  * every score has |x| <= X0 and the tile needs no mask: the cap is an odd polynomial on full-rate FMAs,
+  //    evaluated where the exponent is formed, 2^(s*(A0 + A1 s^2 [+ A2 s^4]) - m) -- one transcendental per score
+  //    as without a cap (tanh is increasing, so the row maximum is the polynomial of the largest raw score);
+  //  * |x| <= 0.4 but beyond X0, or a mask in the way: the two-term polynomial in place, then the plain exponent;
+  //  * otherwise c*log2e*(1 - 2r), r = 1 / (e^(2x) + 1), in place (two transcendentals more per score).
+  // (derived constants are moved back into scalar registers: uniform float arithmetic is done by the vector
+  // ALU, and its results would otherwise occupy a vector register each for the whole kernel)
+  auto uni = [](float x) { return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, x))); };
+  const float cap_a = p.scale / p.softcap;
+  const float cap_a2 = cap_a * cap_a;
+  const float cap_l2 = uni(p.softcap * LF_LOG2E);
+  const float sc_exp = uni(cap_a * (2.0f * LF_LOG2E));            // 2^(s * sc_exp) = e^(2x)
+  const float capA0 = uni(p.scale * LF_LOG2E);                    // = c*log2e * a
+#if LF_CAP_TERMS >= 2
+  const float capA1 = uni(capA0 * cap_a2 * LF_CAP2_B1), capA2 = uni(capA0 * cap_a2 * cap_a2 * LF_CAP2_B2);
+  const float cap_smax = uni(LF_CAP2_X0 / fabsf(cap_a));          // |s| up to which the fused polynomial holds
+#else
+  const float capA1 = uni(capA0 * cap_a2 * LF_CAP1_B1);
+  const float cap_smax = uni(LF_CAP1_X0 / fabsf(cap_a));
+#endif
+  const float capP1 = uni(capA0 * cap_a2 * LF_CAP2_B1), capP2 = uni(capA0 * cap_a2 * cap_a2 * LF_CAP2_B2);
+  const float cap_smax2 = uni(LF_CAP2_X0 / fabsf(cap_a));         // ... the in-place polynomial holds
+  const float cexp = 1.0f;                                       // scores transformed in place are in log2 units
+#elif LF_SOFTCAP
+  // with a score bias: capped score c*tanh(x) = c - 2c*r with r = 1 / (e^(2x) + 1), x = s*scale/c.  The
   // constant c is the same for every key of a row, so the softmax does not see it: the
   // kernel works on -r and folds the factor 2c into the exponent multiplier, which saves
   // the three VALU operations per score that would turn r into the capped score
@@ -185,38 +230,38 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
 #endif
 
   // Fragment addresses inside a tile.  The XOR swizzles (lf_k_phys, lf_v_phys) depend on the lane and on
-  // which 16-dim step (K) / 32-dim block (V) a fragment belongs to, not on its row block: per lane there
-  // are LF_NKS + LF_NDB distinct byte offsets, kept in registers for the whole kernel (laundered through
-  // an empty asm so that they are not recomputed per read); every read is then one of them + the tile's
-  // slot + a constant that fits the instruction's offset field.
-  unsigned kb_off[LF_NKS], vb_off[LF_NDB];
-#pragma unroll
-  for (int ks = 0; ks < LF_NKS; ++ks) {
-    kb_off[ks] = (unsigned)(l32 * LF_D * 2 + 16 * lf_k_phys(l32, 2 * ks + g));
-    asm volatile("" : "+v"(kb_off[ks]));
-  }
-#pragma unroll
-  for (int db = 0; db < LF_NDB; ++db) {
+  // which 16-dim step (K) / 32-dim block (V) a fragment belongs to, not on its row block, and the step /
+  // block enters as an XOR of address bits below the row stride: offset(ks) = offset(0) ^ 32*ks for K,
+  // offset(db) = offset(0) ^ 64*db for V.  A lane keeps the two offsets of step / block 0 (laundered through
+  // an empty asm so that they are not recomputed per read); per tile one add forms base + slot (slots are
+  // multiples of 4 KB), and a read is that ^ a constant, plus a constant in the instruction's offset field.
+  unsigned kb_off0 = (unsigned)(l32 * LF_D * 2 + 16 * lf_k_phys(l32, g));
+  asm volatile("" : "+v"(kb_off0));
+  unsigned vb_off0;
+  {
     const int j16 = lane & 15, dh = (lane >> 4) & 1, row0 = 4 * g + (j16 >> 2);
-    const int col = 32 * db + 16 * dh + 4 * (j16 & 3);
-    vb_off[db] = (unsigned)(row0 * LF_D * 2 + 16 * lf_v_phys(row0, col / 8) + 2 * (col % 8));
-    asm volatile("" : "+v"(vb_off[db]));
+    const int col = 16 * dh + 4 * (j16 & 3);
+    vb_off0 = (unsigned)(row0 * LF_D * 2 + 16 * lf_v_phys(row0, col / 8) + 2 * (col % 8));
+    asm volatile("" : "+v"(vb_off0));
   }
-  // K fragment f = (16-dim step ks, 32-row block kb): rows 32*kb + l32, as lf_read_k_frag
-  auto k_frag = [&](const lf_elem* kbuf, int f) {
+  static_assert((LF_BN * LF_D * 2) % 4096 == 0, "slot strides keep the swizzled address bits clear");
+  typedef __attribute__((address_space(3))) const lf_u32x4* lf_lds_u32x4_ptr;
+  typedef __attribute__((address_space(3))) lf_s16x4* lf_lds_s16x4_ptr;
+  // K fragment f = (16-dim step ks, 32-row block kb): rows 32*kb + l32, as lf_read_k_frag; `ka` = LDS address
+  // of the tile + kb_off0
+  auto k_frag = [&](unsigned ka, int f) {
     const int ks = f / LF_NKB, kb = f % LF_NKB;
-    const char* base = reinterpret_cast<const char*>(kbuf) + kb_off[ks];
-    return *reinterpret_cast<const lf_u32x4*>(base + kb * 32 * LF_D * 2);
+    return *(lf_lds_u32x4_ptr)(size_t)((ka ^ (unsigned)(32 * ks)) + (unsigned)(kb * 32 * LF_D * 2));
   };
-  // V^T fragment f = (16-key step kk, 32-dim block db), two transposed 8-byte reads, as lf_read_v_frag_tr
-  auto v_frag = [&](const lf_elem* vbuf, int f) {
+  // V^T fragment f = (16-key step kk, 32-dim block db), two transposed 8-byte reads, as lf_read_v_frag_tr;
+  // `va` = LDS address of the tile + vb_off0
+  auto v_frag = [&](unsigned va, int f) {
     const int kk = f / LF_NDB, db = f % LF_NDB;
-    const char* base = reinterpret_cast<const char*>(vbuf) + vb_off[db];
     lf_elem8 a;
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
-      const char* src = base + (16 * kk + 8 * half) * LF_D * 2;
-      lf_s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lf_s16x4*)(src));
+      const unsigned src = (va ^ (unsigned)(64 * db)) + (unsigned)((16 * kk + 8 * half) * LF_D * 2);
+      lf_s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lf_lds_s16x4_ptr)(size_t)src);
       lf_elem4 te = __builtin_bit_cast(lf_elem4, t);
       a[4 * half + 0] = te[0];
       a[4 * half + 1] = te[1];
@@ -327,16 +372,16 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
     LF_BARRIER_VM0();
     lf_u32x4 kpre[LF_KPF];
 #pragma unroll
-    for (int f = 0; f < LF_KPF; ++f) kpre[f] = k_frag(lds_k[0], f);
+    for (int f = 0; f < LF_KPF; ++f) kpre[f] = k_frag(k_row_addr(0, 0) + kb_off0, f);
 
     int ks_cur = 0;   // K slot of tile kt
     for (int kt = kt_begin; kt < kt_end; ++kt) {
       const int rel = kt - kt_begin;
       const int ks_nxt = (ks_cur == LF_KSLOTS - 1) ? 0 : ks_cur + 1;   // slot of K(kt+1)
       const int ks_ld = (ks_nxt == LF_KSLOTS - 1) ? 0 : ks_nxt + 1;    // slot K(kt+2) is loaded into
-      const lf_elem* kbuf = lds_k[ks_cur];
-      const lf_elem* knext = lds_k[ks_nxt];
-      const lf_elem* vbuf = lds_v[rel & 1];
+      const unsigned kbuf = k_row_addr(ks_cur, 0) + kb_off0;       // lane's fragment base in K(kt), K(kt+1), V(kt)
+      const unsigned knext = k_row_addr(ks_nxt, 0) + kb_off0;
+      const unsigned vbuf = v_row_addr(rel & 1, 0) + vb_off0;
       const int vs_ld = (rel + 1) & 1;                                 // slot V(kt+1) is loaded into
       // direct load number d of this tile: K(kt+2) passes, then V(kt+1) passes.  Tiles past the
       // last one are asked for with an empty range instead of a test per load: a branch between the
@@ -417,7 +462,51 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
 
         // ---- score modifications and mask; element i of block kb is kv index
         // j = k0 + 32*kb + 8*(i/4) + 4*g + i%4, query my_q.
-#if LF_SOFTCAP
+#if LF_CAPPOLY
+        // largest |raw score| of the wave's tile: decides between the polynomial and the exact form
+        float amax = 0.0f;
+#pragma unroll
+        for (int kb = 0; kb < LF_NKB; ++kb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) amax = fmaxf(amax, fabsf(s[kb][i]));
+        const bool cap_fused = __builtin_amdgcn_ballot_w64(!(amax <= cap_smax)) == 0ull && full;
+        // coefficients of the exponent's polynomial for this tile: the cap's, or the identity for a tile that is
+        // transformed in place (tiny positive instead of 0: a masked score, -inf, then stays -inf instead of NaN)
+        float kA0 = capA0, kA1 = capA1;
+#if LF_CAP_TERMS >= 2
+        float kA2 = capA2;
+#endif
+        if (!cap_fused) {
+          if (__builtin_amdgcn_ballot_w64(!(amax <= cap_smax2)) == 0ull) {
+#pragma unroll
+            for (int kb = 0; kb < LF_NKB; ++kb)
+#pragma unroll
+              for (int i = 0; i < 16; ++i) {
+                const float u = s[kb][i] * s[kb][i];
+                s[kb][i] *= __builtin_fmaf(u, __builtin_fmaf(u, capP2, capP1), capA0);
+              }
+          } else {
+#pragma unroll
+            for (int kb = 0; kb < LF_NKB; ++kb)
+#pragma unroll
+              for (int i = 0; i < 16; ++i)
+                s[kb][i] = __builtin_fmaf(__builtin_amdgcn_rcpf(-1.0f - lf_exp2(s[kb][i] * sc_exp)), 2.0f * cap_l2, cap_l2);
+          }
+          kA0 = 1.0f;
+          kA1 = 1e-30f;
+#if LF_CAP_TERMS >= 2
+          kA2 = 1e-30f;
+#endif
+        }
+        // c*log2e*tanh of a raw score (or the identity), as a factor: score * cap_t(score^2)
+        auto cap_t = [&](float u) {
+#if LF_CAP_TERMS >= 2
+          return __builtin_fmaf(u, __builtin_fmaf(u, kA2, kA1), kA0);
+#else
+          return __builtin_fmaf(u, kA1, kA0);
+#endif
+        };
+#elif LF_SOFTCAP
 #pragma unroll
         for (int kb = 0; kb < LF_NKB; ++kb)
 #pragma unroll
@@ -480,7 +569,11 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
 #pragma unroll
           for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[kb][i]);
         mx = lf_max_halves(mx);
+#if LF_CAPPOLY
+        const float mxc = mx * cap_t(mx * mx);
+#else
         const float mxc = mx * cexp;
+#endif
         if (__builtin_amdgcn_ballot_w64(mxc > mc_ref + (float)LF_LAZY_LOG2) != 0ull) {
           const float mc_new = fmaxf(mc_ref, mxc);
           const float r = (mc_new == LF_NEG_INF) ? 1.0f : lf_exp2(mc_ref - mc_new);
@@ -498,22 +591,27 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
         }
         float rs = 0.0f;
         lf_elem8 pf[LF_NKK];
-        // probabilities of the tile's key block kb, elements [i0, i1)
-        auto exp_block = [&](int kb, int i0, int i1) {
+        // probabilities number [e0, e1) of the tile in the order the second product consumes them:
+        // e = 16 * (key block) + (accumulator element), B operand e / 8
+        auto exp_range = [&](int e0, int e1) {
 #pragma unroll
-          for (int i = i0; i < i1; ++i) {
-            const float e = lf_exp2(s[kb][i] * cexp - mc_sub);
-            rs += e;
-            pf[2 * kb + i / 8][i % 8] = lf_from_float(e);
+          for (int e = e0; e < e1; ++e) {
+#if LF_CAPPOLY
+            const float sv = s[e / 16][e % 16];
+            const float ex = lf_exp2(__builtin_fmaf(sv, cap_t(sv * sv), -mc_sub));
+#else
+            const float ex = lf_exp2(s[e / 16][e % 16] * cexp - mc_sub);
+#endif
+            rs += ex;
+            pf[e / 8][e % 8] = lf_from_float(ex);
           }
         };
 #if LF_SPLIT_EXP
-        // the exponentials of the second key block go between the MFMAs that consume the first:
+        // the exponentials of the tile's second half go between the MFMAs that consume the first:
         // the wave keeps the matrix pipe busy during half of its own softmax
-        exp_block(0, 0, 16);
+        exp_range(0, 8 * LF_NKB);
 #else
-#pragma unroll
-        for (int kb = 0; kb < LF_NKB; ++kb) exp_block(kb, 0, 16);
+        exp_range(0, 16 * LF_NKB);
 #endif
 
         // ---- O^T += V^T P^T; the last steps also read the first fragments of K(kt+1)
@@ -527,7 +625,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
           if (f >= LF_NFV - LF_KPF) kpre[f - (LF_NFV - LF_KPF)] = k_frag(knext, f - (LF_NFV - LF_KPF));
           o[f % LF_NDB] = lf_mfma32(vf[f], pf[f / LF_NDB], o[f % LF_NDB]);
 #if LF_SPLIT_EXP
-          if (f < LF_NFV / 2) exp_block(1, f * 32 / LF_NFV, (f + 1) * 32 / LF_NFV);
+          if (f < LF_NFV / 2) exp_range(8 * LF_NKB + f * (16 * LF_NKB) / LF_NFV, 8 * LF_NKB + (f + 1) * (16 * LF_NKB) / LF_NFV);
 #endif
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -557,7 +655,7 @@ extern "C" __global__ void __launch_bounds__(LF_NT, 8 / LF_NW) lf_attn_prefill_s
     // optional: the row's log-sum-exp of the scaled, masked scores in log2 units (what a
     // backward pass recomputes the probabilities from); -inf for a row that saw no key
     if (p.part_ml != nullptr && g == 0 && my_q < p.Sq)
-#if LF_SOFTCAP
+#if LF_SOFTCAP && !LF_CAPPOLY
       // the kernel's scores are the capped ones minus the cap: the cap comes back in here
       p.part_ml[((long long)b * p.Hq + h) * p.Sq + my_q] = mc_ref + __builtin_log2f(l_tot) + p.softcap * LF_LOG2E;
 #else

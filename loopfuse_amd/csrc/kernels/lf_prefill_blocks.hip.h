@@ -79,6 +79,16 @@ __device__ __forceinline__ void lf_dma_to_lds(const lf_u32x4& rs, unsigned voff,
                : "={m0}"(m0_written) : "s"(m0v), "v"(voff), "s"(rs) : "memory");
 }
 
+// The same with the destination given as an LDS byte address (a wave-uniform integer, see lf_lds_addr): a
+// pointer that went through run-time arithmetic comes back from its generic form with a null test per load.
+__device__ __forceinline__ void lf_dma_to_lds_at(const lf_u32x4& rs, unsigned voff, unsigned lds_addr) {
+  unsigned m0_written;
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tbuffer_load_dwordx4 %2, %3, 0 offen lds"
+               : "={m0}"(m0_written) : "s"(lds_addr), "v"(voff), "s"(rs) : "memory");
+}
+// LDS byte address of a __shared__ object (folds to a constant for the object itself).
+#define lf_lds_addr(obj) ((unsigned)(size_t)(__attribute__((address_space(3))) const void*)(obj))
+
 // Buffer resource over `bytes` bytes from `base` (raw buffer, 32-bit offsets, range checked).
 __device__ __forceinline__ lf_u32x4 lf_make_buffer(const void* base, unsigned bytes) {
   const unsigned long long a = (unsigned long long)base;

@@ -21,6 +21,7 @@
 #include <unordered_set>
 #include <vector>
 
+#include <fcntl.h>
 #include <sys/stat.h>
 #include <unistd.h>
 
@@ -182,6 +183,9 @@ int lf_compile_cached(const char* src, const char* name, const char* const* opts
       void* buf = std::malloc(static_cast<size_t>(n));
       if (buf && std::fread(buf, 1, static_cast<size_t>(n), f) == static_cast<size_t>(n)) {
         std::fclose(f);
+        // a hit refreshes the entry's modification time, so that whoever prunes the directory can
+        // tell the entries still asked for from superseded ones (failure, e.g. a read-only cache, is fine)
+        ::utimensat(AT_FDCWD, path.c_str(), nullptr, 0);
         *code = buf;
         *code_len = static_cast<size_t>(n);
         if (hit) *hit = 1;

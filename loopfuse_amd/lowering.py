@@ -79,6 +79,7 @@ class KernelSpec:
     page_size_v: int = 0   # tokens per page of the V pool when it differs from K's (0 = same)
     d2: int = 0            # prefill: depth of a second score product Q2 K2^T (0, 16, 32, 64)
     safe: bool = False     # rows that saw no key come out as zeros instead of NaN
+    bn: int = 0            # prefill_swp: keys per LDS tile, 32 (three workgroups per CU) or 0 / 64 (two)
     extra: tuple = ()      # further -D options (tuning experiments)
 
     def options(self) -> list[str]:
@@ -106,6 +107,9 @@ class KernelSpec:
             if self.d2:
                 o += [f"-DLF_D2={self.d2}"]
         elif self.family == "prefill_swp":
+            if self.bn == 32:
+                # 32-key tiles: 40 KB of LDS and <= 168 registers, so three workgroups share a CU
+                o += ["-DLF_BN=32", "-DLF_WPE=3", "-DLF_KPF=3", "-DLF_VPF=2"]
             if self.pack:
                 o += [f"-DLF_GQAPACK={int(self.pack)}"]
             if self.bias:
@@ -133,7 +137,7 @@ class KernelSpec:
         return (f"lf_{self.family}_t{self.dtype}_d{self.head_dim}_m{self.mask}_c{int(self.softcap)}"
                 f"_p{self.paged}x{self.page_size}i{int(self.table_i64)}_r{self.rows}w{self.waves}v{int(self.v_tr)}h{int(self.headwave)}b{self.bias}n{int(self.denom)}"
                 + (f"_q{self.d2}" if self.d2 else "") + (f"_gp{int(self.pack)}" if self.pack else "") + (f"_pv{self.page_size_v}" if self.page_size_v else "")
-                + ("_z" if self.safe else "") + ("_co" if self.coop else "") + ("_rl" if self.rowload else "")
+                + ("_z" if self.safe else "") + (f"_bn{self.bn}" if self.bn else "") + ("_co" if self.coop else "") + ("_rl" if self.rowload else "")
                 + "".join("_" + e.replace("-D", "").replace("=", "") for e in self.extra))
 
     def source(self) -> str:
@@ -342,6 +346,20 @@ def _decode_rowload(paged: int, page_size: int, page_size_v: int, bias_bits: int
     return not paged or (page_size % 16 == 0 and (page_size_v or page_size) % 16 == 0)
 
 
+def prefill_kv_tile(D: int, bias_bits: int = 0, choice: Optional[dict] = None) -> int:
+    """Keys per LDS tile of lf_attn_prefill_swp: 0 (the kernel's 64) or 32.  With 32-key tiles a
+    workgroup needs 40 KB of LDS and at most 168 registers per lane, so three workgroups instead of
+    two share a CU; at head dimension 128 that outweighs the second barrier per 64 keys (config 2
+    -2.5 %, config 3 -10 %).  The bias tile classes are per 64 keys, so biased calls keep 64.
+    ``choice["bn"]`` (the tuner) or ``LOOPFUSE_BN`` override the default."""
+    if bias_bits:
+        return 0
+    want = (choice or {}).get("bn", os.environ.get("LOOPFUSE_BN"))
+    if want is not None:
+        return 32 if int(want) == 32 else 0
+    return 32 if D == 128 else 0
+
+
 def prefill_variant(Sq: int, v_tr: bool = True) -> str:
     """Which prefill kernel serves a call.  Default: the software-pipelined kernel
     with direct-to-LDS staging (``prefill_swp``; dense K/V only, ``attention`` falls
@@ -407,9 +425,14 @@ def tuned_attention(q, k, v, plan: AttnPlan, k_table=None, v_table=None, **kw):
             cands = [{"head_per_wave": hw, "splits": sp} for hw in ((False, True) if plan.k_paged and plan.v_paged else (False,))
                      for sp in (None, 1, 2, 4, 8)]
         elif not (plan.k_paged or plan.v_paged):
-            cands = [{"prefill": "swp"}, {"prefill": "w32"}]
+            # kernel family, tile shape (keys per LDS tile, which also sets how many workgroups share a
+            # CU; the reference's tuner searches tile sizes, codegen.py:360-393) and, for grouped query
+            # heads, the packed / unpacked q tile
+            cands = [{"prefill": "swp", "bn": 32}, {"prefill": "swp", "bn": 64}, {"prefill": "w32"}]
             if group % 2 == 0:
-                cands.insert(1, {"prefill": "swp", "pack": False})
+                cands[2:2] = [{"prefill": "swp", "bn": 32, "pack": False}, {"prefill": "swp", "bn": 64, "pack": False}]
+        elif Sq > 1:
+            cands = [{"bn": 32}, {"bn": 64}]
         else:
             cands = [{}]
         best, best_t = cands[0], float("inf")
@@ -746,13 +769,16 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         spec = KernelSpec(family, _DTYPE_CODE[dtype], D, mask, plan.softcap is not None, paged,
                           page_size, table_i64, v_tr=v_tr if family == "prefill" else True, bias=bias_bits,
                           denom=plan.denom_add != 0.0, d2=d2, page_size_v=page_size_v, pack=pack, extra=extra,
-                          safe=plan.zero_blind_rows and bool(bias_bits & 1))
+                          safe=plan.zero_blind_rows and bool(bias_bits & 1),
+                          bn=prefill_kv_tile(D, bias_bits, choice) if family == "prefill_swp" else 0)
         bm, bn = TILE_SHAPES[family]
         nw = 4
         for e in spec.extra:                    # tuning: -DLF_NW=8 doubles the q tile
             if e.startswith("-DLF_NW="):
                 nw = int(e.split("=")[1])
                 bm = 32 * nw
+        if spec.bn:
+            bn = spec.bn
         heads = Hq
         if spec.pack:
             bm, heads = 128 // spec.pack, Hq // spec.pack      # q tiles of 32 rows x 4 heads, or 64 rows x 2 heads
@@ -790,7 +816,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
             get_kernel(spec, "lf_bias_classify").launch((nqt, nb_ * nh_, (nkt + 3) // 4), (256, 1, 1), P)
             names.insert(0, "lf_bias_classify")
         get_kernel(spec, spec.entry()).launch((grid, 1, 1), (64 * nw, 1, 1), P)
-        _last_launch.set({"kernels": names, "grid": grid, "block": 64 * nw, "q_tile_rows": bm,
+        _last_launch.set({"kernels": names, "grid": grid, "block": 64 * nw, "q_tile_rows": bm, "kv_tile_rows": bn,
                                  "heads_per_workgroup": spec.pack or 1})
         return (out, visits) if record_visits else out
 

@@ -62,6 +62,47 @@ def test_causal_prefill(dtype, S, D):
     check(q, k, v, mask="causal")
 
 
+@pytest.mark.parametrize("bn", [32, 64])
+@pytest.mark.parametrize("dtype,D", [(torch.bfloat16, 128), (torch.float16, 128), (torch.bfloat16, 64)])
+def test_prefill_tile_shapes(bn, dtype, D):
+    """Both tile shapes of lf_attn_prefill_swp (32 keys per tile with three workgroups per CU, 64 with two)
+    on every mask, with and without a cap, grouped heads packed and unpacked, page pools, ragged lengths."""
+    c = {"bn": bn}
+    for S in (65, 593):
+        q, k, v = (rand((1, 4, S, D), dtype, s) for s in (1, 2, 3))
+        for mask, window in ((None, 0), ("causal", 0), ("sliding", 100)):
+            for cap in (None, 30.0):
+                check(q, k, v, mask=mask, window=window, softcap=cap, choice=c, force_family="prefill")
+                assert lowering.attention.last_launch["kv_tile_rows"] == bn
+                assert lowering.attention.last_launch["kernels"] == ["lf_attn_prefill_swp"]
+    q = rand((2, 8, 300, D), dtype, 4)
+    k, v = (rand((2, 2, 450, D), dtype, s) for s in (5, 6))
+    for pack in (True, False):
+        check(q, k, v, mask="sliding", window=256, softcap=30.0, choice={**c, "pack": pack})
+        assert lowering.attention.last_launch["kv_tile_rows"] == bn
+    n, P = 2 * 29, 16                                      # page pool [N, P, Hkv, D], 464 tokens per sequence
+    pool_k, pool_v = (rand((n, P, 2, D), dtype, s) for s in (7, 8))
+    table = torch.randperm(n, generator=torch.Generator().manual_seed(9)).view(2, 29).to(torch.int32)
+    check(q, pool_k, pool_v, mask="causal", k_table=table, v_table=table, choice=c)
+    assert lowering.attention.last_launch["kv_tile_rows"] == bn
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("q_scale", [1.0, 4.0, 8.0, 20.0])
+def test_softcap_forms(dtype, q_scale):
+    """The cap is a fused polynomial while a tile's scores are small (|score * scale / cap| <= 0.15), a polynomial
+    in place up to 0.4 and on tiles under a mask, and 1 - 2 / (e^2x + 1) beyond: larger queries move tiles from one
+    form to the next, and rows mix them.  V is scaled down so that the peaked softmax of large scores stays
+    within the storage format's rounding."""
+    for mask, window, S in (("causal", 0, 700), ("sliding", 256, 700), (None, 0, 200)):
+        q = (rand((1, 4, S, 128), torch.float32, 11) * q_scale).to(dtype)
+        k = rand((1, 2, S, 128), dtype, 12)
+        v = (rand((1, 2, S, 128), torch.float32, 13) * 0.25).to(dtype)
+        for cap in (30.0, 5.0):
+            for bn in (32, 64):
+                check(q, k, v, mask=mask, window=window, softcap=cap, choice={"bn": bn}, force_family="prefill")
+
+
 @pytest.mark.parametrize("v_tr", [True, False])
 def test_causal_prefill_v_read_paths(v_tr):
     q, k, v = (rand((1, 2, 320, 128), torch.bfloat16, s) for s in (1, 2, 3))
@@ -329,6 +370,8 @@ def test_visited_tiles_bit_exact(mask, window, S, variant, monkeypatch):
     plan = lowering.AttnPlan(mask=mask, window=window, scale=128 ** -0.5)
     _, visits = lowering.attention(q, k, v, plan, record_visits=True, force_family="prefill")
     torch.cuda.synchronize()
+    bn = lowering.attention.last_launch["kv_tile_rows"]      # 32 or 64 keys per tile, the launch's choice
+    assert lowering.attention.last_launch["q_tile_rows"] == bm
     nqt = skip.cdiv(S, bm)
     visits = visits.cpu().view(2, nqt, -1).bool()
     dense = O.visited_tiles_dense(mask, S, S, window, bm, bn)
@@ -353,6 +396,7 @@ def test_visited_tiles_bit_exact_with_packed_query_heads(mask, window, S, g):
     out, visits = lowering.attention(q, k, v, plan, record_visits=True)
     torch.cuda.synchronize()
     assert lowering.attention.last_launch["heads_per_workgroup"] == g and lowering.attention.last_launch["q_tile_rows"] == bm
+    bn = lowering.attention.last_launch["kv_tile_rows"]
     nqt = skip.cdiv(S, bm)
     visits = visits.cpu().view(2 * (8 // g), nqt, -1).bool()   # (batch x packs of g heads, q tile, kv tile)
     dense = O.visited_tiles_dense(mask, S, S, window, bm, bn)
