@@ -61,6 +61,10 @@ class View:
         return ir.Read(self.buf, self.idx, g)
 
 
+def _is_float(dtype_name: str) -> bool:
+    return dtype_name.startswith(("float", "bfloat", "half", "double"))
+
+
 def _hint(x) -> int:
     if isinstance(x, int):
         return x
@@ -137,11 +141,53 @@ class Parser:
                 if len(outs) != 1 or not isinstance(self.env.get(outs[0]), View):
                     raise Unsupported("graphs with one tensor output only")
                 self.out = self.env[outs[0]]
+                if self.out.buf.kind == "input" and not _is_float(self.out.buf.dtype):
+                    raise Unsupported("integer output")
             else:
                 raise Unsupported(f"node kind {n.op}")
         return self
 
+    # keyword arguments whose given value changes nothing (anything else is refused: the nests below are
+    # built from the positional arguments alone)
+    _NEUTRAL_KWARGS = {"alpha": 1, "beta": 1, "rounding_mode": None, "keepdim": None, "memory_format": None,
+                       "pin_memory": None, "layout": None, "device": None, "non_blocking": False}
+    _VIEW_OPS = None
+
+    def _guard(self, n: torch.fx.Node) -> None:
+        """Refuse what the builder would otherwise get silently wrong: scaled forms of add / sub / addmm
+        (``alpha`` / ``beta``), rounding divisions, conversions to a non-floating type (the kernels compute
+        in fp32 and treat a conversion as the identity), and integer tensors used as values (only gather
+        tables may be integers)."""
+        t, a = n.target, n.args
+        for k, v in n.kwargs.items():
+            if k == "keepdim" or (k == "dtype" and (v is None or (isinstance(v, torch.dtype) and v.is_floating_point))):
+                continue
+            if k in self._NEUTRAL_KWARGS and (v == self._NEUTRAL_KWARGS[k] or v is None):
+                continue
+            if k in ("memory_format", "layout", "device", "pin_memory"):
+                continue                      # where a copy lives, not what it holds
+            raise Unsupported(f"{t}: keyword argument {k}={v!r}")
+        aten = torch.ops.aten
+        if t is torch.ops.prims.convert_element_type.default and len(a) > 1 and isinstance(a[1], torch.dtype) \
+                and not a[1].is_floating_point:
+            raise Unsupported(f"conversion to {a[1]}")
+        if t is aten._softmax.default and len(a) > 2 and a[2]:
+            raise Unsupported("_softmax with half_to_float")
+        if Parser._VIEW_OPS is None:
+            Parser._VIEW_OPS = {aten.transpose.int, aten.permute.default, aten.unsqueeze.default, aten.clone.default,
+                                aten.alias.default, aten.expand.default, aten.view.default, aten._unsafe_view.default,
+                                aten.reshape.default, aten.sym_size.int}
+        if t in Parser._VIEW_OPS:
+            return
+        for k, x in enumerate(a):
+            v = self.env.get(x) if isinstance(x, torch.fx.Node) else None
+            if isinstance(v, View) and v.buf.kind == "input" and not _is_float(v.buf.dtype):
+                if t is torch.ops.loopfuse.paged_load.default and k == 1:
+                    continue                  # the page table
+                raise Unsupported(f"{t}: integer tensor {v.buf.name} used as a value")
+
     def call(self, n: torch.fx.Node):
+        self._guard(n)
         t, a = n.target, n.args
         val = lambda x: self.env[x] if isinstance(x, torch.fx.Node) else x
         # ---- integer arithmetic on sizes

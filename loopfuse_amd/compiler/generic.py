@@ -15,9 +15,12 @@ from .emit import NotLowerable
 
 
 # One thread per output element with sequential inner loops is meant for the small graphs around
-# an attention (epilogues, table look-ups, normalisations); beyond this many inner-loop steps per
-# call the graph is left to the captured ATen ops (rocBLAS for its matmuls).
-MAX_SCALAR_WORK = 1 << 33
+# an attention (epilogues, table look-ups, normalisations).  Element-wise nests move their bytes once,
+# like the ATen ops they replace, at any size; a nest with a reduction or a contraction runs its inner
+# loop per thread with strided reads, which rocBLAS beats by orders of magnitude on anything large:
+# beyond this many inner-loop steps per call (all reducing nests together; 512 x 512 x 512 multiply-adds)
+# the graph is left to the captured ATen ops.
+MAX_SCALAR_WORK = 1 << 27
 
 
 class GenericProgram:
@@ -136,7 +139,9 @@ class GenericProgram:
             for i, s in enumerate(k.scalars):
                 prm.f[i] = float(s.fn(args))
             total = math.prod(ext[a.id] for a in k.par)
-            work += total * math.prod(ext[a.id] for a in k.atoms if not any(a is x for x in k.par))
+            inner = math.prod(ext[a.id] for a in k.atoms if not any(a is x for x in k.par))
+            if inner > 1:
+                work += total * inner
             if work > MAX_SCALAR_WORK:
                 raise NotLowerable("more scalar work than the plain kernels are meant for")
             if total:

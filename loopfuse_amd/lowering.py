@@ -325,7 +325,8 @@ def _decode_headwave(paged: int, page_size: int, Hkv: int, D: int, P: "AttnParam
             and units_hw * max(1, min(8, Sk // 512)) >= cus)
 
 
-def _decode_coop(headwave: bool, page_size: int, page_size_v: int, bias_bits: int, Hkv: int, waves: int) -> bool:
+def _decode_coop(headwave: bool, page_size: int, page_size_v: int, bias_bits: int, Hkv: int, waves: int,
+                 P: "AttnParams", D: int) -> bool:
     """With one kv head per wave the workgroup reads every 16-token block of its 8 heads as one
     contiguous piece and hands the rows to the waves through LDS (``-DLF_COOP=1``) when a block
     lies inside a page (pages of a multiple of 16 tokens) and there is no score bias to carry
@@ -333,7 +334,11 @@ def _decode_coop(headwave: bool, page_size: int, page_size_v: int, bias_bits: in
     tenth of the HBM rate.  LOOPFUSE_DECODE_COOP=0 keeps the per-wave loads."""
     if os.environ.get("LOOPFUSE_DECODE_COOP", "1") != "1":
         return False
-    return headwave and page_size % 16 == 0 and not page_size_v and not bias_bits and Hkv % waves == 0
+    # the block loads take a token's 8 heads as one run of 8 * D elements: the pool must hold the heads of a
+    # token side by side (a permuted [pages, Hkv, page, D] pool view goes to the per-wave loads, which follow
+    # the head stride)
+    token_major = P.k_sh == D and P.v_sh == D and P.k_ss >= Hkv * D and P.v_ss >= Hkv * D
+    return headwave and page_size % 16 == 0 and not page_size_v and not bias_bits and Hkv % waves == 0 and token_major
 
 
 def _decode_rowload(paged: int, page_size: int, page_size_v: int, bias_bits: int) -> bool:
@@ -346,18 +351,20 @@ def _decode_rowload(paged: int, page_size: int, page_size_v: int, bias_bits: int
     return not paged or (page_size % 16 == 0 and (page_size_v or page_size) % 16 == 0)
 
 
-def prefill_kv_tile(D: int, bias_bits: int = 0, choice: Optional[dict] = None) -> int:
+def prefill_kv_tile(D: int, bias_bits: int = 0, choice: Optional[dict] = None, workgroups: int = 1 << 30) -> int:
     """Keys per LDS tile of lf_attn_prefill_swp: 0 (the kernel's 64) or 32.  With 32-key tiles a
     workgroup needs 40 KB of LDS and at most 168 registers per lane, so three workgroups instead of
     two share a CU; at head dimension 128 that outweighs the second barrier per 64 keys (config 2
-    -2.5 %, config 3 -10 %).  The bias tile classes are per 64 keys, so biased calls keep 64.
-    ``choice["bn"]`` (the tuner) or ``LOOPFUSE_BN`` override the default."""
+    -2.5 %, config 3 -10 %) once the launch has three workgroups for every CU -- a launch of 128
+    workgroups is a quarter slower with them -- and at head dimension 64 it does not.  The bias tile
+    classes are per 64 keys, so biased calls keep 64.  ``choice["bn"]`` (the tuner) or
+    ``LOOPFUSE_BN`` override the default."""
     if bias_bits:
         return 0
     want = (choice or {}).get("bn", os.environ.get("LOOPFUSE_BN"))
     if want is not None:
         return 32 if int(want) == 32 else 0
-    return 32 if D == 128 else 0
+    return 32 if D == 128 and workgroups >= 3 * 256 else 0
 
 
 def prefill_variant(Sq: int, v_tr: bool = True) -> str:
@@ -770,7 +777,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
                           page_size, table_i64, v_tr=v_tr if family == "prefill" else True, bias=bias_bits,
                           denom=plan.denom_add != 0.0, d2=d2, page_size_v=page_size_v, pack=pack, extra=extra,
                           safe=plan.zero_blind_rows and bool(bias_bits & 1),
-                          bn=prefill_kv_tile(D, bias_bits, choice) if family == "prefill_swp" else 0)
+                          bn=prefill_kv_tile(D, bias_bits, choice, B * (Hq // (pack or 1)) * (-(-Sq // (128 // (pack or 1)))))
+                          if family == "prefill_swp" else 0)
         bm, bn = TILE_SHAPES[family]
         nw = 4
         for e in spec.extra:                    # tuning: -DLF_NW=8 doubles the q tile
@@ -857,7 +865,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
     P.rows, P.nsplit, P.split_len = rows, nsplit, split_len
     spec = KernelSpec("decode", _DTYPE_CODE[dtype], D, MASK_NONE, plan.softcap is not None, paged,
                       page_size, table_i64, rows=DECODE_QROWS, waves=waves, headwave=headwave, page_size_v=page_size_v,
-                      coop=(coop := _decode_coop(headwave, page_size, page_size_v, bias_bits, Hkv, waves)),
+                      coop=(coop := _decode_coop(headwave, page_size, page_size_v, bias_bits, Hkv, waves, P, D)),
                       rowload=not coop and _decode_rowload(paged, page_size, page_size_v, bias_bits),
                       bias=bias_bits, safe=plan.zero_blind_rows and bool(bias_bits),
                       extra=tuple(os.environ.get("LOOPFUSE_KOPTS", "").split()))

@@ -40,7 +40,8 @@ def attention_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: int, 
                              softcap=float(softcap) if softcap else None)       # 0: no cap
     lse = torch.empty(q.shape[:-1], dtype=torch.float32, device=q.device)
     counters["fwd"] += 1
-    return lowering.attention(_rows(q), _rows(k), _rows(v), plan, lse=lse), lse
+    # the log-sum-exp is written by the direct-to-LDS kernel only: ask for it whatever LOOPFUSE_PREFILL says
+    return lowering.attention(_rows(q), _rows(k), _rows(v), plan, lse=lse, choice={"prefill": "swp"}), lse
 
 
 @attention_fwd.register_fake

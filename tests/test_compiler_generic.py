@@ -172,6 +172,41 @@ def test_graphs_outside_the_builder_are_refused():
         generic.GenericProgram(gm)
 
 
+REFUSED = {
+    "add_alpha": (lambda a, b: torch.add(a, b, alpha=3.0), lambda: (_r(6, 8), _r(6, 8, seed=1))),
+    "sub_alpha": (lambda a, b: torch.sub(a, b, alpha=2.0), lambda: (_r(6, 8), _r(6, 8, seed=1))),
+    "addmm_scaled": (lambda c, a, b: torch.addmm(c, a, b, beta=0.5, alpha=2.0),
+                     lambda: (_r(6, 5, seed=2), _r(6, 8), _r(8, 5, seed=1))),
+    "int64_add": (lambda a: a + 1, lambda: (torch.full((4, 4), 2 ** 30 + 1, dtype=torch.int64),)),
+    "truncation": (lambda a: (a * 2.7).to(torch.int32).float() * 1.5, lambda: (_r(6, 8),)),
+    "rounded_division": (lambda a, b: torch.div(a, b, rounding_mode="floor"), lambda: (_r(6, 8), _r(6, 8, seed=1) + 3.0)),
+    "integer_values": (lambda a, t: a + t, lambda: (_r(3, 5), torch.arange(15, dtype=torch.int32).view(3, 5))),
+}
+
+
+@pytest.mark.parametrize("name", list(REFUSED))
+def test_scaled_rounding_and_integer_forms_are_refused_and_run_as_captured(name):
+    """What the nest builder cannot express -- ``alpha`` / ``beta`` of add / sub / addmm, rounding divisions,
+    conversions to an integer type, integer tensors used as values -- gets no generic program (it would
+    compute something else in fp32); through the backend such a graph runs as captured and agrees with eager."""
+    from loopfuse_amd import loopfuse_backend
+    from loopfuse_amd.torch_backend import interface
+
+    fn, make = REFUSED[name]
+    ins = make()
+    gm, _, _ = _aten_graph(fn, ins)
+    with pytest.raises(emit.NotLowerable):
+        generic.GenericProgram(gm)
+    before = dict(interface.stats)
+    torch._dynamo.reset()
+    got = torch.compile(fn, backend=loopfuse_backend)(*ins)
+    want = fn(*ins)
+    assert got.dtype == want.dtype
+    torch.testing.assert_close(got, want)
+    assert interface.stats["generic_graphs"] == before["generic_graphs"]
+    assert interface.stats["eager_graph"] == before["eager_graph"] + 1
+
+
 def test_backend_takes_the_generic_program_for_graphs_without_attention(monkeypatch):
     """Through ``torch.compile(backend=loopfuse_backend)``: the graph gets a generic program; on
     CPU tensors its kernels cannot run and the call goes to the captured graph (counted, not

@@ -496,6 +496,20 @@ def test_mixed_page_sizes(pk, pv):
     check(rand((B, Hq, S, D), torch.bfloat16, 4), kp, vp, mask="causal", k_table=kt, v_table=vt)
 
 
+def test_decode_head_major_pool_keeps_per_wave_loads():
+    """A page pool whose storage is [pages, Hkv, page, D] (viewed as [pages, page, Hkv, D]): the cooperative
+    block loads assume the heads of a token side by side, so even when one head per wave is asked for the
+    launch must fall to the per-wave loads, which follow the head stride."""
+    w = workloads.make("c5", seed=3, B=2, S=256)
+    kp = w.k.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    vp = w.v.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    assert kp.stride(2) != kp.shape[3] and torch.equal(kp, w.k)
+    check(w.q, kp, vp, k_table=w.k_table, v_table=w.v_table, choice={"head_per_wave": True, "splits": 2})
+    assert lowering.attention.last_launch["head_per_wave"] and not lowering.attention.last_launch["cooperative_loads"]
+    check(w.q, w.k, w.v, k_table=w.k_table, v_table=w.v_table, choice={"head_per_wave": True, "splits": 2})
+    assert lowering.attention.last_launch["cooperative_loads"]
+
+
 def test_decode_paged_identity_table_equals_contiguous(monkeypatch):
     w = workloads.make("c5", seed=2, B=2, S=256)
     n = w.k.shape[0]
