@@ -37,8 +37,26 @@ if ROOT not in sys.path:
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16/fp16, published
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, published
 # HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by a plain copy of known
-# size (the rocprofv3 summaries under profiles/); counters cannot be read from inside this process
-TRAFFIC_BYTES = {"c2": (541 + 128) * (1 << 20), "c5": (513 + 4) * (1 << 20)}
+# size: counters cannot be read from inside this process, so the figures are taken from the line
+# "traffic_bytes_per_launch: <workload>=<bytes> ..." of the counter summary under profiles/
+# (null when the summary or the workload's figure is missing)
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "lf_attn_prefill_swp_c2_and_lf_attn_decode_c5_hbm_traffic_mfma_and_stalls.md")
+
+
+def _traffic_bytes() -> dict:
+    import re
+
+    try:
+        with open(TRAFFIC_SUMMARY) as fh:
+            for line in fh:
+                if line.startswith("traffic_bytes_per_launch:"):
+                    return {k: int(v) for k, v in re.findall(r"(\w+)=(\d+)", line)}
+    except OSError:
+        pass
+    return {}
+
+
+TRAFFIC_BYTES = _traffic_bytes()
 
 
 def time_gpu(fn, steps: int, warmup: int):

@@ -86,6 +86,7 @@ class Parser:
         self.sizes: dict[str, int] = {}  # size symbol -> placeholder index (SymInt inputs), for evaluation per call
         self.ntemp = 0
         self.out: Optional[View] = None
+        self.cur_node: Optional[torch.fx.Node] = None     # the node whose nests are being built
 
     # ------------------------------------------------------------ helpers
     def temp(self, name: str, dims: list[list[Atom]]) -> Buffer:
@@ -103,6 +104,7 @@ class Parser:
 
     def emit(self, name: str, out_dims: list[list[Atom]], red: list[Atom], value: ir.Expr, accum=None) -> View:
         buf = self.temp(name, out_dims)
+        buf.node = self.cur_node
         stmt = ir.Assign(buf, value) if accum is None else ir.Accum(buf, accum[0], value, accum[1])
         self.nests.append(ir.Nest(buf.name, [a for d in out_dims for a in d], red, stmt))
         return View(buf, [list(d) for d in out_dims], [list(d) for d in out_dims])
@@ -134,6 +136,7 @@ class Parser:
                     raise Unsupported(f"placeholder {n.name} of type {type(v).__name__}")
                 ph += 1
             elif n.op == "call_function":
+                self.cur_node = n
                 self.env[n] = self.call(n)
             elif n.op == "output":
                 outs = n.args[0]
@@ -212,6 +215,17 @@ class Parser:
             return ("scalar", (lambda args, c=float(x): c), f"{float(x):g}")
         if t is torch.ops.prims.convert_element_type.default and isinstance(val(a[0]), tuple):
             return val(a[0])
+        if t in (aten.add.Tensor, aten.sub.Tensor, aten.mul.Tensor, aten.div.Tensor) and len(a) == 2 and \
+                all(isinstance(val(x), tuple) and val(x)[0] == "scalar" or isinstance(x, (int, float)) for x in a) and \
+                any(isinstance(val(x), tuple) for x in a):
+            # arithmetic on 0-dim values ((D + D2) ** -0.5)
+            def part(x):
+                v = val(x)
+                return (v[1], v[2]) if isinstance(v, tuple) else ((lambda args, c=float(x): c), f"{float(x):g}")
+            (fa, ta), (fb, tb) = part(a[0]), part(a[1])
+            op, sym = {aten.add.Tensor: (operator.add, "+"), aten.sub.Tensor: (operator.sub, "-"),
+                       aten.mul.Tensor: (operator.mul, "*"), aten.div.Tensor: (operator.truediv, "/")}[t]
+            return ("scalar", (lambda args, f=op, x=fa, y=fb: f(x(args), y(args))), f"({ta}{sym}{tb})")
         if t is aten.pow.Tensor_Tensor and isinstance(val(a[0]), tuple) and isinstance(val(a[1]), tuple):
             x, y = val(a[0]), val(a[1])
             return ("scalar", (lambda args, f=x[1], g=y[1]: f(args) ** g(args)), f"{x[2]}**{y[2]}")
@@ -239,6 +253,8 @@ class Parser:
             dims = [list(d) for d in v.dims]
             dims = [[] for _ in range(len(a[1]) - len(dims))] + dims
             for k, s in enumerate(a[1]):
+                if not isinstance(s, torch.fx.Node) and int(s) == -1:
+                    continue                  # -1: the dimension stays as it is
                 sym, h = self.size_of(s)
                 have = math.prod(x.hint for x in ir.leaves(dims[k])) if dims[k] else 1
                 if have == 1 and h != 1:
@@ -277,9 +293,21 @@ class Parser:
             ir.unify(x.dims[1], y.dims[0])
             prod = self.emit("dot", [x.dims[0], y.dims[1]], [], ir.Dot(x.read(), y.read(), list(x.dims[1])))
             return self.pointwise2("add", val(a[0]).instantiate(), prod.instantiate())
-        if t is aten.exp.default:
+        if t is aten.exp.default or t is aten.exp2.default:
             v = val(a[0]).instantiate()
-            return self.emit("exp", v.dims, [], ir.Un("exp", v.read()))
+            op = "exp" if t is aten.exp.default else "exp2"
+            return self.emit(op, v.dims, [], ir.Un(op, v.read()))
+        if t is torch.ops.loopfuse.scan_max.default:
+            # (running maximum along the last dim, its final value with the dim kept): the final value is a
+            # max nest; the running one gets no nest -- the graphs that use it (the reference's online-softmax
+            # hint exp2(x - run) * exp2(run - max), tests/test_attention.py:95-125) cancel it, which the
+            # simplify pass carries out and insists on
+            x = val(a[0]).instantiate()
+            outer, red = x.dims[:-1], x.dims[-1]
+            m = self.emit("max", list(outer) + [[]], list(red), x.read(), ("max", float("-inf")))
+            run = Buffer(f"scan{self.ntemp}", [list(d) for d in x.dims], "scan")
+            run.scan_of = m.buf
+            return ("tuple", View(run, [list(d) for d in x.dims], [list(d) for d in x.dims]), m)
         if t in (aten.max.dim, aten.sum.dim_IntList, aten.amax.default):
             v = val(a[0]).instantiate()
             dims = a[1] if isinstance(a[1], (list, tuple)) else [a[1]]
@@ -291,9 +319,10 @@ class Parser:
             r = self.emit("sum" if op[0] == "add" else "max", outer, red, v.read(), op)
             return ("tuple", r) if t is aten.max.dim else r
         if t is operator.getitem and isinstance(val(a[0]), tuple) and val(a[0])[0] == "tuple":
-            if a[1] != 0:
+            tup = val(a[0])
+            if a[1] + 1 >= len(tup):
                 raise Unsupported("indices of max are not lowered")
-            return val(a[0])[1]
+            return tup[a[1] + 1]
         if t in (aten.mul.Tensor, aten.div.Tensor):
             x, y = val(a[0]), val(a[1])
             if isinstance(x, View) and not isinstance(y, View):

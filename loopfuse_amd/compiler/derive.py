@@ -28,11 +28,21 @@ class NotDerivable(Exception):
 
 @dataclasses.dataclass
 class OperandLayout:
-    placeholder: int                 # graph input holding the tensor (the pool when paged)
+    placeholder: int                 # graph input holding the tensor (the pool when paged); -1: see node
     perm: tuple = ()                 # dense: permutation of the input's dims giving [B, H, S, D]
     paged: bool = False
     table: int = -1                  # graph input holding the page table
     group: int = 1                   # query heads per kv head at the traced sizes
+    node: object = None              # an operand the graph computes from its inputs (Q + q_bias): the node
+
+
+@dataclasses.dataclass
+class BiasLayout:
+    """An added tensor as a view [B, Hq, rows, X]: per logical dim the source dim that walks it (None = broadcast)."""
+
+    placeholder: int
+    dims: tuple
+    node: object = None
 
 
 @dataclasses.dataclass
@@ -47,6 +57,13 @@ class DerivedAttention:
     v: OperandLayout
     bounds: Optional[TileBounds]
     tile: tuple                      # (BM, BN) the bounds were derived for
+    bias: Optional[BiasLayout] = None        # added to the scaled (capped) scores before the mask
+    out_bias: Optional[BiasLayout] = None    # added to the normalised result
+    q2: Optional[OperandLayout] = None       # second score product: scores = Q K^T + Q2 K2^T
+    k2: Optional[OperandLayout] = None
+    denom_add: tuple = ()                    # ("mul", value | callable) terms added to the softmax denominator
+    base2: bool = False                      # exponentials to base 2
+    late: list = dataclasses.field(default_factory=list)   # the factors of `pre` that the graph applies behind the mask
 
     def number(self, f, args) -> float:
         kind, x = f
@@ -66,15 +83,23 @@ class DerivedAttention:
                 f"post={[f[0] for f in self.post]} Q=in{self.q.placeholder}{self.q.perm} "
                 f"K=in{self.k.placeholder}{'[paged by in%d]' % self.k.table if self.k.paged else self.k.perm} "
                 f"V=in{self.v.placeholder}{'[paged by in%d]' % self.v.table if self.v.paged else self.v.perm} "
-                f"group={self.k.group} kv tiles: {self.bounds.text if self.bounds else 'all'}")
+                f"group={self.k.group} kv tiles: {self.bounds.text if self.bounds else 'all'}"
+                + (" +score_bias" if self.bias else "") + (" +out_bias" if self.out_bias else "")
+                + (" +second product" if self.q2 else "") + (f" denom+{len(self.denom_add)}" if self.denom_add else "")
+                + (" exp2" if self.base2 else ""))
 
 
 def _ids(atoms) -> set:
     return {a.id for a in ir.leaves(atoms) if a.hint != 1}
 
 
+def _has_dot(e: ir.Expr) -> bool:
+    return any(isinstance(x, ir.Dot) for x in ir.walk(e))
+
+
 def _peel(e: ir.Expr):
-    """mods(dot) -> (list of ("mul" | "div" | "tanh", value), the Dot), outermost first."""
+    """mods(core) -> (list of ("mul" | "div" | "tanh", value), core), outermost first; core is a Dot or the
+    sum of two Dots (two-part scores)."""
     ops = []
     while not isinstance(e, ir.Dot):
         if isinstance(e, ir.Un) and e.op == "tanh":
@@ -86,6 +111,8 @@ def _peel(e: ir.Expr):
         elif isinstance(e, ir.Bin) and e.op == "mul" and isinstance(e.a, (ir.Const, ir.Scalar)):
             ops.append(("mul", e.a.value if isinstance(e.a, ir.Const) else e.a.fn))
             e = e.b
+        elif isinstance(e, ir.Bin) and e.op == "add" and isinstance(e.a, ir.Dot) and isinstance(e.b, ir.Dot):
+            break
         else:
             raise NotDerivable(f"score modification {type(e).__name__} is not a scale / softcap chain")
     return ops, e
@@ -108,47 +135,97 @@ def _dense_perm(read: ir.Read, roles: dict, what: str) -> tuple:
 
 
 def attention(nests: list, inputs: list, out_view) -> DerivedAttention:
-    if len(nests) != 1 or not isinstance(nests[0].stmt, ir.Rescaled):
+    from .passes import is_operand_prep
+
+    main = [n for n in nests if isinstance(n.stmt, ir.Rescaled)]
+    rest = [n for n in nests if not isinstance(n.stmt, ir.Rescaled)]
+    if len(main) != 1 or not all(is_operand_prep(n) for n in rest):
         raise NotDerivable(f"{len(nests)} nests left after fusion: not a single attention")
-    nest = nests[0]
+    nest = main[0]
     st = nest.stmt
-    # ---- mask
+    # ---- factors the graph applies to the masked scores (x * c commutes with the mask for c > 0, which
+    # the call checks: -inf must stay -inf)
     score = st.score
+    late = []
+    while isinstance(score, ir.Bin) and score.op in ("mul", "div") and isinstance(score.b, (ir.Const, ir.Scalar)) \
+            and any(isinstance(x, ir.Select) for x in ir.walk(score.a)):
+        late.append((score.op, score.b.value if isinstance(score.b, ir.Const) else score.b.fn))
+        score = score.a
+    # ---- mask
     clauses = []
     if isinstance(score, ir.Select):
         if score.other != float("-inf"):
             raise NotDerivable("masked scores are not -inf")
         clauses, score = score.clauses, score.a
-    ops, dot = _peel(score)
-    if any(isinstance(x, ir.Select) for x in ir.walk(dot)):
+    # ---- an added tensor (score bias): outermost, on top of the scale / softcap chain
+    bias_read = None
+    if isinstance(score, ir.Bin) and score.op == "add":
+        for x, t in ((score.a, score.b), (score.b, score.a)):
+            if isinstance(t, ir.Read) and _has_dot(x) and not isinstance(x, ir.Dot):
+                score, bias_read = x, t
+                break
+            if isinstance(t, ir.Read) and isinstance(x, ir.Dot):
+                score, bias_read = x, t
+                break
+    ops, core = _peel(score)
+    if any(isinstance(x, ir.Select) for x in ir.walk(core)):
         raise NotDerivable("mask below the score product")
-    if not isinstance(dot.a, ir.Read) or not isinstance(dot.b, ir.Read):
-        raise NotDerivable("score product of something else than two tensors")
+    dot, dot2 = core, None
+    if not isinstance(core, ir.Dot):
+        # two-part scores: the product with the deeper contraction is the main one
+        d_a = math.prod(a.hint for a in ir.leaves(core.a.over))
+        d_b = math.prod(a.hint for a in ir.leaves(core.b.over))
+        dot, dot2 = (core.a, core.b) if d_a >= d_b else (core.b, core.a)
+    for d in (dot, dot2):
+        if d is not None and (not isinstance(d.a, ir.Read) or not isinstance(d.b, ir.Read)):
+            raise NotDerivable("score product of something else than two tensors")
     qr, kr, vr = dot.a, dot.b, st.weights
     keys, depth = _ids(nest.red), _ids(dot.over)
-    k_all = set().union(*[_ids(d) for d in kr.idx]) | (set().union(*[_ids(t) for t in kr.gather[2]]) if kr.gather else set())
+
+    def all_ids(r: ir.Read) -> set:
+        out = set().union(*[_ids(d) for d in r.idx]) if r.idx else set()
+        if r.gather:
+            out |= set().union(*[_ids(t) for t in r.gather[2]])
+        return out
+
     if _ids([a for d in qr.idx for a in d]) & keys:
         qr, kr = kr, qr                               # bmm(K, Q^T) spelling
-        k_all = set().union(*[_ids(d) for d in kr.idx])
-    # ---- Q
-    q_roles, group, rows = {}, 1, set()
-    for d, atoms in enumerate(qr.idx):
-        ids = _ids(atoms)
-        if not ids:
-            q_roles[d] = "one"                        # a size-1 dimension
-        elif ids <= depth:
-            q_roles[d] = "depth"
-        elif not (ids & k_all):
-            q_roles[d] = "seq"
-            rows = ids
-        else:
-            q_roles[d] = "batch"
-            group *= math.prod(a.hint for a in ir.leaves(atoms) if a.hint != 1 and a.id not in k_all)
-    if qr.gather is not None:
-        raise NotDerivable("paged queries")
-    q = OperandLayout(qr.buf.placeholder, _dense_perm(qr, q_roles, "Q"))
+    k_all = all_ids(kr)
 
-    def kv_layout(r: ir.Read, dep_ids: set, what: str) -> OperandLayout:
+    def source(r: ir.Read, what: str):
+        """(placeholder, node) of an operand: a graph input, or the node of an element-wise nest over inputs."""
+        if r.buf.kind == "input":
+            return r.buf.placeholder, None
+        if r.buf.node is not None and any(n.writes() is r.buf for n in rest):
+            return -1, r.buf.node
+        raise NotDerivable(f"{what} {r.buf.name} is computed inside the graph")
+
+    # the rows are what the result's second-to-last dim runs over (a key tensor shared by all heads leaves
+    # the head atoms out of K as well, so "not in K" alone does not tell rows from heads)
+    rows_out = _ids(out_view.dims[-2]) if len(out_view.dims) >= 2 else set()
+
+    def q_layout(r: ir.Read, dep_ids: set, k_ids: set, what: str):
+        roles, group, rows = {}, 1, set()
+        for d, atoms in enumerate(r.idx):
+            ids = _ids(atoms)
+            if not ids:
+                roles[d] = "one"                      # a size-1 dimension
+            elif ids <= dep_ids:
+                roles[d] = "depth"
+            elif ids <= rows_out if rows_out else not (ids & k_ids):
+                roles[d] = "seq"
+                rows = ids
+            else:
+                roles[d] = "batch"
+                group *= math.prod(a.hint for a in ir.leaves(atoms) if a.hint != 1 and a.id not in k_ids)
+        if r.gather is not None:
+            raise NotDerivable("paged queries")
+        ph, node = source(r, what)
+        return OperandLayout(ph, _dense_perm(r, roles, what), node=node), group, rows
+
+    q, group, rows = q_layout(qr, depth, k_all, "Q")
+
+    def kv_layout(r: ir.Read, dep_ids: set, what: str, grp: int) -> OperandLayout:
         roles = {}
         for d, atoms in enumerate(r.idx):
             ids = _ids(atoms)
@@ -162,26 +239,58 @@ def attention(nests: list, inputs: list, out_view) -> DerivedAttention:
                 roles[d] = "seq"
             else:
                 roles[d] = "batch"
+        ph, node = source(r, what)
         if r.gather is None:
-            return OperandLayout(r.buf.placeholder, _dense_perm(r, roles, what), group=group)
+            return OperandLayout(ph, _dense_perm(r, roles, what), group=grp, node=node)
         # pool [N, (P,) Hkv, D] gathered through table [B, pages]
         order = [{"one": "batch"}.get(roles[d], roles[d]) for d in range(len(r.idx))]
         if order not in (["page", "seq", "batch", "depth"], ["page", "batch", "depth"]):
             raise NotDerivable(f"{what} pool is not [pages, page size, heads, depth] (roles {order})")
         tbuf, tidx = r.gather[1], r.gather[2]
-        if len(tidx) != 2 or not (_ids(tidx[1]) <= keys) or (_ids(tidx[0]) & keys):
+        if len(tidx) != 2 or not (_ids(tidx[1]) <= keys) or (_ids(tidx[0]) & keys) or tbuf.kind != "input":
             raise NotDerivable(f"{what} page table is not [batch, pages]")
-        return OperandLayout(r.buf.placeholder, (), True, tbuf.placeholder, group)
+        return OperandLayout(ph, (), True, tbuf.placeholder, grp)
 
-    k = kv_layout(kr, depth, "K")
+    k = kv_layout(kr, depth, "K", group)
     out_depth = _ids(out_view.dims[-1])
-    v = kv_layout(vr, out_depth, "V")
-    for r in (qr, kr, vr):
-        if r.buf.kind != "input":
-            raise NotDerivable(f"operand {r.buf.name} is computed inside the graph")
+    v = kv_layout(vr, out_depth, "V", group)
+    # ---- second score product
+    q2 = k2 = None
+    if dot2 is not None:
+        q2r, k2r = dot2.a, dot2.b
+        if _ids([a for d in q2r.idx for a in d]) & keys:
+            q2r, k2r = k2r, q2r
+        depth2 = _ids(dot2.over)
+        q2, group2, rows2 = q_layout(q2r, depth2, all_ids(k2r), "Q2")
+        if rows2 != rows or q2r.gather is not None or k2r.gather is not None:
+            raise NotDerivable("the second score product runs over other rows, or is paged")
+        k2 = kv_layout(k2r, depth2, "K2", group2)      # a positional key may be shared by more heads than K is
     # ---- output: [batch..., rows, depth] in the order the kernel writes
     if len(out_view.dims) != 4 or (rows and _ids(out_view.dims[2]) != rows) or (_ids(out_view.dims[0]) | _ids(out_view.dims[1])) & (rows | out_depth):
         raise NotDerivable("result is not laid out [B, H, rows, depth]")
+
+    def added(r: Optional[ir.Read], last: set, what: str) -> Optional[BiasLayout]:
+        """An added tensor as [B, Hq, rows, last]: which of its dims walks which of the four."""
+        if r is None:
+            return None
+        if r.gather is not None:
+            raise NotDerivable(f"{what} is gathered")
+        ph, node = source(r, what)
+        qb, qh = _ids(qr.idx[q.perm[0]]), _ids(qr.idx[q.perm[1]])
+        dims = [None, None, None, None]
+        for d, atoms in enumerate(r.idx):
+            ids = {a.id for a in ir.leaves(atoms) if a.hint != 1 and not a.broadcast}
+            if not ids:
+                continue                              # size 1 or expanded: broadcast
+            want = [(0, qb), (1, qh), (2, rows), (3, last)]
+            slot = next((i for i, full in want if full and ids == full), None)
+            if slot is None or dims[slot] is not None:
+                raise NotDerivable(f"{what} does not broadcast over [batch, heads, rows, {'keys' if last is keys else 'depth'}]")
+            dims[slot] = d
+        return BiasLayout(ph, tuple(dims), node)
+
+    bias = added(bias_read, keys, "score bias")
+    out_bias = added(st.epilogue, out_depth, "output bias")
     # ---- clauses -> mask kind
     mask, window = None, 0
     for c in clauses:
@@ -204,5 +313,12 @@ def attention(nests: list, inputs: list, out_view) -> DerivedAttention:
     has_tanh = "tanh" in kinds
     cut = kinds.index("tanh") if has_tanh else 0
     post, pre = (ops[:cut], ops[cut + 1:]) if has_tanh else ([], ops)
+    if late and has_tanh:
+        raise NotDerivable("factors behind the mask of capped scores")
+    pre = list(pre) + late
+    if st.base2 and has_tanh:
+        raise NotDerivable("softcap inside an exp2-based softmax")
+    denom = tuple(("mul", t.value if isinstance(t, ir.Const) else t.fn) for t in st.denom_add)
     bounds, tile = (st.tile[2], st.tile[:2]) if st.tile else (None, ())
-    return DerivedAttention(mask, window, list(pre), list(post), has_tanh, q, k, v, bounds, tile)
+    return DerivedAttention(mask, window, list(pre), list(post), has_tanh, q, k, v, bounds, tile,
+                            bias=bias, out_bias=out_bias, q2=q2, k2=k2, denom_add=denom, base2=st.base2, late=late)

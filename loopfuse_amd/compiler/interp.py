@@ -66,7 +66,8 @@ class Interpreter:
             return {"add": a + b, "sub": a - b, "mul": a * b, "div": a / b, "max": torch.maximum(a, b)}[e.op]
         if isinstance(e, ir.Un):
             a = self.value(e.a, want)
-            return {"exp": torch.exp, "tanh": torch.tanh, "neg": torch.neg, "recip": torch.reciprocal}[e.op](a)
+            return {"exp": torch.exp, "exp2": torch.exp2, "tanh": torch.tanh, "neg": torch.neg,
+                    "recip": torch.reciprocal}[e.op](a)
         if isinstance(e, ir.Dot):
             inner = want + [a for a in _axes(e.over) if a.id not in {w.id for w in want}]
             prod = self.value(e.a, inner) * self.value(e.b, inner)
@@ -103,9 +104,17 @@ class Interpreter:
             else:
                 sc = self.value(s.score, par + red).expand([a.hint for a in par + red])
                 flat = sc.reshape([a.hint for a in par] + [-1])
-                p = torch.softmax(flat, dim=-1).reshape(sc.shape)
+                if s.base2:
+                    flat = flat * math.log(2.0)
+                ex = torch.exp(flat - flat.amax(dim=-1, keepdim=True))
+                den = ex.sum(dim=-1, keepdim=True)
+                for t in s.denom_add:
+                    den = den + self.value(t, [])
+                p = (ex / den).reshape(sc.shape)
                 w = self.read(s.weights, par + red)
                 val = (p * w).sum(dim=list(range(len(par), len(par) + len(red))))
+                if s.epilogue is not None:
+                    val = val + self.read(s.epilogue, par)
             buf = n.writes()
             val = val.expand([a.hint for a in par])
             # store shaped like the buffer's dims (atoms of a dim merged, in the buffer's order)

@@ -99,6 +99,8 @@ class Buffer:
     kind: str = "temp"
     dtype: str = "f32"
     placeholder: int = -1            # index among the graph's placeholders (inputs)
+    node: object = None              # temporaries: the graph node whose value this is
+    scan_of: Optional["Buffer"] = None   # kind "scan": the running form of this reduction's result (scan_max)
 
     def __repr__(self) -> str:
         return self.name
@@ -207,6 +209,10 @@ class Rescaled:
     score: Expr                      # per (row, key) value whose softmax is taken
     weights: Read                    # per (key, d) operand of the second product
     tile: Optional[tuple] = None     # (BM, BN, bounds): set by the block-skip pass
+    base2: bool = False              # the graph's exponentials are 2^x: the score is in log2 units
+    denom_add: tuple = ()            # out = acc / (sum + these): Const / Scalar terms, in units where the
+                                     # row maximum contributes 1 (reference tests/test_attention.py:95-125)
+    epilogue: Optional[Read] = None  # added to acc / sum element by element (an output bias)
 
 
 @dataclasses.dataclass(eq=False)
@@ -300,7 +306,10 @@ def show(nests: Sequence[Nest]) -> str:
         else:
             t = f"  tiles {s.tile[0]}x{s.tile[1]}, kv tiles [{s.tile[2].text}]" if s.tile else ""
             out.append(f"{pad}m, l, acc = online_softmax({show_expr(s.score)}) @ {show_expr(s.weights)}{t}")
-            out.append(f"{pad[:-2 * max(len(leaves(n.red)), 0)]}{s.out.name}[...] = acc / l")
+            den = "l" if not s.denom_add else "(l + " + " + ".join(show_expr(t) for t in s.denom_add) + ")"
+            epi = f" + {show_expr(s.epilogue)}" if s.epilogue is not None else ""
+            out.append(f"{pad[:-2 * max(len(leaves(n.red)), 0)]}{s.out.name}[...] = acc / {den}{epi}"
+                       + ("   # exponentials to base 2" if s.base2 else ""))
     return "\n".join(out)
 
 

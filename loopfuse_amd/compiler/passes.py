@@ -83,7 +83,15 @@ def _under_dot(e: ir.Expr, buf: ir.Buffer, inside: bool = False) -> bool:
     return any(_under_dot(c, buf, inside or isinstance(e, ir.Dot)) for c in e.children())
 
 
-def fuse(nests: list[Nest], keep: ir.Buffer, keep_contractions: bool = False) -> list[Nest]:
+def is_operand_prep(nest: Nest) -> bool:
+    """An element-wise nest over graph inputs alone (``Q + q_bias``): when a contraction reads its result,
+    the kernels take that result as an operand, so the nest keeps running as the graph node it came from."""
+    return (isinstance(nest.stmt, ir.Assign) and not nest.red and nest.stmt.buf.node is not None
+            and not any(isinstance(x, (ir.Dot, ir.Select)) for x in ir.walk(nest.stmt.value))
+            and all(r.buf.kind == "input" and r.gather is None for r in ir.reads(nest.stmt.value)))
+
+
+def fuse(nests: list[Nest], keep: ir.Buffer, keep_contractions: bool = False, keep_operands: bool = False) -> list[Nest]:
     """Inline every temporary written by a pointwise (``Assign``) nest into its readers and drop
     its nest; reductions (``Accum``) and the result buffer stay.  Runs to a fixed point.
 
@@ -107,6 +115,9 @@ def fuse(nests: list[Nest], keep: ir.Buffer, keep_contractions: bool = False) ->
                 u = users[0]
                 if len(users) > 1 or not isinstance(u.stmt, ir.Assign) or _under_dot(u.stmt.value, buf):
                     continue
+            if keep_operands and is_operand_prep(prod) and \
+                    all(_only_under_dot(u.stmt.score if isinstance(u.stmt, ir.Rescaled) else u.stmt.value, buf) for u in users):
+                continue                      # an operand of the products: stays a tensor of its own
 
             def inline(x, buf=buf, prod=prod):
                 if isinstance(x, ir.Read) and x.buf is buf:
@@ -124,10 +135,101 @@ def fuse(nests: list[Nest], keep: ir.Buffer, keep_contractions: bool = False) ->
     return nests
 
 
+def _only_under_dot(e: ir.Expr, buf: ir.Buffer, inside: bool = False) -> bool:
+    """Whether every read of ``buf`` in ``e`` is a direct operand of a contraction."""
+    if isinstance(e, ir.Read):
+        return e.buf is not buf or inside
+    if isinstance(e, ir.Dot):
+        return all(_only_under_dot(c, buf, isinstance(c, ir.Read)) for c in e.children())
+    return all(_only_under_dot(c, buf, False) for c in e.children())
+
+
 def _stmt_reads(stmt) -> list[ir.Read]:
     if isinstance(stmt, ir.Rescaled):
-        return ir.reads(stmt.score) + [stmt.weights]
+        return ir.reads(stmt.score) + [stmt.weights] + ([stmt.epilogue] if stmt.epilogue is not None else [])
     return ir.reads(stmt.value)
+
+
+# ---------------------------------------------------------------- simplify
+def _same(a: ir.Expr, b: ir.Expr) -> bool:
+    """Structural equality over the very same atoms."""
+    m: dict = {}
+    if not _struct_eq(a, b, m):
+        return False
+    return True
+
+
+def _terms(e: ir.Expr, sign: int, out: list) -> None:
+    if isinstance(e, ir.Bin) and e.op in ("add", "sub"):
+        _terms(e.a, sign, out)
+        _terms(e.b, sign if e.op == "add" else -sign, out)
+    else:
+        out.append((sign, e))
+
+
+def _cancel(e: ir.Expr) -> ir.Expr:
+    """A sum / difference tree with the terms that occur with both signs removed."""
+    ts: list = []
+    _terms(e, 1, ts)
+    live = [True] * len(ts)
+    for i, (si, ti) in enumerate(ts):
+        if not live[i]:
+            continue
+        for j in range(i + 1, len(ts)):
+            if live[j] and ts[j][0] == -si and _same(ti, ts[j][1]) and _identity_atoms(ti, ts[j][1]):
+                live[i] = live[j] = False
+                break
+    rest = [(sg, t) for (sg, t), ok in zip(ts, live) if ok]
+    if len(rest) == len(ts):
+        return e
+    if not rest:
+        return ir.Const(0.0)
+    pos = [t for sg, t in rest if sg > 0]
+    neg = [t for sg, t in rest if sg < 0]
+    acc = pos[0] if pos else ir.Un("neg", neg.pop(0))
+    for t in pos[1:]:
+        acc = ir.Bin("add", acc, t)
+    for t in neg:
+        acc = ir.Bin("sub", acc, t)
+    return acc
+
+
+def _identity_atoms(a: ir.Expr, b: ir.Expr) -> bool:
+    m: dict = {}
+    _struct_eq(a, b, m)
+    return all(k == v.id for k, v in m.items())
+
+
+def simplify(nests: list[Nest]) -> list[Nest]:
+    """Algebra that makes the graph's own online-softmax hints disappear (reference
+    compiler/passes/cleanup_passes.py + factor_acc.py:140-211 do this with sympy):
+    exp(a) * exp(b) -> exp(a + b) (same for exp2), sums with a term and its negative cancelled,
+    x * 1, x / 1, x + 0.  The running maximum of ``scan_max`` has no nest of its own: it has to
+    cancel, as in exp2(x - run) * exp2(run - max)."""
+    def step(x):
+        if isinstance(x, ir.Bin) and x.op == "mul":
+            a, b = ir.substitute(x.a, step), ir.substitute(x.b, step)
+            if isinstance(a, ir.Un) and isinstance(b, ir.Un) and a.op == b.op and a.op in ("exp", "exp2"):
+                return ir.Un(a.op, _cancel(ir.Bin("add", a.a, b.a)))
+            for u, w in ((a, b), (b, a)):
+                if isinstance(w, ir.Const) and w.value == 1.0:
+                    return u
+            return ir.Bin("mul", a, b)
+        if isinstance(x, ir.Bin) and x.op == "div":
+            a, b = ir.substitute(x.a, step), ir.substitute(x.b, step)
+            if isinstance(b, ir.Const) and b.value == 1.0:
+                return a
+            return ir.Bin("div", a, b)
+        return None
+
+    for n in nests:
+        if isinstance(n.stmt, (ir.Assign, ir.Accum)):
+            n.stmt.value = ir.substitute(n.stmt.value, step)
+    for n in nests:
+        for r in _stmt_reads(n.stmt):
+            if r.buf.kind == "scan":
+                raise PassError("a running maximum (scan_max) is used outside a cancelling online-softmax hint")
+    return nests
 
 
 # ---------------------------------------------------------------- online softmax
@@ -176,27 +278,46 @@ def _struct_eq(a: ir.Expr, b: ir.Expr, m: dict) -> bool:
 def online_softmax(nests: list[Nest], keep: ir.Buffer) -> list[Nest]:
     """After ``fuse`` an attention graph is three nests over the same rows:
 
-        m[r]    = max_j  x[r, j]                                  (Accum max)
-        l[r]    = sum_j  exp(x[r, j] - m[r])                      (Accum add)
-        o[r, d] = dot_j( exp(x[r, j] - m[r]) / l[r],  v[j, d] )   (Assign of a Dot over j)
+        m[r]    = max_j  x[r, j]                                        (Accum max)
+        l[r]    = sum_j  e(x[r, j] - m[r])                              (Accum add; e = exp or exp2)
+        o[r, d] = dot_j( e(x[r, j] - m[r]) / (l[r] + c),  v[j, d] ) + b[r, d]
 
-    The divisor l[r] does not depend on j, so it moves out of the contraction; what remains of
-    the second and third nest are sums over j of terms that carry the same factor exp(-m[r]).
-    With a running maximum in place of m, growing it from m_old to m_new multiplies every term
-    already summed by exp(m_old - m_new) -- a factor free of j -- so one pass that rescales both
-    accumulators whenever the maximum grows computes the same values (the "online hoist" of the
-    reference, factor_acc.py:23-109).  The pass checks that the three nests have exactly this
-    form, with the same x, and replaces them by one ``Rescaled`` nest."""
+    (c and b optional).  The divisor does not depend on j, so it moves out of the contraction, and
+    so does b; what remains of the second and third nest are sums over j of terms that carry the
+    same factor e(-m[r]).  With a running maximum in place of m, growing it from m_old to m_new
+    multiplies every term already summed by e(m_old - m_new) -- a factor free of j -- so one pass
+    that rescales both accumulators whenever the maximum grows computes the same values (the
+    "online hoist" of the reference, factor_acc.py:23-109, 140-211).  x is whatever the graph makes
+    of its score products -- scales, a cap, added tensors, a second product, masks -- and is carried
+    over as it is.  The pass checks that the nests have this form, with the same x, and replaces
+    them by one ``Rescaled`` nest."""
     out_nest = next((n for n in nests if n.writes() is keep), None)
-    if out_nest is None or not isinstance(out_nest.stmt, ir.Assign) or not isinstance(out_nest.stmt.value, ir.Dot):
+    if out_nest is None or not isinstance(out_nest.stmt, ir.Assign):
+        raise PassError("the result is not written by an element-wise nest")
+    val, epilogue = out_nest.stmt.value, None
+    if isinstance(val, ir.Bin) and val.op == "add":
+        # result = contraction + tensor: the tensor is added once per element after the normalisation
+        for d, t in ((val.a, val.b), (val.b, val.a)):
+            if isinstance(d, ir.Dot) and isinstance(t, ir.Read):
+                val, epilogue = d, t
+                break
+    if not isinstance(val, ir.Dot):
         raise PassError("the result is not a contraction")
-    dot = out_nest.stmt.value
+    dot = val
     p, v = dot.a, dot.b
-    # p = exp(x - m[r]) / l[r]
-    if not (isinstance(p, ir.Bin) and p.op == "div" and isinstance(p.b, ir.Read)):
+    # p = e(x - m[r]) / (l[r] + c...)
+    if not (isinstance(p, ir.Bin) and p.op == "div"):
         raise PassError("left operand of the contraction is not a normalised value")
-    e, l_read = p.a, p.b
-    if not (isinstance(e, ir.Un) and e.op == "exp" and isinstance(e.a, ir.Bin) and e.a.op == "sub" and isinstance(e.a.b, ir.Read)):
+    e, den = p.a, p.b
+    den_terms: list = []
+    _terms(den, 1, den_terms)
+    l_reads = [t for sg, t in den_terms if isinstance(t, ir.Read)]
+    extra = [t for sg, t in den_terms if not isinstance(t, ir.Read)]
+    if len(l_reads) != 1 or any(sg < 0 for sg, _ in den_terms) or not all(isinstance(t, (ir.Const, ir.Scalar)) for t in extra):
+        raise PassError("the normaliser is not the row sum plus constants")
+    l_read = l_reads[0]
+    if not (isinstance(e, ir.Un) and e.op in ("exp", "exp2") and isinstance(e.a, ir.Bin) and e.a.op == "sub"
+            and isinstance(e.a.b, ir.Read)):
         raise PassError("numerator is not exp(x - m)")
     x, m_read = e.a.a, e.a.b
     if not isinstance(v, ir.Read):
@@ -218,7 +339,10 @@ def online_softmax(nests: list[Nest], keep: ir.Buffer) -> list[Nest]:
     # x may not depend on the statistics themselves
     if any(r.buf in (l_read.buf, m_read.buf) for r in ir.reads(x)):
         raise PassError("scores depend on their own statistics")
-    new = Nest(out_nest.name, out_nest.par, list(dot.over), ir.Rescaled(keep, x, v))
+    if epilogue is not None and any(r.buf in (l_read.buf, m_read.buf) for r in [epilogue]):
+        raise PassError("the added tensor is a row statistic")
+    new = Nest(out_nest.name, out_nest.par, list(dot.over),
+               ir.Rescaled(keep, x, v, base2=(e.op == "exp2"), denom_add=tuple(extra), epilogue=epilogue))
     return [n for n in nests if n not in (out_nest, l_nest, m_nest)] + [new]
 
 

@@ -24,9 +24,10 @@ def compile_graph(gm: torch.fx.GraphModule, bm: int = 128, bn: int = 64) -> Comp
     try:
         p = build.parse(gm)
         before = ir.show(p.nests)
-        nests = passes.fuse(p.nests, p.out.buf)
+        nests = passes.fuse(p.nests, p.out.buf, keep_operands=True)
+        nests = passes.simplify(nests)
         nests = passes.online_softmax(nests, p.out.buf)
-        nests = passes.fuse(nests, p.out.buf)
+        nests = passes.fuse(nests, p.out.buf, keep_operands=True)
         nests = passes.block_skip(nests, bm, bn)
         att = derive.attention(nests, p.inputs, p.out)
     except (build.Unsupported, passes.PassError, ValueError) as e:

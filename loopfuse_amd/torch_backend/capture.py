@@ -418,8 +418,11 @@ class AttentionMatch:
             grp = q.shape[1] // max(kd.shape[1], 1)
             if q.shape[1] % max(kd.shape[1], 1) == 0 and grp % 2 == 0:
                 pack = 4 if grp % 4 == 0 else 2
+        bn = 0
+        if family == "prefill_swp":       # the tile shape the launch would take for a grid of this size
+            bn = lowering.prefill_kv_tile(D, bias, None, B * (Hq // (pack or 1)) * (-(-Sq // (128 // (pack or 1)))))
         return [lowering.KernelSpec(family, dt, D, mask, plan.softcap is not None, paged, ps, i64, bias=bias, d2=d2,
-                                    page_size_v=psv, pack=pack, extra=extra,
+                                    page_size_v=psv, pack=pack, extra=extra, bn=bn,
                                     safe=plan.zero_blind_rows and bool(bias & 1) and family == "prefill")]
 
 

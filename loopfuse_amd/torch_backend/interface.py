@@ -54,12 +54,13 @@ stats = {"fused": 0, "eager_graph": 0, "eager_runtime": 0, "eager_training": 0, 
 
 
 def _frontend() -> str:
-    """Which front end turns the graph into fused calls: "match" (default) = the sub-graph
-    matcher of capture.py; "ir" = the loop-nest front end (loopfuse_amd/compiler: per-op nests,
-    fusion, online-softmax and block-skip passes, plan read off the fused nest), with the matcher
-    as fallback for graphs it does not cover; "check" = the matcher, cross-checked against the
-    loop-nest front end wherever that derives a plan."""
-    return os.environ.get("LOOPFUSE_FRONTEND", "match")
+    """Which front end turns the graph into fused calls: "ir" (default) = the loop-nest front end
+    (loopfuse_amd/compiler: per-op nests, fusion, online-softmax and block-skip passes, plan read
+    off the fused nest), with the sub-graph matcher of capture.py as fallback for graphs it does not
+    cover (an attention inside a larger graph, several attentions, torch's fused attention ops, mask
+    tensors); "match" = the matcher alone; "check" = the matcher, cross-checked against the loop-nest
+    front end wherever that derives a plan."""
+    return os.environ.get("LOOPFUSE_FRONTEND", "ir")
 
 
 def match_from_nests(gm: torch.fx.GraphModule, comp: "compiler.pipeline.Compiled") -> capture.AttentionMatch:
@@ -68,20 +69,82 @@ def match_from_nests(gm: torch.fx.GraphModule, comp: "compiler.pipeline.Compiled
     placeholders = [n for n in gm.graph.nodes if n.op == "placeholder"]
     out_node = next(n for n in gm.graph.nodes if n.op == "output").args[0]
     out_node = out_node[0] if isinstance(out_node, (tuple, list)) else out_node
+    inputs = list(placeholders)
 
-    def operand(o) -> capture.Operand:
-        return capture.Operand(o.placeholder, tuple(o.perm), o.paged, o.table, o.group)
+    def index_of(o) -> int:
+        """Position of an operand among the fused call's inputs: a placeholder, or a node of the graph
+        that keeps running (an operand computed from the inputs, such as Q + q_bias)."""
+        if o.node is None:
+            return o.placeholder
+        if o.node not in inputs:
+            inputs.append(o.node)
+        return inputs.index(o.node)
+
+    def operand(o):
+        return None if o is None else capture.Operand(index_of(o), tuple(o.perm), o.paged, o.table, o.group)
+
+    def added(bl):
+        return None if bl is None else capture.BiasOperand(index_of(bl), tuple(bl.dims))
 
     def factor(f):
         kind, x = f
         x = ("fn", x) if callable(x) else float(x)
         return ("recip", x) if kind == "div" else x
 
-    return capture.AttentionMatch(out_node=out_node, inputs=placeholders, q=operand(att.q), k=operand(att.k),
+    return capture.AttentionMatch(out_node=out_node, inputs=inputs, q=operand(att.q), k=operand(att.k),
                                   v=operand(att.v), factors=[factor(f) for f in att.pre],
                                   post_factors=[factor(f) for f in att.post], has_tanh=att.has_tanh,
                                   mask=att.mask, window=("fn", att.window) if callable(att.window) else att.window,
-                                  out_rank=4)
+                                  out_rank=4, bias=added(att.bias), out_bias=added(att.out_bias),
+                                  q2=operand(att.q2), k2=operand(att.k2),
+                                  denom_add=tuple(factor(f) for f in att.denom_add), base2=att.base2,
+                                  late_factors=tuple(factor(f) for f in att.late))
+
+
+def _differences(m: capture.AttentionMatch, d: capture.AttentionMatch) -> str:
+    """What two descriptions of one attention disagree on ("" = nothing): mask, window, cap, the number
+    and the static values of the factors, operand sources / layouts / paging / head grouping, added
+    tensors, second product, denominator terms and exponent base.  (LOOPFUSE_FRONTEND=check.)"""
+    def static(fs):
+        """(product of the factors known at trace time, number of the others)"""
+        known = [float(f) for f in fs if isinstance(f, (int, float))]
+        rec = [1.0 / float(f[1]) for f in fs if isinstance(f, tuple) and f[0] == "recip" and isinstance(f[1], (int, float))]
+        r = 1.0
+        for x in known + rec:
+            r *= x
+        return round(r, 9), len(fs) - len(known) - len(rec)
+
+    def op(o):
+        return None if o is None else (o.index, tuple(o.perm), o.paged, o.group)
+
+    def table(match, o):
+        return None if o is None or not o.paged else match.inputs[o.table_index].name
+
+    def src(match, o):
+        return None if o is None else match.inputs[o.index].name
+
+    def added(b):
+        return None if b is None else (tuple(b.dims), b.keep)
+
+    checks = [
+        ("mask", m.mask, d.mask), ("cap", m.has_tanh, d.has_tanh),
+        ("factors before the cap", static(m.factors), static(d.factors)),
+        ("factors behind the cap", static(m.post_factors), static(d.post_factors)),
+        ("denominator terms", sorted(float(t) for t in m.denom_add if isinstance(t, (int, float))),
+         sorted(float(t) for t in d.denom_add if isinstance(t, (int, float)))), ("exponent base", m.base2, d.base2),
+        ("score bias", added(m.bias), added(d.bias)), ("output bias", added(m.out_bias), added(d.out_bias)),
+    ]
+    if m.mask == "sliding" and isinstance(m.window, int) and isinstance(d.window, int):
+        checks.append(("window", m.window, d.window))
+    for name in ("q", "k", "v", "q2", "k2"):
+        om, od = getattr(m, name), getattr(d, name)
+        checks.append((f"{name} source", src(m, om), src(d, od)))
+        checks.append((f"{name} layout", op(om) and op(om)[1:], op(od) and op(od)[1:]))
+        checks.append((f"{name} page table", table(m, om), table(d, od)))
+    for name in ("bias", "out_bias"):
+        bm_, bd = getattr(m, name), getattr(d, name)
+        checks.append((f"{name} source", bm_ and m.inputs[bm_.index].name, bd and d.inputs[bd.index].name))
+    return "; ".join(f"{what}: {x!r} vs {y!r}" for what, x, y in checks if x != y)
 
 
 def _strict() -> bool:
@@ -306,6 +369,10 @@ def loopfuse_compiler(gm: torch.fx.GraphModule, sample_inputs, input_names: list
             log.info("loop-nest front end: %s", e)
             if DEBUG:
                 print(f"---- loopfuse_amd: loop-nest front end does not cover this graph ({e})")
+        except Exception as e:                     # a front-end bug must not take the graph down: the matcher gets it
+            log.warning("loop-nest front end failed on this graph (%s: %s); the sub-graph matcher takes it",
+                        type(e).__name__, e)
+            stats["match_errors"] += 1
         else:
             stats["derived_graphs"] += 1
             if DEBUG:
@@ -330,13 +397,11 @@ def loopfuse_compiler(gm: torch.fx.GraphModule, sample_inputs, input_names: list
         else:
             reason = ""
         if frontend == "check" and derived is not None:
-            a = derived.attention
-            same = (len(matches) == 1 and matches[0].mask == a.mask and matches[0].has_tanh == a.has_tanh
-                    and matches[0].k.paged == a.k.paged and matches[0].v.paged == a.v.paged
-                    and (a.mask != "sliding" or callable(a.window) or matches[0].window == a.window))
-            if not same:
-                raise AssertionError("loopfuse_amd: the two front ends disagree: matcher "
-                                     f"{[m.describe() for m in matches]} vs loop nests {a.describe()}")
+            d = match_from_nests(gm, derived)
+            why = "the matcher finds %d attentions" % len(matches) if len(matches) != 1 else _differences(matches[0], d)
+            if why:
+                raise AssertionError(f"loopfuse_amd: the two front ends disagree ({why}): matcher "
+                                     f"{[m.describe() for m in matches]} vs loop nests {d.describe()}")
     if not matches:
         if _strict():
             raise NotImplementedError(f"loopfuse_amd: no fused-attention pattern in the graph: {reason}")

@@ -23,12 +23,15 @@ def rand(shape, dtype=torch.bfloat16, seed=0):
     return torch.randn(shape, generator=g, dtype=torch.float32).to(dtype)
 
 
-def run_fused(fn, inputs, mode=None):
+def run_fused(fn, inputs, mode=None, derived=None):
+    """``derived``: True / False = the loop-nest front end must / cannot have produced the plan."""
     torch._dynamo.reset()
     before = dict(interface.stats)
     out = torch.compile(fn, backend=loopfuse_backend, dynamic=True, mode=mode)(*[t.to(DEV) for t in inputs])
     torch.cuda.synchronize()
     assert interface.stats["fused"] == before["fused"] + 1, "the fused HIP path was not taken"
+    if derived is not None:
+        assert interface.stats["derived_graphs"] == before["derived_graphs"] + int(derived)
     assert interface.stats["eager_graph"] == before["eager_graph"]
     assert interface.stats["eager_runtime"] == before["eager_runtime"]
     return out.float().cpu()
@@ -43,7 +46,7 @@ def test_standard_attn(S):
     Q, K, V = (rand((4, 8, S, 64), seed=s) for s in (1, 2, 3))
     torch._dynamo.mark_static(Q, 3)
     torch._dynamo.mark_dynamic(Q, 2)
-    got = run_fused(fn, (Q, K, V))
+    got = run_fused(fn, (Q, K, V), derived=True)
     assert (got - O.attention_reference(Q, K, V, mask="causal")).abs().max() <= TOL
 
 
@@ -57,7 +60,7 @@ def test_gqa_attn():
 
     Q = rand((4, 8, 1024, 64), seed=1)
     K, V = (rand((4, 4, 1024, 64), seed=s) for s in (2, 3))
-    got = run_fused(fn, (Q, K, V))
+    got = run_fused(fn, (Q, K, V), derived=True)
     assert (got - O.attention_reference(Q, K, V, mask="causal")).abs().max() <= TOL
 
 
@@ -72,7 +75,7 @@ def test_sliding_mask_softcap_gqa():
 
     Q = rand((2, 32, 1024, 128), seed=1)
     K, V = (rand((2, 8, 1024, 128), seed=s) for s in (2, 3))
-    got = run_fused(fn, (Q, K, V), mode="max-autotune")
+    got = run_fused(fn, (Q, K, V), mode="max-autotune", derived=True)
     want = O.attention_reference(Q, K, V, mask="sliding", window=256, softcap=30.0)
     assert (got - want).abs().max() <= TOL
 
@@ -88,7 +91,7 @@ def test_paged_attention_k_only():
     Kc = rand((n, H, D), seed=1)
     tab = torch.randint(0, n, (B, S), generator=torch.Generator().manual_seed(5), dtype=torch.int32)
     Q, V = rand((B, H, S, D), seed=2), rand((B, H, S, D), seed=3)
-    got = run_fused(fn, (Q, Kc, tab, V))
+    got = run_fused(fn, (Q, Kc, tab, V), derived=True)
     want = O.attention_reference(Q, Kc, V, mask="causal", k_table=tab)
     assert (got - want).abs().max() <= TOL
 
@@ -110,7 +113,7 @@ def test_paged_attention_gqa():
     Q, V = rand((B, Hq, S, D), seed=2), rand((B, Hk, S, D), seed=3)
     torch._dynamo.mark_static(Q, 3)
     torch._dynamo.mark_dynamic(Q, 2)
-    got = run_fused(fn, (Q, Kc, tab, V))
+    got = run_fused(fn, (Q, Kc, tab, V), derived=True)
     want = O.attention_reference(Q, Kc, V, mask="causal", k_table=tab)
     assert (got - want).abs().max() <= TOL
 
@@ -127,7 +130,7 @@ def test_modified_attn():
     sb, ob = rand((B, H, S, S), seed=5), rand((B, H, S, D), seed=6)
     torch._dynamo.mark_static(Q, 3)
     torch._dynamo.mark_dynamic(Q, 2)
-    got = run_fused(fn, (Q, K, V, qb, sb, ob))
+    got = run_fused(fn, (Q, K, V, qb, sb, ob), derived=True)
     # the graph adds the query bias in bf16 before the first product; so does the oracle input
     want = O.attention_reference(Q + qb, K, V, mask="causal", scale=3.5 * D ** -0.5, score_bias=sb, out_bias=ob)
     excess = ((got - want).abs() - 2.0 ** -8 * want.abs()).max()     # bf16 rounding of the shifted output
@@ -149,7 +152,7 @@ def test_broadcast_score_bias_gqa():
     pos = torch.arange(S)
     slopes = 2.0 ** -(torch.arange(1, Hq + 1).float())
     bias = (-(pos[:, None] - pos[None, :]).abs().float() * slopes[:, None, None]).to(torch.bfloat16)[None]
-    got = run_fused(fn, (Q, K, V, bias))
+    got = run_fused(fn, (Q, K, V, bias), derived=True)
     want = O.attention_reference(Q, K, V, mask="causal", score_bias=bias)
     assert (got - want).abs().max() <= TOL
 
@@ -172,7 +175,7 @@ def test_explicit_softmax_shifted_denominator():
     Q, K, V = (rand((2, 8, 700, 128), seed=s) for s in (1, 2, 3))
     torch._dynamo.mark_static(Q, 3)
     torch._dynamo.mark_dynamic(Q, 2)
-    got = run_fused(fn, (Q, K, V))
+    got = run_fused(fn, (Q, K, V), derived=True)
     assert (got - O.attention_reference(Q, K, V, mask="causal", denom_add=1.0)).abs().max() <= TOL
 
 
@@ -187,7 +190,7 @@ def test_prefix_attention_two_fused_calls():
     B, H, Sq, Sp, D = 3, 4, 320, 512, 128
     Q, Ks, Vs = (rand((B, H, Sq, D), seed=s) for s in (1, 2, 3))
     Kp, Vp = (rand((B, H, Sp, D), seed=s) for s in (4, 5))
-    got = run_fused(fn, (Q, Kp, Vp, Ks, Vs))
+    got = run_fused(fn, (Q, Kp, Vp, Ks, Vs), derived=False)       # two attentions in one graph: the matcher's
     assert len(interface.last_matches) == 2
     want = O.attention_reference(Q, Kp, Vp) + O.attention_reference(Q, Ks, Vs, mask="causal")
     assert (got - want).abs().max() <= 2 * TOL      # two bf16 results added in bf16
@@ -211,7 +214,7 @@ def test_mla_two_part_scores(shared_rope):
     torch._dynamo.mark_static(Qn, 3)
     torch._dynamo.mark_static(Qp, 3)
     torch._dynamo.mark_dynamic(Qn, 2)
-    got = run_fused(fn, (Qn, Qp, Kn, Kp, V))
+    got = run_fused(fn, (Qn, Qp, Kn, Kp, V), derived=True)
     want = O.attention_reference(Qn, Kn, V, mask="causal", scale=(D + Dp) ** -0.5, q2=Qp, k2=Kp)
     assert (got - want).abs().max() <= TOL
 

@@ -158,6 +158,102 @@ def test_derived_tile_ranges_are_bit_exact(mask, window, bm, bn):
             assert torch.equal(got, dense[qt]), (Sq, Sk, qt, b, e)
 
 
+# ---- the graphs the reference modifies its attention into (tests/test_accuracy.py:172-196,
+# tests/test_attention.py:95-151): added tensors, an operand computed in the graph, the explicit
+# exp2 softmax with its scan_max hint and a shifted denominator, two-part scores
+def _modified(Q, K, V, q_bias, scores_bias, out_bias):
+    QK = (Q + q_bias) @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+    QK = QK * 3.5 + scores_bias
+    return torch.softmax(torch.ops.loopfuse.causal_mask(QK), dim=-1) @ V + out_bias
+
+
+def _explicit(Q, K, V):
+    import math
+
+    def _softmax(X):
+        Xf = X.to(torch.float32)
+        Xf_scaled = Xf * 1 / math.log(2)
+        X_mik, X_mi = torch.ops.loopfuse.scan_max(Xf_scaled)
+        expX = torch.exp2(Xf_scaled - X_mik) * torch.exp2(X_mik - X_mi)
+        return expX / (torch.sum(expX, dim=-1, keepdim=True) + 1)
+    QK = Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)
+    return _softmax(torch.ops.loopfuse.causal_mask(QK)).to(Q.dtype) @ V
+
+
+def _mla(Q_nope, Q_pe, K_nope, K_pe, V):
+    qk = Q_nope @ K_nope.transpose(-2, -1) + Q_pe @ K_pe.expand(-1, Q_pe.shape[1], -1, -1).transpose(-2, -1)
+    qk *= (Q_nope.shape[-1] + Q_pe.shape[-1]) ** (-0.5)
+    return torch.softmax(torch.ops.loopfuse.causal_mask(qk), dim=-1) @ V
+
+
+def _bias_gqa(Q, K, V, bias):
+    g = Q.shape[1] // K.shape[1]
+    K, V = K.repeat_interleave(g, dim=1), V.repeat_interleave(g, dim=1)
+    QK = torch.tanh((Q @ K.transpose(-2, -1) * (Q.shape[-1] ** -0.5)) / 20.0) * 20.0 + bias
+    return torch.softmax(torch.ops.loopfuse.sliding_mask(QK, 17), dim=-1) @ V
+
+
+WIDER = {
+    "modified": (_modified, lambda: tuple(_r(2, 3, 40, 16, seed=s) for s in (1, 2, 3, 4)) + (_r(2, 3, 40, 40, seed=5), _r(2, 3, 40, 16, seed=6))),
+    "explicit": (_explicit, lambda: tuple(_r(2, 3, 40, 16, seed=s) for s in (1, 2, 3))),
+    "mla": (_mla, lambda: (_r(2, 4, 40, 16, seed=1), _r(2, 4, 40, 8, seed=2), _r(2, 4, 40, 16, seed=3), _r(2, 1, 40, 8, seed=4), _r(2, 4, 40, 16, seed=5))),
+    "bias_gqa": (_bias_gqa, lambda: (_r(2, 8, 40, 16, seed=1), _r(2, 2, 40, 16, seed=2), _r(2, 2, 40, 16, seed=3), _r(1, 8, 40, 40, seed=4))),
+}
+
+
+@pytest.mark.parametrize("name", list(WIDER))
+def test_modified_attentions_fall_out_of_the_same_passes(name):
+    """fuse -> simplify -> online softmax leave one rescaled nest (plus the nest of an operand the graph
+    computes from its inputs), which evaluates to what torch computes for the traced graph; the derived
+    plan and operands equal what the sub-graph matcher extracts independently."""
+    fn, make = WIDER[name]
+    gm, args, out = _aten_graph(fn, make())
+    comp = compiler.compile_graph(gm)
+    p = compiler.build.parse(gm)                                     # the pipeline's steps, once more, for the interpreter
+    nests = passes.fuse(p.nests, p.out.buf, keep_operands=True)
+    nests = passes.online_softmax(passes.simplify(nests), p.out.buf)
+    assert sum(isinstance(n.stmt, ir.Rescaled) for n in nests) == 1
+    assert len(nests) == (2 if name == "modified" else 1)
+    feeds = {b.name: args[b.placeholder] for b in p.inputs}
+    got = interp.Interpreter(feeds).run(nests, args)[p.out.buf.name]
+    assert (got - out.double().reshape(got.shape)).abs().max().item() <= 1e-5
+    att = comp.attention
+    assert (att.bias is not None) == (name in ("modified", "bias_gqa")) and (att.out_bias is not None) == (name == "modified")
+    assert (att.q2 is not None) == (name == "mla") and att.base2 == (name == "explicit") and len(att.denom_add) == (name == "explicit")
+    assert (att.q.node is not None) == (name == "modified")
+    # against the matcher
+    derived = interface.match_from_nests(gm, comp)
+    matched = capture.match_attention(gm)
+    assert len(matched) == 1
+    m = matched[0]
+    vals_d, vals_m = derived.input_values(gm, args), m.input_values(gm, args)
+    a, b = derived.plan_for(vals_d), m.plan_for(vals_m)
+    assert (a.mask, a.window, a.denom_add) == (b.mask, b.window, b.denom_add)
+    assert a.scale == pytest.approx(b.scale, rel=1e-6) and a.softcap == (pytest.approx(b.softcap) if b.softcap else None)
+    pairs = [(derived.q, m.q), (derived.k, m.k), (derived.v, m.v)]
+    if name == "mla":
+        pairs += [(derived.q2, m.q2), (derived.k2, m.k2)]
+    for od, om in pairs:
+        td, tm = derived._operand(od, vals_d)[0], m._operand(om, vals_m)[0]
+        assert td.shape == tm.shape and td.stride() == tm.stride() and torch.equal(td, tm)
+    B, Hq, Sq, Sk, D = derived._shapes(vals_d)
+    for bd, bm_, shape in ((derived.bias, m.bias, (B, Hq, Sq, Sk)), (derived.out_bias, m.out_bias, (B, Hq, Sq, D))):
+        assert (bd is None) == (bm_ is None)
+        if bd is not None:
+            assert torch.equal(derived._bias_view(bd, vals_d, shape), m._bias_view(bm_, vals_m, shape))
+
+
+def test_a_running_maximum_that_does_not_cancel_is_refused():
+    def fn(Q, K, V):
+        x = Q @ K.transpose(-2, -1)
+        run, mx = torch.ops.loopfuse.scan_max(x)
+        e = torch.exp2(x - run)                       # not the hint: the running maximum stays in the value
+        return (e / torch.sum(e, dim=-1, keepdim=True)) @ V
+    gm, _, _ = _aten_graph(fn, tuple(_r(1, 2, 8, 8, seed=s) for s in (1, 2, 3)))
+    with pytest.raises(compiler.NotDerivable, match="running maximum"):
+        compiler.compile_graph(gm)
+
+
 def test_graphs_that_are_not_one_attention_are_refused():
     for fn, ins in ((lambda a, b: a + b, (_r(4, 8), _r(4, 8))),
                     (lambda x, y: torch.softmax(x, dim=-1) @ y, (_r(2, 4, 8, 8), _r(2, 4, 8, 16))),
