@@ -556,7 +556,23 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan,
         raise UnsupportedPlan("Q must be [B, Hq, Sq, D]")
     B, Hq, Sq, D = q.shape
     if D not in (64, 128):
-        raise UnsupportedPlan(f"head dim {D} not supported (64, 128)")
+        # Other head dimensions up to 128 (the reference takes any static D, ops.py:370-397): dense operands
+        # are copied into zero-padded rows of 64 / 128 elements -- zeros add nothing to Q K^T, and the padded
+        # columns of V give output columns that are cut off again -- at O(S D) beside the O(S^2 D) attention.
+        Dp = 64 if D < 64 else 128
+        if D > 128 or D < 1 or plan.k_paged or plan.v_paged or lse is not None or q2 is not None or static_scratch \
+                or k.dim() != 4 or v.dim() != 4 or k.shape[-1] != D or v.shape[-1] != D:
+            raise UnsupportedPlan(f"head dim {D} not supported (64 and 128; up to 128 by padding for dense operands)")
+        grow = lambda t: None if t is None else torch.nn.functional.pad(t, (0, Dp - D))
+        res = attention(grow(q), grow(k), grow(v), plan, None, None, record_visits=record_visits, score_bias=score_bias,
+                        out_bias=grow(out_bias), force_family=force_family, num_splits=num_splits, v_tr=v_tr,
+                        choice=choice, merge_splits=merge_splits)
+        o_p, vis = res if record_visits else (res, None)
+        if out is None:
+            out = o_p[..., :D].contiguous()
+        else:
+            out.copy_(o_p[..., :D])
+        return (out, vis) if record_visits else out
     if not (plan.scale > 0.0) or not math.isfinite(plan.scale):
         raise UnsupportedPlan("score scale must be positive and finite")
     softcap = None

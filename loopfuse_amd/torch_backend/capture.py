@@ -378,8 +378,10 @@ class AttentionMatch:
         k = vals[self.k.index]
         D = q.shape[-1]
         dt = lowering._DTYPE_CODE.get(q.dtype)
-        if dt is None or D not in (64, 128):
+        if dt is None or D > 128 or (D not in (64, 128) and (self.k.paged or self.v.paged or self.q2 is not None)):
             raise lowering.UnsupportedPlan("dtype/head dim not served by the HIP kernels")
+        if D not in (64, 128):
+            D = 64 if D < 64 else 128          # dense operands of other head dims run zero-padded
         paged = (1 if self.k.paged else 0) | (2 if self.v.paged else 0)
         ps = 1
         i64 = False

@@ -103,6 +103,25 @@ def test_softcap_forms(dtype, q_scale):
                 check(q, k, v, mask=mask, window=window, softcap=cap, choice={"bn": bn}, force_family="prefill")
 
 
+@pytest.mark.parametrize("D", [40, 80, 96, 120])
+def test_other_head_dims_run_zero_padded(D):
+    """Head dims other than 64 / 128 (up to 128, dense operands): the rows are zero-padded to the next kernel
+    width, which changes neither Q K^T nor the kept columns of P V."""
+    q = rand((2, 4, 300, D), torch.bfloat16, 1)
+    k, v = (rand((2, 2, 300, D), torch.bfloat16, s) for s in (2, 3))
+    check(q, k, v, mask="causal")
+    check(q, k, v, mask="sliding", window=64, softcap=20.0)
+    check(rand((2, 4, 1, D), torch.float16, 4), k.half(), v.half())          # decode shape
+    out = torch.full((2, 4, 300, D), 7.0, dtype=torch.bfloat16, device=dev())
+    got = lowering.attention(q.to(dev()), k.to(dev()), v.to(dev()), lowering.AttnPlan(mask="causal", scale=D ** -0.5), out=out)
+    assert got is out and (out.float().cpu() - O.attention_reference(q, k, v, mask="causal")).abs().max().item() <= 2e-2
+    pool = rand((40, 16, 2, D), torch.bfloat16, 5)
+    table = torch.arange(40, dtype=torch.int32).view(2, 20)
+    with pytest.raises(lowering.UnsupportedPlan):
+        lowering.attention(q.to(dev()), pool.to(dev()), pool.to(dev()), lowering.AttnPlan(scale=0.1, k_paged=True, v_paged=True),
+                           table.to(dev()), table.to(dev()))
+
+
 @pytest.mark.parametrize("v_tr", [True, False])
 def test_causal_prefill_v_read_paths(v_tr):
     q, k, v = (rand((1, 2, 320, 128), torch.bfloat16, s) for s in (1, 2, 3))
