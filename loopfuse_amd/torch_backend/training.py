@@ -20,7 +20,7 @@ log = logging.getLogger("loopfuse_amd")
 
 _MASK_CODE = {None: 0, "none": 0, "causal": 1, "sliding": 2}
 _MASK_NAME = {0: None, 1: "causal", 2: "sliding"}
-counters = {"fwd": 0, "bwd": 0}
+counters = {"fwd": 0, "bwd": 0, "repacked": 0}
 
 
 def _rows(t: torch.Tensor) -> torch.Tensor:
@@ -41,7 +41,13 @@ def attention_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: int, 
     lse = torch.empty(q.shape[:-1], dtype=torch.float32, device=q.device)
     counters["fwd"] += 1
     # the log-sum-exp is written by the direct-to-LDS kernel only: ask for it whatever LOOPFUSE_PREFILL says
-    return lowering.attention(_rows(q), _rows(k), _rows(v), plan, lse=lse, choice={"prefill": "swp"}), lse
+    try:
+        return lowering.attention(_rows(q), _rows(k), _rows(v), plan, lse=lse, choice={"prefill": "swp"}), lse
+    except lowering.UnsupportedPlan:
+        # views whose rows lie beyond the direct loads' 32-bit reach: packed copies are always within it
+        counters["repacked"] += 1
+        return lowering.attention(q.contiguous(), k.contiguous(), v.contiguous(), plan, lse=lse,
+                                  choice={"prefill": "swp"}), lse
 
 
 @attention_fwd.register_fake
@@ -58,7 +64,12 @@ def attention_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Te
     plan = lowering.AttnPlan(mask=_MASK_NAME[mask], window=int(window), scale=float(scale),
                              softcap=float(softcap) if softcap else None)
     counters["bwd"] += 1
-    return lowering.attention_backward(_rows(q), _rows(k), _rows(v), _rows(o), lse.contiguous(), _rows(dout), plan)
+    try:
+        return lowering.attention_backward(_rows(q), _rows(k), _rows(v), _rows(o), lse.contiguous(), _rows(dout), plan)
+    except lowering.UnsupportedPlan:
+        counters["repacked"] += 1
+        return lowering.attention_backward(q.contiguous(), k.contiguous(), v.contiguous(), o.contiguous(),
+                                           lse.contiguous(), dout.contiguous(), plan)
 
 
 @attention_bwd.register_fake

@@ -168,6 +168,33 @@ def test_backward_is_reproducible_and_refuses_what_it_does_not_serve():
         lowering.attention_backward(q, k, v, o, lse, dout, lowering.AttnPlan(mask="causal", scale=0.1, softcap=0.0))
 
 
+def test_training_ops_repack_views_beyond_the_direct_loads_reach():
+    """K rows 4 MiB apart (a view into a 4 GiB tensor) lie beyond the 32-bit offsets of the direct-to-LDS loads:
+    the operator refuses them, and the custom ops of a training graph go through packed copies instead of
+    aborting -- same values as on packed operands."""
+    from loopfuse_amd.torch_backend import training
+
+    S, D, R = 1025, 128, 1 << 21
+    g = torch.Generator().manual_seed(9)
+    q, k, v, dout = (torch.randn((1, 1, S, D), generator=g).to(torch.bfloat16).to(DEV) for _ in range(4))
+    wide = torch.empty((1, 1, S, R), dtype=torch.bfloat16, device=DEV)
+    wide[..., :D] = k
+    k_view = wide[..., :D]
+    plan = lowering.AttnPlan(mask="causal", scale=D ** -0.5)
+    lse = torch.empty((1, 1, S), dtype=torch.float32, device=DEV)
+    with pytest.raises(lowering.UnsupportedPlan):
+        lowering.attention(q, k_view, v, plan, lse=lse, choice={"prefill": "swp"})
+    before = training.counters["repacked"]
+    o1, lse1 = torch.ops.loopfuse_amd.attention_fwd(q, k_view, v, 1, 0, D ** -0.5, 0.0)
+    o2, lse2 = torch.ops.loopfuse_amd.attention_fwd(q, k, v, 1, 0, D ** -0.5, 0.0)
+    assert torch.equal(o1, o2) and torch.equal(lse1, lse2)
+    g1 = torch.ops.loopfuse_amd.attention_bwd(q, k_view, v, o1, lse1, dout, 1, 0, D ** -0.5, 0.0)
+    g2 = torch.ops.loopfuse_amd.attention_bwd(q, k, v, o2, lse2, dout, 1, 0, D ** -0.5, 0.0)
+    assert all(torch.equal(a, b) for a, b in zip(g1, g2))
+    assert training.counters["repacked"] == before + 2
+    del wide
+
+
 # ---- through torch.compile(backend=loopfuse_backend): graphs traced for training
 def _train_case(name):
     from loopfuse_amd import workloads  # noqa: F401

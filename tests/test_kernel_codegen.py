@@ -8,7 +8,9 @@ to one register file, the live ranges fit), and this test holds the generated co
 compiled as the library compiles them (hipRTC, no GPU needed), disassembled, and checked for
   * no scratch-memory access at all (no spills),
   * every read of an MFMA's AGPR result by a non-MFMA instruction at least MIN_GAP
-    instructions behind the MFMA that wrote it, or behind an explicit drain (s_nop >= 9).
+    instructions behind the MFMA that wrote it, or behind an explicit drain (s_nop >= 9),
+  * no instruction other than the chain's own MFMAs touching the VGPR destination of an MFMA
+    between that MFMA and the drain behind its chain.
 """
 import os
 import re
@@ -63,6 +65,27 @@ def _check(name, lines):
         drained = any(re.match(r"s_nop (\d+)", x) and int(re.match(r"s_nop (\d+)", x).group(1)) >= 9 for x in between)
         assert drained or len(between) >= MIN_GAP, \
             f"{name}: '{ln}' reads a{reg} {len(between)} instructions behind the MFMA that writes it ('{lines[j]}')"
+    if not mfma_dst:
+        return          # MFMAs issued through the builtin only: the compiler places their wait states itself
+    # MFMAs with a VGPR destination (S^T / dP^T): until the drain behind the chain -- or MIN_GAP instructions --
+    # nothing but the chain's own MFMAs may touch the destination registers (a copy or a live-range split the
+    # compiler placed there would read or overwrite an accumulator that is not written yet)
+    for j, ln in enumerate(lines):
+        m = re.match(r"v_mfma_\S+ v\[(\d+):(\d+)\]", ln)
+        if not m:
+            continue
+        lo, hi = int(m.group(1)), int(m.group(2))
+        for gap, x in enumerate(lines[j + 1:j + 1 + MIN_GAP]):
+            nop = re.match(r"s_nop (\d+)", x)
+            if nop and int(nop.group(1)) >= 9:
+                break
+            if x.startswith("v_mfma"):
+                continue
+            regs = {int(r) for r in re.findall(r"\bv(\d+)\b", x)}
+            for a, b in re.findall(r"\bv\[(\d+):(\d+)\]", x):
+                regs.update(range(int(a), int(b) + 1))
+            hit = sorted(r for r in regs if lo <= r <= hi)
+            assert not hit, f"{name}: '{x}' touches v{hit[0]} {gap} instructions behind '{ln}', before its drain"
 
 
 SPECS = [
@@ -95,3 +118,12 @@ def test_the_check_sees_an_early_read():
     _check("probe", lines[:1] + ["v_mov_b32_e32 v0, v0"] * MIN_GAP + lines[2:])
     with pytest.raises(AssertionError):
         _check("probe", lines[:2] + ["scratch_load_dword v1, off, s0"])
+    # a VGPR-destination MFMA of such a kernel: a copy of its accumulator before the drain is seen, one behind it is not
+    chain = ["v_mfma_f32_32x32x16_bf16 a[0:15], v[0:3], v[4:7], a[0:15]",
+             "v_mfma_f32_32x32x16_bf16 v[16:31], v[0:3], a[16:19], 0",
+             "v_mfma_f32_32x32x16_bf16 v[16:31], v[4:7], a[20:23], v[16:31]"]
+    with pytest.raises(AssertionError):
+        _check("probe", chain + ["v_mov_b32_e32 v40, v17", "s_nop 9", "s_nop 9"])
+    with pytest.raises(AssertionError):
+        _check("probe", chain + ["global_load_dwordx4 v[28:31], v[0:1], off", "s_nop 9", "s_nop 9"])
+    _check("probe", chain + ["v_add_u32_e32 v1, v2, v3", "s_nop 9", "s_nop 9", "v_mov_b32_e32 v40, v17"])
