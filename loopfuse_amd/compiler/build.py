@@ -177,7 +177,7 @@ class Parser:
         if t is aten._softmax.default and len(a) > 2 and a[2]:
             raise Unsupported("_softmax with half_to_float")
         if Parser._VIEW_OPS is None:
-            Parser._VIEW_OPS = {aten.transpose.int, aten.permute.default, aten.unsqueeze.default, aten.clone.default,
+            Parser._VIEW_OPS = {aten.transpose.int, aten.t.default, aten.permute.default, aten.unsqueeze.default, aten.clone.default,
                                 aten.alias.default, aten.expand.default, aten.view.default, aten._unsafe_view.default,
                                 aten.reshape.default, aten.sym_size.int}
         if t in Parser._VIEW_OPS:
@@ -236,6 +236,11 @@ class Parser:
             dims = list(v.dims)
             dims[d0], dims[d1] = dims[d1], dims[d0]
             return dataclasses.replace(v, dims=dims)
+        if t is aten.t.default:
+            v = val(a[0])
+            if len(v.dims) > 2:
+                raise Unsupported("t() of a tensor with more than two dims")
+            return dataclasses.replace(v, dims=list(reversed(v.dims)))
         if t is aten.permute.default:
             v = val(a[0])
             return dataclasses.replace(v, dims=[v.dims[p % len(v.dims)] for p in a[1]])

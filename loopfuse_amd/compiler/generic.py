@@ -10,7 +10,7 @@ from typing import Sequence
 
 import torch
 
-from . import build, emit, ir, passes
+from . import build, emit, emit_gemm, ir, passes
 from .emit import NotLowerable
 
 
@@ -21,6 +21,8 @@ from .emit import NotLowerable
 # beyond this many inner-loop steps per call (all reducing nests together; 512 x 512 x 512 multiply-adds)
 # the graph is left to the captured ATen ops.
 MAX_SCALAR_WORK = 1 << 27
+
+counters = {"mfma": 0, "plain": 0}      # kernel launches by kind (tests read them)
 
 
 class GenericProgram:
@@ -49,20 +51,55 @@ class GenericProgram:
         self.dtypes[p.out.buf.name] = emit._DT.get(self.out_dtype, 0)
         self.kernels = [emit.Emitter(n, self.dtypes, f"lf_gen_{i}").emit() for i, n in enumerate(nests)]
         self.source = emit.PRELUDE + "\n".join(k.source for k in self.kernels)
+        # contractions of bf16 / fp16 operands also get an MFMA kernel with the nest's epilogue fused; the plain
+        # kernel of the same nest serves the calls whose strides or extents it cannot take
+        self.gemm: dict = {}
+        for i, n in enumerate(nests):
+            info = emit_gemm.match(n, self.dtypes)
+            if info is not None:
+                try:
+                    self.gemm[i] = (emit_gemm.GemmEmitter(n, self.dtypes, f"lf_gen_{i}_mfma", info).emit(), info)
+                except NotLowerable:
+                    pass
+        self.gpu_source = self.source
+        if self.gemm:
+            self.gpu_source = emit.PRELUDE + emit_gemm.GEMM_PRELUDE + "\n".join(
+                [k.source for k in self.kernels] + [k.source for k, _ in self.gemm.values()])
         self._loaded: dict = {}
 
     @property
     def code(self) -> str:
-        return self.source
+        return self.gpu_source
 
     def _module(self):
         from .. import lowering, runtime
         dev = torch.cuda.current_device()
         if dev not in self._loaded:
-            code, _, _ = runtime.compile_source(self.source, "lf_generic", list(lowering.COMMON_OPTS))
+            code, _, _ = runtime.compile_source(self.gpu_source, "lf_generic", list(lowering.COMMON_OPTS))
             mod = runtime.Module(code)
-            self._loaded[dev] = [mod.kernel(k.name) for k in self.kernels]
+            self._loaded[dev] = ([mod.kernel(k.name) for k in self.kernels],
+                                 {i: mod.kernel(k.name) for i, (k, _) in self.gemm.items()})
         return self._loaded[dev]
+
+    @staticmethod
+    def _gemm_layouts(info, bufs: dict, ext: dict):
+        """(A is k-contiguous, B is k-contiguous) when the MFMA kernel can read both operands of this call with
+        16-byte pieces, else None."""
+        M, N, K = ext[info.m.id], ext[info.n.id], ext[info.k.id]
+        flags = []
+        for buf, (d_outer, d_k), batch_dims, outer in ((info.a_buf, info.a_dims, info.a_batch_dims, M),
+                                                      (info.b_buf, info.b_dims, info.b_batch_dims, N)):
+            t = bufs[buf.name]
+            if t.data_ptr() % 16 or any(t.stride(d) % 8 for d in batch_dims if t.shape[d] > 1):
+                return None
+            s_outer, s_k = t.stride(d_outer), t.stride(d_k)
+            if (s_k == 1 or K == 1) and K % 8 == 0 and (s_outer % 8 == 0 or outer == 1):
+                flags.append(1)
+            elif (s_outer == 1 or outer == 1) and outer % 8 == 0 and (s_k % 8 == 0 or K == 1):
+                flags.append(0)
+            else:
+                return None
+        return flags
 
     def _solve(self, nest: ir.Nest, bufs: dict, known: dict, syms: dict) -> None:
         """Run-time extent of every leaf atom of ``nest`` into ``known``: each dimension of a
@@ -114,13 +151,15 @@ class GenericProgram:
         if launchers is None:
             if dev.type != "cuda":
                 raise NotLowerable("tensors are not on the GPU")
-            kernels = self._module()
+            kernels, mfma = self._module()
             launchers = [lambda blocks, prm, fn=fn: fn.launch((blocks, 1, 1), (256, 1, 1), prm) for fn in kernels]
+        else:
+            mfma = {}
         ext: dict = {}
         syms: dict = {name: int(args[i]) for name, i in self.parsed.sizes.items()}
         work = 0
         bufs: dict = {b.name: args[b.placeholder] for b in self.parsed.inputs}
-        for nest, k, fn in zip(self.nests, self.kernels, launchers):
+        for ni, (nest, k, fn) in enumerate(zip(self.nests, self.kernels, launchers)):
             out = nest.writes()
             self._solve(nest, bufs, ext, syms)
             try:
@@ -129,6 +168,15 @@ class GenericProgram:
                 raise NotLowerable("an extent could not be derived from the argument shapes") from e
             dt = self.out_dtype if out is self.parsed.out.buf else torch.float32
             bufs[out.name] = torch.empty(shape, dtype=dt, device=dev)
+            if ni in mfma:
+                try:
+                    layouts = self._gemm_layouts(self.gemm[ni][1], bufs, ext)
+                except KeyError:
+                    layouts = None
+                if layouts is not None and all(ext.get(a.id, 0) > 0 for a in self.gemm[ni][0].atoms):
+                    self._launch_gemm(mfma[ni], *self.gemm[ni], layouts, bufs, ext, args)
+                    counters["mfma"] += 1
+                    continue
             prm = emit.GenParams()
             for i, b in enumerate(k.bufs):
                 prm.ptr[i] = bufs[b.name].data_ptr()
@@ -148,6 +196,26 @@ class GenericProgram:
                 if (total + 255) // 256 >= 1 << 31:
                     raise NotLowerable("more output elements than one grid dimension holds")
                 fn((total + 255) // 256, prm)
+                counters["plain"] += 1
         res = bufs[self.parsed.out.buf.name]
         view = [math.prod(1 if a.hint == 1 else ext[a.id] for a in ir.leaves(d)) for d in self.parsed.out.dims]
         return res.view(view)
+
+    @staticmethod
+    def _launch_gemm(fn, k, info, layouts, bufs: dict, ext: dict, args) -> None:
+        prm = emit.GenParams()
+        for i, b in enumerate(k.bufs):
+            prm.ptr[i] = bufs[b.name].data_ptr()
+        for i, a in enumerate(k.atoms):
+            prm.n[i] = ext[a.id]
+        for i, (b, d) in enumerate(k.strides):
+            prm.n[len(k.atoms) + i] = bufs[b.name].stride(d)
+        prm.n[info.flags_at], prm.n[info.flags_at + 1] = layouts
+        for i, s in enumerate(k.scalars):
+            prm.f[i] = float(s.fn(args))
+        tiles = -(-ext[info.m.id] // emit_gemm.BM) * -(-ext[info.n.id] // emit_gemm.BN) * \
+            math.prod(ext[a.id] for a in info.batch)
+        blocks = 8 * -(-tiles // 8)
+        if blocks >= 1 << 31:
+            raise NotLowerable("more tiles than one grid dimension holds")
+        fn.launch((blocks, 1, 1), (256, 1, 1), prm)

@@ -1,0 +1,116 @@
+"""Contractions in graphs without an attention on the MFMA path (``compiler/emit_gemm.py``): the
+reference emits ``tl.dot`` for every contraction (``loopfuse/codegen.py:658-668``) and checks
+``a @ b + c`` in two and three dims (``tests/test_accuracy.py:56-82``).  Expected values are float64
+einsums on the CPU; the tolerance is the output format's rounding (2^-8 relative for bf16, 2^-11 for
+fp16) plus the fp32 accumulation of K products of rounded operands."""
+import pytest
+import torch
+
+import loopfuse_amd  # noqa: F401
+from loopfuse_amd import loopfuse_backend
+from loopfuse_amd.compiler import generic
+from loopfuse_amd.torch_backend import interface
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+BF, HF = torch.bfloat16, torch.float16
+
+
+def rand(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+def _close(got, want, dtype):
+    rel = 2.0 ** -8 if dtype == BF else 2.0 ** -11
+    err = (got.double().cpu() - want).abs()
+    budget = rel * want.abs() + 2e-3 * max(1.0, want.abs().max().item()) * (1.0 if dtype == BF else 0.25)
+    assert torch.isfinite(got).all()
+    assert (err <= budget).all(), f"max excess {(err - budget).max().item()}"
+
+
+def _compiled(fn):
+    torch._dynamo.reset()
+    return torch.compile(fn, backend=loopfuse_backend, dynamic=True)
+
+
+CASES = [
+    # name, shapes of a, b (as stored), how the graph views them, epilogue operand shape
+    ("ref_2dim", (1024, 64), (64, 128), "ab", (1024, 128)),            # reference tests/test_accuracy.py:56-64
+    ("ref_3dim", (4, 1024, 64), (4, 64, 128), "ab", (4, 1024, 128)),   # reference tests/test_accuracy.py:69-82
+    ("b_transposed", (300, 72), (136, 72), "abT", (300, 136)),         # B stored [N, K]: k-contiguous on both sides
+    ("a_transposed", (200, 264), (200, 96), "aTb", (264, 96)),         # A stored [K, M]: transposed reads on both sides
+    ("both_transposed", (64, 520), (40, 64), "aTbT", (520, 40)),
+    ("ragged_rows", (777, 128), (128, 200), "ab", (777, 200)),         # M odd (A k-contiguous), N a multiple of 8 only
+    ("odd_n_b_kcontig", (130, 64), (77, 64), "abT", (130, 77)),        # N odd with B k-contiguous
+    ("long_k", (256, 4096), (4096, 256), "ab", (256, 256)),
+    ("batch_broadcast_b", (3, 2, 160, 64), (64, 96), "ab", (96,)),     # B shared by every batch element; bias over n
+    ("tiny", (8, 8), (8, 8), "ab", (8, 8)),
+]
+
+
+@pytest.mark.parametrize("dtype", [BF, HF])
+@pytest.mark.parametrize("name,sa,sb,form,sc", CASES, ids=[c[0] for c in CASES])
+def test_matmul_with_epilogue_runs_on_mfma(name, sa, sb, form, sc, dtype):
+    a, b, c = rand(sa, dtype, 1, 0.5), rand(sb, dtype, 2, 0.5), rand(sc, dtype, 3)
+    va = (lambda t: t.transpose(-1, -2)) if form.startswith("aT") else (lambda t: t)
+    vb = (lambda t: t.transpose(-1, -2)) if form.endswith("bT") else (lambda t: t)
+    fn = lambda a, b, c: (va(a) @ vb(b)) * 0.25 + c           # noqa: E731
+    ins = [t.to(DEV) for t in (a, b, c)]
+    before, stats = dict(generic.counters), dict(interface.stats)
+    got = _compiled(fn)(*ins)
+    assert interface.stats["fused_generic"] == stats["fused_generic"] + 1
+    assert generic.counters["mfma"] == before["mfma"] + 1 and generic.counters["plain"] == before["plain"]
+    want = torch.matmul(va(a.double()), vb(b.double())) * 0.25 + c.double()
+    assert got.dtype == dtype and tuple(got.shape) == tuple(want.shape)
+    _close(got, want, dtype)
+
+
+def test_calls_the_mfma_kernel_cannot_read_take_the_plain_kernel():
+    """k not a multiple of 8, a misaligned base, an operand stride that is not a multiple of 8: same program, the
+    one-thread-per-element kernel of the nest serves the call."""
+    fn = lambda a, b, c: a @ b + c        # noqa: E731
+    a, b, c = rand((64, 32), BF, 1).to(DEV), rand((32, 48), BF, 2).to(DEV), rand((64, 48), BF, 3).to(DEV)
+    run = _compiled(fn)
+    cases = [
+        (rand((64, 20), BF, 4).to(DEV), rand((20, 48), BF, 5).to(DEV), c),                     # K = 20
+        (rand((64, 33), BF, 6).to(DEV)[:, 1:], b, c),                                          # base 2 bytes off, row stride 33
+        (a, rand((32, 52), BF, 7).to(DEV)[:, :48], c),                                         # row stride 52
+    ]
+    for x, y, z in cases:
+        before = dict(generic.counters)
+        got = run(x, y, z)
+        assert generic.counters["mfma"] == before["mfma"] and generic.counters["plain"] == before["plain"] + 1
+        _close(got, x.double().cpu() @ y.double().cpu() + z.double().cpu(), BF)
+    before = dict(generic.counters)
+    _close(run(a, b, c), a.double().cpu() @ b.double().cpu() + c.double().cpu(), BF)
+    assert generic.counters["mfma"] == before["mfma"] + 1
+
+
+def test_large_matmul_is_no_longer_left_to_the_captured_graph():
+    """2048 x 2048 x 2048 is 2^33 multiply-adds, far beyond what the plain kernels are allowed: on the MFMA path the
+    backend keeps the graph (counted as a generated-kernel run), a tanh epilogue and a bias over n fused."""
+    fn = lambda a, b, bias: torch.tanh(a @ b.t() * 0.02 + bias)      # noqa: E731
+    a, b, bias = rand((2048, 2048), BF, 1), rand((2048, 2048), BF, 2), rand((2048,), BF, 3)
+    torch._dynamo.reset()
+    before, kinds = dict(interface.stats), dict(generic.counters)
+    got = torch.compile(fn, backend=loopfuse_backend)(a.to(DEV), b.to(DEV), bias.to(DEV))
+    assert interface.stats["fused_generic"] == before["fused_generic"] + 1
+    assert interface.stats["eager_runtime"] == before["eager_runtime"]
+    assert generic.counters["mfma"] == kinds["mfma"] + 1 and generic.counters["plain"] == kinds["plain"]
+    want = torch.tanh(a.double() @ b.double().t() * 0.02 + bias.double())
+    _close(got, want, BF)
+
+
+def test_two_products_in_a_row_keep_the_intermediate_and_both_run_on_mfma():
+    """(a @ b) @ c (reference tests/test_accuracy.py:85-100, commented out there): the first product stays a
+    temporary -- fp32, so the second contraction reads it through the plain kernel unless it is small; here only
+    the first runs on MFMA and the result still matches."""
+    fn = lambda a, b, c: (a @ b) @ c      # noqa: E731
+    a, b, c = rand((256, 64), BF, 1, 0.3), rand((64, 128), BF, 2, 0.3), rand((128, 64), BF, 3, 0.3)
+    ins = [t.to(DEV) for t in (a, b, c)]
+    before = dict(generic.counters)
+    got = _compiled(fn)(*ins)
+    assert generic.counters["mfma"] + generic.counters["plain"] == before["mfma"] + before["plain"] + 2
+    assert generic.counters["mfma"] >= before["mfma"] + 1
+    _close(got, (a.double() @ b.double()) @ c.double(), BF)
