@@ -3,18 +3,20 @@
 cases ``tests/test_accuracy.py:56-82``: ``a @ b + c`` in two and three dims).
 
 A nest ``out[batch.., m, n] = f(sum_k A[batch.., m, k] * B[batch.., k, n], other reads)`` with bf16 /
-fp16 operands becomes one kernel: a workgroup of four waves owns a 128 x 128 tile of the output and walks
-k in steps of 64; both operand tiles go global -> registers -> LDS (16-byte pieces, XOR-swizzled,
-double-buffered, one barrier per step) and come back as ``v_mfma_f32_32x32x16`` operands -- by plain
-16-byte reads where k is the contiguous dimension of the operand in memory, by transposed reads
-(``ds_read_b64_tr_b16``) where m / n is.  The product is formed transposed (C^T = B^T A^T), so a lane
-ends up with four consecutive n of one m: the epilogue expression -- whatever the fused nest holds
-around the contraction -- is evaluated per element on the fp32 accumulators and stored from there.
+fp16 operands becomes one kernel: a workgroup of four waves owns a 128 x 128 tile of the output (64 x 64
+per wave, four accumulators) and walks k in steps of 64; both operand tiles go global -> registers -> LDS
+(16-byte pieces, XOR-swizzled, double-buffered, one barrier per step) and come back as
+``v_mfma_f32_32x32x16`` operands -- by plain 16-byte reads where k is the contiguous dimension of the
+operand in memory, by transposed reads (``ds_read_b64_tr_b16``) where m / n is.  The product is formed
+transposed (C^T = B^T A^T); the fp32 accumulators then pass through LDS once so that a lane holds four
+consecutive n of one m and neighbouring lanes neighbouring n: the epilogue expression -- whatever the
+fused nest holds around the contraction -- is evaluated there per element, its reads coalesced, and the
+results leave in 8- or 16-byte stores along the rows of the output.
 
-Which of the two layouts an operand has is decided per call from its strides (a flag in the
-parameter block, uniform over the launch).  Calls the kernel cannot serve (strides that are not
-multiples of 8 elements, k or the contiguous extent not a multiple of 8, unaligned bases) take the
-plain one-thread-per-element kernel of the same nest.
+Which of the two layouts an operand has is a compile-time flag of the kernel (``-DLFG_A_ROWS``,
+``-DLFG_B_ROWS``); the launcher picks the code object per call from the strides.  Calls the kernel
+cannot serve (strides that are not multiples of 8 elements, k or the contiguous extent not a multiple
+of 8, unaligned bases) take the plain one-thread-per-element kernel of the same nest.
 """
 from __future__ import annotations
 
@@ -31,6 +33,7 @@ GEMM_PRELUDE = r"""
 typedef float lfg_f32x16 __attribute__((ext_vector_type(16)));
 typedef unsigned int lfg_u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int lfg_u32x2 __attribute__((ext_vector_type(2)));
+typedef float lfg_f32x4 __attribute__((ext_vector_type(4)));
 typedef short lfg_s16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 lfg_bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 lfg_f16x8 __attribute__((ext_vector_type(8)));
@@ -47,36 +50,19 @@ __device__ __forceinline__ lfg_f32x16 lfg_mfma(_Float16, lfg_u32x4 a, lfg_u32x4 
 //   transposed reads (4 consecutive rows x 64 contiguous bytes per 32 lanes).
 __device__ __forceinline__ int lfg_rows_at(int row, int piece) { return row * 64 + 8 * (piece ^ ((row >> 1) & 7)); }
 __device__ __forceinline__ int lfg_cols_at(int row, int piece) { return row * 128 + 8 * (piece ^ (4 * (row & 3))); }
-// global -> registers: the four 16-byte pieces of a 128 x 64 / 64 x 128 tile that thread `tid` stages; pieces outside
-// [0, lim_outer) x [0, lim_k) arrive as zeros (extents are multiples of 8 along the contiguous dimension)
-template <typename T>
-__device__ __forceinline__ void lfg_fetch(lfg_u32x4 (&st)[4], const T* base, bool rows, long long s_outer, long long s_k,
-                                          long long o0, long long lim_outer, long long k0, long long lim_k, int tid) {
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int idx = tid + 256 * j;
-    long long o, k;
-    if (rows) { o = o0 + (idx >> 3); k = k0 + 8 * (idx & 7); }
-    else { k = k0 + (idx >> 4); o = o0 + 8 * (idx & 15); }
-    const bool ok = o < lim_outer && k < lim_k;
-    const T* src = base + (ok ? o * s_outer + k * s_k : 0ll);
-    const lfg_u32x4 v = *reinterpret_cast<const lfg_u32x4*>(src);
-    st[j] = ok ? v : lfg_u32x4{0u, 0u, 0u, 0u};
-  }
-}
-__device__ __forceinline__ void lfg_stage(unsigned short* tile, const lfg_u32x4 (&st)[4], bool rows, int tid) {
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int idx = tid + 256 * j;
-    const int at = rows ? lfg_rows_at(idx >> 3, idx & 7) : lfg_cols_at(idx >> 4, idx & 15);
-    *reinterpret_cast<lfg_u32x4*>(&tile[at]) = st[j];
-  }
-}
+// The four 16-byte pieces of a 128 x 64 / 64 x 128 tile that thread `tid` stages: where they lie relative to the tile's
+// origin (outer = m or n, k), as element offsets.
+template <bool kRows> struct LfgPiece {
+  static __device__ __forceinline__ int outer(int idx) { return kRows ? (idx >> 3) : 8 * (idx & 15); }
+  static __device__ __forceinline__ int k(int idx) { return kRows ? 8 * (idx & 7) : (idx >> 4); }
+  static __device__ __forceinline__ int lds(int idx) { return kRows ? lfg_rows_at(idx >> 3, idx & 7) : lfg_cols_at(idx >> 4, idx & 15); }
+};
 // MFMA operand (either side: 32 rows or columns `blk`, lane % 32 picks one, lane / 32 the half of the 16-step `ks`):
 // k = 16 * ks + 8 * (lane / 32) .. + 7 in both layouts
-__device__ __forceinline__ lfg_u32x4 lfg_operand(const unsigned short* tile, bool rows, int blk, int ks, int lane) {
+template <bool kRows>
+__device__ __forceinline__ lfg_u32x4 lfg_operand(const unsigned short* tile, int blk, int ks, int lane) {
   const int l32 = lane & 31, g = lane >> 5;
-  if (rows) return *reinterpret_cast<const lfg_u32x4*>(&tile[lfg_rows_at(32 * blk + l32, 2 * ks + g)]);
+  if (kRows) return *reinterpret_cast<const lfg_u32x4*>(&tile[lfg_rows_at(32 * blk + l32, 2 * ks + g)]);
   const int j16 = lane & 15, dh = (lane >> 4) & 1;
   const int col = 32 * blk + 16 * dh + 4 * (j16 & 3);
   lfg_u32x2 h[2];
@@ -88,6 +74,17 @@ __device__ __forceinline__ lfg_u32x4 lfg_operand(const unsigned short* tile, boo
     h[half] = __builtin_bit_cast(lfg_u32x2, t);
   }
   return lfg_u32x4{h[0][0], h[0][1], h[1][0], h[1][1]};
+}
+// four consecutive results of one output row: one store when the row is contiguous and aligned, else element-wise
+template <typename T> struct LfgPack;
+template <> struct LfgPack<float> { typedef lfg_u32x4 type; };
+template <> struct LfgPack<__bf16> { typedef lfg_u32x2 type; };
+template <> struct LfgPack<_Float16> { typedef lfg_u32x2 type; };
+template <typename T>
+__device__ __forceinline__ void lfg_st4(void* p, long long at, const float (&r)[4]) {
+  T t[4] = {(T)r[0], (T)r[1], (T)r[2], (T)r[3]};
+  typedef typename LfgPack<T>::type pack_t;
+  *reinterpret_cast<pack_t*>(reinterpret_cast<T*>(p) + at) = __builtin_bit_cast(pack_t, t);
 }
 """
 
@@ -105,7 +102,9 @@ class GemmInfo:
     b_dims: tuple               # (dim of B indexed by n, dim indexed by k)
     a_batch_dims: list          # dims of A indexed by a batch atom
     b_batch_dims: list
-    flags_at: int = 0           # n[flags_at], n[flags_at + 1]: A / B are k-contiguous
+    flags_at: int = 0           # n[flags_at]: the output's rows are contiguous and aligned for 8- / 16-byte stores
+    out_buf: object = None
+    out_n_dim: int = -1         # dimension of the output indexed by n alone (-1: none)
 
 
 def _single(atoms) -> Optional[ir.Atom]:
@@ -200,9 +199,14 @@ class GemmEmitter(Emitter):
         out = n.writes()
         o = self.buf(out)
         ooff = self.offset(out, out.dims, None)
+        g.out_buf = out
+        for d, atoms in enumerate(out.dims):
+            xs = [a for a in ir.leaves(atoms) if a.hint != 1]
+            if len(xs) == 1 and xs[0] is g.n:
+                g.out_n_dim = d
         na, ns = len(self.atoms), len(self.strides)
         g.flags_at = na + ns
-        if na + ns + 2 > MAX_N or len(self.bufs) > MAX_PTR:
+        if na + ns + 1 > MAX_N or len(self.bufs) > MAX_PTR:
             raise NotLowerable("nest touches too many buffers / dimensions")
         defs = [f"const long long N{k} = p.n[{k}];" for k in range(na)] + \
                [f"const long long S{k} = p.n[{na + k}];" for k in range(ns)]
@@ -210,12 +214,14 @@ class GemmEmitter(Emitter):
         for a in reversed(g.batch):
             k = self.atom(a)
             batch_decode.append(f"const long long i{k} = blk % N{k}; blk /= N{k};")
+        out_t = _CT[self.dtypes[out.name]]
         src = f"""extern "C" __global__ void __launch_bounds__(256, 2) {self.name}(const LfGenParams p) {{
   {' '.join(defs)}
-  const bool a_rows = p.n[{g.flags_at}] != 0, b_rows = p.n[{g.flags_at + 1}] != 0;
-  __shared__ __attribute__((aligned(16))) unsigned short tile_a[2][8192];
-  __shared__ __attribute__((aligned(16))) unsigned short tile_b[2][8192];
+  constexpr bool a_rows = LFG_A_ROWS != 0, b_rows = LFG_B_ROWS != 0;
+  const bool row_stores = p.n[{g.flags_at}] != 0;
+  __shared__ __attribute__((aligned(16))) unsigned short lds[32768];        // A tiles [2][8192], B tiles [2][8192]
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave & 1, wn = wave >> 1;                                   // the wave's 64 x 64 quarter of the tile
   const long long M = N{km}, Nn = N{kn}, K = N{kk};
   const long long mt = (M + {BM - 1}) / {BM}, nt = (Nn + {BN - 1}) / {BN};
   long long total = mt * nt;
@@ -231,51 +237,105 @@ class GemmEmitter(Emitter):
   const long long m0 = tm * {BM}, n0 = tn * {BN};
   const {elem}* A = {a_base};
   const {elem}* B = {b_base};
-  lfg_f32x16 acc[4];
+  // this thread's pieces: pointer at k = 0, whether the row / column group exists, k offset inside a step
+  const {elem}* pa[4];
+  const {elem}* pb[4];
+  bool oka[4], okb[4];
 #pragma unroll
-  for (int nb = 0; nb < 4; ++nb)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) acc[nb][i] = 0.0f;
+  for (int j = 0; j < 4; ++j) {{
+    const int idx = tid + 256 * j;
+    const long long oa = m0 + LfgPiece<a_rows>::outer(idx), ob = n0 + LfgPiece<b_rows>::outer(idx);
+    oka[j] = oa < M;
+    okb[j] = ob < Nn;
+    pa[j] = A + (oka[j] ? oa : 0ll) * S{sam} + (long long)LfgPiece<a_rows>::k(idx) * S{sak};
+    pb[j] = B + (okb[j] ? ob : 0ll) * S{sbn} + (long long)LfgPiece<b_rows>::k(idx) * S{sbk};
+  }}
   lfg_u32x4 sa[4], sb[4];
-  lfg_fetch<{elem}>(sa, A, a_rows, S{sam}, S{sak}, m0, M, 0, K, tid);
-  lfg_fetch<{elem}>(sb, B, b_rows, S{sbn}, S{sbk}, n0, Nn, 0, K, tid);
-  lfg_stage(tile_a[0], sa, a_rows, tid);
-  lfg_stage(tile_b[0], sb, b_rows, tid);
+  auto fetch = [&](long long k0) {{
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {{
+      const int idx = tid + 256 * j;
+      const bool va = oka[j] && k0 + LfgPiece<a_rows>::k(idx) < K, vb = okb[j] && k0 + LfgPiece<b_rows>::k(idx) < K;
+      sa[j] = va ? *reinterpret_cast<const lfg_u32x4*>(pa[j]) : lfg_u32x4{{0u, 0u, 0u, 0u}};
+      sb[j] = vb ? *reinterpret_cast<const lfg_u32x4*>(pb[j]) : lfg_u32x4{{0u, 0u, 0u, 0u}};
+      pa[j] += {BK} * S{sak};
+      pb[j] += {BK} * S{sbk};
+    }}
+  }};
+  auto stage = [&](int buf) {{
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {{
+      const int idx = tid + 256 * j;
+      *reinterpret_cast<lfg_u32x4*>(&lds[buf * 8192 + LfgPiece<a_rows>::lds(idx)]) = sa[j];
+      *reinterpret_cast<lfg_u32x4*>(&lds[16384 + buf * 8192 + LfgPiece<b_rows>::lds(idx)]) = sb[j];
+    }}
+  }};
+  lfg_f32x16 acc[2][2];
+#pragma unroll
+  for (int x = 0; x < 4; ++x)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[x / 2][x % 2][i] = 0.0f;
+  fetch(0);
+  stage(0);
   __syncthreads();
   const long long steps = (K + {BK - 1}) / {BK};
   for (long long st = 0; st < steps; ++st) {{
     const int cur = (int)(st & 1);
-    if (st + 1 < steps) {{
-      lfg_fetch<{elem}>(sa, A, a_rows, S{sam}, S{sak}, m0, M, (st + 1) * {BK}, K, tid);
-      lfg_fetch<{elem}>(sb, B, b_rows, S{sbn}, S{sbk}, n0, Nn, (st + 1) * {BK}, K, tid);
-    }}
+    if (st + 1 < steps) fetch((st + 1) * {BK});
+    const unsigned short* ta = &lds[cur * 8192];
+    const unsigned short* tb = &lds[16384 + cur * 8192];
 #pragma unroll
     for (int ks = 0; ks < {BK // 16}; ++ks) {{
-      const lfg_u32x4 fm = lfg_operand(tile_a[cur], a_rows, wave, ks, lane);       // A rows of this wave: lane = m
+      lfg_u32x4 fm[2], fn[2];
 #pragma unroll
-      for (int nb = 0; nb < 4; ++nb)
-        acc[nb] = lfg_mfma(({elem})0.0f, lfg_operand(tile_b[cur], b_rows, nb, ks, lane), fm, acc[nb]);
+      for (int x = 0; x < 2; ++x) {{
+        fm[x] = lfg_operand<a_rows>(ta, 2 * wm + x, ks, lane);       // lane = m
+        fn[x] = lfg_operand<b_rows>(tb, 2 * wn + x, ks, lane);       // lane = n: the A operand of C^T = B^T A^T
+      }}
+#pragma unroll
+      for (int x = 0; x < 4; ++x)
+        acc[x / 2][x % 2] = lfg_mfma(({elem})0.0f, fn[x % 2], fm[x / 2], acc[x / 2][x % 2]);
     }}
-    if (st + 1 < steps) {{
-      lfg_stage(tile_a[cur ^ 1], sa, a_rows, tid);
-      lfg_stage(tile_b[cur ^ 1], sb, b_rows, tid);
-    }}
+    if (st + 1 < steps) stage(cur ^ 1);
     __syncthreads();
   }}
-  // C^T[n][m]: lane holds m = m0 + 32 * wave + lane % 32; element i of block nb is n = n0 + 32 * nb + 8 * (i / 4) + 4 * (lane / 32) + i % 4
-  const long long i{km} = m0 + 32 * wave + (lane & 31);
-  if (i{km} >= M) return;
+  // acc[mb][nb][i] = C[m][n], m = 64 * wm + 32 * mb + lane % 32, n = 64 * wn + 32 * nb + 8 * (i / 4) + 4 * (lane / 32) + i % 4.
+  // Through the wave's own 16 KB of LDS ([64 m][64 n] fp32, 16-byte pieces permuted by the row): afterwards a lane
+  // holds four consecutive n of one m and 16 neighbouring lanes cover 64 consecutive n.
+  float* mine = reinterpret_cast<float*>(lds) + wave * 4096;
+  {{
+    const int l32 = lane & 31, gg = lane >> 5;
 #pragma unroll
-  for (int nb = 0; nb < 4; ++nb)
+    for (int x = 0; x < 4; ++x)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {{
-      const long long i{kn} = n0 + 32 * nb + 8 * (i / 4) + 4 * (lane >> 5) + (i % 4);
-      if (i{kn} < Nn) {{
-        const float accv = acc[nb][i];
-        const float result = {val};
-        lfg_st<{_CT[self.dtypes[out.name]]}>(p.ptr[{o}], {ooff}, result);
+      for (int q = 0; q < 4; ++q) {{
+        const int row = 32 * (x / 2) + l32, piece = 8 * (x % 2) + 2 * q + gg;
+        const lfg_f32x16& c = acc[x / 2][x % 2];
+        *reinterpret_cast<lfg_u32x4*>(&mine[row * 64 + 4 * (piece ^ (row & 15))]) =
+            __builtin_bit_cast(lfg_u32x4, lfg_f32x4{{c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]}});
+      }}
+  }}
+  __syncthreads();
+  auto epilogue = [&](float accv, long long i{km}, long long i{kn}) -> float {{ return {val}; }};
+  auto out_at = [&](long long i{km}, long long i{kn}) -> long long {{ return {ooff}; }};
+#pragma unroll 4
+  for (int j = 0; j < 16; ++j) {{
+    const int row = 4 * j + (lane >> 4), piece = lane & 15;
+    const lfg_f32x4 c = __builtin_bit_cast(lfg_f32x4, *reinterpret_cast<const lfg_u32x4*>(&mine[row * 64 + 4 * (piece ^ (row & 15))]));
+    const long long m = m0 + 64 * wm + row, n = n0 + 64 * wn + 4 * piece;
+    if (m < M && n < Nn) {{
+      float r[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) r[e] = epilogue(c[e], m, n + e < Nn ? n + e : n);
+      if (row_stores && n + 3 < Nn) {{
+        lfg_st4<{out_t}>(p.ptr[{o}], out_at(m, n), r);
+      }} else {{
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (n + e < Nn) lfg_st<{out_t}>(p.ptr[{o}], out_at(m, n + e), r[e]);
       }}
     }}
+  }}
 }}
 """
         return Kernel(self.name, src, self.bufs, self.atoms, self.strides, self.scalars, par)

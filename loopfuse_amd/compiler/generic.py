@@ -61,25 +61,34 @@ class GenericProgram:
                     self.gemm[i] = (emit_gemm.GemmEmitter(n, self.dtypes, f"lf_gen_{i}_mfma", info).emit(), info)
                 except NotLowerable:
                     pass
-        self.gpu_source = self.source
-        if self.gemm:
-            self.gpu_source = emit.PRELUDE + emit_gemm.GEMM_PRELUDE + "\n".join(
-                [k.source for k in self.kernels] + [k.source for k, _ in self.gemm.values()])
+        # the MFMA kernels are specialised by operand layout at compile time: one code object per layout pair,
+        # built when a call first needs it
+        self.gemm_source = emit.PRELUDE + emit_gemm.GEMM_PRELUDE + "\n".join(k.source for k, _ in self.gemm.values())
         self._loaded: dict = {}
+        self._gemm_loaded: dict = {}
 
     @property
     def code(self) -> str:
-        return self.gpu_source
+        return self.source + (self.gemm_source if self.gemm else "")
 
     def _module(self):
         from .. import lowering, runtime
         dev = torch.cuda.current_device()
         if dev not in self._loaded:
-            code, _, _ = runtime.compile_source(self.gpu_source, "lf_generic", list(lowering.COMMON_OPTS))
+            code, _, _ = runtime.compile_source(self.source, "lf_generic", list(lowering.COMMON_OPTS))
             mod = runtime.Module(code)
-            self._loaded[dev] = ([mod.kernel(k.name) for k in self.kernels],
-                                 {i: mod.kernel(k.name) for i, (k, _) in self.gemm.items()})
+            self._loaded[dev] = [mod.kernel(k.name) for k in self.kernels]
         return self._loaded[dev]
+
+    def _gemm_kernel(self, ni: int, layouts):
+        from .. import lowering, runtime
+        key = (torch.cuda.current_device(), tuple(layouts))
+        if key not in self._gemm_loaded:
+            opts = list(lowering.COMMON_OPTS) + [f"-DLFG_A_ROWS={layouts[0]}", f"-DLFG_B_ROWS={layouts[1]}"]
+            code, _, _ = runtime.compile_source(self.gemm_source, "lf_generic_mfma", opts)
+            mod = runtime.Module(code)
+            self._gemm_loaded[key] = {i: mod.kernel(k.name) for i, (k, _) in self.gemm.items()}
+        return self._gemm_loaded[key][ni]
 
     @staticmethod
     def _gemm_layouts(info, bufs: dict, ext: dict):
@@ -151,8 +160,9 @@ class GenericProgram:
         if launchers is None:
             if dev.type != "cuda":
                 raise NotLowerable("tensors are not on the GPU")
-            kernels, mfma = self._module()
+            kernels = self._module()
             launchers = [lambda blocks, prm, fn=fn: fn.launch((blocks, 1, 1), (256, 1, 1), prm) for fn in kernels]
+            mfma = self.gemm
         else:
             mfma = {}
         ext: dict = {}
@@ -174,7 +184,7 @@ class GenericProgram:
                 except KeyError:
                     layouts = None
                 if layouts is not None and all(ext.get(a.id, 0) > 0 for a in self.gemm[ni][0].atoms):
-                    self._launch_gemm(mfma[ni], *self.gemm[ni], layouts, bufs, ext, args)
+                    self._launch_gemm(self._gemm_kernel(ni, layouts), *self.gemm[ni], bufs, ext, args)
                     counters["mfma"] += 1
                     continue
             prm = emit.GenParams()
@@ -202,7 +212,7 @@ class GenericProgram:
         return res.view(view)
 
     @staticmethod
-    def _launch_gemm(fn, k, info, layouts, bufs: dict, ext: dict, args) -> None:
+    def _launch_gemm(fn, k, info, bufs: dict, ext: dict, args) -> None:
         prm = emit.GenParams()
         for i, b in enumerate(k.bufs):
             prm.ptr[i] = bufs[b.name].data_ptr()
@@ -210,7 +220,12 @@ class GenericProgram:
             prm.n[i] = ext[a.id]
         for i, (b, d) in enumerate(k.strides):
             prm.n[len(k.atoms) + i] = bufs[b.name].stride(d)
-        prm.n[info.flags_at], prm.n[info.flags_at + 1] = layouts
+        # rows of the output contiguous along n, every row start and the extent a multiple of four elements:
+        # results leave four at a time
+        o = bufs[info.out_buf.name]
+        prm.n[info.flags_at] = int(info.out_n_dim >= 0 and o.stride(info.out_n_dim) == 1 and ext[info.n.id] % 4 == 0
+                                   and o.data_ptr() % 16 == 0
+                                   and all(st % 4 == 0 for d, st in enumerate(o.stride()) if d != info.out_n_dim and o.shape[d] > 1))
         for i, s in enumerate(k.scalars):
             prm.f[i] = float(s.fn(args))
         tiles = -(-ext[info.m.id] // emit_gemm.BM) * -(-ext[info.n.id] // emit_gemm.BN) * \
