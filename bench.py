@@ -274,6 +274,40 @@ def cpu_baseline(seconds: float = 12.0) -> dict:
     }
 
 
+def generated_matmul(args, dev) -> dict:
+    """Contractions of graphs without an attention on the generated MFMA kernels (loopfuse_amd/compiler/emit_gemm.py):
+    ``a @ b.t() + bias`` on bf16 operands through the backend with its tuning off, against the same function run
+    eagerly (library matmul + add) on the same GPU."""
+    import torch
+
+    from loopfuse_amd import loopfuse_backend
+    from loopfuse_amd.compiler import generic
+
+    res = {}
+    old = os.environ.get("LOOPFUSE_AUTOTUNE")
+    os.environ["LOOPFUSE_AUTOTUNE"] = "0"
+    try:
+        for m, n, k in ((4096, 4096, 4096), (8192, 8192, 8192), (16384, 4096, 1024)):
+            g = torch.Generator().manual_seed(0)
+            a, b, bias = (torch.randn(s, generator=g).to(torch.bfloat16).to(dev) for s in ((m, k), (n, k), (n,)))
+            fn = lambda a, b, bias: a @ b.t() + bias      # noqa: E731
+            torch._dynamo.reset()
+            cf = torch.compile(fn, backend=loopfuse_backend)
+            before = generic.counters["mfma"]
+            cf(a, b, bias)
+            assert generic.counters["mfma"] == before + 1, "the contraction did not run on the generated MFMA kernel"
+            t, _ = time_gpu(lambda i: cf(a, b, bias), 30, 10)
+            te, _ = time_gpu(lambda i: fn(a, b, bias), 30, 10)
+            res[f"{m}x{n}x{k}"] = {"us_per_call": t * 1e6, "tflops": 2.0 * m * n * k / t / 1e12,
+                                   "eager_us_per_call": te * 1e6, "eager_tflops": 2.0 * m * n * k / te / 1e12}
+    finally:
+        if old is None:
+            os.environ.pop("LOOPFUSE_AUTOTUNE", None)
+        else:
+            os.environ["LOOPFUSE_AUTOTUNE"] = old
+    return res
+
+
 def torch_sdpa(args, dev) -> dict:
     """PyTorch's own fused attention on the same GPU and inputs: a same-hardware point of
     comparison (not the reference, which has no AMD path).  Softcap and the sliding window
@@ -324,6 +358,8 @@ def main() -> int:
     ap.add_argument("--mfma-ceiling", action="store_true",
                     help="also run the MFMA-only probe on zeros and on N(0,1) operands (the data-dependent clock ceiling), and "
                          "the prefill kernel on zero operands, without the mask and at S = 8192")
+    ap.add_argument("--generated-matmul", action="store_true",
+                    help="also time a @ b.t() + bias on the generated MFMA kernels of the non-attention path")
     ap.add_argument("--backward", action="store_true",
                     help="also time the forward with its log-sum-exp output and the backward kernels on config 2")
     ap.add_argument("--workload", default="c2", help="prefill workload: c2 | c2_softcap | c3 | c2_mask (the causal mask given as a tensor)")
@@ -436,6 +472,8 @@ def main() -> int:
         out["backward"] = backward_leg(dev)
     if args.torch_sdpa:
         out["torch_sdpa"] = torch_sdpa(args, dev)
+    if args.generated_matmul:
+        out["generated_matmul"] = generated_matmul(args, dev)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))

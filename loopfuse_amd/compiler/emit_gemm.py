@@ -50,13 +50,34 @@ __device__ __forceinline__ lfg_f32x16 lfg_mfma(_Float16, lfg_u32x4 a, lfg_u32x4 
 //   transposed reads (4 consecutive rows x 64 contiguous bytes per 32 lanes).
 __device__ __forceinline__ int lfg_rows_at(int row, int piece) { return row * 64 + 8 * (piece ^ ((row >> 1) & 7)); }
 __device__ __forceinline__ int lfg_cols_at(int row, int piece) { return row * 128 + 8 * (piece ^ (4 * (row & 3))); }
-// The four 16-byte pieces of a 128 x 64 / 64 x 128 tile that thread `tid` stages: where they lie relative to the tile's
-// origin (outer = m or n, k), as element offsets.
+// Tiles arrive by direct global -> LDS loads: a wave-level load writes 64 lanes x 16 bytes at M0 + 16 * lane, i.e. the
+// 64 consecutive 16-byte positions `idx` = 64 * (wave + 4 * j) + lane of the tile, and the permutation is applied on
+// the global side: the lane that fills position idx fetches the piece (outer = m or n, k) that lives there.
 template <bool kRows> struct LfgPiece {
-  static __device__ __forceinline__ int outer(int idx) { return kRows ? (idx >> 3) : 8 * (idx & 15); }
-  static __device__ __forceinline__ int k(int idx) { return kRows ? 8 * (idx & 7) : (idx >> 4); }
-  static __device__ __forceinline__ int lds(int idx) { return kRows ? lfg_rows_at(idx >> 3, idx & 7) : lfg_cols_at(idx >> 4, idx & 15); }
+  static __device__ __forceinline__ int outer(int idx) {
+    return kRows ? (idx >> 3) : 8 * ((idx & 15) ^ (4 * ((idx >> 4) & 3)));
+  }
+  static __device__ __forceinline__ int k(int idx) {
+    return kRows ? 8 * ((idx & 7) ^ ((idx >> 4) & 7)) : (idx >> 4);
+  }
 };
+// Buffer resource over `bytes` bytes from `base` (raw buffer, 32-bit offsets, range checked: a load beyond the range
+// delivers zeros)
+__device__ __forceinline__ lfg_u32x4 lfg_make_buffer(const void* base, unsigned bytes) {
+  const unsigned long long a = (unsigned long long)base;
+  lfg_u32x4 rs;
+  rs[0] = __builtin_amdgcn_readfirstlane((unsigned)a);
+  rs[1] = __builtin_amdgcn_readfirstlane((unsigned)(a >> 32) & 0xffffu);
+  rs[2] = __builtin_amdgcn_readfirstlane(bytes);
+  rs[3] = 0x00020000u;
+  return rs;
+}
+// One wave-level direct-to-LDS load (not tracked by the compiler's wait counters: callers wait with s_waitcnt vmcnt)
+__device__ __forceinline__ void lfg_dma(const lfg_u32x4& rs, unsigned voff, unsigned lds_addr) {
+  unsigned m0_written;
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tbuffer_load_dwordx4 %2, %3, 0 offen lds"
+               : "={m0}"(m0_written) : "s"(lds_addr), "v"(voff), "s"(rs) : "memory");
+}
 // MFMA operand (either side: 32 rows or columns `blk`, lane % 32 picks one, lane / 32 the half of the 16-step `ks`):
 // k = 16 * ks + 8 * (lane / 32) .. + 7 in both layouts
 template <bool kRows>
@@ -102,7 +123,8 @@ class GemmInfo:
     b_dims: tuple               # (dim of B indexed by n, dim indexed by k)
     a_batch_dims: list          # dims of A indexed by a batch atom
     b_batch_dims: list
-    flags_at: int = 0           # n[flags_at]: the output's rows are contiguous and aligned for 8- / 16-byte stores
+    flags_at: int = 0           # n[flags_at]: the output's rows are contiguous and aligned for 8- / 16-byte stores;
+                                # n[flags_at + 1], n[flags_at + 2]: bytes of A / B reachable from a batch element's base
     out_buf: object = None
     out_n_dim: int = -1         # dimension of the output indexed by n alone (-1: none)
 
@@ -206,7 +228,7 @@ class GemmEmitter(Emitter):
                 g.out_n_dim = d
         na, ns = len(self.atoms), len(self.strides)
         g.flags_at = na + ns
-        if na + ns + 1 > MAX_N or len(self.bufs) > MAX_PTR:
+        if na + ns + 3 > MAX_N or len(self.bufs) > MAX_PTR:
             raise NotLowerable("nest touches too many buffers / dimensions")
         defs = [f"const long long N{k} = p.n[{k}];" for k in range(na)] + \
                [f"const long long S{k} = p.n[{na + k}];" for k in range(ns)]
@@ -237,37 +259,31 @@ class GemmEmitter(Emitter):
   const long long m0 = tm * {BM}, n0 = tn * {BN};
   const {elem}* A = {a_base};
   const {elem}* B = {b_base};
-  // this thread's pieces: pointer at k = 0, whether the row / column group exists, k offset inside a step
-  const {elem}* pa[4];
-  const {elem}* pb[4];
-  bool oka[4], okb[4];
+  // this thread's pieces of a tile: byte offset at k = 0 and how many k are left from the piece's own k (0 or less:
+  // the piece lies outside the operand and is asked for beyond the buffer's range, i.e. arrives as zeros)
+  const lfg_u32x4 rs_a = lfg_make_buffer(A, (unsigned)p.n[{g.flags_at + 1}]), rs_b = lfg_make_buffer(B, (unsigned)p.n[{g.flags_at + 2}]);
+  unsigned offa[4], offb[4];
+  int rooma[4], roomb[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {{
     const int idx = tid + 256 * j;
     const long long oa = m0 + LfgPiece<a_rows>::outer(idx), ob = n0 + LfgPiece<b_rows>::outer(idx);
-    oka[j] = oa < M;
-    okb[j] = ob < Nn;
-    pa[j] = A + (oka[j] ? oa : 0ll) * S{sam} + (long long)LfgPiece<a_rows>::k(idx) * S{sak};
-    pb[j] = B + (okb[j] ? ob : 0ll) * S{sbn} + (long long)LfgPiece<b_rows>::k(idx) * S{sbk};
+    const int ka = LfgPiece<a_rows>::k(idx), kb = LfgPiece<b_rows>::k(idx);
+    offa[j] = (unsigned)(2 * (oa * S{sam} + ka * S{sak}));
+    offb[j] = (unsigned)(2 * (ob * S{sbn} + kb * S{sbk}));
+    rooma[j] = oa < M ? (int)min(K - ka, (long long)0x7fffffff) : 0;
+    roomb[j] = ob < Nn ? (int)min(K - kb, (long long)0x7fffffff) : 0;
   }}
-  lfg_u32x4 sa[4], sb[4];
-  auto fetch = [&](long long k0) {{
+  const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) const void*)lds;
+  const unsigned stepa = (unsigned)(2 * {BK} * S{sak}), stepb = (unsigned)(2 * {BK} * S{sbk});
+  // tile of k step `st` into buffer `buf`
+  auto fetch = [&](int st, int buf) {{
+    const int k0 = st * {BK};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {{
-      const int idx = tid + 256 * j;
-      const bool va = oka[j] && k0 + LfgPiece<a_rows>::k(idx) < K, vb = okb[j] && k0 + LfgPiece<b_rows>::k(idx) < K;
-      sa[j] = va ? *reinterpret_cast<const lfg_u32x4*>(pa[j]) : lfg_u32x4{{0u, 0u, 0u, 0u}};
-      sb[j] = vb ? *reinterpret_cast<const lfg_u32x4*>(pb[j]) : lfg_u32x4{{0u, 0u, 0u, 0u}};
-      pa[j] += {BK} * S{sak};
-      pb[j] += {BK} * S{sbk};
-    }}
-  }};
-  auto stage = [&](int buf) {{
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {{
-      const int idx = tid + 256 * j;
-      *reinterpret_cast<lfg_u32x4*>(&lds[buf * 8192 + LfgPiece<a_rows>::lds(idx)]) = sa[j];
-      *reinterpret_cast<lfg_u32x4*>(&lds[16384 + buf * 8192 + LfgPiece<b_rows>::lds(idx)]) = sb[j];
+      const unsigned at = 16u * (unsigned)(64 * (wave + 4 * j));
+      lfg_dma(rs_a, k0 < rooma[j] ? offa[j] + (unsigned)st * stepa : 0xffffffffu, lds0 + 16384u * (unsigned)buf + at);
+      lfg_dma(rs_b, k0 < roomb[j] ? offb[j] + (unsigned)st * stepb : 0xffffffffu, lds0 + 32768u + 16384u * (unsigned)buf + at);
     }}
   }};
   lfg_f32x16 acc[2][2];
@@ -275,13 +291,12 @@ class GemmEmitter(Emitter):
   for (int x = 0; x < 4; ++x)
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[x / 2][x % 2][i] = 0.0f;
-  fetch(0);
-  stage(0);
-  __syncthreads();
-  const long long steps = (K + {BK - 1}) / {BK};
-  for (long long st = 0; st < steps; ++st) {{
-    const int cur = (int)(st & 1);
-    if (st + 1 < steps) fetch((st + 1) * {BK});
+  fetch(0, 0);
+  asm volatile("s_waitcnt vmcnt(0)\\n\\ts_barrier" ::: "memory");
+  const int steps = (int)((K + {BK - 1}) / {BK});
+  for (int st = 0; st < steps; ++st) {{
+    const int cur = st & 1;
+    if (st + 1 < steps) fetch(st + 1, cur ^ 1);
     const unsigned short* ta = &lds[cur * 8192];
     const unsigned short* tb = &lds[16384 + cur * 8192];
 #pragma unroll
@@ -296,8 +311,8 @@ class GemmEmitter(Emitter):
       for (int x = 0; x < 4; ++x)
         acc[x / 2][x % 2] = lfg_mfma(({elem})0.0f, fn[x % 2], fm[x / 2], acc[x / 2][x % 2]);
     }}
-    if (st + 1 < steps) stage(cur ^ 1);
-    __syncthreads();
+    // this wave's loads of the next tile have landed, every wave is done reading this one
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\\n\\ts_barrier" ::: "memory");
   }}
   // acc[mb][nb][i] = C[m][n], m = 64 * wm + 32 * mb + lane % 32, n = 64 * wn + 32 * nb + 8 * (i / 4) + 4 * (lane / 32) + i % 4.
   // Through the wave's own 16 KB of LDS ([64 m][64 n] fp32, 16-byte pieces permuted by the row): afterwards a lane

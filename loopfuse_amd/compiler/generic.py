@@ -66,6 +66,7 @@ class GenericProgram:
         self.gemm_source = emit.PRELUDE + emit_gemm.GEMM_PRELUDE + "\n".join(k.source for k, _ in self.gemm.values())
         self._loaded: dict = {}
         self._gemm_loaded: dict = {}
+        self.last_mfma_flop = 0.0           # flop the MFMA kernels of the last run() were launched for
 
     @property
     def code(self) -> str:
@@ -102,6 +103,8 @@ class GenericProgram:
             if t.data_ptr() % 16 or any(t.stride(d) % 8 for d in batch_dims if t.shape[d] > 1):
                 return None
             s_outer, s_k = t.stride(d_outer), t.stride(d_k)
+            if s_outer < 0 or s_k < 0 or 2 * ((outer + 128) * s_outer + (K + 64) * s_k) >= 1 << 32:
+                return None                  # the direct loads address a batch element's operand with 32-bit byte offsets
             if (s_k == 1 or K == 1) and K % 8 == 0 and (s_outer % 8 == 0 or outer == 1):
                 flags.append(1)
             elif (s_outer == 1 or outer == 1) and outer % 8 == 0 and (s_k % 8 == 0 or K == 1):
@@ -165,6 +168,7 @@ class GenericProgram:
             mfma = self.gemm
         else:
             mfma = {}
+        self.last_mfma_flop = 0.0
         ext: dict = {}
         syms: dict = {name: int(args[i]) for name, i in self.parsed.sizes.items()}
         work = 0
@@ -186,6 +190,8 @@ class GenericProgram:
                 if layouts is not None and all(ext.get(a.id, 0) > 0 for a in self.gemm[ni][0].atoms):
                     self._launch_gemm(self._gemm_kernel(ni, layouts), *self.gemm[ni], bufs, ext, args)
                     counters["mfma"] += 1
+                    info = self.gemm[ni][1]
+                    self.last_mfma_flop += 2.0 * math.prod(ext[a.id] for a in [info.m, info.n, info.k] + list(info.batch))
                     continue
             prm = emit.GenParams()
             for i, b in enumerate(k.bufs):
@@ -226,6 +232,10 @@ class GenericProgram:
         prm.n[info.flags_at] = int(info.out_n_dim >= 0 and o.stride(info.out_n_dim) == 1 and ext[info.n.id] % 4 == 0
                                    and o.data_ptr() % 16 == 0
                                    and all(st % 4 == 0 for d, st in enumerate(o.stride()) if d != info.out_n_dim and o.shape[d] > 1))
+        for j, (buf, (d_outer, d_k), outer) in enumerate(((info.a_buf, info.a_dims, ext[info.m.id]),
+                                                          (info.b_buf, info.b_dims, ext[info.n.id]))):
+            t = bufs[buf.name]
+            prm.n[info.flags_at + 1 + j] = 2 * ((outer - 1) * t.stride(d_outer) + (ext[info.k.id] - 1) * t.stride(d_k) + 1)
         for i, s in enumerate(k.scalars):
             prm.f[i] = float(s.fn(args))
         tiles = -(-ext[info.m.id] // emit_gemm.BM) * -(-ext[info.n.id] // emit_gemm.BN) * \

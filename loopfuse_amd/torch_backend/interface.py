@@ -49,7 +49,7 @@ USE_HARDCODE_KERNEL = os.environ.get("USE_HARDCODE_KERNEL", "0") == "1"
 # "eager_training" = graph traced with gradients enabled (forward or backward half)
 # "refused_signatures" = argument layouts latched as not servable (see optimized_fn)
 stats = {"fused": 0, "eager_graph": 0, "eager_runtime": 0, "eager_training": 0, "compiled_graphs": 0, "matched_graphs": 0,
-         "refused_signatures": 0, "derived_graphs": 0, "generic_graphs": 0, "fused_generic": 0,
+         "refused_signatures": 0, "derived_graphs": 0, "generic_graphs": 0, "fused_generic": 0, "tuned_captured": 0,
          "training_graphs": 0, "fused_training": 0, "match_errors": 0}
 
 
@@ -307,7 +307,25 @@ def rewrite_graph(gm: torch.fx.GraphModule, matches: list, call=None) -> torch.f
     return fused
 
 
-def _generic_program(gm: torch.fx.GraphModule):
+# A graph whose contractions run on the generated MFMA kernels competes with the captured graph's library
+# matmuls: under "max-autotune" a call shape with at least this many flop in such kernels is measured both ways
+# once and keeps the faster route (smaller ones are bound by launches, where one fused kernel wins)
+GENERIC_TUNE_MIN_FLOP = float(1 << 32)
+
+
+def _time_call(fn, reps: int = 3) -> float:
+    fn()
+    torch.cuda.synchronize()
+    t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0.record()
+    for _ in range(reps):
+        fn()
+    t1.record()
+    torch.cuda.synchronize()
+    return t0.elapsed_time(t1) / reps
+
+
+def _generic_program(gm: torch.fx.GraphModule, tune: bool = False):
     """A graph without an attention in it: its loop nests, fused, as one plain HIP kernel per
     nest (loopfuse_amd/compiler/generic.py) -- what the reference's code generator does for every
     graph (loopfuse/codegen.py:100-404).  None when the nest builder does not cover the graph or
@@ -333,11 +351,27 @@ def _generic_program(gm: torch.fx.GraphModule):
     if CODEGEN_ONLY:
         return lambda *args: [prog] if as_tuple else prog
     refused: list = []
+    routes: dict = {}          # call signature -> "generated" | "captured" (measured choice)
 
     def generic_fn(*args):
+        key = None
+        if tune and prog.gemm and not refused:
+            key = tuple((tuple(a.shape), tuple(a.stride())) if isinstance(a, torch.Tensor) else a for a in args)
+            if routes.get(key) == "captured":
+                stats["tuned_captured"] += 1
+                return gm(*args)
         if not refused:
             try:
                 out = prog.run(args)
+                if key is not None and key not in routes:
+                    if len(routes) >= 256:
+                        routes.clear()
+                    routes[key] = "generated"
+                    if prog.last_mfma_flop >= GENERIC_TUNE_MIN_FLOP:
+                        t_gen, t_cap = _time_call(lambda: prog.run(args)), _time_call(lambda: gm(*args))
+                        log.info("generated kernels %.3f ms, captured graph %.3f ms", t_gen, t_cap)
+                        if t_cap < 0.95 * t_gen:
+                            routes[key] = "captured"
             except generic.NotLowerable as e:
                 if _strict():
                     raise
@@ -405,7 +439,7 @@ def loopfuse_compiler(gm: torch.fx.GraphModule, sample_inputs, input_names: list
     if not matches:
         if _strict():
             raise NotImplementedError(f"loopfuse_amd: no fused-attention pattern in the graph: {reason}")
-        generic = _generic_program(gm)
+        generic = _generic_program(gm, tune=(mode == "max-autotune") and os.environ.get("LOOPFUSE_AUTOTUNE", "1") == "1")
         if generic is not None:
             return generic
         log.info("graph not recognised (%s); running it unfused", reason)

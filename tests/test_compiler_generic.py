@@ -251,3 +251,64 @@ def test_codegen_only_hands_back_the_generated_source(monkeypatch):
     prg = torch.compile(lambda a, b, c: a @ b + c, backend=loopfuse_backend, dynamic=True)(
         _r(16, 8), _r(8, 12, seed=1), _r(16, 12, seed=2))
     assert prg.code.count("__global__") == 1 and "lf_gen_0" in prg.code and "LfGenParams" in prg.code
+
+
+# ---- contractions on the MFMA path (compiler/emit_gemm.py): recognition and code generation, no GPU needed
+def _bf16_graph(fn, shapes):
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from torch.fx.experimental.proxy_tensor import make_fx
+    with FakeTensorMode():
+        return make_fx(fn, tracing_mode="fake")(*[torch.empty(s, dtype=torch.bfloat16) for s in shapes])
+
+
+def test_contractions_of_half_precision_operands_get_an_mfma_kernel():
+    """``a @ b + c`` (reference tests/test_accuracy.py:56-82) on bf16 operands: the nest is recognised as a batched
+    matrix product with a pointwise epilogue -- which atoms are rows, columns, the contraction and the batch, and
+    which dimension of each operand they index -- and gets a second, MFMA kernel beside the plain one.  fp32
+    operands, a gathered operand and a contraction whose operand is computed in the nest keep the plain kernel only."""
+    from loopfuse_amd.compiler import emit_gemm
+
+    prog = generic.GenericProgram(_bf16_graph(lambda a, b, c: (a @ b.transpose(-1, -2)) * 0.5 + c,
+                                              [(4, 96, 64), (4, 40, 64), (40,)]))
+    assert list(prog.gemm) == [0]
+    k, info = prog.gemm[0]
+    assert (info.m.hint, info.n.hint, info.k.hint, [a.hint for a in info.batch]) == (96, 40, 64, [4])
+    assert info.a_dims == (1, 2) and info.b_dims == (1, 2) and info.a_batch_dims == [0] and info.b_batch_dims == [0]
+    assert "v_mfma" not in k.source and "lfg_mfma" in k.source and "__launch_bounds__(256, 2)" in k.source
+    assert "accv * 0.5f" in k.source                     # the epilogue is evaluated on the accumulator
+    assert prog.code.count("__global__") == 2            # plain + MFMA
+    # rows of a [.., M, K] view that matmul flattened: the outer ones count as batch
+    prog = generic.GenericProgram(_bf16_graph(lambda a, b: a @ b, [(3, 2, 160, 64), (64, 96)]))
+    info = prog.gemm[0][1]
+    assert (info.m.hint, info.n.hint, info.k.hint, sorted(a.hint for a in info.batch)) == (160, 96, 64, [2, 3])
+    assert info.b_batch_dims == []
+    # not served: fp32 operands; softmax(x) @ y (an operand computed in the nest)
+    with_fp32 = generic.GenericProgram(_aten_graph(lambda a, b, c: a @ b + c, (_r(16, 8), _r(8, 12, seed=1), _r(16, 12, seed=2)))[0])
+    assert not with_fp32.gemm
+    sm = generic.GenericProgram(_bf16_graph(lambda x, y: torch.softmax(x, dim=-1) @ y, [(2, 64, 32), (2, 32, 48)]))
+    assert not sm.gemm
+
+
+@pytest.mark.parametrize("layouts", [(1, 1), (1, 0), (0, 1), (0, 0)])
+def test_mfma_kernel_compiles_for_every_operand_layout(shim_built, layouts):
+    """The generated source builds for gfx950 with hipRTC in all four layout specialisations, without scratch
+    memory and within the registers of two workgroups per CU."""
+    import re
+    import subprocess
+
+    prog = generic.GenericProgram(_bf16_graph(lambda a, b, c: torch.tanh(a @ b + c), [(256, 128), (128, 192), (192,)]))
+    opts = list(lowering.COMMON_OPTS) + [f"-DLFG_A_ROWS={layouts[0]}", f"-DLFG_B_ROWS={layouts[1]}"]
+    code, _, _ = runtime.compile_source(prog.gemm_source, "lf_generic_mfma", opts)
+    readelf = "/opt/rocm/llvm/bin/llvm-readelf"
+    if not os.path.exists(readelf):
+        return
+    path = os.path.join(os.environ.get("TMPDIR", "/tmp"), f"lf_gemm_{os.getpid()}.hsaco")
+    with open(path, "wb") as fh:
+        fh.write(code)
+    try:
+        notes = subprocess.run([readelf, "--notes", path], capture_output=True, text=True, check=True).stdout
+    finally:
+        os.unlink(path)
+    assert int(re.search(r"\.private_segment_fixed_size:\s+(\d+)", notes).group(1)) == 0
+    assert int(re.search(r"\.vgpr_count:\s+(\d+)", notes).group(1)) <= 256
+    assert int(re.search(r"\.group_segment_fixed_size:\s+(\d+)", notes).group(1)) == 65536

@@ -87,9 +87,10 @@ def test_calls_the_mfma_kernel_cannot_read_take_the_plain_kernel():
     assert generic.counters["mfma"] == before["mfma"] + 1
 
 
-def test_large_matmul_is_no_longer_left_to_the_captured_graph():
+def test_large_matmul_is_no_longer_left_to_the_captured_graph(monkeypatch):
     """2048 x 2048 x 2048 is 2^33 multiply-adds, far beyond what the plain kernels are allowed: on the MFMA path the
     backend keeps the graph (counted as a generated-kernel run), a tanh epilogue and a bias over n fused."""
+    monkeypatch.setenv("LOOPFUSE_AUTOTUNE", "0")
     fn = lambda a, b, bias: torch.tanh(a @ b.t() * 0.02 + bias)      # noqa: E731
     a, b, bias = rand((2048, 2048), BF, 1), rand((2048, 2048), BF, 2), rand((2048,), BF, 3)
     torch._dynamo.reset()
@@ -114,3 +115,25 @@ def test_two_products_in_a_row_keep_the_intermediate_and_both_run_on_mfma():
     assert generic.counters["mfma"] + generic.counters["plain"] == before["mfma"] + before["plain"] + 2
     assert generic.counters["mfma"] >= before["mfma"] + 1
     _close(got, (a.double() @ b.double()) @ c.double(), BF)
+
+
+def test_max_autotune_measures_large_products_against_the_captured_graph():
+    """Under mode="max-autotune" (the default) a call with 2^32 flop or more in generated MFMA kernels is timed
+    against the captured graph once; later calls of that signature take the faster route.  Either way the values
+    are right and every call is accounted for."""
+    fn = lambda a, b, bias: a @ b.t() + bias      # noqa: E731
+    a, b, bias = rand((4096, 2048), BF, 1, 0.5), rand((4096, 2048), BF, 2, 0.5), rand((4096,), BF, 3)
+    ins = [t.to(DEV) for t in (a, b, bias)]
+    want = a.double() @ b.double().t() + bias.double()
+    torch._dynamo.reset()
+    run = torch.compile(fn, backend=loopfuse_backend)
+    before = dict(interface.stats)
+    for _ in range(3):
+        got = run(*ins)
+        # the captured graph rounds the product to bf16 before the bias is added: one more half-ulp
+        err = (got.double().cpu() - want).abs()
+        assert (err <= 2.0 ** -7 * want.abs() + 0.02 * want.abs().max()).all()
+    routed = {k: interface.stats[k] - before[k] for k in ("fused_generic", "tuned_captured", "eager_runtime", "eager_graph")}
+    assert routed["fused_generic"] + routed["tuned_captured"] == 3 and routed["fused_generic"] >= 1, routed
+    assert routed["eager_runtime"] == 0 and routed["eager_graph"] == 0, routed
+    assert routed["tuned_captured"] in (0, 2), routed
