@@ -26,8 +26,20 @@ from typing import Optional
 from . import ir
 from .emit import _CT, MAX_N, MAX_PTR, Emitter, Kernel, NotLowerable
 
-BM = BN = 128
 BK = 64
+# workgroup tiles (waves along m, waves along n, 32 x 32 blocks per wave along m, along n): 128 x 128 on four waves at
+# two workgroups per CU; 256 x 256 on eight waves, one per CU, with half the L2 -> LDS bytes per flop
+TILES = {"s": (2, 2, 2, 2), "l": (4, 2, 2, 4)}
+
+
+def tile_extent(shape: str) -> tuple:
+    wm, wn, mb, nb = TILES[shape]
+    return 32 * wm * mb, 32 * wn * nb
+
+
+def tile_options(shape: str) -> list:
+    wm, wn, mb, nb = TILES[shape]
+    return [f"-DLFG_WGM={wm}", f"-DLFG_WGN={wn}", f"-DLFG_MB={mb}", f"-DLFG_NB={nb}"]
 
 GEMM_PRELUDE = r"""
 typedef float lfg_f32x16 __attribute__((ext_vector_type(16)));
@@ -43,22 +55,23 @@ __device__ __forceinline__ lfg_f32x16 lfg_mfma(__bf16, lfg_u32x4 a, lfg_u32x4 b,
 __device__ __forceinline__ lfg_f32x16 lfg_mfma(_Float16, lfg_u32x4 a, lfg_u32x4 b, lfg_f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(lfg_f16x8, a), __builtin_bit_cast(lfg_f16x8, b), c, 0, 0, 0);
 }
-// Operand tiles in LDS, 8192 two-byte elements each.
-//   k-contiguous operand ("rows"): [128 rows (m or n)][64 k]; the eight 16-byte pieces of a row are permuted by the
+// Operand tiles in LDS; `kExtent` = rows / columns of the workgroup's tile along m (A) or n (B), 64 k per step.
+//   k-contiguous operand ("rows"): [kExtent rows][64 k]; the eight 16-byte pieces of a row are permuted by the
 //   row pair, so that the 16-byte reads of 16 consecutive rows touch every bank once.
-//   m/n-contiguous operand ("cols"): [64 k][128 m or n]; the 64-byte groups of a row are permuted by the row, for the
+//   m/n-contiguous operand ("cols"): [64 k][kExtent]; the 64-byte groups of a row are permuted by the row, for the
 //   transposed reads (4 consecutive rows x 64 contiguous bytes per 32 lanes).
 __device__ __forceinline__ int lfg_rows_at(int row, int piece) { return row * 64 + 8 * (piece ^ ((row >> 1) & 7)); }
-__device__ __forceinline__ int lfg_cols_at(int row, int piece) { return row * 128 + 8 * (piece ^ (4 * (row & 3))); }
-// Tiles arrive by direct global -> LDS loads: a wave-level load writes 64 lanes x 16 bytes at M0 + 16 * lane, i.e. the
-// 64 consecutive 16-byte positions `idx` = 64 * (wave + 4 * j) + lane of the tile, and the permutation is applied on
-// the global side: the lane that fills position idx fetches the piece (outer = m or n, k) that lives there.
-template <bool kRows> struct LfgPiece {
+template <int kExtent>
+__device__ __forceinline__ int lfg_cols_at(int row, int piece) { return row * kExtent + 8 * (piece ^ (4 * (row & 3))); }
+// Tiles arrive by direct global -> LDS loads: a wave-level load writes 64 lanes x 16 bytes at M0 + 16 * lane, i.e. 64
+// consecutive 16-byte positions `idx` of the tile, and the permutation is applied on the global side: the lane that
+// fills position idx fetches the piece (outer = m or n, k) that lives there.
+template <bool kRows, int kExtent> struct LfgPiece {
   static __device__ __forceinline__ int outer(int idx) {
-    return kRows ? (idx >> 3) : 8 * ((idx & 15) ^ (4 * ((idx >> 4) & 3)));
+    return kRows ? (idx >> 3) : 8 * ((idx % (kExtent / 8)) ^ (4 * ((idx / (kExtent / 8)) & 3)));
   }
   static __device__ __forceinline__ int k(int idx) {
-    return kRows ? 8 * ((idx & 7) ^ ((idx >> 4) & 7)) : (idx >> 4);
+    return kRows ? 8 * ((idx & 7) ^ ((idx >> 4) & 7)) : idx / (kExtent / 8);
   }
 };
 // Buffer resource over `bytes` bytes from `base` (raw buffer, 32-bit offsets, range checked: a load beyond the range
@@ -80,7 +93,7 @@ __device__ __forceinline__ void lfg_dma(const lfg_u32x4& rs, unsigned voff, unsi
 }
 // MFMA operand (either side: 32 rows or columns `blk`, lane % 32 picks one, lane / 32 the half of the 16-step `ks`):
 // k = 16 * ks + 8 * (lane / 32) .. + 7 in both layouts
-template <bool kRows>
+template <bool kRows, int kExtent>
 __device__ __forceinline__ lfg_u32x4 lfg_operand(const unsigned short* tile, int blk, int ks, int lane) {
   const int l32 = lane & 31, g = lane >> 5;
   if (kRows) return *reinterpret_cast<const lfg_u32x4*>(&tile[lfg_rows_at(32 * blk + l32, 2 * ks + g)]);
@@ -90,7 +103,7 @@ __device__ __forceinline__ lfg_u32x4 lfg_operand(const unsigned short* tile, int
 #pragma unroll
   for (int half = 0; half < 2; ++half) {
     const int row = 16 * ks + 8 * g + 4 * half + (j16 >> 2);
-    const unsigned short* src = &tile[lfg_cols_at(row, col >> 3) + (col & 7)];
+    const unsigned short* src = &tile[lfg_cols_at<kExtent>(row, col >> 3) + (col & 7)];
     const lfg_s16x4 t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) lfg_s16x4*)(src));
     h[half] = __builtin_bit_cast(lfg_u32x2, t);
   }
@@ -237,15 +250,23 @@ class GemmEmitter(Emitter):
             k = self.atom(a)
             batch_decode.append(f"const long long i{k} = blk % N{k}; blk /= N{k};")
         out_t = _CT[self.dtypes[out.name]]
-        src = f"""extern "C" __global__ void __launch_bounds__(256, 2) {self.name}(const LfGenParams p) {{
+        src = f"""extern "C" __global__ void __launch_bounds__(64 * LFG_WGM * LFG_WGN, 2)
+{self.name}(const LfGenParams p) {{
   {' '.join(defs)}
   constexpr bool a_rows = LFG_A_ROWS != 0, b_rows = LFG_B_ROWS != 0;
+  // the workgroup's tile: kWM x kWN waves, each kMB x kNB blocks of 32 x 32
+  constexpr int kWM = LFG_WGM, kWN = LFG_WGN, kMB = LFG_MB, kNB = LFG_NB;
+  constexpr int kBM = 32 * kWM * kMB, kBN = 32 * kWN * kNB, kWaves = kWM * kWN, kNT = 64 * kWaves;
+  constexpr int kTileA = kBM * {BK}, kTileB = kBN * {BK};                    // elements of one operand tile
+  constexpr int kPA = kBM * 8 / kNT, kPB = kBN * 8 / kNT;                   // 16-byte pieces per thread and tile
+  static_assert(kNB % 2 == 0 && kBM * 8 % kNT == 0 && kBN * 8 % kNT == 0, "tile shape");
+  static_assert(kWaves * kMB * 8192 <= 4 * (kTileA + kTileB), "the accumulators pass through the tiles' LDS");
   const bool row_stores = p.n[{g.flags_at}] != 0;
-  __shared__ __attribute__((aligned(16))) unsigned short lds[32768];        // A tiles [2][8192], B tiles [2][8192]
+  __shared__ __attribute__((aligned(16))) unsigned short lds[2 * (kTileA + kTileB)];     // A tiles [2], then B tiles [2]
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave & 1, wn = wave >> 1;                                   // the wave's 64 x 64 quarter of the tile
+  const int wm = wave % kWM, wn = wave / kWM;
   const long long M = N{km}, Nn = N{kn}, K = N{kk};
-  const long long mt = (M + {BM - 1}) / {BM}, nt = (Nn + {BN - 1}) / {BN};
+  const long long mt = (M + kBM - 1) / kBM, nt = (Nn + kBN - 1) / kBN;
   long long total = mt * nt;
   {' '.join(f'total *= N{self.atom(a)};' for a in g.batch)}
   // workgroups go to the 8 XCDs round-robin: each XCD takes a contiguous run of tiles (n fastest), so the
@@ -256,22 +277,28 @@ class GemmEmitter(Emitter):
   const long long tn = blk % nt; blk /= nt;
   const long long tm = blk % mt; blk /= mt;
   {' '.join(batch_decode)}
-  const long long m0 = tm * {BM}, n0 = tn * {BN};
+  const long long m0 = tm * kBM, n0 = tn * kBN;
   const {elem}* A = {a_base};
   const {elem}* B = {b_base};
-  // this thread's pieces of a tile: byte offset at k = 0 and how many k are left from the piece's own k (0 or less:
-  // the piece lies outside the operand and is asked for beyond the buffer's range, i.e. arrives as zeros)
+  // this thread's pieces of a tile: byte offset at k = 0 and how many k are left from the piece's own k (0: the
+  // piece lies outside the operand and is asked for beyond the buffer's range, i.e. arrives as zeros)
   const lfg_u32x4 rs_a = lfg_make_buffer(A, (unsigned)p.n[{g.flags_at + 1}]), rs_b = lfg_make_buffer(B, (unsigned)p.n[{g.flags_at + 2}]);
-  unsigned offa[4], offb[4];
-  int rooma[4], roomb[4];
+  unsigned offa[kPA], offb[kPB];
+  int rooma[kPA], roomb[kPB];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {{
-    const int idx = tid + 256 * j;
-    const long long oa = m0 + LfgPiece<a_rows>::outer(idx), ob = n0 + LfgPiece<b_rows>::outer(idx);
-    const int ka = LfgPiece<a_rows>::k(idx), kb = LfgPiece<b_rows>::k(idx);
+  for (int j = 0; j < kPA; ++j) {{
+    const int idx = tid + kNT * j;
+    const long long oa = m0 + LfgPiece<a_rows, kBM>::outer(idx);
+    const int ka = LfgPiece<a_rows, kBM>::k(idx);
     offa[j] = (unsigned)(2 * (oa * S{sam} + ka * S{sak}));
-    offb[j] = (unsigned)(2 * (ob * S{sbn} + kb * S{sbk}));
     rooma[j] = oa < M ? (int)min(K - ka, (long long)0x7fffffff) : 0;
+  }}
+#pragma unroll
+  for (int j = 0; j < kPB; ++j) {{
+    const int idx = tid + kNT * j;
+    const long long ob = n0 + LfgPiece<b_rows, kBN>::outer(idx);
+    const int kb = LfgPiece<b_rows, kBN>::k(idx);
+    offb[j] = (unsigned)(2 * (ob * S{sbn} + kb * S{sbk}));
     roomb[j] = ob < Nn ? (int)min(K - kb, (long long)0x7fffffff) : 0;
   }}
   const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) const void*)lds;
@@ -280,74 +307,84 @@ class GemmEmitter(Emitter):
   auto fetch = [&](int st, int buf) {{
     const int k0 = st * {BK};
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {{
-      const unsigned at = 16u * (unsigned)(64 * (wave + 4 * j));
-      lfg_dma(rs_a, k0 < rooma[j] ? offa[j] + (unsigned)st * stepa : 0xffffffffu, lds0 + 16384u * (unsigned)buf + at);
-      lfg_dma(rs_b, k0 < roomb[j] ? offb[j] + (unsigned)st * stepb : 0xffffffffu, lds0 + 32768u + 16384u * (unsigned)buf + at);
-    }}
+    for (int j = 0; j < kPA; ++j)
+      lfg_dma(rs_a, k0 < rooma[j] ? offa[j] + (unsigned)st * stepa : 0xffffffffu,
+              lds0 + 2u * (unsigned)(kTileA * buf) + 1024u * (unsigned)(wave + kWaves * j));
+#pragma unroll
+    for (int j = 0; j < kPB; ++j)
+      lfg_dma(rs_b, k0 < roomb[j] ? offb[j] + (unsigned)st * stepb : 0xffffffffu,
+              lds0 + 2u * (unsigned)(2 * kTileA + kTileB * buf) + 1024u * (unsigned)(wave + kWaves * j));
   }};
-  lfg_f32x16 acc[2][2];
+  lfg_f32x16 acc[kMB][kNB];
 #pragma unroll
-  for (int x = 0; x < 4; ++x)
+  for (int x = 0; x < kMB; ++x)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) acc[x / 2][x % 2][i] = 0.0f;
+    for (int y = 0; y < kNB; ++y)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[x][y][i] = 0.0f;
   fetch(0, 0);
   asm volatile("s_waitcnt vmcnt(0)\\n\\ts_barrier" ::: "memory");
   const int steps = (int)((K + {BK - 1}) / {BK});
   for (int st = 0; st < steps; ++st) {{
     const int cur = st & 1;
     if (st + 1 < steps) fetch(st + 1, cur ^ 1);
-    const unsigned short* ta = &lds[cur * 8192];
-    const unsigned short* tb = &lds[16384 + cur * 8192];
+    const unsigned short* ta = &lds[kTileA * cur];
+    const unsigned short* tb = &lds[2 * kTileA + kTileB * cur];
 #pragma unroll
     for (int ks = 0; ks < {BK // 16}; ++ks) {{
-      lfg_u32x4 fm[2], fn[2];
+      lfg_u32x4 fm[kMB], fn[kNB];
 #pragma unroll
-      for (int x = 0; x < 2; ++x) {{
-        fm[x] = lfg_operand<a_rows>(ta, 2 * wm + x, ks, lane);       // lane = m
-        fn[x] = lfg_operand<b_rows>(tb, 2 * wn + x, ks, lane);       // lane = n: the A operand of C^T = B^T A^T
-      }}
+      for (int x = 0; x < kMB; ++x) fm[x] = lfg_operand<a_rows, kBM>(ta, kMB * wm + x, ks, lane);       // lane = m
 #pragma unroll
-      for (int x = 0; x < 4; ++x)
-        acc[x / 2][x % 2] = lfg_mfma(({elem})0.0f, fn[x % 2], fm[x / 2], acc[x / 2][x % 2]);
+      for (int y = 0; y < kNB; ++y) fn[y] = lfg_operand<b_rows, kBN>(tb, kNB * wn + y, ks, lane);       // lane = n: the A operand of C^T = B^T A^T
+#pragma unroll
+      for (int x = 0; x < kMB; ++x)
+#pragma unroll
+        for (int y = 0; y < kNB; ++y) acc[x][y] = lfg_mfma(({elem})0.0f, fn[y], fm[x], acc[x][y]);
     }}
     // this wave's loads of the next tile have landed, every wave is done reading this one
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\\n\\ts_barrier" ::: "memory");
   }}
-  // acc[mb][nb][i] = C[m][n], m = 64 * wm + 32 * mb + lane % 32, n = 64 * wn + 32 * nb + 8 * (i / 4) + 4 * (lane / 32) + i % 4.
-  // Through the wave's own 16 KB of LDS ([64 m][64 n] fp32, 16-byte pieces permuted by the row): afterwards a lane
-  // holds four consecutive n of one m and 16 neighbouring lanes cover 64 consecutive n.
-  float* mine = reinterpret_cast<float*>(lds) + wave * 4096;
-  {{
-    const int l32 = lane & 31, gg = lane >> 5;
-#pragma unroll
-    for (int x = 0; x < 4; ++x)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {{
-        const int row = 32 * (x / 2) + l32, piece = 8 * (x % 2) + 2 * q + gg;
-        const lfg_f32x16& c = acc[x / 2][x % 2];
-        *reinterpret_cast<lfg_u32x4*>(&mine[row * 64 + 4 * (piece ^ (row & 15))]) =
-            __builtin_bit_cast(lfg_u32x4, lfg_f32x4{{c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]}});
-      }}
-  }}
-  __syncthreads();
+  // acc[x][y][i] = C[m][n], m = 32 * (kMB * wm + x) + lane % 32, n = 32 * (kNB * wn + y) + 8 * (i / 4) + 4 * (lane / 32) + i % 4.
+  // Two n blocks at a time through the wave's own part of LDS ([32 * kMB m][64 n] fp32, 16-byte pieces permuted by the
+  // row): afterwards a lane holds four consecutive n of one m and 16 neighbouring lanes cover 64 consecutive n.
+  float* mine = reinterpret_cast<float*>(lds) + wave * (kMB * 2048);
   auto epilogue = [&](float accv, long long i{km}, long long i{kn}) -> float {{ return {val}; }};
   auto out_at = [&](long long i{km}, long long i{kn}) -> long long {{ return {ooff}; }};
+#pragma unroll
+  for (int pass = 0; pass < kNB / 2; ++pass) {{
+    if (pass) __syncthreads();
+    {{
+      const int l32 = lane & 31, gg = lane >> 5;
+#pragma unroll
+      for (int x = 0; x < kMB; ++x)
+#pragma unroll
+        for (int y = 0; y < 2; ++y)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {{
+            const int row = 32 * x + l32, piece = 8 * y + 2 * q + gg;
+            const lfg_f32x16& c = acc[x][2 * pass + y];
+            *reinterpret_cast<lfg_u32x4*>(&mine[row * 64 + 4 * (piece ^ (row & 15))]) =
+                __builtin_bit_cast(lfg_u32x4, lfg_f32x4{{c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]}});
+          }}
+    }}
+    __syncthreads();
 #pragma unroll 4
-  for (int j = 0; j < 16; ++j) {{
-    const int row = 4 * j + (lane >> 4), piece = lane & 15;
-    const lfg_f32x4 c = __builtin_bit_cast(lfg_f32x4, *reinterpret_cast<const lfg_u32x4*>(&mine[row * 64 + 4 * (piece ^ (row & 15))]));
-    const long long m = m0 + 64 * wm + row, n = n0 + 64 * wn + 4 * piece;
-    if (m < M && n < Nn) {{
-      float r[4];
+    for (int j = 0; j < 8 * kMB; ++j) {{
+      const int row = 4 * j + (lane >> 4), piece = lane & 15;
+      const lfg_f32x4 c = __builtin_bit_cast(lfg_f32x4, *reinterpret_cast<const lfg_u32x4*>(&mine[row * 64 + 4 * (piece ^ (row & 15))]));
+      const long long m = m0 + 32 * kMB * wm + row, n = n0 + 32 * kNB * wn + 64 * pass + 4 * piece;
+      if (m < M && n < Nn) {{
+        float r[4];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) r[e] = epilogue(c[e], m, n + e < Nn ? n + e : n);
-      if (row_stores && n + 3 < Nn) {{
-        lfg_st4<{out_t}>(p.ptr[{o}], out_at(m, n), r);
-      }} else {{
+        for (int e = 0; e < 4; ++e) r[e] = epilogue(c[e], m, n + e < Nn ? n + e : n);
+        if (row_stores && n + 3 < Nn) {{
+          lfg_st4<{out_t}>(p.ptr[{o}], out_at(m, n), r);
+        }} else {{
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (n + e < Nn) lfg_st<{out_t}>(p.ptr[{o}], out_at(m, n + e), r[e]);
+          for (int e = 0; e < 4; ++e)
+            if (n + e < Nn) lfg_st<{out_t}>(p.ptr[{o}], out_at(m, n + e), r[e]);
+        }}
       }}
     }}
   }}

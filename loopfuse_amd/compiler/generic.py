@@ -81,15 +81,27 @@ class GenericProgram:
             self._loaded[dev] = [mod.kernel(k.name) for k in self.kernels]
         return self._loaded[dev]
 
-    def _gemm_kernel(self, ni: int, layouts):
+    def _gemm_kernel(self, ni: int, layouts, shape: str):
         from .. import lowering, runtime
-        key = (torch.cuda.current_device(), tuple(layouts))
+        key = (torch.cuda.current_device(), tuple(layouts), shape)
         if key not in self._gemm_loaded:
-            opts = list(lowering.COMMON_OPTS) + [f"-DLFG_A_ROWS={layouts[0]}", f"-DLFG_B_ROWS={layouts[1]}"]
+            opts = list(lowering.COMMON_OPTS) + [f"-DLFG_A_ROWS={layouts[0]}", f"-DLFG_B_ROWS={layouts[1]}"] + \
+                emit_gemm.tile_options(shape)
             code, _, _ = runtime.compile_source(self.gemm_source, "lf_generic_mfma", opts)
             mod = runtime.Module(code)
             self._gemm_loaded[key] = {i: mod.kernel(k.name) for i, (k, _) in self.gemm.items()}
         return self._gemm_loaded[key][ni]
+
+    @staticmethod
+    def _gemm_shape(info, ext: dict) -> str:
+        """256 x 256 tiles when they fill most of the CUs, else 128 x 128."""
+        import os
+        forced = os.environ.get("LOOPFUSE_GEMM_TILE")
+        if forced in emit_gemm.TILES:
+            return forced
+        bm, bn = emit_gemm.tile_extent("l")
+        tiles = -(-ext[info.m.id] // bm) * -(-ext[info.n.id] // bn) * math.prod(ext[a.id] for a in info.batch)
+        return "l" if tiles >= 192 and ext[info.m.id] >= bm and ext[info.n.id] >= bn else "s"
 
     @staticmethod
     def _gemm_layouts(info, bufs: dict, ext: dict):
@@ -103,7 +115,7 @@ class GenericProgram:
             if t.data_ptr() % 16 or any(t.stride(d) % 8 for d in batch_dims if t.shape[d] > 1):
                 return None
             s_outer, s_k = t.stride(d_outer), t.stride(d_k)
-            if s_outer < 0 or s_k < 0 or 2 * ((outer + 128) * s_outer + (K + 64) * s_k) >= 1 << 32:
+            if s_outer < 0 or s_k < 0 or 2 * ((outer + 256) * s_outer + (K + 64) * s_k) >= 1 << 32:
                 return None                  # the direct loads address a batch element's operand with 32-bit byte offsets
             if (s_k == 1 or K == 1) and K % 8 == 0 and (s_outer % 8 == 0 or outer == 1):
                 flags.append(1)
@@ -188,7 +200,8 @@ class GenericProgram:
                 except KeyError:
                     layouts = None
                 if layouts is not None and all(ext.get(a.id, 0) > 0 for a in self.gemm[ni][0].atoms):
-                    self._launch_gemm(self._gemm_kernel(ni, layouts), *self.gemm[ni], bufs, ext, args)
+                    shape = self._gemm_shape(self.gemm[ni][1], ext)
+                    self._launch_gemm(self._gemm_kernel(ni, layouts, shape), shape, *self.gemm[ni], bufs, ext, args)
                     counters["mfma"] += 1
                     info = self.gemm[ni][1]
                     self.last_mfma_flop += 2.0 * math.prod(ext[a.id] for a in [info.m, info.n, info.k] + list(info.batch))
@@ -218,7 +231,7 @@ class GenericProgram:
         return res.view(view)
 
     @staticmethod
-    def _launch_gemm(fn, k, info, bufs: dict, ext: dict, args) -> None:
+    def _launch_gemm(fn, shape: str, k, info, bufs: dict, ext: dict, args) -> None:
         prm = emit.GenParams()
         for i, b in enumerate(k.bufs):
             prm.ptr[i] = bufs[b.name].data_ptr()
@@ -238,9 +251,10 @@ class GenericProgram:
             prm.n[info.flags_at + 1 + j] = 2 * ((outer - 1) * t.stride(d_outer) + (ext[info.k.id] - 1) * t.stride(d_k) + 1)
         for i, s in enumerate(k.scalars):
             prm.f[i] = float(s.fn(args))
-        tiles = -(-ext[info.m.id] // emit_gemm.BM) * -(-ext[info.n.id] // emit_gemm.BN) * \
-            math.prod(ext[a.id] for a in info.batch)
+        bm, bn = emit_gemm.tile_extent(shape)
+        tiles = -(-ext[info.m.id] // bm) * -(-ext[info.n.id] // bn) * math.prod(ext[a.id] for a in info.batch)
         blocks = 8 * -(-tiles // 8)
         if blocks >= 1 << 31:
             raise NotLowerable("more tiles than one grid dimension holds")
-        fn.launch((blocks, 1, 1), (256, 1, 1), prm)
+        wm, wn, _, _ = emit_gemm.TILES[shape]
+        fn.launch((blocks, 1, 1), (64 * wm * wn, 1, 1), prm)

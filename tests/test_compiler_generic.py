@@ -274,7 +274,7 @@ def test_contractions_of_half_precision_operands_get_an_mfma_kernel():
     k, info = prog.gemm[0]
     assert (info.m.hint, info.n.hint, info.k.hint, [a.hint for a in info.batch]) == (96, 40, 64, [4])
     assert info.a_dims == (1, 2) and info.b_dims == (1, 2) and info.a_batch_dims == [0] and info.b_batch_dims == [0]
-    assert "v_mfma" not in k.source and "lfg_mfma" in k.source and "__launch_bounds__(256, 2)" in k.source
+    assert "v_mfma" not in k.source and "lfg_mfma" in k.source and "__launch_bounds__(64 * LFG_WGM * LFG_WGN, 2)" in k.source
     assert "accv * 0.5f" in k.source                     # the epilogue is evaluated on the accumulator
     assert prog.code.count("__global__") == 2            # plain + MFMA
     # rows of a [.., M, K] view that matmul flattened: the outer ones count as batch
@@ -289,15 +289,18 @@ def test_contractions_of_half_precision_operands_get_an_mfma_kernel():
     assert not sm.gemm
 
 
+@pytest.mark.parametrize("shape", ["s", "l"])
 @pytest.mark.parametrize("layouts", [(1, 1), (1, 0), (0, 1), (0, 0)])
-def test_mfma_kernel_compiles_for_every_operand_layout(shim_built, layouts):
-    """The generated source builds for gfx950 with hipRTC in all four layout specialisations, without scratch
-    memory and within the registers of two workgroups per CU."""
+def test_mfma_kernel_compiles_for_every_operand_layout(shim_built, layouts, shape):
+    """The generated source builds for gfx950 with hipRTC in all four layout specialisations and both tile shapes,
+    without scratch memory and within the registers of two waves per SIMD."""
     import re
     import subprocess
 
+    from loopfuse_amd.compiler import emit_gemm
+
     prog = generic.GenericProgram(_bf16_graph(lambda a, b, c: torch.tanh(a @ b + c), [(256, 128), (128, 192), (192,)]))
-    opts = list(lowering.COMMON_OPTS) + [f"-DLFG_A_ROWS={layouts[0]}", f"-DLFG_B_ROWS={layouts[1]}"]
+    opts = list(lowering.COMMON_OPTS) + [f"-DLFG_A_ROWS={layouts[0]}", f"-DLFG_B_ROWS={layouts[1]}"] + emit_gemm.tile_options(shape)
     code, _, _ = runtime.compile_source(prog.gemm_source, "lf_generic_mfma", opts)
     readelf = "/opt/rocm/llvm/bin/llvm-readelf"
     if not os.path.exists(readelf):
@@ -311,4 +314,4 @@ def test_mfma_kernel_compiles_for_every_operand_layout(shim_built, layouts):
         os.unlink(path)
     assert int(re.search(r"\.private_segment_fixed_size:\s+(\d+)", notes).group(1)) == 0
     assert int(re.search(r"\.vgpr_count:\s+(\d+)", notes).group(1)) <= 256
-    assert int(re.search(r"\.group_segment_fixed_size:\s+(\d+)", notes).group(1)) == 65536
+    assert int(re.search(r"\.group_segment_fixed_size:\s+(\d+)", notes).group(1)) == {"s": 65536, "l": 131072}[shape]

@@ -16,6 +16,13 @@ DEV = "cuda:0"
 BF, HF = torch.bfloat16, torch.float16
 
 
+@pytest.fixture(autouse=True)
+def _fixed_route(monkeypatch):
+    """The route of a call is asserted below: the measured choice between generated and captured graph stays off
+    except in the test of that choice."""
+    monkeypatch.setenv("LOOPFUSE_AUTOTUNE", "0")
+
+
 def rand(shape, dtype, seed, scale=1.0):
     g = torch.Generator().manual_seed(seed)
     return (torch.randn(shape, generator=g) * scale).to(dtype)
@@ -46,6 +53,11 @@ CASES = [
     ("long_k", (256, 4096), (4096, 256), "ab", (256, 256)),
     ("batch_broadcast_b", (3, 2, 160, 64), (64, 96), "ab", (96,)),     # B shared by every batch element; bias over n
     ("tiny", (8, 8), (8, 8), "ab", (8, 8)),
+    # enough 256 x 256 tiles to fill the CUs: the eight-wave kernel, ragged at both edges, in every layout
+    ("large_tiles", (3592, 192), (192, 3600), "ab", (3600,)),
+    ("large_tiles_bT", (3592, 136), (3601, 136), "abT", (3592, 3601)),
+    ("large_tiles_aT", (72, 3600), (72, 3592), "aTb", (3592,)),
+    ("large_tiles_aTbT", (200, 3592), (3608, 200), "aTbT", (3592, 3608)),
 ]
 
 
@@ -87,10 +99,9 @@ def test_calls_the_mfma_kernel_cannot_read_take_the_plain_kernel():
     assert generic.counters["mfma"] == before["mfma"] + 1
 
 
-def test_large_matmul_is_no_longer_left_to_the_captured_graph(monkeypatch):
+def test_large_matmul_is_no_longer_left_to_the_captured_graph():
     """2048 x 2048 x 2048 is 2^33 multiply-adds, far beyond what the plain kernels are allowed: on the MFMA path the
     backend keeps the graph (counted as a generated-kernel run), a tanh epilogue and a bias over n fused."""
-    monkeypatch.setenv("LOOPFUSE_AUTOTUNE", "0")
     fn = lambda a, b, bias: torch.tanh(a @ b.t() * 0.02 + bias)      # noqa: E731
     a, b, bias = rand((2048, 2048), BF, 1), rand((2048, 2048), BF, 2), rand((2048,), BF, 3)
     torch._dynamo.reset()
@@ -117,10 +128,11 @@ def test_two_products_in_a_row_keep_the_intermediate_and_both_run_on_mfma():
     _close(got, (a.double() @ b.double()) @ c.double(), BF)
 
 
-def test_max_autotune_measures_large_products_against_the_captured_graph():
+def test_max_autotune_measures_large_products_against_the_captured_graph(monkeypatch):
     """Under mode="max-autotune" (the default) a call with 2^32 flop or more in generated MFMA kernels is timed
     against the captured graph once; later calls of that signature take the faster route.  Either way the values
     are right and every call is accounted for."""
+    monkeypatch.setenv("LOOPFUSE_AUTOTUNE", "1")
     fn = lambda a, b, bias: a @ b.t() + bias      # noqa: E731
     a, b, bias = rand((4096, 2048), BF, 1, 0.5), rand((4096, 2048), BF, 2, 0.5), rand((4096,), BF, 3)
     ins = [t.to(DEV) for t in (a, b, bias)]
