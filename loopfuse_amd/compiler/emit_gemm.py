@@ -274,8 +274,13 @@ class GemmEmitter(Emitter):
   const long long per_xcd = (total + 7) / 8;
   long long blk = (long long)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if ((long long)(blockIdx.x >> 3) >= per_xcd || blk >= total) return;
-  const long long tn = blk % nt; blk /= nt;
-  const long long tm = blk % mt; blk /= mt;
+  // inside a batch element the tiles run in bands of kBand tile rows, column by column: the workgroups resident
+  // on an XCD at a time (32 or 64 consecutive tiles) then cover a block of the output that is a few tiles tall and
+  // wide, and read correspondingly few rows of A and columns of B past its L2
+  constexpr long long kBand = kNT <= 256 ? 8 : 4;
+  const long long t = blk % (mt * nt); blk /= mt * nt;
+  const long long first = t / (kBand * nt) * kBand, tall = min(mt - first, kBand);
+  const long long tm = first + (t % (kBand * nt)) % tall, tn = (t % (kBand * nt)) / tall;
   {' '.join(batch_decode)}
   const long long m0 = tm * kBM, n0 = tn * kBN;
   const {elem}* A = {a_base};
