@@ -169,6 +169,8 @@ class Parser:
                 continue
             if k in ("memory_format", "layout", "device", "pin_memory"):
                 continue                      # where a copy lives, not what it holds
+            if k == "approximate" and t is torch.ops.aten.gelu.default and v in ("none", "tanh"):
+                continue                      # read by the gelu handler
             raise Unsupported(f"{t}: keyword argument {k}={v!r}")
         aten = torch.ops.aten
         if t is torch.ops.prims.convert_element_type.default and len(a) > 1 and isinstance(a[1], torch.dtype) \
@@ -342,6 +344,14 @@ class Parser:
         if t is aten.tanh.default:
             v = val(a[0]).instantiate()
             return self.emit("tanh", v.dims, [], ir.Un("tanh", v.read()))
+        # ---- the activations of the layers around an attention (pointwise, one operand)
+        unary = {aten.relu.default: "relu", aten.sigmoid.default: "sigmoid", aten.silu.default: "silu",
+                 aten.neg.default: "neg", aten.reciprocal.default: "recip", aten.sqrt.default: "sqrt",
+                 aten.rsqrt.default: "rsqrt", aten.abs.default: "abs"}
+        if t in unary or t is aten.gelu.default:
+            op = unary.get(t) or ("gelu_tanh" if n.kwargs.get("approximate", "none") == "tanh" else "gelu")
+            v = val(a[0]).instantiate()
+            return self.emit(op, v.dims, [], ir.Un(op, v.read()))
         if t is torch.ops.loopfuse.causal_mask.default:
             v = val(a[0]).instantiate()
             row, col = v.dims[-2], v.dims[-1]

@@ -33,6 +33,10 @@ struct LfGenParams {{ void* ptr[{MAX_PTR}]; long long n[{MAX_N}]; float f[{MAX_F
 template <typename T> __device__ __forceinline__ float lfg_ld(const void* p, long long i) {{ return (float)reinterpret_cast<const T*>(p)[i]; }}
 template <typename T> __device__ __forceinline__ long long lfg_ldi(const void* p, long long i) {{ return (long long)reinterpret_cast<const T*>(p)[i]; }}
 template <typename T> __device__ __forceinline__ void lfg_st(void* p, long long i, float v) {{ reinterpret_cast<T*>(p)[i] = (T)v; }}
+__device__ __forceinline__ float lfg_sigmoid(float x) {{ return 1.0f / (1.0f + __expf(-x)); }}
+__device__ __forceinline__ float lfg_silu(float x) {{ return x / (1.0f + __expf(-x)); }}
+__device__ __forceinline__ float lfg_gelu(float x) {{ return 0.5f * x * (1.0f + erff(x * 0.70710678f)); }}
+__device__ __forceinline__ float lfg_gelu_tanh(float x) {{ return 0.5f * x * (1.0f + tanhf(0.79788456f * (x + 0.044715f * x * x * x))); }}
 """
 
 
@@ -132,7 +136,11 @@ class Emitter:
             return f"fmaxf({a}, {b})" if e.op == "max" else f"({a} {dict(add='+', sub='-', mul='*', div='/')[e.op]} {b})"
         if isinstance(e, ir.Un):
             a = self.expr(e.a)
-            return {"exp": f"__expf({a})", "tanh": f"tanhf({a})", "neg": f"(-{a})", "recip": f"(1.0f / {a})"}[e.op]
+            if e.op in ("sigmoid", "silu", "gelu", "gelu_tanh"):
+                return f"lfg_{e.op}({a})"
+            return {"exp": f"__expf({a})", "exp2": f"exp2f({a})", "tanh": f"tanhf({a})", "neg": f"(-{a})",
+                    "recip": f"(1.0f / {a})", "relu": f"fmaxf({a}, 0.0f)", "sqrt": f"sqrtf({a})",
+                    "rsqrt": f"(1.0f / sqrtf({a}))", "abs": f"fabsf({a})"}[e.op]
         if isinstance(e, ir.Select):
             conds = [f"({c.ci}ll * {self.index(c.row)} + {c.cj}ll * {self.index(c.col)} + {c.c0}ll <= 0)" for c in e.clauses]
             other = "(-__builtin_inff())" if e.other == float("-inf") else f"{float(e.other)!r}f"

@@ -46,8 +46,23 @@ class GenericProgram:
         self.dtypes = {b.name: emit._DT.get(getattr(torch, b.dtype, None), None) for b in p.inputs}
         if any(v is None for v in self.dtypes.values()):
             raise NotLowerable("an input dtype the emitted kernels do not read")
+        # temporaries are fp32, except one that another nest reads as a direct operand of a contraction and that
+        # the traced graph holds in bf16 / fp16: it is stored as the graph stores it (the rounding eager does), so
+        # that the contraction can take it on the MFMA path
+        operand_of_dot = set()
         for n in nests:
-            self.dtypes.setdefault(n.writes().name, 0)               # temporaries are fp32
+            for e in ir.walk(n.stmt.value):
+                if isinstance(e, ir.Dot):
+                    operand_of_dot.update(x.buf.name for x in (e.a, e.b) if isinstance(x, ir.Read))
+        self.torch_dtypes: dict = {}
+        for n in nests:
+            b = n.writes()
+            traced = getattr(getattr(b, "node", None), "meta", {}).get("val", None)
+            tdt = getattr(traced, "dtype", None)
+            if b is not p.out.buf and b.name in operand_of_dot and tdt in (torch.bfloat16, torch.float16):
+                self.dtypes.setdefault(b.name, emit._DT[tdt])
+                self.torch_dtypes[b.name] = tdt
+            self.dtypes.setdefault(b.name, 0)
         self.dtypes[p.out.buf.name] = emit._DT.get(self.out_dtype, 0)
         self.kernels = [emit.Emitter(n, self.dtypes, f"lf_gen_{i}").emit() for i, n in enumerate(nests)]
         self.source = emit.PRELUDE + "\n".join(k.source for k in self.kernels)
@@ -204,7 +219,7 @@ class GenericProgram:
                 shape = [math.prod(1 if a.hint == 1 else ext[a.id] for a in ir.leaves(d)) for d in out.dims]
             except KeyError as e:
                 raise NotLowerable("an extent could not be derived from the argument shapes") from e
-            dt = self.out_dtype if out is self.parsed.out.buf else torch.float32
+            dt = self.out_dtype if out is self.parsed.out.buf else self.torch_dtypes.get(out.name, torch.float32)
             bufs[out.name] = torch.empty(shape, dtype=dt, device=dev)
             allocs.append((len(steps), out.name, tuple(shape), dt))
             if ni in mfma:

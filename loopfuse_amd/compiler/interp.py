@@ -67,7 +67,10 @@ class Interpreter:
         if isinstance(e, ir.Un):
             a = self.value(e.a, want)
             return {"exp": torch.exp, "exp2": torch.exp2, "tanh": torch.tanh, "neg": torch.neg,
-                    "recip": torch.reciprocal}[e.op](a)
+                    "recip": torch.reciprocal, "relu": torch.relu, "sigmoid": torch.sigmoid,
+                    "silu": torch.nn.functional.silu, "gelu": torch.nn.functional.gelu,
+                    "gelu_tanh": lambda x: torch.nn.functional.gelu(x, approximate="tanh"),
+                    "sqrt": torch.sqrt, "rsqrt": torch.rsqrt, "abs": torch.abs}[e.op](a)
         if isinstance(e, ir.Dot):
             inner = want + [a for a in _axes(e.over) if a.id not in {w.id for w in want}]
             prod = self.value(e.a, inner) * self.value(e.b, inner)

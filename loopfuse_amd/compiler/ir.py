@@ -148,7 +148,7 @@ class Bin(Expr):
 
 @dataclasses.dataclass(eq=False)
 class Un(Expr):
-    op: str                          # exp tanh neg recip
+    op: str                          # exp exp2 tanh neg recip relu sigmoid silu gelu gelu_tanh sqrt rsqrt abs
     a: Expr
 
     def children(self):

@@ -100,6 +100,17 @@ CASES = {
     "modified_attn": (_modified, lambda: tuple(_r(2, 2, 16, 8, seed=s) for s in (1, 2, 3, 4)) + (_r(2, 2, 16, 16, seed=5), _r(2, 2, 16, 8, seed=6)),
                       _modified_ref, 4),
     "simplified_attn": (_simplified, lambda: tuple(_r(2, 2, 16, 8, seed=s) * 0.2 for s in (1, 2, 3)), _simplified_ref, 4),
+    # the layers around an attention: linear + activation + linear; every activation the builder knows, each written
+    # out differently for the expected value
+    "mlp_gelu": (lambda x, w1, b1, w2, b2: torch.nn.functional.linear(torch.nn.functional.gelu(torch.nn.functional.linear(x, w1, b1)), w2, b2),
+                 lambda: (_r(3, 10, 8), _r(12, 8, seed=1), _r(12, seed=2), _r(6, 12, seed=3), _r(6, seed=4)),
+                 lambda x, w1, b1, w2, b2: torch.einsum("bsh,oh->bso", (lambda h: 0.5 * h * (1 + torch.erf(h / 2 ** 0.5)))(
+                     torch.einsum("bsk,hk->bsh", x, w1) + b1), w2) + b2, 2),
+    "activations": (lambda x: torch.nn.functional.gelu(x, approximate="tanh") + torch.relu(x) * torch.sigmoid(x) -
+                    torch.nn.functional.silu(x) + torch.rsqrt(torch.abs(x) + 1.0) * torch.sqrt(torch.abs(x)) + torch.reciprocal(-x - 3.0 * torch.abs(x) - 1.0),
+                    lambda: (_r(5, 7),),
+                    lambda x: 0.5 * x * (1 + torch.tanh((2 / torch.pi) ** 0.5 * (x + 0.044715 * x ** 3))) + x.clamp(min=0) / (1 + torch.exp(-x))
+                    - x / (1 + torch.exp(-x)) + (x.abs() / (x.abs() + 1)) ** 0.5 + 1 / (-x - 3 * x.abs() - 1), 1),
 }
 
 

@@ -149,3 +149,28 @@ def test_max_autotune_measures_large_products_against_the_captured_graph(monkeyp
     assert routed["fused_generic"] + routed["tuned_captured"] == 3 and routed["fused_generic"] >= 1, routed
     assert routed["eager_runtime"] == 0 and routed["eager_graph"] == 0, routed
     assert routed["tuned_captured"] in (0, 2), routed
+
+
+@pytest.mark.parametrize("act", ["gelu_tanh", "relu", "silu"])
+def test_mlp_block_runs_both_products_on_mfma(act):
+    """linear -> activation -> linear (the layers around an attention): bias and activation are the first
+    product's epilogue, its result is stored in the graph's own dtype -- the rounding eager does -- and read by
+    the second product as an MFMA operand.  Expected: float64 with the hidden activations rounded the same way."""
+    import torch.nn.functional as F
+    fa = {"gelu_tanh": lambda h: F.gelu(h, approximate="tanh"), "relu": F.relu, "silu": F.silu}[act]
+
+    def mlp(x, w1, b1, w2, b2):
+        return F.linear(fa(F.linear(x, w1, b1)), w2, b2)
+
+    x, w1, b1 = rand((4, 300, 256), BF, 1), rand((1024, 256), BF, 2, 0.06), rand((1024,), BF, 3, 0.1)
+    w2, b2 = rand((256, 1024), BF, 4, 0.03), rand((256,), BF, 5, 0.1)
+    ins = [t.to(DEV) for t in (x, w1, b1, w2, b2)]
+    before, stats = dict(generic.counters), dict(interface.stats)
+    got = _compiled(mlp)(*ins)
+    assert interface.stats["fused_generic"] == stats["fused_generic"] + 1
+    assert generic.counters["mfma"] == before["mfma"] + 2 and generic.counters["plain"] == before["plain"]
+    h = fa(x.double() @ w1.double().t() + b1.double()).to(BF).double()
+    want = h @ w2.double().t() + b2.double()
+    assert got.dtype == BF and tuple(got.shape) == (4, 300, 256)
+    # a hidden value that falls next to a rounding boundary may round the other way: one bf16 ulp of one of 1024 terms
+    _close(got, want, BF)
