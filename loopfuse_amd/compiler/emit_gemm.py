@@ -3,20 +3,25 @@
 cases ``tests/test_accuracy.py:56-82``: ``a @ b + c`` in two and three dims).
 
 A nest ``out[batch.., m, n] = f(sum_k A[batch.., m, k] * B[batch.., k, n], other reads)`` with bf16 /
-fp16 operands becomes one kernel: a workgroup of four waves owns a 128 x 128 tile of the output (64 x 64
-per wave, four accumulators) and walks k in steps of 64; both operand tiles go global -> registers -> LDS
-(16-byte pieces, XOR-swizzled, double-buffered, one barrier per step) and come back as
+fp16 operands becomes one kernel.  A workgroup owns a tile of the output -- 128 x 128 on four waves (two
+workgroups per CU) or 256 x 256 on eight (one per CU, half the L2 -> LDS bytes per flop; ``TILES``), a
+compile-time choice -- and walks k in steps of 64.  Both operand tiles arrive by direct global -> LDS loads
+(``buffer_load_dwordx4 ... lds``: 16-byte pieces, range-checked so that the edges arrive as zeros, the XOR
+permutation applied on the global side), double-buffered, one barrier per step, and come back as
 ``v_mfma_f32_32x32x16`` operands -- by plain 16-byte reads where k is the contiguous dimension of the
 operand in memory, by transposed reads (``ds_read_b64_tr_b16``) where m / n is.  The product is formed
 transposed (C^T = B^T A^T); the fp32 accumulators then pass through LDS once so that a lane holds four
 consecutive n of one m and neighbouring lanes neighbouring n: the epilogue expression -- whatever the
 fused nest holds around the contraction -- is evaluated there per element, its reads coalesced, and the
-results leave in 8- or 16-byte stores along the rows of the output.
+results leave in 8- or 16-byte stores along the rows of the output.  Tiles are walked in bands of a few
+tile rows, an XCD taking a contiguous run of them, so that its resident workgroups share operand rows and
+columns in its L2.
 
 Which of the two layouts an operand has is a compile-time flag of the kernel (``-DLFG_A_ROWS``,
 ``-DLFG_B_ROWS``); the launcher picks the code object per call from the strides.  Calls the kernel
 cannot serve (strides that are not multiples of 8 elements, k or the contiguous extent not a multiple
-of 8, unaligned bases) take the plain one-thread-per-element kernel of the same nest.
+of 8, unaligned bases, an operand beyond the 32-bit byte offsets of the loads) take the plain
+one-thread-per-element kernel of the same nest.
 """
 from __future__ import annotations
 
