@@ -174,3 +174,48 @@ def test_mlp_block_runs_both_products_on_mfma(act):
     assert got.dtype == BF and tuple(got.shape) == (4, 300, 256)
     # a hidden value that falls next to a rounding boundary may round the other way: one bf16 ulp of one of 1024 terms
     _close(got, want, BF)
+
+
+@pytest.mark.parametrize("chunk", range(3))
+def test_random_products_on_mfma(chunk, monkeypatch):
+    """Seeded shapes, layouts, batch forms, epilogues and tile shapes: every call that satisfies the kernel's
+    alignment rules runs on MFMA and equals float64; operands are slices of larger tensors half of the time, so
+    that row strides differ from extents."""
+    import random
+
+    rng = random.Random(4000 + chunk)
+    for n in range(12):
+        dtype = rng.choice([BF, BF, HF])
+        M = rng.choice([8, 64, 100, 129, 250, 256, 300, 511, 777])
+        N = rng.choice([8, 40, 128, 136, 256, 264, 520])
+        K = rng.choice([8, 16, 64, 72, 128, 200, 1024])
+        batch = rng.choice([(), (), (2,), (3,), (2, 2)])
+        a_t, b_t = rng.random() < 0.4, rng.random() < 0.5
+        if a_t:
+            M = -(-M // 8) * 8                       # m is the contiguous dimension of A: pieces of 8
+        if not b_t:
+            N = -(-N // 8) * 8
+        pad_a, pad_b = rng.choice([0, 8, 24]), rng.choice([0, 8, 16])
+        tile = rng.choice(["s", "l", None])
+        monkeypatch.setenv("LOOPFUSE_GEMM_TILE", tile or "")
+        sa = batch + ((K, M + pad_a) if a_t else (M, K + pad_a))
+        b_batched = bool(batch) and rng.random() < 0.5
+        sb = (batch if b_batched else ()) + ((N, K + pad_b) if b_t else (K, N + pad_b))
+        a_full, b_full = rand(sa, dtype, 100 * chunk + n, 0.5).to(DEV), rand(sb, dtype, 100 * chunk + n + 50, 0.5).to(DEV)
+        a = a_full[..., :M] if a_t else a_full[..., :K]
+        b = b_full[..., :K] if b_t else b_full[..., :N]
+        bias_shape = rng.choice([(N,), (M, N), (1, N), batch + (M, N), (M, 1)])
+        bias = rand(bias_shape, dtype, 100 * chunk + n + 70).to(DEV)
+        epi = rng.choice(["affine", "tanh", "relu", "gelu"])
+        va = (lambda t: t.transpose(-1, -2)) if a_t else (lambda t: t)
+        vb = (lambda t: t.transpose(-1, -2)) if b_t else (lambda t: t)
+        act = {"affine": lambda x: x, "tanh": torch.tanh, "relu": torch.relu, "gelu": torch.nn.functional.gelu}[epi]
+        fn = lambda a, b, c: act((va(a) @ vb(b)) * 0.125 + c)      # noqa: E731
+        print(f"case {chunk}.{n}: {dtype} M{M} N{N} K{K} batch{batch} b_batched={b_batched} aT={a_t} bT={b_t} pads {pad_a},{pad_b} "
+              f"bias{bias_shape} {epi} tile={tile}", flush=True)
+        before = dict(generic.counters)
+        got = _compiled(fn)(a, b, bias)
+        assert generic.counters["mfma"] == before["mfma"] + 1 and generic.counters["plain"] == before["plain"]
+        want = act((va(a.double().cpu()) @ vb(b.double().cpu())) * 0.125 + bias.double().cpu())
+        assert tuple(got.shape) == tuple(want.shape)
+        _close(got, want, dtype)
