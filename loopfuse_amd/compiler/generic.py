@@ -25,11 +25,20 @@ MAX_SCALAR_WORK = 1 << 27
 counters = {"mfma": 0, "plain": 0}      # kernel launches by kind (tests read them)
 
 
+def _half_operand(nest: ir.Nest) -> bool:
+    """A pointwise nest without a contraction of its own whose value the traced graph holds in bf16 / fp16."""
+    val = getattr(getattr(nest.stmt.buf, "node", None), "meta", {}).get("val", None)
+    return (isinstance(nest.stmt, ir.Assign) and not nest.red and getattr(val, "dtype", None) in (torch.bfloat16, torch.float16)
+            and not any(isinstance(x, ir.Dot) for x in ir.walk(nest.stmt.value)))
+
+
 class GenericProgram:
     def __init__(self, gm: torch.fx.GraphModule):
         try:
             p = build.parse(gm)
-            nests = passes.fuse(p.nests, p.out.buf, keep_contractions=True)
+            # a half-precision tensor that only contractions read stays a tensor (stored as the graph stores it):
+            # the contraction then has two plain operands and can run on MFMA
+            nests = passes.fuse(p.nests, p.out.buf, keep_contractions=True, keep_operands=True, operand_pred=_half_operand)
         except (build.Unsupported, passes.PassError, ValueError) as e:
             raise NotLowerable(str(e)) from e
         if any(isinstance(n.stmt, ir.Rescaled) for n in nests):

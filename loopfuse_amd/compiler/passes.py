@@ -91,7 +91,8 @@ def is_operand_prep(nest: Nest) -> bool:
             and all(r.buf.kind == "input" and r.gather is None for r in ir.reads(nest.stmt.value)))
 
 
-def fuse(nests: list[Nest], keep: ir.Buffer, keep_contractions: bool = False, keep_operands: bool = False) -> list[Nest]:
+def fuse(nests: list[Nest], keep: ir.Buffer, keep_contractions: bool = False, keep_operands: bool = False,
+         operand_pred=None) -> list[Nest]:
     """Inline every temporary written by a pointwise (``Assign``) nest into its readers and drop
     its nest; reductions (``Accum``) and the result buffer stay.  Runs to a fixed point.
 
@@ -99,7 +100,10 @@ def fuse(nests: list[Nest], keep: ir.Buffer, keep_contractions: bool = False, ke
     pointwise reader (the epilogue of a matmul); where it would be recomputed per element of
     another contraction or reduction, or by several readers, it stays a temporary.  The
     attention pipeline inlines everything (its kernels keep the score tile on chip); the plain
-    one-thread-per-element kernels would repeat the contraction instead."""
+    one-thread-per-element kernels would repeat the contraction instead.
+
+    ``keep_operands``: a pointwise producer that is read only as a direct operand of contractions stays a tensor
+    of its own when ``operand_pred(producer)`` holds (default: ``is_operand_prep``)."""
     nests = list(nests)
     changed = True
     while changed:
@@ -115,7 +119,7 @@ def fuse(nests: list[Nest], keep: ir.Buffer, keep_contractions: bool = False, ke
                 u = users[0]
                 if len(users) > 1 or not isinstance(u.stmt, ir.Assign) or _under_dot(u.stmt.value, buf):
                     continue
-            if keep_operands and is_operand_prep(prod) and \
+            if keep_operands and (operand_pred or is_operand_prep)(prod) and \
                     all(_only_under_dot(u.stmt.score if isinstance(u.stmt, ir.Rescaled) else u.stmt.value, buf) for u in users):
                 continue                      # an operand of the products: stays a tensor of its own
 

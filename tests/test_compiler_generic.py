@@ -276,7 +276,7 @@ def test_contractions_of_half_precision_operands_get_an_mfma_kernel():
     """``a @ b + c`` (reference tests/test_accuracy.py:56-82) on bf16 operands: the nest is recognised as a batched
     matrix product with a pointwise epilogue -- which atoms are rows, columns, the contraction and the batch, and
     which dimension of each operand they index -- and gets a second, MFMA kernel beside the plain one.  fp32
-    operands, a gathered operand and a contraction whose operand is computed in the nest keep the plain kernel only."""
+    operands and a gathered operand keep the plain kernel only."""
     from loopfuse_amd.compiler import emit_gemm
 
     prog = generic.GenericProgram(_bf16_graph(lambda a, b, c: (a @ b.transpose(-1, -2)) * 0.5 + c,
@@ -296,8 +296,14 @@ def test_contractions_of_half_precision_operands_get_an_mfma_kernel():
     # not served: fp32 operands; softmax(x) @ y (an operand computed in the nest)
     with_fp32 = generic.GenericProgram(_aten_graph(lambda a, b, c: a @ b + c, (_r(16, 8), _r(8, 12, seed=1), _r(16, 12, seed=2)))[0])
     assert not with_fp32.gemm
+    # softmax(x) @ y (reference tests/test_accuracy.py:197-211) in bf16: the probabilities stay a bf16 tensor of their
+    # own (the rounding eager does) instead of being recomputed inside the contraction, which then runs on MFMA;
+    # in fp32 they are inlined as before and the plain kernels serve the graph
     sm = generic.GenericProgram(_bf16_graph(lambda x, y: torch.softmax(x, dim=-1) @ y, [(2, 64, 32), (2, 32, 48)]))
-    assert not sm.gemm
+    assert [type(n.stmt).__name__ for n in sm.nests] == ["Accum", "Accum", "Assign", "Assign"] and list(sm.gemm) == [3]
+    assert list(sm.torch_dtypes.values()) == [torch.bfloat16]
+    sm32 = generic.GenericProgram(_aten_graph(lambda x, y: torch.softmax(x, dim=-1) @ y, (_r(2, 16, 8), _r(2, 8, 12, seed=1)))[0])
+    assert len(sm32.nests) == 3 and not sm32.gemm
 
 
 @pytest.mark.parametrize("shape", ["s", "l"])

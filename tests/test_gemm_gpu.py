@@ -219,3 +219,16 @@ def test_random_products_on_mfma(chunk, monkeypatch):
         want = act((va(a.double().cpu()) @ vb(b.double().cpu())) * 0.125 + bias.double().cpu())
         assert tuple(got.shape) == tuple(want.shape)
         _close(got, want, dtype)
+
+
+def test_softmax_times_matrix_at_the_reference_size():
+    """``softmax(x) @ y`` with x [4, 8, 1024, 64], y [4, 8, 64, 1024] in bf16 (reference tests/test_accuracy.py:197-211,
+    its own size): 2^31 multiply-adds, which the plain kernels are not allowed.  The row maxima and sums are plain
+    reductions, the probabilities a bf16 tensor, the product an MFMA launch."""
+    x, y = rand((4, 8, 1024, 64), BF, 1), rand((4, 8, 64, 1024), BF, 2)
+    before, stats = dict(generic.counters), dict(interface.stats)
+    got = _compiled(lambda x, y: torch.softmax(x, dim=-1) @ y)(x.to(DEV), y.to(DEV))
+    assert interface.stats["fused_generic"] == stats["fused_generic"] + 1 and interface.stats["eager_runtime"] == stats["eager_runtime"]
+    assert generic.counters["mfma"] == before["mfma"] + 1 and generic.counters["plain"] == before["plain"] + 3
+    p = torch.softmax(x.double(), dim=-1).to(BF).double()
+    _close(got, p @ y.double(), BF)
