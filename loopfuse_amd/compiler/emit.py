@@ -57,6 +57,7 @@ class Kernel:
     strides: list                   # (buffer, dim) pairs whose element strides follow in n[]
     scalars: list                   # ir.Scalar nodes filling f[]
     par: list                       # parallel leaf atoms (thread index, outer to inner)
+    lanes_per_output: int = 1       # 64: one wave per output element (a reduction shared by its lanes)
 
 
 class Emitter:
@@ -161,7 +162,10 @@ class Emitter:
             return v
         raise NotLowerable(f"expression {type(e).__name__}")
 
-    def emit(self) -> Kernel:
+    def emit(self, wave_reduce: bool = False) -> Kernel:
+        """``wave_reduce``: a reduction nest as one wave per output element -- the 64 lanes stride over the reduced
+        index space (innermost reduced atom fastest, so rows that are contiguous in memory are read coalesced) and
+        combine through ``ds_bpermute`` -- instead of one thread walking it alone.  GPU only."""
         n = self.nest
         s = n.stmt
         if isinstance(s, ir.Rescaled):
@@ -171,7 +175,28 @@ class Emitter:
         for a in par:
             self.atom(a)
         body: list = []
-        if isinstance(s, ir.Assign):
+        if wave_reduce:
+            if not isinstance(s, ir.Accum) or not red:
+                raise NotLowerable("not a reduction")
+            init = "(-__builtin_inff())" if s.init == float("-inf") else f"{float(s.init)!r}f"
+            comb = (lambda a, b: f"fmaxf({a}, {b})") if s.op == "max" else (lambda a, b: f"{a} + {b}")
+            ks = [self.atom(a) for a in red]
+            self.lines.append(f"float result = {init};")
+            self.lines.append(f"const long long R = {' * '.join(f'N{k}' for k in ks)};")
+            self.lines.append("for (long long r = lane; r < R; r += 64) {")
+            self.lines.append("long long rr = r;")
+            for k in reversed(ks):
+                self.lines.append(f"const long long i{k} = rr % N{k}; rr /= N{k};")
+            val = self.expr(s.value)
+            self.lines.append(f"result = {comb('result', val)};")
+            self.lines.append("}")
+            self.lines.append("#pragma unroll")
+            self.lines.append("for (int off = 32; off > 0; off >>= 1) {")
+            self.lines.append("const float other = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ off) << 2, __builtin_bit_cast(int, result)));")
+            self.lines.append(f"result = {comb('result', 'other')};")
+            self.lines.append("}")
+            body = self.lines
+        elif isinstance(s, ir.Assign):
             val = self.expr(s.value)
             body = self.lines + [f"const float result = {val};"]
         else:
@@ -188,7 +213,10 @@ class Emitter:
         o = self.buf(out)
         ooff = self.offset(out, out.dims, None)
         # thread -> parallel atoms (inner atom fastest)
-        dec = ["long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;"]
+        if wave_reduce:
+            dec = ["long long t = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);", "const int lane = threadIdx.x & 63;"]
+        else:
+            dec = ["long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;"]
         total = " * ".join(f"N{self.atom(a)}" for a in par) or "1"
         dec.append(f"if (t >= {total}) return;")
         for a in reversed(par):
@@ -201,5 +229,5 @@ class Emitter:
                [f"const long long S{k} = p.n[{na + k}];" for k in range(len(self.strides))]
         src = (f'extern "C" __global__ void __launch_bounds__(256) {self.name}(const LfGenParams p) {{\n  ' +
                "\n  ".join(defs + dec + body) +
-               f"\n  lfg_st<{_CT[self.dtypes[out.name]]}>(p.ptr[{o}], {ooff}, result);\n}}\n")
-        return Kernel(self.name, src, self.bufs, self.atoms, self.strides, self.scalars, par)
+               f"\n  {'if (lane == 0) ' if wave_reduce else ''}lfg_st<{_CT[self.dtypes[out.name]]}>(p.ptr[{o}], {ooff}, result);\n}}\n")
+        return Kernel(self.name, src, self.bufs, self.atoms, self.strides, self.scalars, par, 64 if wave_reduce else 1)

@@ -22,7 +22,8 @@ from .emit import NotLowerable
 # the graph is left to the captured ATen ops.
 MAX_SCALAR_WORK = 1 << 27
 
-counters = {"mfma": 0, "plain": 0}      # kernel launches by kind (tests read them)
+counters = {"mfma": 0, "plain": 0, "wave": 0}      # kernel launches by kind (tests read them; "wave" launches count as "plain" too)
+WAVE_REDUCE_MIN = 128       # reduced elements per output from which a reduction takes the one-wave-per-output kernel
 
 
 def _half_operand(nest: ir.Nest) -> bool:
@@ -75,6 +76,15 @@ class GenericProgram:
         self.dtypes[p.out.buf.name] = emit._DT.get(self.out_dtype, 0)
         self.kernels = [emit.Emitter(n, self.dtypes, f"lf_gen_{i}").emit() for i, n in enumerate(nests)]
         self.source = emit.PRELUDE + "\n".join(k.source for k in self.kernels)
+        # reductions also get a one-wave-per-output form (GPU only), taken when the reduced extent is long
+        self.wave: dict = {}
+        for i, n in enumerate(nests):
+            if isinstance(n.stmt, ir.Accum) and [a for a in ir.leaves(n.red) if a.hint != 1]:
+                try:
+                    self.wave[i] = emit.Emitter(n, self.dtypes, f"lf_gen_{i}_wave").emit(wave_reduce=True)
+                except NotLowerable:
+                    pass
+        self.gpu_source = self.source + "\n".join(k.source for k in self.wave.values())
         # contractions of bf16 / fp16 operands also get an MFMA kernel with the nest's epilogue fused; the plain
         # kernel of the same nest serves the calls whose strides or extents it cannot take
         self.gemm: dict = {}
@@ -95,15 +105,15 @@ class GenericProgram:
 
     @property
     def code(self) -> str:
-        return self.source + (self.gemm_source if self.gemm else "")
+        return self.gpu_source + (self.gemm_source if self.gemm else "")
 
     def _module(self):
         from .. import lowering, runtime
         dev = torch.cuda.current_device()
         if dev not in self._loaded:
-            code, _, _ = runtime.compile_source(self.source, "lf_generic", list(lowering.COMMON_OPTS))
+            code, _, _ = runtime.compile_source(self.gpu_source, "lf_generic", list(lowering.COMMON_OPTS))
             mod = runtime.Module(code)
-            self._loaded[dev] = [mod.kernel(k.name) for k in self.kernels]
+            self._loaded[dev] = ([mod.kernel(k.name) for k in self.kernels], {i: mod.kernel(k.name) for i, k in self.wave.items()})
         return self._loaded[dev]
 
     def _gemm_kernel(self, ni: int, layouts, shape: str):
@@ -208,12 +218,12 @@ class GenericProgram:
             plan = self._plans.get(key)
             if plan is not None:
                 return self._replay(plan, args, dev)
-            kernels = self._module()
+            kernels, wave_fns = self._module()
             launchers = [lambda blocks, prm, fn=fn: (fn.launch((blocks, 1, 1), (256, 1, 1), prm),
                                                      steps.append((fn, blocks, 256, prm)))[0] for fn in kernels]
             mfma = self.gemm
         else:
-            mfma = {}
+            mfma, wave_fns = {}, {}
         self.last_mfma_flop = 0.0
         n_mfma = n_plain = 0
         allocs: list = []                  # (steps before it, buffer name, shape, dtype)
@@ -245,6 +255,13 @@ class GenericProgram:
                     info = self.gemm[ni][1]
                     self.last_mfma_flop += 2.0 * math.prod(ext[a.id] for a in [info.m, info.n, info.k] + list(info.batch))
                     continue
+            if ni in wave_fns:
+                # a long reduction: one wave per output element (the plain kernel's thread would walk it alone)
+                wk = self.wave[ni]
+                reduced = math.prod(ext[a.id] for a in ir.leaves(nest.red) if a.hint != 1)
+                if reduced >= WAVE_REDUCE_MIN:
+                    k, fn = wk, (lambda blocks, prm, f=wave_fns[ni]: (f.launch((blocks, 1, 1), (256, 1, 1), prm),
+                                                                     steps.append((f, blocks, 256, prm)))[0])
             prm = emit.GenParams()
             for i, b in enumerate(k.bufs):
                 prm.ptr[i] = bufs[b.name].data_ptr()
@@ -257,16 +274,18 @@ class GenericProgram:
             total = math.prod(ext[a.id] for a in k.par)
             inner = math.prod(ext[a.id] for a in k.atoms if not any(a is x for x in k.par))
             if inner > 1:
-                work += total * inner
+                work += total * inner // k.lanes_per_output
             if work > MAX_SCALAR_WORK:
                 raise NotLowerable("more scalar work than the plain kernels are meant for")
             if total:
-                if (total + 255) // 256 >= 1 << 31:
+                per_block = 256 // k.lanes_per_output
+                if (total + per_block - 1) // per_block >= 1 << 31:
                     raise NotLowerable("more output elements than one grid dimension holds")
-                fn((total + 255) // 256, prm)
+                fn((total + per_block - 1) // per_block, prm)
                 if key is not None:
                     steps[-1] = steps[-1] + ([b.name for b in k.bufs],)
                 counters["plain"] += 1
+                counters["wave"] += int(k.lanes_per_output == 64)
                 n_plain += 1
         res = bufs[self.parsed.out.buf.name]
         view = [math.prod(1 if a.hint == 1 else ext[a.id] for a in ir.leaves(d)) for d in self.parsed.out.dims]

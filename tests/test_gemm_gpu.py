@@ -232,3 +232,49 @@ def test_softmax_times_matrix_at_the_reference_size():
     assert generic.counters["mfma"] == before["mfma"] + 1 and generic.counters["plain"] == before["plain"] + 3
     p = torch.softmax(x.double(), dim=-1).to(BF).double()
     _close(got, p @ y.double(), BF)
+
+
+def test_long_reductions_take_one_wave_per_output():
+    """A reduction over 128 or more elements per output runs one wave per output element (lanes stride over the
+    reduced index space, combine through ds_bpermute); shorter ones keep one thread per output.  Sums, maxima, a
+    reduction over two merged dims and one whose reduced dim is not the contiguous one."""
+    x = rand((3, 5, 700), torch.float32, 1)
+    y = rand((3, 5, 700), torch.float32, 2)
+    cases = [
+        ("sum", lambda a, b: (a * b).sum(-1), 1),
+        ("max", lambda a, b: (a + b).max(-1).values, 1),
+        ("two dims", lambda a, b: (a - b).sum(dim=(1, 2)), 1),
+        ("strided", lambda a, b: (a * 2.0 + b).sum(dim=0), 0),                    # 3 elements per output: plain kernel
+        ("through a transposed view", lambda a, b: torch.exp(a * 0.1).transpose(1, 2).sum(dim=1), 1),   # the 700-long dim again
+        ("long and strided", lambda a, b: (a.permute(2, 0, 1) * 0.5 - b.permute(2, 0, 1)).sum(dim=0), 1),  # the long dim, reduced through permuted views
+        ("short middle dim", lambda a, b: (a + b).sum(dim=1), 0),                    # 5 per output: plain
+        ("softmax by hand", lambda a, b: torch.exp(a - a.max(-1, keepdim=True).values)
+         / torch.exp(a - a.max(-1, keepdim=True).values).sum(-1, keepdim=True) + b, 3),      # the maximum is written twice
+    ]
+    for name, fn, n_wave in cases:
+        before = dict(generic.counters)
+        got = _compiled(fn)(x.to(DEV), y.to(DEV))
+        want = fn(x.double(), y.double())
+        assert generic.counters["wave"] == before["wave"] + n_wave, name
+        torch.testing.assert_close(got.double().cpu(), want, rtol=1e-5, atol=1e-4)
+
+
+def test_simplified_attention_at_the_reference_size():
+    """(Q K^T / (max + sum + 1e-3)) V, no exponential (reference tests/test_accuracy.py:314-333, B4 H8 S1024 D64,
+    bf16): both products on MFMA, the two row reductions over 1024 scores one wave per row, the quotient a bf16
+    tensor.  The reference checks this case at rtol 1e-2."""
+    def fn(Q, K, V):
+        QK = Q @ K.transpose(-2, -1)
+        m = torch.max(QK, dim=-1, keepdim=True)[0] + torch.sum(QK, dim=-1, keepdim=True)
+        return (QK / (m + 1e-3)) @ V
+
+    Q, K, V = (rand((4, 8, 1024, 64), BF, s, 0.2) for s in (1, 2, 3))
+    before, stats = dict(generic.counters), dict(interface.stats)
+    got = _compiled(fn)(Q.to(DEV), K.to(DEV), V.to(DEV))
+    assert interface.stats["fused_generic"] == stats["fused_generic"] + 1 and interface.stats["eager_runtime"] == stats["eager_runtime"]
+    assert generic.counters["mfma"] == before["mfma"] + 2 and generic.counters["wave"] == before["wave"] + 2
+    s = torch.einsum("bhid,bhjd->bhij", Q.double(), K.double())
+    den = s.amax(dim=-1) + s.sum(dim=-1) + 1e-3
+    want = torch.einsum("bhij,bhjd->bhid", (s / den[..., None]).to(BF).double(), V.double())
+    err = (got.double().cpu() - want).abs()
+    assert (err <= 1e-2 * want.abs() + 1e-2 * want.abs().max()).all(), err.max().item()
